@@ -1,0 +1,215 @@
+"""Python mirror of the reference's native module ``dhellam._Clib``.
+
+The reference exports six functions from a pybind11 torch extension
+(csrc/torchapi.cpp:2-9, signatures csrc/operators/ops.h:18-81).  The same names
+with the same positional arguments and return conventions are provided here as
+thin shims over the C ABI of ``libdhellam_hip.so``; tensors are only carriers
+of device pointers.  Functions the reference does not have (RMSNorm, RoPE,
+merge, MoE, grouped GEMM) are exported under ``py*`` names in the same style.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+__all__ = ["add_tensors", "pygemm", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge"]
+
+
+def _timed(profiling: bool, stream, fn):
+    """Run fn(); with ``profiling`` bracket it with events on ``stream`` and return ms
+    (the reference brackets with cudaEvent and synchronises only when profiling,
+    csrc/operators/gemm.cu:101-131)."""
+    if not profiling:
+        fn()
+        return 0.0
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    fn()
+    end.record(stream)
+    end.synchronize()
+    return float(start.elapsed_time(end))
+
+
+def add_tensors(a, b):
+    """ops.h:67-69."""
+    return a + b
+
+
+def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, transb, grad_accumulate, math_sm_count,
+           profiling):
+    """csrc/operators/gemm.cu:3-170.  Column-major cuBLASLt convention of the reference:
+    with row-major tensors A [m?,k?], B, the result is D = op(B) @ op(A) written into
+    ``outputD`` (accumulated when ``grad_accumulate``), i.e.
+
+        transa  transb   D
+        True    False    B   @ A.T     ("TN": input @ weight.T)
+        False   False    B   @ A       ("NN": dgrad)
+        False   True     B.T @ A       ("NT": wgrad)
+
+    Dense GEMM is a library call on this path (hipBLASLt through torch.matmul);
+    ``input_workspace`` / ``workspaceSize`` / ``math_sm_count`` are accepted and unused.
+    """
+    _lib.need_cuda(inputA, inputB, outputD)
+    a = inputA.t() if transa else inputA
+    b = inputB.t() if transb else inputB
+    stream = torch.cuda.current_stream()
+
+    def run():
+        if grad_accumulate:
+            outputD.addmm_(b, a)
+        else:
+            torch.matmul(b, a, out=outputD)
+
+    return _timed(profiling, stream, run)
+
+
+def pygelu(input, output, profiling):
+    """csrc/operators/gelu.cu:17-43 (tanh-approximation GELU into ``output``)."""
+    _lib.need_cuda(input, output)
+    assert input.is_contiguous() and output.is_contiguous() and input.numel() == output.numel()
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    return _timed(profiling, stream, lambda: _lib.check(
+        lib.dh_gelu(input.data_ptr(), output.data_ptr(), input.numel(), _lib.dt(input), stream.cuda_stream)))
+
+
+def pybda(input, bias, residual, output, prob, profiling):
+    """csrc/operators/bda.cu:18-62: output = mask * (input + bias) + residual.  Only
+    prob = 0 (mask of ones) is implemented; the reference draws its mask with
+    torch::dropout."""
+    if prob != 0.0:
+        raise RuntimeError("pybda: only prob = 0 is implemented")
+    _lib.need_cuda(input, bias, residual, output)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    return _timed(profiling, stream, lambda: _lib.check(
+        lib.dh_bias_mask_add(input.data_ptr(), bias.data_ptr(), residual.data_ptr(), None, output.data_ptr(),
+                             input.numel(), _lib.dt(input), stream.cuda_stream)))
+
+
+# ---------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------
+def _tok_stride(t: torch.Tensor) -> int:
+    if not (t.dim() == 3 and t.stride(2) == 1 and t.stride(1) == t.shape[2]):
+        raise RuntimeError("attention tensors must be [tokens, heads, d] with contiguous (heads, d)")
+    return t.stride(0)
+
+
+def _attn_fwd_raw(q, k, v, out, lse, cu_q, cu_k, max_q, max_k, scale, causal, stream_ptr):
+    lib = _lib.load()
+    _lib.check(lib.dh_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                               cu_q.data_ptr(), cu_k.data_ptr(), cu_q.numel() - 1, int(max_q), int(max_k),
+                               q.shape[1], k.shape[1], q.shape[2], _tok_stride(q), _tok_stride(k), _tok_stride(v),
+                               _tok_stride(out), float(scale), int(bool(causal)), _lib.dt(q), stream_ptr))
+
+
+def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+                     is_causal, return_softmax, math_sm_count, profiling):
+    """ops.h:18-32 / flash_atten.cu:436-477.  Runs on the current stream.
+
+    Returns [out, q, k, v, out, softmax_lse, p, rng_state] (+ a CPU fp32 [1] tensor of
+    milliseconds when ``profiling``), positions as in flash_atten.cu:429-433.  The
+    reference pads the head dim to a multiple of 8 and returns the padded tensors; the
+    supported head dims need no padding, so the inputs themselves are returned.
+    ``p`` is an empty tensor (return_softmax is only meaningful with dropout) and
+    ``rng_state`` is a zero int64[2].  Dropout is not implemented: p_dropout must be 0.
+    """
+    if p_dropout != 0.0:
+        raise RuntimeError("pymha_varlen_fwd: dropout is not implemented (p_dropout must be 0)")
+    if return_softmax:
+        raise RuntimeError("pymha_varlen_fwd: return_softmax is only supported with dropout in the reference")
+    _lib.need_cuda(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    if cu_seqlens_q.dtype != torch.int32 or cu_seqlens_k.dtype != torch.int32:
+        raise RuntimeError("cu_seqlens must be int32")
+    stream = torch.cuda.current_stream()
+    b = cu_seqlens_q.numel() - 1
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
+    ms = _timed(profiling, stream, lambda: _attn_fwd_raw(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k,
+                                                        max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
+                                                        stream.cuda_stream))
+    p = torch.empty(0, dtype=q.dtype, device=q.device)
+    rng_state = torch.zeros(2, dtype=torch.int64, device=q.device)
+    res = [out, q, k, v, out, lse, p, rng_state]
+    if profiling:
+        res.append(torch.tensor([ms], dtype=torch.float32))
+    return res
+
+
+_bwd_ws: dict = {}
+
+
+def _attn_bwd_workspace(nbytes: int, device, stream_ptr: int) -> torch.Tensor:
+    key = (str(device), stream_ptr)
+    ws = _bwd_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _bwd_ws[key] = ws
+    return ws
+
+
+def _attn_bwd_raw(dout, q, k, v, out, lse, dq, dk, dv, delta, cu_q, cu_k, max_q, max_k, scale, causal, stream_ptr):
+    lib = _lib.load()
+    b = cu_q.numel() - 1
+    nbytes = lib.dh_attn_bwd_workspace_bytes(q.shape[0], k.shape[0], b, int(max_q), q.shape[1], k.shape[1],
+                                             q.shape[2], _lib.dt(q))
+    ws = _attn_bwd_workspace(nbytes, q.device, stream_ptr)
+    _lib.check(lib.dh_attn_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                               lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.ptr(delta),
+                               ws.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(), b, int(max_q), int(max_k),
+                               q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2], _tok_stride(q),
+                               _tok_stride(k), _tok_stride(v), _tok_stride(out), _tok_stride(dout),
+                               _tok_stride(dq), _tok_stride(dk), _tok_stride(dv), float(scale), int(bool(causal)),
+                               _lib.dt(q), stream_ptr))
+
+
+def pymha_varlen_bwd(dout, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                     p_dropout, softmax_scale, is_causal, rng_state, deterministic, math_sm_count, profiling,
+                     stream_ptr):
+    """ops.h:34-52 / flash_atten.cu:760-813.  Unlike the forward it launches on the raw
+    stream handle ``stream_ptr`` (flash_atten.cu:784).  Returns [dq, dk, dv, softmax_d]
+    (+ CPU ms tensor when profiling).  The result is deterministic regardless of
+    ``deterministic`` (no floating-point atomics are used)."""
+    if p_dropout != 0.0:
+        raise RuntimeError("pymha_varlen_bwd: dropout is not implemented (p_dropout must be 0)")
+    _lib.need_cuda(dout, q, k, v, out, softmax_lse)
+    b = cu_seqlens_q.numel() - 1
+    ext = torch.cuda.ExternalStream(stream_ptr) if stream_ptr else torch.cuda.default_stream()
+    with torch.cuda.stream(ext):
+        dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+        dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+        softmax_d = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
+        ms = _timed(profiling, ext, lambda: _attn_bwd_raw(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d,
+                                                          cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                                          softmax_scale, is_causal, int(stream_ptr or 0)))
+    res = [dq, dk, dv, softmax_d]
+    if profiling:
+        res.append(torch.tensor([ms], dtype=torch.float32))
+    return res
+
+
+def pyattn_merge(outs, lses, row_begin, rows, out, lse):
+    """Fused merge of ring-attention partial results (dhellam/operators/ring_attn.py:26-40
+    applied as in :146-195) on the current stream.  outs[s] [b*rows[s], hq, d], lses[s]
+    fp32 [b, hq, rows[s]]; out [b*sq, hq, d]; lse fp32 [b, hq, sq]."""
+    lib = _lib.load()
+    n = len(outs)
+    b, hq, sq = lse.shape
+    d = out.shape[-1]
+    po = (C.c_void_p * n)(*[o.data_ptr() for o in outs])
+    pl = (C.c_void_p * n)(*[l.data_ptr() for l in lses])
+    rb = (C.c_int32 * n)(*[int(x) for x in row_begin])
+    rr = (C.c_int32 * n)(*[int(x) for x in rows])
+    for s in range(n):
+        assert outs[s].is_contiguous() and lses[s].is_contiguous() and lses[s].dtype == torch.float32
+        assert outs[s].shape == (b * rows[s], hq, d) and lses[s].shape == (b, hq, rows[s])
+    assert out.is_contiguous() and lse.is_contiguous()
+    _lib.check(lib.dh_attn_merge(C.cast(po, C.c_void_p), C.cast(pl, C.c_void_p), C.cast(rb, C.c_void_p),
+                                 C.cast(rr, C.c_void_p), n, out.data_ptr(), lse.data_ptr(), b, sq, hq, d,
+                                 _lib.dt(out), torch.cuda.current_stream().cuda_stream))

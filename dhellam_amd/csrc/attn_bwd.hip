@@ -1,0 +1,597 @@
+// Flash-attention backward on bf16/fp16 MFMA (gfx950), deterministic (no
+// floating-point atomics).
+//
+// Three kernels:
+//   delta   : delta_i = sum_d dO[i,d] * O[i,d]                      (streaming)
+//   dK/dV   : a workgroup owns 32*NW key/value rows (K, V fragments stay in
+//             registers), walks the query heads of its GQA group and the query
+//             tiles that attend to it; S = Q K^T and dP = dO V^T are computed
+//             with the key index on lanes so that P and dS feed dV^T += dO^T P
+//             and dK^T += Q^T dS straight from their accumulators, with the
+//             transposed Q / dO fragments coming from LDS transpose reads.
+//             The GQA group sum happens in the accumulators; when the grid
+//             would be too small the group is split over workgroups and a small
+//             kernel adds the fp32 partials in a fixed order.
+//   dQ      : a workgroup owns 32*NW query rows (Q, dO fragments in registers),
+//             walks the key tiles; S^T, dP^T have the query index on lanes and
+//             dS^T feeds dQ^T += K^T dS^T.
+// Recomputing S and dP in both passes costs 7 matrix products instead of 5 but
+// needs no fp32 dQ accumulator in memory and no atomics.
+#include "mma.h"
+
+namespace dh {
+
+struct AttnBwdParams {
+  const void *dout, *q, *k, *v;
+  const float *lse, *delta;
+  void *dq, *dk, *dv;
+  float *dk_part, *dv_part;  // fp32 [hsplit][total_k][hk][d] when hsplit > 1
+  const int32_t *cu_q, *cu_k;
+  int max_sq, hq, hk, hsplit;
+  int64_t total_k;
+  int64_t q_stride, k_stride, v_stride, do_stride, dq_stride, dk_stride, dv_stride;
+  float scale, scale_log2;
+  int causal;
+};
+
+// ---- delta = rowsum(dO * O) ---------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *__restrict__ delta,
+                  const int32_t *__restrict__ cu_q, int max_sq, int hq, int d, int lanes_per, int64_t do_stride,
+                  int64_t o_stride) {
+  constexpr int N = Vec<T>::N;
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], sq = cu_q[b + 1] - q0;
+  const int per_block = 256 / lanes_per;
+  const int sub = threadIdx.x / lanes_per, ln = threadIdx.x % lanes_per;
+  const int nvec = d / N;
+  for (int64_t item = (int64_t)blockIdx.x * per_block + sub; item < (int64_t)sq * hq;
+       item += (int64_t)gridDim.x * per_block) {
+    const int i = (int)(item / hq), h = (int)(item % hq);
+    float s = 0.f;
+    for (int c = ln; c < nvec; c += lanes_per) {
+      const Vec<T> a = ldg(dout + (int64_t)(q0 + i) * do_stride + (int64_t)h * d + c * N);
+      const Vec<T> o = ldg(out + (int64_t)(q0 + i) * o_stride + (int64_t)h * d + c * N);
+#pragma unroll
+      for (int j = 0; j < N; ++j) s += to_f(a.v[j]) * to_f(o.v[j]);
+    }
+    for (int o = lanes_per >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if (ln == 0) delta[((int64_t)b * hq + h) * max_sq + i] = s;
+  }
+}
+
+// ---- dK, dV ---------------------------------------------------------------------------------
+template <typename T, int D, int NW>
+__global__ void __launch_bounds__(64 * NW) attn_bwd_dkv_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int BN = 32 * NW, BM = 32, NT = 64 * NW;
+  constexpr int QS = D + 16;  // row stride of the Q / dO tiles (row reads and transpose reads)
+  constexpr int VPR = D / 8;
+  constexpr int LPT = BM * VPR / NT;
+  static_assert(BM * VPR % NT == 0, "tile must divide over the block");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *sQ = reinterpret_cast<T *>(smem_raw);        // [2][BM*QS]
+  T *sdO = sQ + 2 * BM * QS;                      // [2][BM*QS]
+  float *sLse = reinterpret_cast<float *>(sdO + 2 * BM * QS);  // [2][BM]  (lse * log2e, +inf for rows >= sq)
+  float *sDel = sLse + 2 * BM;                                 // [2][BM]
+
+  const int b = blockIdx.z;
+  const int hkv = blockIdx.y / p.hsplit, hs = blockIdx.y % p.hsplit;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int j0 = blockIdx.x * BN;  // causal: low tiles carry the most work and come first
+  if (j0 >= sk) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int jw0 = j0 + 32 * w;
+  const int jrow = jw0 + c;
+  const int ratio = p.hq / p.hk;
+  const int hper = ratio / p.hsplit;
+
+  Frag Kf[D / 16], Vf[D / 16];
+  {
+    const int jl = jrow < sk ? jrow : sk - 1;
+    const T *kp = reinterpret_cast<const T *>(p.k) + (int64_t)(k0 + jl) * p.k_stride + (int64_t)hkv * D;
+    const T *vp = reinterpret_cast<const T *>(p.v) + (int64_t)(k0 + jl) * p.v_stride + (int64_t)hkv * D;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      Kf[ks] = frag_ld<T>(kp + ks * 16 + 8 * hh);
+      Vf[ks] = frag_ld<T>(vp + ks * 16 + 8 * hh);
+    }
+  }
+  floatx16 dKt[D / 32], dVt[D / 32];
+#pragma unroll
+  for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      dKt[t][v] = 0.f;
+      dVt[t][v] = 0.f;
+    }
+
+  const int i_begin = p.causal ? (j0 / BM) * BM : 0;
+  const int ntq = i_begin < sq ? (sq - i_begin + BM - 1) / BM : 0;
+  const int nsteps = ntq * hper;
+
+  uint4 rq[LPT], rdo[LPT];
+  float rl = 0.f, rd = 0.f;
+  auto gload = [&](int step) {
+    const int g = step / ntq, ti = step % ntq;
+    const int h = hkv * ratio + hs * hper + g;
+    const int i0 = i_begin + ti * BM;
+    const T *qg = reinterpret_cast<const T *>(p.q) + (int64_t)q0 * p.q_stride + (int64_t)h * D;
+    const T *dg = reinterpret_cast<const T *>(p.dout) + (int64_t)q0 * p.do_stride + (int64_t)h * D;
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / VPR, cv = idx % VPR;
+      const int ir = i0 + r;
+      if (ir < sq) {
+        rq[i] = *reinterpret_cast<const uint4 *>(qg + (int64_t)ir * p.q_stride + cv * 8);
+        rdo[i] = *reinterpret_cast<const uint4 *>(dg + (int64_t)ir * p.do_stride + cv * 8);
+      } else {
+        rq[i] = make_uint4(0, 0, 0, 0);
+        rdo[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    if (tid < BM) {
+      const int ir = i0 + tid;
+      if (ir < sq) {
+        rl = p.lse[((int64_t)b * p.hq + h) * p.max_sq + ir] * 1.4426950408889634f;
+        rd = p.delta[((int64_t)b * p.hq + h) * p.max_sq + ir];
+      } else {
+        rl = INFINITY;
+        rd = 0.f;
+      }
+    }
+  };
+  auto sstore = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / VPR, cv = idx % VPR;
+      *reinterpret_cast<uint4 *>(sQ + st * BM * QS + r * QS + cv * 8) = rq[i];
+      *reinterpret_cast<uint4 *>(sdO + st * BM * QS + r * QS + cv * 8) = rdo[i];
+    }
+    if (tid < BM) {
+      sLse[st * BM + tid] = rl;
+      sDel[st * BM + tid] = rd;
+    }
+  };
+
+  if (nsteps > 0) {
+    gload(0);
+    sstore(0);
+  }
+  __syncthreads();
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int st = step & 1;
+    if (step + 1 < nsteps) gload(step + 1);
+    const int i0 = i_begin + (step % ntq) * BM;
+    // causal: the whole 32-row query block lies above this wavefront's keys -> nothing to add
+    const bool skip = p.causal && i0 + BM - 1 < jw0;
+    if (!skip) {
+      const T *tQ = sQ + st * BM * QS;
+      const T *tdO = sdO + st * BM * QS;
+      floatx16 S, dP;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        S[v] = 0.f;
+        dP[v] = 0.f;
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const Frag aq = frag_ld<T>(tQ + c * QS + ks * 16 + 8 * hh);
+        S = M::mma(aq, Kf[ks], S);
+        const Frag ad = frag_ld<T>(tdO + c * QS + ks * 16 + 8 * hh);
+        dP = M::mma(ad, Vf[ks], dP);
+      }
+      const bool need_mask = p.causal && i0 < jw0 + 31;
+      float pv[16], dsv[16];
+#pragma unroll
+      for (int vb = 0; vb < 4; ++vb) {
+        const float4 l4 = *reinterpret_cast<const float4 *>(sLse + st * BM + 8 * vb + 4 * hh);
+        const float4 d4 = *reinterpret_cast<const float4 *>(sDel + st * BM + 8 * vb + 4 * hh);
+        const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
+        const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * vb + e;
+          float pe = fast_exp2(S[v] * p.scale_log2 - ls[e]);
+          if (need_mask && jrow > i0 + acc_row(v, hh)) pe = 0.f;
+          pv[v] = pe;
+          dsv[v] = pe * (dP[v] - dl[e]);
+        }
+      }
+      Frag Pb[2], dSb[2];
+      Pb[0] = frag_pack<T>(pv);
+      Pb[1] = frag_pack<T>(pv + 8);
+      dSb[0] = frag_pack<T>(dsv);
+      dSb[1] = frag_pack<T>(dsv + 8);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t) {
+          const int n0 = 32 * t + 16 * ((lane >> 4) & 1);
+          const Frag ad = frag_ld_tr<T>(tdO, QS, 16 * s + 4 * hh, 16 * s + 8 + 4 * hh, n0, lane);
+          dVt[t] = M::mma(ad, Pb[s], dVt[t]);
+          const Frag aq = frag_ld_tr<T>(tQ, QS, 16 * s + 4 * hh, 16 * s + 8 + 4 * hh, n0, lane);
+          dKt[t] = M::mma(aq, dSb[s], dKt[t]);
+        }
+      }
+    }
+    if (step + 1 < nsteps) sstore(st ^ 1);
+    __syncthreads();
+  }
+
+  if (jrow < sk) {
+    if (p.hsplit == 1) {
+      T *dkp = reinterpret_cast<T *>(p.dk) + (int64_t)(k0 + jrow) * p.dk_stride + (int64_t)hkv * D;
+      T *dvp = reinterpret_cast<T *>(p.dv) + (int64_t)(k0 + jrow) * p.dv_stride + (int64_t)hkv * D;
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          struct alignas(8) { T v[4]; } a, bq;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            a.v[e] = static_cast<T>(dKt[t][4 * vb + e] * p.scale);
+            bq.v[e] = static_cast<T>(dVt[t][4 * vb + e]);
+          }
+          *reinterpret_cast<decltype(a) *>(dkp + 32 * t + 8 * vb + 4 * hh) = a;
+          *reinterpret_cast<decltype(bq) *>(dvp + 32 * t + 8 * vb + 4 * hh) = bq;
+        }
+    } else {
+      const int64_t off = (((int64_t)hs * p.total_k + (k0 + jrow)) * p.hk + hkv) * D;
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          *reinterpret_cast<float4 *>(p.dk_part + off + 32 * t + 8 * vb + 4 * hh) =
+              make_float4(dKt[t][4 * vb] * p.scale, dKt[t][4 * vb + 1] * p.scale, dKt[t][4 * vb + 2] * p.scale,
+                          dKt[t][4 * vb + 3] * p.scale);
+          *reinterpret_cast<float4 *>(p.dv_part + off + 32 * t + 8 * vb + 4 * hh) =
+              make_float4(dVt[t][4 * vb], dVt[t][4 * vb + 1], dVt[t][4 * vb + 2], dVt[t][4 * vb + 3]);
+        }
+    }
+  }
+}
+
+// Sum of the head-split partials, in split order: part fp32 [hsplit][total_k][hk][d] -> dst (T, strided rows).
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_bwd_gqa_sum_kernel(const float *__restrict__ dk_part, const float *__restrict__ dv_part, T *__restrict__ dk,
+                        T *__restrict__ dv, int64_t total_k, int hk, int d, int hsplit, int64_t dk_stride,
+                        int64_t dv_stride) {
+  const int dv4 = d / 4;
+  const int64_t nitems = total_k * hk * dv4;
+  for (int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x; it < nitems; it += (int64_t)gridDim.x * 256) {
+    const int cc = (int)(it % dv4);
+    const int64_t r = it / dv4;
+    const int h = (int)(r % hk);
+    const int64_t j = r / hk;
+    float4 a = make_float4(0, 0, 0, 0), bb = make_float4(0, 0, 0, 0);
+    for (int s = 0; s < hsplit; ++s) {
+      const int64_t off = (((int64_t)s * total_k + j) * hk + h) * d + cc * 4;
+      const float4 x = *reinterpret_cast<const float4 *>(dk_part + off);
+      const float4 y = *reinterpret_cast<const float4 *>(dv_part + off);
+      a.x += x.x; a.y += x.y; a.z += x.z; a.w += x.w;
+      bb.x += y.x; bb.y += y.y; bb.z += y.z; bb.w += y.w;
+    }
+    T *pk = dk + j * dk_stride + (int64_t)h * d + cc * 4;
+    T *pv = dv + j * dv_stride + (int64_t)h * d + cc * 4;
+    pk[0] = from_f<T>(a.x); pk[1] = from_f<T>(a.y); pk[2] = from_f<T>(a.z); pk[3] = from_f<T>(a.w);
+    pv[0] = from_f<T>(bb.x); pv[1] = from_f<T>(bb.y); pv[2] = from_f<T>(bb.z); pv[3] = from_f<T>(bb.w);
+  }
+}
+
+// ---- dQ ---------------------------------------------------------------------------------------
+template <typename T, int D, int NW>
+__global__ void __launch_bounds__(64 * NW) attn_bwd_dq_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int BM = 32 * NW, BN = 32, NT = 64 * NW;
+  constexpr int KS = D + 16;  // K tile: row reads and transpose reads
+  constexpr int VS = D + 8;   // V tile: row reads only
+  constexpr int VPR = D / 8;
+  constexpr int LPT = BN * VPR / NT;
+  static_assert(BN * VPR % NT == 0, "tile must divide over the block");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *sK = reinterpret_cast<T *>(smem_raw);  // [2][BN*KS]
+  T *sV = sK + 2 * BN * KS;                 // [2][BN*VS]
+
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int mt = gridDim.x - 1 - blockIdx.x;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int m0 = mt * BM;
+  if (m0 >= sq) return;
+  const int hkv = h / (p.hq / p.hk);
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int wrow0 = m0 + w * 32;
+  const int row_q = wrow0 + c;
+  const bool row_ok = row_q < sq;
+  const int row_ld = row_ok ? row_q : sq - 1;
+
+  Frag Qf[D / 16], dOf[D / 16];
+  {
+    const T *qp = reinterpret_cast<const T *>(p.q) + (int64_t)(q0 + row_ld) * p.q_stride + (int64_t)h * D;
+    const T *dp = reinterpret_cast<const T *>(p.dout) + (int64_t)(q0 + row_ld) * p.do_stride + (int64_t)h * D;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      Qf[ks] = frag_ld<T>(qp + ks * 16 + 8 * hh);
+      dOf[ks] = frag_ld<T>(dp + ks * 16 + 8 * hh);
+    }
+  }
+  const float lse_c = row_ok ? p.lse[((int64_t)b * p.hq + h) * p.max_sq + row_q] * 1.4426950408889634f : INFINITY;
+  const float del_c = row_ok ? p.delta[((int64_t)b * p.hq + h) * p.max_sq + row_q] : 0.f;
+
+  const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
+  const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
+  int nk_end = sk;
+  if (p.causal && m0 + BM < nk_end) nk_end = m0 + BM;
+  const int ntiles = (nk_end + BN - 1) / BN;
+
+  floatx16 dQt[D / 32];
+#pragma unroll
+  for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dQt[t][v] = 0.f;
+
+  uint4 rk[LPT], rv[LPT];
+  auto gload = [&](int n0) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / VPR, cv = idx % VPR;
+      const int kr = n0 + r;
+      if (kr < sk) {
+        rk[i] = *reinterpret_cast<const uint4 *>(kg + (int64_t)kr * p.k_stride + cv * 8);
+        rv[i] = *reinterpret_cast<const uint4 *>(vg + (int64_t)kr * p.v_stride + cv * 8);
+      } else {
+        rk[i] = make_uint4(0, 0, 0, 0);
+        rv[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto sstore = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * NT;
+      const int r = idx / VPR, cv = idx % VPR;
+      *reinterpret_cast<uint4 *>(sK + st * BN * KS + r * KS + cv * 8) = rk[i];
+      *reinterpret_cast<uint4 *>(sV + st * BN * VS + r * VS + cv * 8) = rv[i];
+    }
+  };
+  if (ntiles > 0) {
+    gload(0);
+    sstore(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < ntiles; ++it) {
+    const int n0 = it * BN;
+    const int st = it & 1;
+    if (it + 1 < ntiles) gload(n0 + BN);
+    const bool skip = p.causal && n0 > wrow0 + 31;
+    if (!skip) {
+      const T *tK = sK + st * BN * KS;
+      const T *tV = sV + st * BN * VS;
+      floatx16 S, dP;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        S[v] = 0.f;
+        dP[v] = 0.f;
+      }
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const Frag ak = frag_ld<T>(tK + c * KS + ks * 16 + 8 * hh);
+        S = M::mma(ak, Qf[ks], S);
+        const Frag av = frag_ld<T>(tV + c * VS + ks * 16 + 8 * hh);
+        dP = M::mma(av, dOf[ks], dP);
+      }
+      const bool need_mask = (p.causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+      float dsv[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float pe = fast_exp2(S[v] * p.scale_log2 - lse_c);
+        if (need_mask) {
+          const int kv = n0 + acc_row(v, hh);
+          if (kv >= sk || (p.causal && kv > row_q)) pe = 0.f;
+        }
+        dsv[v] = pe * (dP[v] - del_c);
+      }
+      Frag dSb[2];
+      dSb[0] = frag_pack<T>(dsv);
+      dSb[1] = frag_pack<T>(dsv + 8);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t) {
+          const Frag ak = frag_ld_tr<T>(tK, KS, 16 * s + 4 * hh, 16 * s + 8 + 4 * hh, 32 * t + 16 * ((lane >> 4) & 1), lane);
+          dQt[t] = M::mma(ak, dSb[s], dQt[t]);
+        }
+      }
+    }
+    if (it + 1 < ntiles) sstore(st ^ 1);
+    __syncthreads();
+  }
+
+  if (row_ok) {
+    T *dqp = reinterpret_cast<T *>(p.dq) + (int64_t)(q0 + row_q) * p.dq_stride + (int64_t)h * D;
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int vb = 0; vb < 4; ++vb) {
+        struct alignas(8) { T v[4]; } a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+        *reinterpret_cast<decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh) = a;
+      }
+  }
+}
+
+// ---- host -------------------------------------------------------------------------------------
+static int pick_hsplit(int max_sk, int batch, int hq, int hk, int bn) {
+  const int ratio = hq / hk;
+  if (ratio == 1) return 1;
+  const int64_t blocks = cdiv(max_sk, bn) * hk * batch;
+  int hsplit = 1;
+  for (int s = 1; s <= ratio; ++s)
+    if (ratio % s == 0 && blocks * s <= 1024) hsplit = s;
+  return hsplit;
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+template <typename T, int D, int NW>
+static int launch_dkv(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
+  constexpr int BN = 32 * NW, BM = 32;
+  constexpr size_t smem = 2 * 2 * BM * (D + 16) * sizeof(T) + 4 * BM * sizeof(float);
+  static bool attr_set = false;
+  if (!attr_set) {
+    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dkv_kernel<T, D, NW>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_set = true;
+  }
+  dim3 grid((unsigned)cdiv(max_sk, BN), (unsigned)(p.hk * p.hsplit), (unsigned)batch);
+  hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, D, NW>), grid, dim3(64 * NW), smem, st, p);
+  return DH_OK;
+}
+
+template <typename T, int D, int NW>
+static int launch_dq(const AttnBwdParams &p, int batch, hipStream_t st) {
+  constexpr int BM = 32 * NW, BN = 32;
+  constexpr size_t smem = 2 * BN * ((D + 16) + (D + 8)) * sizeof(T);
+  static bool attr_set = false;
+  if (!attr_set) {
+    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<T, D, NW>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_set = true;
+  }
+  dim3 grid((unsigned)cdiv(p.max_sq, BM), (unsigned)p.hq, (unsigned)batch);
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, NW>), grid, dim3(64 * NW), smem, st, p);
+  return DH_OK;
+}
+
+template <typename T>
+static int launch_delta(const void *dout, const void *out, float *delta, const int32_t *cu_q, int batch, int max_sq,
+                        int hq, int d, int64_t do_stride, int64_t o_stride, hipStream_t st) {
+  const int nvec = d / Vec<T>::N;
+  int lanes_per = 1;
+  while (lanes_per < nvec && lanes_per < 64) lanes_per <<= 1;
+  const int per_block = 256 / lanes_per;
+  int64_t blocks = cdiv((int64_t)max_sq * hq, per_block);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL((attn_delta_kernel<T>), dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, st,
+                     (const T *)dout, (const T *)out, delta, cu_q, max_sq, hq, d, lanes_per, do_stride, o_stride);
+  return DH_OK;
+}
+
+int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, const float *lse, const float *delta,
+                 void *dq, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k, int batch, int max_sq,
+                 int max_sk, int hq, int hk, int d, int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                 int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int causal,
+                 hipStream_t st);
+
+constexpr int DKV_NW = 2;  // wavefronts per dK/dV workgroup (64 key rows)
+
+}  // namespace dh
+
+extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch, int max_seqlen_q, int hq,
+                                              int hk, int d, int dtype) {
+  using namespace dh;
+  (void)total_q;
+  size_t n = align256((size_t)batch * hq * (max_seqlen_q > 0 ? max_seqlen_q : 0) * sizeof(float));
+  if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
+    n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
+  return n + 256;
+}
+
+extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                           const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
+                           const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
+                           int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                           int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                           int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                           float softmax_scale, int causal, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(batch >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0 && total_q >= 0 && total_k >= 0, "negative size");
+  DH_CHECK(hq > 0 && hk > 0 && hq % hk == 0, "hq=%d must be a positive multiple of hk=%d", hq, hk);
+  if (batch == 0) return DH_OK;
+  DH_CHECK(dout && q && k && v && out && lse && dq && dk && dv && workspace && cu_seqlens_q && cu_seqlens_k,
+           "null pointer");
+  DH_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  uint8_t *ws = (uint8_t *)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  float *delta = delta_out ? delta_out : (float *)ws;
+  ws += align256((size_t)batch * hq * max_seqlen_q * sizeof(float));
+
+  const int n = 16 / (int)dtype_size(dtype);
+  DH_CHECK(d % n == 0 || dtype == DH_F32, "head dim %d must be a multiple of %d", d, n);
+  DH_CHECK(do_stride % n == 0 && o_stride % n == 0 && aligned16(dout) && aligned16(out),
+           "dout/out rows must be 16-byte aligned");
+  if (max_seqlen_q > 0) {
+    DH_DISPATCH_DTYPE(dtype, {
+      launch_delta<T>(dout, out, delta, cu_seqlens_q, batch, max_seqlen_q, hq, d, do_stride, o_stride, st);
+    });
+  }
+  if (dtype == DH_F32) {
+    DH_CHECK(d > 0 && d <= 256 && d % 4 == 0, "fp32 attention needs d %% 4 == 0 and d <= 256 (got %d)", d);
+    return attn_bwd_f32(dout, q, k, v, lse, delta, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, batch, max_seqlen_q,
+                        max_seqlen_k, hq, hk, d, q_stride, k_stride, v_stride, do_stride, dq_stride, dk_stride,
+                        dv_stride, softmax_scale, causal, st);
+  }
+  DH_CHECK(d == 64 || d == 128, "bf16/fp16 attention supports head dim 64 or 128 (got %d)", d);
+  DH_CHECK(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && dq_stride % 4 == 0 && dk_stride % 4 == 0 &&
+               dv_stride % 4 == 0,
+           "token strides must keep rows aligned");
+  DH_CHECK(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(dq) && aligned16(dk) && aligned16(dv),
+           "pointers must be 16-byte aligned");
+  AttnBwdParams p;
+  p.dout = dout; p.q = q; p.k = k; p.v = v; p.lse = lse; p.delta = delta;
+  p.dq = dq; p.dk = dk; p.dv = dv;
+  p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
+  p.max_sq = max_seqlen_q; p.hq = hq; p.hk = hk;
+  p.total_k = total_k;
+  p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride; p.do_stride = do_stride;
+  p.dq_stride = dq_stride; p.dk_stride = dk_stride; p.dv_stride = dv_stride;
+  p.scale = softmax_scale;
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  p.causal = causal;
+  p.hsplit = pick_hsplit(max_seqlen_k, batch, hq, hk, 32 * DKV_NW);
+  p.dk_part = nullptr;
+  p.dv_part = nullptr;
+  if (p.hsplit > 1) {
+    const size_t part = align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
+    p.dk_part = (float *)ws;
+    p.dv_part = (float *)(ws + part);
+  }
+  const bool small_q = cdiv(max_seqlen_q, 128) * hq * batch < 2 * 256;
+  int rc = DH_OK;
+#define DH_BWD(TT, DD)                                                                         \
+  do {                                                                                         \
+    if (max_seqlen_k > 0) rc = launch_dkv<TT, DD, DKV_NW>(p, batch, max_seqlen_k, st);         \
+    if (rc == DH_OK && p.hsplit > 1 && total_k > 0) {                                          \
+      int64_t blocks = cdiv(total_k * hk * (DD / 4), 256);                                     \
+      if (blocks > 256 * 16) blocks = 256 * 16;                                                \
+      hipLaunchKernelGGL((attn_bwd_gqa_sum_kernel<TT>), dim3((unsigned)blocks), dim3(256), 0, st, p.dk_part, \
+                         p.dv_part, (TT *)dk, (TT *)dv, total_k, hk, DD, p.hsplit, dk_stride, dv_stride);    \
+    }                                                                                          \
+    if (rc == DH_OK && max_seqlen_q > 0)                                                       \
+      rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st);  \
+  } while (0)
+  if (dtype == DH_BF16) {
+    if (d == 128) DH_BWD(bf16_t, 128); else DH_BWD(bf16_t, 64);
+  } else {
+    if (d == 128) DH_BWD(f16_t, 128); else DH_BWD(f16_t, 64);
+  }
+#undef DH_BWD
+  if (rc != DH_OK) return rc;
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}

@@ -1,0 +1,262 @@
+// Streaming elementwise kernels: SwiGLU forward/backward, residual add, and the
+// two legacy kernels of the binding surface (tanh-GELU, bias-mask-add).
+// All are HBM-bound: 16-byte accesses, several independent loads in flight per
+// lane, fp32 math, one rounding on store.
+#include "common.h"
+
+namespace dh {
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// One "item" = one 16-byte vector of the output row; rows x fv items in total.
+template <typename T, int UNROLL>
+__global__ void __launch_bounds__(256)
+swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems, int fv) {
+  constexpr int N = Vec<T>::N;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; it < nitems; it += stride * UNROLL) {
+    Vec<T> a[UNROLL], b[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nitems) {
+        const int64_t r = id / fv;
+        const int c = (int)(id - r * fv);
+        const T *row = y + r * (2 * (int64_t)fv * N);
+        a[u] = ldg(row + (int64_t)c * N);
+        b[u] = ldg(row + ((int64_t)fv + c) * N);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nitems) {
+        Vec<T> o;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float g = to_f(a[u].v[j]);
+          o.v[j] = from_f<T>(g * sigmoidf_(g) * to_f(b[u].v[j]));
+        }
+        stg(out + id * N, o);
+      }
+    }
+  }
+}
+
+template <typename T, int UNROLL>
+__global__ void __launch_bounds__(256)
+swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, int64_t nitems, int fv) {
+  constexpr int N = Vec<T>::N;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; it < nitems; it += stride * UNROLL) {
+    Vec<T> a[UNROLL], b[UNROLL], gv[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nitems) {
+        const int64_t r = id / fv;
+        const int c = (int)(id - r * fv);
+        const T *row = y + r * (2 * (int64_t)fv * N);
+        a[u] = ldg(row + (int64_t)c * N);
+        b[u] = ldg(row + ((int64_t)fv + c) * N);
+        gv[u] = ldg(g + id * N);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nitems) {
+        const int64_t r = id / fv;
+        const int c = (int)(id - r * fv);
+        Vec<T> d1, d2;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float y1 = to_f(a[u].v[j]), y2 = to_f(b[u].v[j]), gg = to_f(gv[u].v[j]);
+          const float s = sigmoidf_(y1);
+          d1.v[j] = from_f<T>(gg * s * (1.0f + y1 * (1.0f - s)) * y2);
+          d2.v[j] = from_f<T>(gg * (y1 * s));
+        }
+        T *row = dy + r * (2 * (int64_t)fv * N);
+        stg(row + (int64_t)c * N, d1);
+        stg(row + ((int64_t)fv + c) * N, d2);
+      }
+    }
+  }
+}
+
+// Scalar fallbacks (f not a multiple of the vector width, or unaligned pointers).
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_fwd_scalar_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t n, int64_t f) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / f, c = i - r * f;
+    const float g = to_f(y[r * 2 * f + c]);
+    out[i] = from_f<T>(g * sigmoidf_(g) * to_f(y[r * 2 * f + f + c]));
+  }
+}
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_bwd_scalar_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, int64_t n,
+                         int64_t f) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / f, c = i - r * f;
+    const float y1 = to_f(y[r * 2 * f + c]), y2 = to_f(y[r * 2 * f + f + c]), gg = to_f(g[i]);
+    const float s = sigmoidf_(y1);
+    dy[r * 2 * f + c] = from_f<T>(gg * s * (1.0f + y1 * (1.0f - s)) * y2);
+    dy[r * 2 * f + f + c] = from_f<T>(gg * (y1 * s));
+  }
+}
+
+enum { EW_ADD = 0, EW_GELU = 1, EW_BMA = 2 };
+
+template <typename T, int OP>
+__device__ __forceinline__ float ew_apply(float x, float b, float r, float m) {
+  if (OP == EW_ADD) return x + r;
+  if (OP == EW_GELU) return x * (0.5f + 0.5f * tanhf(x * (0.79788456f + 0.03567741f * x * x)));
+  return m * (x + b) + r;
+}
+
+template <typename T, int OP, int UNROLL>
+__global__ void __launch_bounds__(256)
+ew_kernel(const T *__restrict__ x, const T *__restrict__ bias, const T *__restrict__ res, const T *__restrict__ mask,
+          T *__restrict__ out, int64_t nvec, int64_t n) {
+  constexpr int N = Vec<T>::N;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; it < nvec; it += stride * UNROLL) {
+    Vec<T> xv[UNROLL], bv[UNROLL], rv[UNROLL], mv[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nvec) {
+        xv[u] = ldg(x + id * N);
+        if (OP != EW_GELU) rv[u] = ldg(res + id * N);
+        if (OP == EW_BMA) {
+          bv[u] = ldg(bias + id * N);
+          if (mask) mv[u] = ldg(mask + id * N);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t id = it + u * stride;
+      if (id < nvec) {
+        Vec<T> o;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float m = (OP == EW_BMA && mask) ? to_f(mv[u].v[j]) : 1.0f;
+          o.v[j] = from_f<T>(ew_apply<T, OP>(to_f(xv[u].v[j]), OP == EW_BMA ? to_f(bv[u].v[j]) : 0.f,
+                                             OP != EW_GELU ? to_f(rv[u].v[j]) : 0.f, m));
+        }
+        stg(out + id * N, o);
+      }
+    }
+  }
+  // tail elements (n % N) and everything when nvec == 0
+  const int64_t t0 = nvec * N;
+  if (blockIdx.x == 0) {
+    for (int64_t i = t0 + threadIdx.x; i < n; i += 256) {
+      const float m = (OP == EW_BMA && mask) ? to_f(mask[i]) : 1.0f;
+      out[i] = from_f<T>(ew_apply<T, OP>(to_f(x[i]), OP == EW_BMA ? to_f(bias[i]) : 0.f,
+                                         OP != EW_GELU ? to_f(res[i]) : 0.f, m));
+    }
+  }
+}
+
+static inline unsigned stream_grid(int64_t items, int per_thread) {
+  int64_t b = cdiv(items, 256ll * per_thread);
+  if (b < 1) b = 1;
+  if (b > 256 * 32) b = 256 * 32;
+  return (unsigned)b;
+}
+
+template <typename T, int OP>
+static int launch_ew(const void *x, const void *bias, const void *res, const void *mask, void *out, int64_t n,
+                     hipStream_t st) {
+  constexpr int N = Vec<T>::N;
+  bool al = aligned16(x) && aligned16(out) && (!bias || aligned16(bias)) && (!res || aligned16(res)) &&
+            (!mask || aligned16(mask));
+  const int64_t nvec = al ? n / N : 0;
+  hipLaunchKernelGGL((ew_kernel<T, OP, 4>), dim3(stream_grid(nvec, 4)), dim3(256), 0, st, (const T *)x,
+                     (const T *)bias, (const T *)res, (const T *)mask, (T *)out, nvec, n);
+  return 0;
+}
+
+}  // namespace dh
+
+extern "C" int dh_swiglu_fwd(const void *y, void *out, int64_t rows, int64_t f, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(rows >= 0 && f >= 0, "bad shape rows=%lld f=%lld", (long long)rows, (long long)f);
+  if (rows == 0 || f == 0) return DH_OK;
+  DH_CHECK(y && out, "null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  DH_DISPATCH_DTYPE(dtype, {
+    constexpr int N = Vec<T>::N;
+    if (f % N == 0 && aligned16(y) && aligned16(out) && f / N < (1ll << 31)) {
+      const int64_t nitems = rows * (f / N);
+      hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4>), dim3(stream_grid(nitems, 4)), dim3(256), 0, st, (const T *)y,
+                         (T *)out, nitems, (int)(f / N));
+    } else {
+      hipLaunchKernelGGL((swiglu_fwd_scalar_kernel<T>), dim3(stream_grid(rows * f, 4)), dim3(256), 0, st,
+                         (const T *)y, (T *)out, rows * f, f);
+    }
+  });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t rows, int64_t f, int dtype,
+                             void *stream) {
+  using namespace dh;
+  DH_CHECK(rows >= 0 && f >= 0, "bad shape rows=%lld f=%lld", (long long)rows, (long long)f);
+  if (rows == 0 || f == 0) return DH_OK;
+  DH_CHECK(g && y && dy, "null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  DH_DISPATCH_DTYPE(dtype, {
+    constexpr int N = Vec<T>::N;
+    if (f % N == 0 && aligned16(y) && aligned16(g) && aligned16(dy) && f / N < (1ll << 31)) {
+      const int64_t nitems = rows * (f / N);
+      hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2>), dim3(stream_grid(nitems, 2)), dim3(256), 0, st, (const T *)g,
+                         (const T *)y, (T *)dy, nitems, (int)(f / N));
+    } else {
+      hipLaunchKernelGGL((swiglu_bwd_scalar_kernel<T>), dim3(stream_grid(rows * f, 4)), dim3(256), 0, st,
+                         (const T *)g, (const T *)y, (T *)dy, rows * f, f);
+    }
+  });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_residual_add(const void *x, const void *residual, void *out, int64_t n, int dtype,
+                               void *stream) {
+  using namespace dh;
+  DH_CHECK(n >= 0, "n must be >= 0");
+  if (n == 0) return DH_OK;
+  DH_CHECK(x && residual && out, "null pointer");
+  DH_DISPATCH_DTYPE(dtype, { launch_ew<T, EW_ADD>(x, nullptr, residual, nullptr, out, n, (hipStream_t)stream); });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_gelu(const void *x, void *out, int64_t n, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(n >= 0, "n must be >= 0");
+  if (n == 0) return DH_OK;
+  DH_CHECK(x && out, "null pointer");
+  DH_DISPATCH_DTYPE(dtype, { launch_ew<T, EW_GELU>(x, nullptr, nullptr, nullptr, out, n, (hipStream_t)stream); });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_bias_mask_add(const void *x, const void *bias, const void *residual, const void *mask, void *out,
+                                int64_t n, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(n >= 0, "n must be >= 0");
+  if (n == 0) return DH_OK;
+  DH_CHECK(x && bias && residual && out, "null pointer");
+  DH_DISPATCH_DTYPE(dtype, { launch_ew<T, EW_BMA>(x, bias, residual, mask, out, n, (hipStream_t)stream); });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}

@@ -1,0 +1,80 @@
+"""Norm forward/backward with the reference's wrapper signatures.
+
+Mirrors dhellam/operators/layernorm.py:6-45 (``pylayernorm_fwd``) and :47-91
+(``pylayernorm_bwd``).  ``ln_bias=None`` selects RMSNorm (returned ``mu`` is
+None); a bias selects LayerNorm.  ``fwd_sm_margin`` / ``bwd_sm_margin`` are
+accepted and ignored (every reference call site passes 0, dstb.py:70,77,388).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ._util import on_stream
+
+_workspaces: dict = {}
+
+
+def _workspace(nbytes: int, device, stream) -> torch.Tensor:
+    """fp32 scratch for the dgamma partial rows, cached per (device, stream)."""
+    key = (device, stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() * 4 < nbytes:
+        ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_gamma, stream, profiling=False):
+    in_features = ln_weight.numel()
+    assert inp.is_cuda, "dhellam needs a GPU."
+    assert inp.shape[-1] == in_features, "LayerNorm not possible"
+    assert inp.is_contiguous() and ln_weight.is_contiguous()
+    lib = _lib.load()
+    inputmat = inp.view((-1, in_features))
+    rows = inputmat.shape[0]
+    el: list = []
+    with on_stream(stream, profiling, el) as st:
+        ln_out = torch.empty_like(inputmat)
+        rsigma = torch.empty(rows, dtype=torch.float32, device=inp.device)
+        mu = torch.empty(rows, dtype=torch.float32, device=inp.device) if ln_bias is not None else None
+        _lib.check(lib.dh_norm_fwd(inputmat.data_ptr(), ln_weight.data_ptr(), _lib.ptr(ln_bias), ln_out.data_ptr(),
+                                   _lib.ptr(mu), rsigma.data_ptr(), rows, in_features, float(eps),
+                                   int(bool(zero_centered_gamma)), _lib.dt(inp), st.cuda_stream))
+    return ln_out.view_as(inp), mu, rsigma, el[0]
+
+
+def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_centered_gamma, stream,
+                    profiling=False, add_to_dgrad=None, dgamma_out=None, dbeta_out=None):
+    """Returns (dinp, dgamma, dbeta, ms).
+
+    Extensions over the reference signature (all optional): ``add_to_dgrad`` is
+    added to dinp inside the kernel (the residual-branch gradient the reference
+    adds afterwards, dstb.py:391,401); ``dgamma_out`` / ``dbeta_out`` are
+    accumulated into in place (the reference's ``main_grad.add_``, dstb.py:392-393).
+    """
+    in_features = ln_weight.numel()
+    assert inp.is_cuda, "dhellam needs a GPU."
+    assert inp.shape[-1] == in_features, "LayerNorm not possible"
+    lib = _lib.load()
+    inputmat = inp.view((-1, in_features))
+    d_ln_out = d_ln_out.view((-1, in_features))
+    assert inputmat.is_contiguous() and d_ln_out.is_contiguous()
+    rows = inputmat.shape[0]
+    el: list = []
+    with on_stream(stream, profiling, el) as st:
+        dinp = torch.empty_like(inputmat)
+        accumulate = dgamma_out is not None
+        dgamma = dgamma_out if accumulate else torch.empty_like(ln_weight)
+        if mu is not None:
+            dbeta = dbeta_out if dbeta_out is not None else torch.empty_like(ln_weight)
+            assert (dbeta_out is not None) == accumulate, "pass both or neither of dgamma_out/dbeta_out"
+        else:
+            dbeta = None
+        ws = _workspace(lib.dh_norm_bwd_workspace_bytes(rows, in_features), inp.device, st)
+        add = add_to_dgrad.view((-1, in_features)) if add_to_dgrad is not None else None
+        _lib.check(lib.dh_norm_bwd(d_ln_out.data_ptr(), inputmat.data_ptr(), _lib.ptr(mu), rsigma.data_ptr(),
+                                   ln_weight.data_ptr(), _lib.ptr(add), dinp.data_ptr(), dgamma.data_ptr(),
+                                   _lib.ptr(dbeta), ws.data_ptr(), rows, in_features,
+                                   int(bool(zero_centered_gamma)), int(accumulate), _lib.dt(inp), st.cuda_stream))
+    return dinp.view_as(inp), dgamma, dbeta, el[0]

@@ -1,0 +1,40 @@
+"""SwiGLU forward/backward: dhellam/operators/swiglu.py:28-62.
+
+``y`` has the gate in the first half of the last dim and the up projection in
+the second half (swiglu.py:15).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ._util import on_stream
+
+
+def swiglu(y, stream=None, profiling=False):
+    assert y.is_cuda and y.is_contiguous() and y.shape[-1] % 2 == 0
+    lib = _lib.load()
+    f = y.shape[-1] // 2
+    rows = y.numel() // (2 * f) if f else 0
+    el: list = []
+    with on_stream(stream, profiling, el) as st:
+        out = torch.empty(*y.shape[:-1], f, dtype=y.dtype, device=y.device)
+        _lib.check(lib.dh_swiglu_fwd(y.data_ptr(), out.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
+    return out, el[0]
+
+
+def swiglu_back(g, y, o=None, stream=None, profiling=False):
+    """``o`` (optional) receives the result; the reference allocates it but its kernel
+    ignores it (swiglu.py:48-55)."""
+    assert y.is_cuda and y.is_contiguous() and g.is_contiguous() and y.shape[-1] % 2 == 0
+    lib = _lib.load()
+    f = y.shape[-1] // 2
+    rows = y.numel() // (2 * f) if f else 0
+    assert g.numel() == rows * f, "grad shape does not match swiglu input"
+    el: list = []
+    with on_stream(stream, profiling, el) as st:
+        if o is None:
+            o = torch.empty_like(y)
+        assert o.is_contiguous() and o.shape == y.shape
+        _lib.check(lib.dh_swiglu_bwd(g.data_ptr(), y.data_ptr(), o.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
+    return o, el[0]

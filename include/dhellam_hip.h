@@ -1,0 +1,235 @@
+/*
+ * dhellam_hip.h -- C ABI of the MI355X (gfx950) operator library behind the
+ * DHeLlam per-rank operator hot path.
+ *
+ * Every entry point takes raw DEVICE pointers, plain sizes and a HIP stream
+ * handle (hipStream_t passed as void*; NULL = the null stream).  All kernels
+ * are enqueued asynchronously on that stream; nothing here synchronises and,
+ * unless an entry says so, nothing here allocates.  Return value: 0 on
+ * success, a negative dh_status otherwise; dh_last_error() then holds a
+ * "file:line in function: message" string for the calling thread (the
+ * reference's DHELLAM_CHECK style, csrc/operators/logging.h:53-86, without the
+ * C++ exception).
+ *
+ * The reference binds this path through a pybind11 torch extension
+ * (csrc/torchapi.cpp:2-9, csrc/operators/ops.h:18-81); each declaration below
+ * cites the reference interface it stands behind.  The Python mirror of that
+ * extension (dhellam_amd/_Clib.py) is a thin ctypes shim over these symbols.
+ */
+#ifndef DHELLAM_HIP_H
+#define DHELLAM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { DH_F32 = 0, DH_BF16 = 1, DH_F16 = 2 } dh_dtype;
+
+typedef enum {
+  DH_OK = 0,
+  DH_ERR_INVALID = -1,   /* bad argument / unsupported shape */
+  DH_ERR_HIP = -2,       /* a HIP runtime call failed */
+  DH_ERR_UNSUPPORTED = -3
+} dh_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int dh_version(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char *dh_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Normalisation.  Stands behind dhellam/operators/layernorm.py:6-45
+ * (pylayernorm_fwd -> tex.layernorm_fwd) and :47-91 (pylayernorm_bwd ->
+ * tex.layernorm_bwd).  beta == NULL selects RMSNorm (y = x * rsigma * gamma,
+ * mu unused); beta != NULL selects LayerNorm (y = (x-mu)*rsigma*gamma+beta).
+ * x, y, gamma, beta share `dtype`; mu/rsigma are fp32 [rows].
+ * zero_centered_gamma: gamma is stored as (gamma - 1).
+ * ---------------------------------------------------------------------- */
+int dh_norm_fwd(const void *x, const void *gamma, const void *beta, void *y,
+                float *mu, float *rsigma, int64_t rows, int64_t cols,
+                float eps, int zero_centered_gamma, int dtype, void *stream);
+
+/* Bytes of fp32 scratch dh_norm_bwd needs for its dgamma/dbeta partial sums. */
+size_t dh_norm_bwd_workspace_bytes(int64_t rows, int64_t cols);
+
+/* dx = d(loss)/dx (+ add_to_dx if non-NULL: the residual-branch gradient the
+ * reference adds in a separate launch, dhellam/core/dstb.py:387-405).
+ * dgamma/dbeta [cols] in `dtype`; mu == NULL selects RMSNorm (dbeta may be
+ * NULL).  accumulate_wgrad != 0: dgamma/dbeta are added to instead of
+ * overwritten.  workspace: dh_norm_bwd_workspace_bytes() bytes. */
+int dh_norm_bwd(const void *dy, const void *x, const float *mu,
+                const float *rsigma, const void *gamma, const void *add_to_dx,
+                void *dx, void *dgamma, void *dbeta, void *workspace,
+                int64_t rows, int64_t cols, int zero_centered_gamma,
+                int accumulate_wgrad, int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * SwiGLU.  dhellam/operators/swiglu.py:13-16 (fwd) and :21-26 (bwd).
+ * y [rows, 2*f]: gate = first f columns, up = last f.  out [rows, f].
+ * bwd: dy [rows, 2*f] = cat(g*sig(y1)*(1+y1*(1-sig(y1)))*y2, g*silu(y1)).
+ * ---------------------------------------------------------------------- */
+int dh_swiglu_fwd(const void *y, void *out, int64_t rows, int64_t f, int dtype,
+                  void *stream);
+int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t rows,
+                  int64_t f, int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Residual add (bias-dropout-add with dropout disabled).
+ * dhellam/operators/bda.py:3-12.  out = x + residual (out may alias x: the
+ * reference op is in-place on its input).  n = element count.
+ * ---------------------------------------------------------------------- */
+int dh_residual_add(const void *x, const void *residual, void *out, int64_t n,
+                    int dtype, void *stream);
+
+/* Legacy elementwise kernels of the binding surface, fp16/bf16/fp32.
+ * csrc/operators/gelu.cu:10-15 (tanh GELU) and csrc/operators/bda.cu:10-16
+ * (out = mask*(x+bias)+residual; mask == NULL means all-ones). */
+int dh_gelu(const void *x, void *out, int64_t n, int dtype, void *stream);
+int dh_bias_mask_add(const void *x, const void *bias, const void *residual,
+                     const void *mask, void *out, int64_t n, int dtype,
+                     void *stream);
+
+/* ------------------------------------------------------------------------
+ * Rotary position embedding (rotate-half, non-interleaved).  The reference has
+ * no RoPE; its slot is between the q/k/v split and the attention call
+ * (dhellam/core/dstb.py:122-126) and, in backward, before the dq/dk/dv concat
+ * (:376-382).  q [tokens, hq, d], k [tokens, hk, d] (k may be NULL), token
+ * stride given in elements so q/k may be views into a packed qkv row.
+ * inv_freq: fp32 [d/2] on device; angle = (float)pos * inv_freq[j].
+ * positions: int32 [tokens] or NULL (then pos = t % seq_len, or t if
+ * seq_len <= 0).  backward != 0 applies the inverse rotation (sin -> -sin).
+ * Output may alias input.
+ * ---------------------------------------------------------------------- */
+int dh_rope(const void *q, const void *k, void *q_out, void *k_out,
+            const float *inv_freq, const int32_t *positions, int64_t tokens,
+            int hq, int hk, int d, int64_t q_stride, int64_t k_stride,
+            int64_t qo_stride, int64_t ko_stride, int64_t seq_len,
+            int backward, int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Variable-length flash attention.  csrc/operators/ops.h:18-32 /
+ * csrc/operators/flash_atten.cu:220-434 (forward) and ops.h:34-52 /
+ * flash_atten.cu:479-757 (backward).
+ * q [total_q, hq, d], k/v [total_k, hk, d], out like q; token strides are in
+ * elements (head stride is d, last dim contiguous).  cu_seqlens_* int32 [b+1]
+ * on device.  lse fp32 [b, hq, max_seqlen_q] = natural-log logsumexp of the
+ * scaled scores (-inf rows never occur for causal sq == sk).  causal requires
+ * per-sequence sq == sk.  hq % hk == 0 (GQA).  d in {64, 128} for bf16/fp16,
+ * any d <= 256 with d % 4 == 0 for fp32.
+ * ---------------------------------------------------------------------- */
+int dh_attn_fwd(const void *q, const void *k, const void *v, void *out,
+                float *lse, const int32_t *cu_seqlens_q,
+                const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
+                int max_seqlen_k, int hq, int hk, int d, int64_t q_stride,
+                int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                float softmax_scale, int causal, int dtype, void *stream);
+
+/* Bytes of scratch dh_attn_bwd needs (delta = rowsum(dO*O), and fp32 dK/dV
+ * partials when a GQA group is split over workgroups). */
+size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
+                                   int max_seqlen_q, int hq, int hk, int d,
+                                   int dtype);
+
+/* dq like q, dk/dv like k/v (GQA groups are reduced inside the kernel; the
+ * reference sums an expanded buffer afterwards, flash_atten.cu:646-652).
+ * delta_out (fp32 [b, hq, max_seqlen_q], may be NULL) receives rowsum(dO*O),
+ * the reference's softmax_d. */
+int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v,
+                const void *out, const float *lse, void *dq, void *dk,
+                void *dv, float *delta_out, void *workspace,
+                const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                int batch, int max_seqlen_q, int max_seqlen_k,
+                int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                int64_t o_stride, int64_t do_stride, int64_t dq_stride,
+                int64_t dk_stride, int64_t dv_stride, float softmax_scale,
+                int causal, int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Ring-attention merge of per-step partial results.
+ * dhellam/operators/ring_attn.py:26-40 (lse and out correction) applied as in
+ * :146-195, in one pass and in fp32.  Step s contributes rows
+ * [row_begin[s], row_begin[s]+rows[s]) of every sequence (the reference's
+ * "second half of q" steps have row_begin = sq/2).  outs[s]: [b*rows[s], hq,
+ * d] contiguous; lses[s]: fp32 [b, hq, rows[s]].  out [b*sq, hq, d];
+ * lse fp32 [b, hq, sq].  n_steps <= 8.  Host arrays of device pointers.
+ * ---------------------------------------------------------------------- */
+int dh_attn_merge(const void *const *outs, const float *const *lses,
+                  const int32_t *row_begin, const int32_t *rows, int n_steps,
+                  void *out, float *lse, int batch, int sq, int hq, int d,
+                  int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * MoE routing and token permutation.  No counterpart in the reference (it has
+ * no MoE); semantics are Mixtral/Megatron-core dropless top-k routing.
+ * ---------------------------------------------------------------------- */
+/* logits fp32 [tokens, experts] -> topk_idx int32 [tokens, k] (descending
+ * logit, ties to the lower expert id), gates fp32 [tokens, k] = softmax over
+ * the k selected logits.  experts <= 64, k <= 8. */
+int dh_moe_route_topk(const float *logits, int32_t *topk_idx, float *gates,
+                      int64_t tokens, int experts, int k, void *stream);
+
+size_t dh_moe_sort_workspace_bytes(int64_t n_assign, int experts);
+/* Stable counting sort of the flat assignment list topk_idx [n_assign] by
+ * expert id.  tokens_per_expert int32 [experts]; sorted_idx int32 [n_assign]
+ * (flat assignment ids in sorted order); dest_row int32 [n_assign] (position
+ * of each assignment in the sorted order). */
+int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert,
+                int32_t *sorted_idx, int32_t *dest_row, void *workspace,
+                int64_t n_assign, int experts, void *stream);
+
+/* permuted[r] = scale * x[src_assign[r] / k] for r in [0, n_rows), where
+ * src_assign = sorted_idx + first_row (a device pointer offset by the caller)
+ * and scale = row_scale[src_assign[r]] if row_scale != NULL else 1.
+ * n_rows is read ON DEVICE from *n_rows_dev (no host sync); the launch covers
+ * max_rows. */
+int dh_moe_gather_rows(const void *x, const int32_t *src_assign,
+                       const float *row_scale, void *permuted,
+                       const int32_t *n_rows_dev, int64_t max_rows, int k,
+                       int64_t hidden, int dtype, void *stream);
+
+/* out[t] = sum_j w(t,j) * y[dest_row[t*k+j] - first_row] over the j whose
+ * sorted position falls in [first_row, first_row + n_rows); w = gates[t*k+j]
+ * or 1 if gates == NULL.  Tokens with no local assignment get zeros.
+ * first_row / n_rows are read on device from range_dev[0..1]. */
+int dh_moe_scatter_rows(const void *y, const int32_t *dest_row,
+                        const float *gates, void *out,
+                        const int32_t *range_dev, int64_t tokens, int k,
+                        int64_t hidden, int dtype, void *stream);
+
+/* dgates[t*k+j] = <dout[t], y[dest_row[t*k+j]-first_row]> (0 if not local). */
+int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *dest_row,
+                     float *dgates, const int32_t *range_dev, int64_t tokens,
+                     int k, int64_t hidden, int dtype, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Grouped GEMM on MFMA (bf16/fp16 in, fp32 accumulate).  No counterpart in
+ * the reference.  Group g owns rows [offs[g], offs[g+1]) (device int32
+ * [groups+1], read on device).
+ *   NT: c[rows_g, n] = a[rows_g, k] * b[g][n, k]^T          (forward)
+ *   NN: c[rows_g, n] = a[rows_g, k] * b[g][k, n]            (dgrad)
+ *   TN: c[g][m, n] (+)= a[rows_g, m]^T * b[rows_g, n]       (wgrad)
+ * max_rows bounds the launch grid.
+ * ---------------------------------------------------------------------- */
+int dh_grouped_gemm_nt(const void *a, const void *b, void *c,
+                       const int32_t *offs, int groups, int64_t max_rows,
+                       int64_t n, int64_t k, int dtype, void *stream);
+int dh_grouped_gemm_nn(const void *a, const void *b, void *c,
+                       const int32_t *offs, int groups, int64_t max_rows,
+                       int64_t n, int64_t k, int dtype, void *stream);
+int dh_grouped_gemm_tn(const void *a, const void *b, void *c,
+                       const int32_t *offs, int groups, int64_t max_rows,
+                       int64_t m, int64_t n, int accumulate, int dtype,
+                       void *stream);
+
+/* Plain device-to-device copy kernel (a known-size streaming kernel used to
+ * calibrate the profiler's HBM byte counters). */
+int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DHELLAM_HIP_H */

@@ -1,0 +1,200 @@
+"""GPU parity of flash attention (fwd, bwd), the merge and the ring step against the oracle.
+
+All calls go through the C ABI via the reference-named shims (pymha_varlen_fwd/bwd,
+fa_cp_block_fwd/bwd).  Inputs are seeded N(0,1), rounded to the run dtype and fed
+identically to the HIP path and to the oracle.  Tolerances: rel-err <= 1e-2
+(bf16/fp16), <= 1e-5 (fp32) on outputs and gradients.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import attention as OA
+from tests.util import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+
+
+def _cu(lens):
+    c = [0]
+    for n in lens:
+        c.append(c[-1] + n)
+    return torch.tensor(c, dtype=torch.int32)
+
+
+def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.float64, packed=False, seed=0):
+    from dhellam_amd import _Clib
+    cq, ck = _cu(lens_q), _cu(lens_k)
+    tq, tk = int(cq[-1]), int(ck[-1])
+    scale = 1.0 / math.sqrt(d)
+    if packed:
+        # q, k, v as strided views of one [T, (hq + 2 hk) d] projection output (self-attention only)
+        assert tq == tk
+        qkv = randn((tq, (hq + 2 * hk) * d), dtype, seed)
+        qkv_g = qkv.cuda()
+        sl = lambda t, a, n: t[:, a * d:(a + n) * d].view(t.shape[0], n, d)
+        q, k, v = sl(qkv, 0, hq), sl(qkv, hq, hk), sl(qkv, hq + hk, hk)
+        qg, kg, vg = sl(qkv_g, 0, hq), sl(qkv_g, hq, hk), sl(qkv_g, hq + hk, hk)
+    else:
+        q, k, v = randn((tq, hq, d), dtype, seed), randn((tk, hk, d), dtype, seed + 1), randn((tk, hk, d), dtype, seed + 2)
+        qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    do = randn((tq, hq, d), dtype, seed + 3)
+    mq, mk = max(lens_q), max(lens_k)
+    res = _Clib.pymha_varlen_fwd(qg, kg, vg, cq.cuda(), ck.cuda(), mq, mk, 0.0, scale, causal, False, 0, False)
+    assert len(res) == 8
+    out, lse = res[0], res[5]
+    assert res[4] is out and res[1] is qg
+    oo, lo = OA.attn_fwd(q, k, v, cq, ck, scale, causal, oracle_dtype)
+    assert_close(out, oo, dtype, "out")
+    for i, n in enumerate(lens_q):
+        if n:
+            assert_close(lse[i, :, :n], lo[i, :, :n], torch.float32, f"lse[{i}]", scale=1e3 if dtype != torch.float32 else 1)
+    # backward consumes the forward's own (rounded) out and lse, like the layer does
+    stream = torch.cuda.current_stream()
+    r = _Clib.pymha_varlen_bwd(do.cuda(), qg, kg, vg, out, lse, cq.cuda(), ck.cuda(), mq, mk, 0.0, scale, causal,
+                               None, False, 0, False, stream.cuda_stream)
+    assert len(r) == 4
+    dq, dk, dv, dl = r
+    lse_cpu = lse.cpu().double()
+    dqo, dko, dvo, dlo = OA.attn_bwd(do, q, k, v, out.cpu(), lse_cpu, cq, ck, scale, causal, oracle_dtype)
+    assert_close(dq, dqo, dtype, "dq")
+    assert_close(dk, dko, dtype, "dk")
+    assert_close(dv, dvo, dtype, "dv")
+    for i, n in enumerate(lens_q):
+        if n:
+            assert_close(dl[i, :, :n], dlo[i, :, :n], torch.float32, f"delta[{i}]", scale=1e3 if dtype != torch.float32 else 10)
+    return out, lse, dq, dk, dv
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("lens_q,lens_k,hq,hk,d,causal", [
+    ([1024], [1024], 8, 1, 128, True),          # the 70B shard's head layout, shortened
+    ([512, 512], [512, 512], 16, 16, 64, True),  # MHA, d 64, two sequences
+    ([100, 257, 64, 1], [100, 257, 64, 1], 4, 2, 128, True),   # ragged
+    ([300], [200], 4, 2, 128, False),            # rectangular, non-causal
+    ([128, 77], [640, 33], 6, 3, 64, False),
+    ([2048], [1024], 8, 2, 128, False),          # ring 'lower' shape
+    ([1024], [2048], 8, 2, 128, False),          # ring 'upper' shape
+])
+def test_attention_16bit(dtype, lens_q, lens_k, hq, hk, d, causal):
+    _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal)
+
+
+def test_attention_packed_qkv_views():
+    _run_fwd_bwd(torch.bfloat16, [384, 128], [384, 128], 8, 1, 128, True, packed=True)
+
+
+def test_attention_full_70b_shard_shape():
+    # 8 q heads + 1 kv head, d 128, 4096 tokens, causal, bf16; oracle in fp32 to keep the CPU time in seconds
+    _run_fwd_bwd(torch.bfloat16, [4096], [4096], 8, 1, 128, True, oracle_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("lens_q,lens_k,hq,hk,d,causal", [
+    ([512, 512], [512, 512], 16, 16, 64, True),  # the fp32 parity configuration
+    ([130, 7], [130, 7], 4, 2, 32, True),
+    ([50], [200], 2, 1, 256, False),
+    ([70], [70], 3, 3, 20, True),
+])
+def test_attention_fp32(lens_q, lens_k, hq, hk, d, causal):
+    _run_fwd_bwd(torch.float32, lens_q, lens_k, hq, hk, d, causal)
+
+
+def test_attention_is_deterministic():
+    a = _run_fwd_bwd(torch.bfloat16, [700], [700], 8, 2, 128, True)
+    b = _run_fwd_bwd(torch.bfloat16, [700], [700], 8, 2, 128, True)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_attention_profiling_and_errors():
+    from dhellam_amd import _Clib
+    q = randn((256, 4, 128), torch.bfloat16, 0).cuda()
+    cu = _cu([256]).cuda()
+    res = _Clib.pymha_varlen_fwd(q, q, q, cu, cu, 256, 256, 0.0, 0.1, True, False, 0, True)
+    assert len(res) == 9 and res[8].device.type == "cpu" and res[8].item() > 0
+    with pytest.raises(RuntimeError):
+        _Clib.pymha_varlen_fwd(q, q, q, cu, cu, 256, 256, 0.1, 0.1, True, False, 0, False)   # dropout
+    q96 = randn((256, 4, 96), torch.bfloat16, 0).cuda()
+    with pytest.raises(RuntimeError, match="head dim"):
+        _Clib.pymha_varlen_fwd(q96, q96, q96, cu, cu, 256, 256, 0.0, 0.1, True, False, 0, False)
+    k3 = randn((256, 3, 128), torch.bfloat16, 0).cuda()
+    with pytest.raises(RuntimeError, match="multiple"):
+        _Clib.pymha_varlen_fwd(q, k3, k3, cu, cu, 256, 256, 0.0, 0.1, True, False, 0, False)
+
+
+# ------------------------------------------------------------------------------------------
+# merge and ring step
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_merge_kernel(dtype):
+    from dhellam_amd import _Clib
+    b, sq, hq, d = 2, 96, 3, 64
+    row_begin, rows = [0, 0, 48, 48], [96, 96, 48, 48]
+    outs = [randn((b * n, hq, d), dtype, 10 + i) for i, n in enumerate(rows)]
+    lses = [randn((b, hq, n), torch.float32, 20 + i, std=3.0) for i, n in enumerate(rows)]
+    out = torch.empty((b * sq, hq, d), dtype=dtype, device="cuda")
+    lse = torch.empty((b, hq, sq), dtype=torch.float32, device="cuda")
+    _Clib.pyattn_merge([o.cuda() for o in outs], [l.cuda() for l in lses], row_begin, rows, out, lse)
+    oo, lo = OA.merge(outs, lses, row_begin, rows, b, sq, hq, d)
+    assert_close(out, oo, dtype, "merged out")
+    assert_close(lse, lo, torch.float32, "merged lse", scale=2)
+
+
+def _ring_inputs(dtype, b, c, hq, hk, d, cp, seed=0):
+    q = randn((b, 2, c, hq, d), dtype, seed)
+    chunks = [(randn((b, 2, c, hk, d), dtype, seed + 10 + 2 * i), randn((b, 2, c, hk, d), dtype, seed + 11 + 2 * i))
+              for i in range(cp)]
+    dout = randn((b, 2, c, hq, d), dtype, seed + 99)
+    return q, chunks, dout
+
+
+def _ring_gpu(q, chunks, dout, rank, cp):
+    from dhellam_amd.operators.ring_attn import RingGroup, fa_cp_block_bwd, fa_cp_block_fwd
+    b, _, c = q.shape[:3]
+    s = 2 * c
+    grp = RingGroup(rank, cp)
+    cu = torch.arange(0, (b + 1) * s, s, dtype=torch.int32).cuda()
+    bufs = [torch.stack((k, v)).cuda() for k, v in chunks]
+    qg = q.cuda()
+    carry = [qg, bufs, None, None, None, None, None, 0]
+    for i in range(cp):
+        r = fa_cp_block_fwd(carry[0], cu, cu, s, s, carry[1], carry[2], carry[3], carry[4], carry[5], carry[6], i,
+                            True, grp, list(range(cp)), None)
+        if i < cp - 1:
+            carry, reqs = r
+            assert reqs == [] and carry[-1] == i + 1
+        else:
+            out, q_ret, kv_ret, lse, rng = r
+    assert q_ret is qg and kv_ret is bufs[-1]
+    state = [dout.cuda(), None, None, bufs, 0]
+    for i in range(cp + 1):
+        r = fa_cp_block_bwd(state[0], out, qg, state[1], None, state[2], lse, rng, cu, cu, s, s, state[3], i, True,
+                            grp, list(range(cp)), None)
+        if i < cp:
+            state, reqs = r
+        else:
+            dq, dkv = r
+    return out, lse, dq, dkv
+
+
+@pytest.mark.parametrize("dtype,b,c,hq,hk,d", [(torch.bfloat16, 1, 128, 4, 2, 128), (torch.bfloat16, 1, 96, 2, 2, 64),
+                                                 (torch.float32, 1, 48, 2, 1, 32)])
+@pytest.mark.parametrize("rank", [0, 1, 3])
+def test_ring_step_matches_oracle_and_dense(dtype, b, c, hq, hk, d, rank):
+    cp = 4
+    q, chunks, dout = _ring_inputs(dtype, b, c, hq, hk, d, cp)
+    scale = 1.0 / math.sqrt(d)
+    out, lse, dq, dkv = _ring_gpu(q, chunks, dout, rank, cp)
+    oo, lo, _ = OA.ring_fwd(q, chunks, rank, scale)
+    assert_close(out, oo, dtype, "ring out")
+    assert_close(lse, lo, torch.float32, "ring lse", scale=1e3 if dtype != torch.float32 else 2)
+    # the same thing as ONE dense causal attention over the zig-zag order
+    do_, lo_ = OA.zigzag_dense(q, chunks, rank, scale)
+    assert_close(out.view(b, 2 * c, hq, d), do_, dtype, "ring out vs dense")
+    # backward: oracle ring with the GPU's own merged out/lse
+    dqo, dkvo = OA.ring_bwd(dout, out.cpu(), lse.cpu().double(), q, chunks, rank, scale)
+    assert_close(dq.view(q.shape), dqo, dtype, "ring dq")
+    for s in range(cp):
+        assert_close(dkv[s][0], dkvo[s][0], dtype, f"ring dk[{s}]")
+        assert_close(dkv[s][1], dkvo[s][1], dtype, f"ring dv[{s}]")

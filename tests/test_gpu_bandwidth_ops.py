@@ -1,0 +1,144 @@
+"""GPU parity of the bandwidth-bound operators against the CPU oracle.
+
+Each test feeds the SAME seeded tensors (already rounded to the run dtype) to the
+HIP path (through the C ABI, via the reference-named wrappers) and to the oracle
+in fp64.  Tolerances: rel-err <= 1e-5 (fp32), <= 1e-2 (bf16/fp16).
+"""
+import pytest
+import torch
+
+from oracle import ops as O
+from tests.util import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1024, 1024), (512, 8192), (37, 256), (5, 4096), (3, 100), (2, 24576), (64, 64)])
+@pytest.mark.parametrize("ln", [False, True])
+def test_norm_fwd_bwd(dtype, rows, cols, ln):
+    from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
+    x = randn((rows, cols), dtype, 0)
+    gamma = (1.0 + 0.1 * randn((cols,), torch.float32, 1)).to(dtype)
+    beta = (0.1 * randn((cols,), torch.float32, 2)).to(dtype) if ln else None
+    dy = randn((rows, cols), dtype, 3)
+    res = randn((rows, cols), dtype, 4)
+    y, mu, rs, ms = pylayernorm_fwd(x.cuda(), gamma.cuda(), beta.cuda() if ln else None, 1e-5, 0, False, None)
+    yo, muo, rso = O.norm_fwd(x, gamma, beta, 1e-5)
+    assert ms == 0
+    assert_close(y, yo, dtype, "y")
+    assert_close(rs, rso, torch.float32, "rsigma", scale=4)
+    if ln:
+        assert_close(mu, muo, torch.float32, "mu", scale=4)
+    else:
+        assert mu is None
+    # backward uses the oracle's statistics rounded to fp32, as the forward would hand over
+    rs32 = rso.float()
+    mu32 = muo.float() if ln else None
+    dx, dg, db, _ = pylayernorm_bwd(dy.cuda(), x.cuda(), mu32.cuda() if ln else None, rs32.cuda(), gamma.cuda(), 0,
+                                    False, None)
+    dxo, dgo, dbo = O.norm_bwd(dy, x, mu32, rs32, gamma)
+    assert_close(dx, dxo, dtype, "dx")
+    assert_close(dg, dgo, dtype, "dgamma")
+    if ln:
+        assert_close(db, dbo, dtype, "dbeta")
+    else:
+        assert db is None
+    # fused residual-gradient add and in-place accumulation of the weight gradients
+    acc_g = randn((cols,), dtype, 5).cuda()
+    acc_b = randn((cols,), dtype, 6).cuda() if ln else None
+    acc_g0, acc_b0 = acc_g.clone(), (acc_b.clone() if ln else None)
+    dx2, dg2, db2, _ = pylayernorm_bwd(dy.cuda(), x.cuda(), mu32.cuda() if ln else None, rs32.cuda(), gamma.cuda(),
+                                       0, False, None, add_to_dgrad=res.cuda(), dgamma_out=acc_g, dbeta_out=acc_b)
+    assert_close(dx2, dxo + res.double(), dtype, "dx+res")
+    assert dg2 is acc_g
+    assert_close(acc_g, dgo + acc_g0.double().cpu(), dtype, "dgamma accumulate")
+    if ln:
+        assert_close(acc_b, dbo + acc_b0.double().cpu(), dtype, "dbeta accumulate")
+
+
+def test_norm_zero_centered_gamma_and_empty():
+    from dhellam_amd.operators.layernorm import pylayernorm_fwd
+    x = randn((16, 512), torch.float32, 0)
+    g = 0.1 * randn((512,), torch.float32, 1)
+    y, _, _, _ = pylayernorm_fwd(x.cuda(), g.cuda(), None, 1e-5, 0, True, None)
+    yo, _, _ = O.norm_fwd(x, g, None, 1e-5, zero_centered_gamma=True)
+    assert_close(y, yo, torch.float32)
+    e = torch.empty((0, 512), device="cuda")
+    y, mu, rs, _ = pylayernorm_fwd(e, g.cuda(), None, 1e-5, 0, False, None)
+    assert y.shape == (0, 512) and rs.shape == (0,)
+
+
+def test_norm_profiling_returns_ms():
+    from dhellam_amd.operators.layernorm import pylayernorm_fwd
+    x = randn((512, 8192), torch.bfloat16, 0).cuda()
+    g = torch.ones(8192, dtype=torch.bfloat16, device="cuda")
+    *_, ms = pylayernorm_fwd(x, g, None, 1e-5, 0, False, None, profiling=True)
+    assert 0 < ms < 50
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 512, 5632), (1, 4096, 7168), (7, 30), (3, 5, 2), (0, 64)])
+def test_swiglu(dtype, shape):
+    from dhellam_amd.operators.swiglu import swiglu, swiglu_back
+    y = randn(shape, dtype, 0)
+    g = randn(shape[:-1] + (shape[-1] // 2,), dtype, 1)
+    out, ms = swiglu(y.cuda())
+    assert ms == 0 and out.shape == g.shape
+    assert_close(out, O.swiglu_fwd(y), dtype, "swiglu")
+    dy, _ = swiglu_back(g.cuda().view(-1, g.shape[-1]), y.cuda().view(-1, shape[-1]))
+    assert_close(dy, O.swiglu_bwd(g, y).view(-1, shape[-1]), dtype, "swiglu_back")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [1 * 512 * 8192, 1000003, 7, 0])
+def test_bda(dtype, n):
+    from dhellam_amd.operators.bda import bda_bwd, bda_fwd
+    x, r = randn((n,), dtype, 0), randn((n,), dtype, 1)
+    xg = x.cuda()
+    out, mask, ms = bda_fwd(xg, r.cuda())
+    assert out.data_ptr() == xg.data_ptr(), "bda_fwd is in place on its input"
+    assert mask is None and ms == 0
+    assert_close(out, O.bda_fwd(x, r), dtype, "bda", scale=1.0)
+    dres, din, _ = bda_bwd(out, None)
+    assert torch.equal(dres, out) and torch.equal(din, out)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,hq,hk,d,theta,seq", [(1024, 16, 16, 64, 1e4, 512), (4096, 8, 1, 128, 5e5, None),
+                                                  (33, 3, 1, 32, 1e4, None), (16, 2, 0, 16, 1e4, None)])
+def test_rope(dtype, T, hq, hk, d, theta, seq):
+    from dhellam_amd.operators.rope import rope_bwd, rope_fwd
+    # q and k are views into one packed [T, (hq + 2 hk) * d] row, as the layer produces them
+    packed = randn((T, (hq + 2 * hk) * d), dtype, 0)
+    pg = packed.cuda()
+    q = packed[:, : hq * d].view(T, hq, d)
+    k = packed[:, hq * d: (hq + hk) * d].view(T, hk, d) if hk else None
+    qg = pg[:, : hq * d].view(T, hq, d)
+    kg = pg[:, hq * d: (hq + hk) * d].view(T, hk, d) if hk else None
+    pos = torch.arange(T) % seq if seq else torch.arange(T)
+    qr, kr, _ = rope_fwd(qg, kg, None, theta, seq)
+    assert_close(qr, O.rope(q, pos, theta), dtype, "q")
+    if hk:
+        assert_close(kr, O.rope(k, pos, theta), dtype, "k")
+    # explicit positions, backward, in place
+    pos32 = pos.to(torch.int32).cuda()
+    dq, dk, _ = rope_bwd(qr, kr, pos32, theta, None)
+    assert_close(dq, O.rope(O.rope(q, pos, theta).to(dtype), pos, theta, backward=True), dtype, "bwd")
+    # inverse rotation recovers the input up to two roundings
+    assert_close(dq, q, dtype, "roundtrip", scale=3)
+
+
+def test_legacy_kernels():
+    from dhellam_amd import _Clib
+    x = randn((4096, 33), torch.float16, 0)
+    o = torch.empty_like(x).cuda()
+    assert _Clib.pygelu(x.cuda(), o, False) == 0
+    assert_close(o, O.gelu_tanh(x), torch.float16)
+    b, r = randn((4096, 33), torch.float16, 1), randn((4096, 33), torch.float16, 2)
+    assert _Clib.pybda(x.cuda(), b.cuda(), r.cuda(), o, 0.0, False) == 0
+    assert_close(o, O.bias_mask_add(x, b, r), torch.float16)
+    s = _Clib.add_tensors(x.cuda(), b.cuda())
+    assert torch.equal(s.cpu(), x + b)

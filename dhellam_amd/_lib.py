@@ -38,10 +38,10 @@ SIGNATURES = {
     "dh_attn_merge": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
     "dh_moe_route_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "dh_moe_sort_workspace_bytes": (_sz, [_i64, _i32]),
-    "dh_moe_sort": (_i32, [_vp] * 5 + [_i64, _i32, _vp]),
-    "dh_moe_gather_rows": (_i32, [_vp] * 5 + [_i64, _i32, _i64, _i32, _vp]),
-    "dh_moe_scatter_rows": (_i32, [_vp] * 5 + [_i64, _i32, _i64, _i32, _vp]),
-    "dh_moe_gate_grad": (_i32, [_vp] * 5 + [_i64, _i32, _i64, _i32, _vp]),
+    "dh_moe_sort": (_i32, [_vp] * 6 + [_i64, _i32, _vp]),
+    "dh_moe_gather_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
+    "dh_moe_scatter_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
+    "dh_moe_gate_grad": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
     "dh_grouped_gemm_nt": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp]),
     "dh_grouped_gemm_nn": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp]),
     "dh_grouped_gemm_tn": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _i32, _vp]),

@@ -1,0 +1,333 @@
+// Grouped GEMM on gfx950 MFMA (bf16/fp16 inputs, fp32 accumulate) for one
+// expert-parallel rank: every local expert multiplies its own contiguous block
+// of permuted rows.
+//
+// One template covers the three products a SwiGLU expert needs:
+//   NT  c[r, n]  = sum_k a[r, k] * w[g][n, k]      forward  (both k-contiguous)
+//   NN  c[r, n]  = sum_k a[r, k] * w[g][k, n]      dgrad    (w strided in k)
+//   TN  c[g][m,n] = sum_r a[r, m] * b[r, n]        wgrad    (both strided in k = r)
+// A workgroup is 2x2 wavefronts, each owning a (32*WM) x (32*WN) output block
+// kept in accumulators; 64-deep k slices of both operands are staged in LDS
+// (two stages, one barrier per slice).  k-contiguous operands are read from LDS
+// as 16-byte row fragments; k-strided operands stay row-major in LDS and are
+// read with transpose loads, so no operand is ever transposed in memory.
+// The product is formed as C^T (weights in the MFMA A slot) so that each lane
+// ends up with runs of 4 consecutive output columns of one row: 8-byte stores.
+// Group row ranges are read on the device from the offsets table.
+#include "mma.h"
+
+namespace dh {
+
+constexpr int GG_BK = 64;
+constexpr int GG_MAX_GROUPS = 64;
+
+struct GGParams {
+  const void *a, *b;
+  void *c;
+  const int32_t *offs;
+  int groups;
+  int64_t m_dim;   // TN: columns of a (= rows of c[g]); NT/NN: unused
+  int64_t n_dim;   // output columns
+  int64_t k_dim;   // NT/NN: reduction length; TN: unused (comes from offs)
+  int64_t lda, ldb, ldc;
+  int64_t b_group_stride, c_group_stride;
+  int tiles_m, tiles_n;  // grid extents (tiles_m is an upper bound for NT/NN)
+  int accumulate;
+};
+
+// Load one 64-deep k slice of an operand into registers.
+//   KC (k-contiguous): tile [R rows][64 k]; element (row, k) at src[row * ld + k]
+//   KS (k-strided)   : tile [64 k][R cols]; element (k, col) at src[k * ld + col]
+template <typename T, int R, bool KSTRIDED>
+struct TileLoader {
+  static constexpr int VECS = R * GG_BK / 8;
+  static constexpr int LPT = VECS / 256;
+  static_assert(VECS % 256 == 0, "tile must divide over 256 threads");
+  // rows: extent along the R dimension still valid (from tile origin); kext: valid k extent from this slice's origin
+  static __device__ __forceinline__ void gload(uint4 (&reg)[LPT], const T *src, int64_t ld, int rext, int kext, int tid) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * 256;
+      int r, k;
+      if (KSTRIDED) {
+        k = idx / (R / 8);
+        r = (idx % (R / 8)) * 8;
+        reg[i] = (k < kext && r < rext) ? *reinterpret_cast<const uint4 *>(src + (int64_t)k * ld + r) : make_uint4(0, 0, 0, 0);
+      } else {
+        r = idx / (GG_BK / 8);
+        k = (idx % (GG_BK / 8)) * 8;
+        reg[i] = (r < rext && k < kext) ? *reinterpret_cast<const uint4 *>(src + (int64_t)r * ld + k) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  }
+  static constexpr int LD = KSTRIDED ? R + 32 : GG_BK + 8;          // LDS row stride (elements)
+  static constexpr int ELEMS = KSTRIDED ? GG_BK * LD : R * LD;      // LDS elements per stage
+  static __device__ __forceinline__ void sstore(const uint4 (&reg)[LPT], T *dst, int tid) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int idx = tid + i * 256;
+      if (KSTRIDED) {
+        const int k = idx / (R / 8), r = (idx % (R / 8)) * 8;
+        *reinterpret_cast<uint4 *>(dst + k * LD + r) = reg[i];
+      } else {
+        const int r = idx / (GG_BK / 8), k = (idx % (GG_BK / 8)) * 8;
+        *reinterpret_cast<uint4 *>(dst + r * LD + k) = reg[i];
+      }
+    }
+  }
+  // Fragment for the 32 rows/cols starting at r0, k-step ks (16 values of k): slot j of lane half hh is k = 16ks + 8hh + j.
+  static __device__ __forceinline__ typename Mma<T>::Frag frag(const T *tile, int r0, int ks, int lane) {
+    const int c = lane & 31, hh = lane >> 5;
+    if (KSTRIDED) return frag_ld_tr<T>(tile, LD, 16 * ks + 8 * hh, 16 * ks + 8 * hh + 4, r0 + 16 * ((lane >> 4) & 1), lane);
+    return frag_ld<T>(tile + (r0 + c) * LD + ks * 16 + 8 * hh);
+  }
+};
+
+template <typename T, bool TA, bool TB, int WM, int WN, bool GROUPED_OUT>
+__global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  using LA = TileLoader<T, BM, TA>;
+  using LB = TileLoader<T, BN, TB>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  T *sA = reinterpret_cast<T *>(smem_raw);   // [2][LA::ELEMS]
+  T *sB = sA + 2 * LA::ELEMS;                // [2][LB::ELEMS]
+
+  // XCD-aware tile order: consecutive workgroup ids land on different XCDs, so give
+  // each XCD a contiguous run of tiles; inside a run the m tile moves fastest (tiles
+  // that share a weight panel are neighbours in one L2).
+  const int ntiles = p.tiles_m * p.tiles_n;
+  int pid = blockIdx.x;
+  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  int tm = pid % p.tiles_m;
+  const int tn = pid / p.tiles_m;
+
+  const int base = p.offs[0];
+  int g = 0, row_begin = 0, row_end = 0;
+  if (GROUPED_OUT) {
+    // wgrad: one full [m_dim, n_dim] output per group; blockIdx.y = group
+    g = blockIdx.y;
+    row_begin = p.offs[g] - base;
+    row_end = p.offs[g + 1] - base;
+  } else {
+    bool found = false;
+    for (int gi = 0; gi < p.groups; ++gi) {
+      const int rb = p.offs[gi] - base, re = p.offs[gi + 1] - base;
+      const int t = (re - rb + BM - 1) / BM;
+      if (!found && tm < t) {
+        g = gi; row_begin = rb; row_end = re; found = true;
+      } else if (!found) {
+        tm -= t;
+      }
+    }
+    if (!found) return;
+  }
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int wm = w >> 1, wn = w & 1;
+  const int n0 = tn * BN;
+
+  // Operand origins and extents.
+  const T *ag, *bg;
+  int a_rext, b_rext;       // valid extent along the tile's non-k dimension
+  int64_t k_total;
+  if (GROUPED_OUT) {
+    // a [rows, m_dim] (k = row), b [rows, n_dim]
+    const int m0 = tm * BM;
+    ag = reinterpret_cast<const T *>(p.a) + (int64_t)row_begin * p.lda + m0;
+    bg = reinterpret_cast<const T *>(p.b) + (int64_t)row_begin * p.ldb + n0;
+    a_rext = (int)(p.m_dim - m0);
+    b_rext = (int)(p.n_dim - n0);
+    k_total = row_end - row_begin;
+  } else {
+    const int m0 = row_begin + tm * BM;
+    ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
+    a_rext = row_end - m0;
+    bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (TB ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+    b_rext = (int)(p.n_dim - n0);
+    k_total = p.k_dim;
+  }
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  uint4 ra[LA::LPT], rb[LB::LPT];
+  const int nslices = (int)((k_total + GG_BK - 1) / GG_BK);
+  auto gload = [&](int s) {
+    const int64_t k0 = (int64_t)s * GG_BK;
+    const int kext = (int)(k_total - k0 < GG_BK ? k_total - k0 : GG_BK);
+    LA::gload(ra, TA ? ag + k0 * p.lda : ag + k0, p.lda, a_rext, kext, tid);
+    LB::gload(rb, TB ? bg + k0 * p.ldb : bg + k0, p.ldb, b_rext, kext, tid);
+  };
+  if (nslices > 0) {
+    gload(0);
+    LA::sstore(ra, sA, tid);
+    LB::sstore(rb, sB, tid);
+  }
+  __syncthreads();
+
+  for (int s = 0; s < nslices; ++s) {
+    const int st = s & 1;
+    if (s + 1 < nslices) gload(s + 1);
+    const T *tA = sA + st * LA::ELEMS;
+    const T *tB = sB + st * LB::ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < GG_BK / 16; ++ks) {
+      Frag fa[WM], fb[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) fa[i] = LA::frag(tA, wm * 32 * WM + 32 * i, ks, lane);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) fb[j] = LB::frag(tB, wn * 32 * WN + 32 * j, ks, lane);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = M::mma(fb[j], fa[i], acc[i][j]);  // C^T block: rows n, cols m
+    }
+    if (s + 1 < nslices) {
+      LA::sstore(ra, sA + (st ^ 1) * LA::ELEMS, tid);
+      LB::sstore(rb, sB + (st ^ 1) * LB::ELEMS, tid);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
+  T *cg;
+  int m_lim;
+  if (GROUPED_OUT) {
+    cg = reinterpret_cast<T *>(p.c) + (int64_t)g * p.c_group_stride + (int64_t)(tm * BM) * p.ldc + n0;
+    m_lim = a_rext;
+  } else {
+    cg = reinterpret_cast<T *>(p.c) + (int64_t)(row_begin + tm * BM) * p.ldc + n0;
+    m_lim = a_rext;
+  }
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int m = wm * 32 * WM + 32 * i + c;
+    if (m < m_lim) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          const int n = wn * 32 * WN + 32 * j + 8 * vb + 4 * hh;
+          if (n < b_rext) {
+            struct alignas(8) Q4 { T v[4]; };
+            Q4 *dst = reinterpret_cast<Q4 *>(cg + (int64_t)m * p.ldc + n);
+            Q4 o;
+            if (p.accumulate) {
+              const Q4 old = *dst;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e] + static_cast<float>(old.v[e]));
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e]);
+            }
+            *dst = o;
+          }
+        }
+    }
+  }
+}
+
+template <typename T, bool TA, bool TB, int WM, int WN, bool GROUPED_OUT>
+static int launch_gg(GGParams p, int64_t m_extent, hipStream_t st) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  using LA = TileLoader<T, BM, TA>;
+  using LB = TileLoader<T, BN, TB>;
+  constexpr size_t smem = 2 * (LA::ELEMS + LB::ELEMS) * sizeof(T);
+  static_assert(smem <= 160 * 1024, "LDS budget");
+  static bool attr_set = false;
+  if (!attr_set) {
+    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&grouped_gemm_kernel<T, TA, TB, WM, WN, GROUPED_OUT>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    attr_set = true;
+  }
+  p.tiles_n = (int)cdiv(p.n_dim, BN);
+  p.tiles_m = GROUPED_OUT ? (int)cdiv(m_extent, BM) : (int)(cdiv(m_extent, BM) + p.groups);
+  if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), GROUPED_OUT ? (unsigned)p.groups : 1u);
+  hipLaunchKernelGGL((grouped_gemm_kernel<T, TA, TB, WM, WN, GROUPED_OUT>), grid, dim3(256), smem, st, p);
+  return DH_OK;
+}
+
+template <bool TA, bool TB, bool GROUPED_OUT>
+static int dispatch_gg(const GGParams &p, int64_t m_extent, int dtype, hipStream_t st) {
+  // 256x256 workgroup tiles when there is enough work to fill the chip with them, else 128x128.
+  const int64_t big_tiles = cdiv(m_extent, 256) * cdiv(p.n_dim, 256) * (GROUPED_OUT ? p.groups : 1);
+  const bool big = big_tiles >= 256;
+  if (dtype == DH_BF16)
+    return big ? launch_gg<bf16_t, TA, TB, 4, 4, GROUPED_OUT>(p, m_extent, st)
+               : launch_gg<bf16_t, TA, TB, 2, 2, GROUPED_OUT>(p, m_extent, st);
+  return big ? launch_gg<f16_t, TA, TB, 4, 4, GROUPED_OUT>(p, m_extent, st)
+             : launch_gg<f16_t, TA, TB, 2, 2, GROUPED_OUT>(p, m_extent, st);
+}
+
+static int gg_common_checks(const void *a, const void *b, void *c, const int32_t *offs, int groups, int dtype) {
+  DH_CHECK(groups >= 1 && groups <= GG_MAX_GROUPS, "groups=%d must be in [1, %d]", groups, GG_MAX_GROUPS);
+  DH_CHECK(dtype == DH_BF16 || dtype == DH_F16, "grouped GEMM supports bf16/fp16 (dtype %d)", dtype);
+  DH_CHECK(a && b && c && offs, "null pointer");
+  DH_CHECK(aligned16(a) && aligned16(b) && aligned16(c), "operands must be 16-byte aligned");
+  return DH_OK;
+}
+
+}  // namespace dh
+
+extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const int32_t *offs, int groups,
+                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(max_rows >= 0 && n >= 0 && k >= 0, "negative size");
+  if (max_rows == 0 || n == 0) return DH_OK;
+  int rc = gg_common_checks(a, b, c, offs, groups, dtype);
+  if (rc) return rc;
+  DH_CHECK(n % 8 == 0 && k % 8 == 0, "n=%lld and k=%lld must be multiples of 8", (long long)n, (long long)k);
+  GGParams p{};
+  p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
+  p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
+  p.b_group_stride = n * k; p.accumulate = 0;
+  rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
+  if (rc) return rc;
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const int32_t *offs, int groups,
+                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(max_rows >= 0 && n >= 0 && k >= 0, "negative size");
+  if (max_rows == 0 || n == 0) return DH_OK;
+  int rc = gg_common_checks(a, b, c, offs, groups, dtype);
+  if (rc) return rc;
+  DH_CHECK(n % 8 == 0 && k % 8 == 0, "n=%lld and k=%lld must be multiples of 8", (long long)n, (long long)k);
+  GGParams p{};
+  p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
+  p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = n; p.ldc = n;
+  p.b_group_stride = n * k; p.accumulate = 0;
+  rc = dispatch_gg<false, true, false>(p, max_rows, dtype, (hipStream_t)stream);
+  if (rc) return rc;
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_grouped_gemm_tn(const void *a, const void *b, void *c, const int32_t *offs, int groups,
+                                  int64_t max_rows, int64_t m, int64_t n, int accumulate, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(max_rows >= 0 && n >= 0 && m >= 0, "negative size");
+  if (m == 0 || n == 0) return DH_OK;
+  int rc = gg_common_checks(a, b, c, offs, groups, dtype);
+  if (rc) return rc;
+  DH_CHECK(n % 8 == 0 && m % 8 == 0, "m=%lld and n=%lld must be multiples of 8", (long long)m, (long long)n);
+  GGParams p{};
+  p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
+  p.m_dim = m; p.n_dim = n; p.lda = m; p.ldb = n; p.ldc = n;
+  p.c_group_stride = m * n; p.accumulate = accumulate;
+  rc = dispatch_gg<true, true, true>(p, m, dtype, (hipStream_t)stream);
+  if (rc) return rc;
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}

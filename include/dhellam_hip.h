@@ -173,42 +173,48 @@ int dh_moe_route_topk(const float *logits, int32_t *topk_idx, float *gates,
                       int64_t tokens, int experts, int k, void *stream);
 
 size_t dh_moe_sort_workspace_bytes(int64_t n_assign, int experts);
-/* Stable counting sort of the flat assignment list topk_idx [n_assign] by
- * expert id.  tokens_per_expert int32 [experts]; sorted_idx int32 [n_assign]
- * (flat assignment ids in sorted order); dest_row int32 [n_assign] (position
- * of each assignment in the sorted order). */
+/* Stable counting sort of the flat assignment list topk_idx [n_assign]
+ * (assignment a = token*k + j) by expert id.  tokens_per_expert int32
+ * [experts]; expert_offsets int32 [experts+1] (exclusive scan of the counts);
+ * sorted_idx int32 [n_assign] (assignment ids in sorted order); dest_row int32
+ * [n_assign] (position of each assignment in the sorted order). */
 int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert,
-                int32_t *sorted_idx, int32_t *dest_row, void *workspace,
-                int64_t n_assign, int experts, void *stream);
+                int32_t *expert_offsets, int32_t *sorted_idx, int32_t *dest_row,
+                void *workspace, int64_t n_assign, int experts, void *stream);
 
-/* permuted[r] = scale * x[src_assign[r] / k] for r in [0, n_rows), where
- * src_assign = sorted_idx + first_row (a device pointer offset by the caller)
- * and scale = row_scale[src_assign[r]] if row_scale != NULL else 1.
- * n_rows is read ON DEVICE from *n_rows_dev (no host sync); the launch covers
- * max_rows. */
-int dh_moe_gather_rows(const void *x, const int32_t *src_assign,
+/* The rows of local experts [e_lo, e_hi) are the sorted positions
+ * [first, first + n_rows) with first = expert_offsets[e_lo] and n_rows =
+ * expert_offsets[e_hi] - first, both read ON DEVICE (no host sync); launches
+ * cover max_rows / tokens.
+ *
+ * gather: permuted[r] = scale * x[sorted_idx[first + r] / k] for r < n_rows,
+ * scale = row_scale[sorted_idx[first + r]] if row_scale != NULL else 1. */
+int dh_moe_gather_rows(const void *x, const int32_t *sorted_idx,
                        const float *row_scale, void *permuted,
-                       const int32_t *n_rows_dev, int64_t max_rows, int k,
-                       int64_t hidden, int dtype, void *stream);
+                       const int32_t *expert_offsets, int e_lo, int e_hi,
+                       int64_t max_rows, int k, int64_t hidden, int dtype,
+                       void *stream);
 
-/* out[t] = sum_j w(t,j) * y[dest_row[t*k+j] - first_row] over the j whose
- * sorted position falls in [first_row, first_row + n_rows); w = gates[t*k+j]
- * or 1 if gates == NULL.  Tokens with no local assignment get zeros.
- * first_row / n_rows are read on device from range_dev[0..1]. */
+/* scatter: out[t] = sum_j w(t,j) * y[dest_row[t*k+j] - first] over the j whose
+ * sorted position is local; w = gates[t*k+j], or 1 if gates == NULL.  Tokens
+ * with no local assignment get zeros.  j order is fixed (deterministic). */
 int dh_moe_scatter_rows(const void *y, const int32_t *dest_row,
                         const float *gates, void *out,
-                        const int32_t *range_dev, int64_t tokens, int k,
-                        int64_t hidden, int dtype, void *stream);
+                        const int32_t *expert_offsets, int e_lo, int e_hi,
+                        int64_t tokens, int k, int64_t hidden, int dtype,
+                        void *stream);
 
-/* dgates[t*k+j] = <dout[t], y[dest_row[t*k+j]-first_row]> (0 if not local). */
+/* dgates[t*k+j] = <dout[t], y[dest_row[t*k+j]-first]> (0 if not local). */
 int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *dest_row,
-                     float *dgates, const int32_t *range_dev, int64_t tokens,
-                     int k, int64_t hidden, int dtype, void *stream);
+                     float *dgates, const int32_t *expert_offsets, int e_lo,
+                     int e_hi, int64_t tokens, int k, int64_t hidden, int dtype,
+                     void *stream);
 
 /* ------------------------------------------------------------------------
  * Grouped GEMM on MFMA (bf16/fp16 in, fp32 accumulate).  No counterpart in
- * the reference.  Group g owns rows [offs[g], offs[g+1]) (device int32
- * [groups+1], read on device).
+ * the reference.  Group g owns rows [offs[g]-offs[0], offs[g+1]-offs[0]) of
+ * the stacked row dimension (offs: device int32 [groups+1], read on device,
+ * so a slice of expert_offsets can be passed as is).
  *   NT: c[rows_g, n] = a[rows_g, k] * b[g][n, k]^T          (forward)
  *   NN: c[rows_g, n] = a[rows_g, k] * b[g][k, n]            (dgrad)
  *   TN: c[g][m, n] (+)= a[rows_g, m]^T * b[rows_g, n]       (wgrad)

@@ -1,0 +1,158 @@
+"""GPU parity of MoE routing / sort / permute / unpermute (bit-exact indices) and of the
+MFMA grouped GEMM and expert FFN against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe as OM
+from tests.util import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+
+
+def _logits(T, E, seed, ties=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((T, E), generator=g, dtype=torch.float32)
+    if ties:
+        x = torch.round(x * 2) / 2          # many exact ties
+    return x
+
+
+@pytest.mark.parametrize("T,E,k,ties", [(8192, 8, 2, False), (1000, 8, 2, True), (33, 64, 8, True), (5, 3, 1, False),
+                                         (4096, 16, 4, True)])
+def test_route_topk_bit_exact(T, E, k, ties):
+    from dhellam_amd.operators.moe import route_topk
+    lg = _logits(T, E, 1, ties)
+    idx, gates, ms = route_topk(lg.cuda(), k)
+    io, go = OM.route_topk(lg.numpy(), k)
+    assert np.array_equal(idx.cpu().numpy(), io), "top-k indices must be bit-exact"
+    assert_close(gates, torch.from_numpy(go), torch.float32, "gates", scale=2)
+    assert torch.allclose(gates.sum(1).cpu(), torch.ones(T), atol=1e-6)
+
+
+@pytest.mark.parametrize("T,E,k", [(8192, 8, 2), (1000, 8, 2), (3000, 64, 8), (1, 4, 1), (1025, 5, 3)])
+def test_sort_bit_exact(T, E, k):
+    from dhellam_amd.operators.moe import sort_assignments
+    io, _ = OM.route_topk(_logits(T, E, 2, True).numpy(), k)
+    plan, _ = sort_assignments(torch.from_numpy(io).cuda(), E)
+    tpe, offs, sidx, dest = OM.sort_assignments(io, E)
+    assert np.array_equal(plan.tokens_per_expert.cpu().numpy(), tpe)
+    assert np.array_equal(plan.expert_offsets.cpu().numpy(), offs)
+    assert np.array_equal(plan.sorted_idx.cpu().numpy(), sidx), "stable sort order must be bit-exact"
+    assert np.array_equal(plan.dest_row.cpu().numpy(), dest)
+
+
+def test_sort_skewed_and_empty_experts():
+    from dhellam_amd.operators.moe import sort_assignments
+    idx = np.zeros((5000, 2), dtype=np.int32)
+    idx[:, 1] = 7                                  # experts 1..6 receive nothing
+    plan, _ = sort_assignments(torch.from_numpy(idx).cuda(), 8)
+    tpe, offs, sidx, dest = OM.sort_assignments(idx, 8)
+    assert np.array_equal(plan.tokens_per_expert.cpu().numpy(), tpe)
+    assert np.array_equal(plan.sorted_idx.cpu().numpy(), sidx)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,H,E,k,e_lo,e_hi", [(8192, 4096, 8, 2, 0, 2), (777, 520, 8, 2, 2, 5), (300, 100, 4, 1, 0, 4),
+                                                (64, 256, 8, 2, 7, 8)])
+def test_permute_unpermute(dtype, T, H, E, k, e_lo, e_hi):
+    from dhellam_amd.operators import moe
+    lg = _logits(T, E, 3)
+    idx, gates, _ = moe.route_topk(lg.cuda(), k)
+    plan, _ = moe.sort_assignments(idx, E)
+    io, go = OM.route_topk(lg.numpy(), k)
+    tpe, offs, sidx, dest = OM.sort_assignments(io, E)
+    R = int(offs[e_hi] - offs[e_lo])
+    max_rows = R + 37
+    x = randn((T, H), dtype, 4)
+    xp, _ = moe.permute_fwd(x.cuda(), plan, e_lo, e_hi, max_rows)
+    xo = OM.permute(x, sidx, offs, e_lo, e_hi, k)
+    assert torch.equal(xp[:R].cpu(), xo.to(dtype)), "permute is a pure row copy: must be bit-exact"
+    assert xp[R:].abs().max().item() == 0 if max_rows > R else True
+    # unpermute with gates
+    y = randn((max_rows, H), dtype, 5)
+    out, _ = moe.unpermute_fwd(y.cuda(), plan, gates, e_lo, e_hi)
+    oo = OM.unpermute(y[:R], dest, offs, e_lo, e_hi, T, k, gates.cpu())
+    assert_close(out, oo, dtype, "unpermute")
+    # backward pieces
+    dxo = OM.unpermute(y[:R], dest, offs, e_lo, e_hi, T, k, None)
+    dx, _ = moe.permute_bwd(y.cuda(), plan, e_lo, e_hi)
+    assert_close(dx, dxo, dtype, "permute_bwd")
+    dout = randn((T, H), dtype, 6)
+    dy, dg, _ = moe.unpermute_bwd(dout.cuda(), y.cuda(), plan, gates, e_lo, e_hi, max_rows)
+    dyo = OM.permute(dout, sidx, offs, e_lo, e_hi, k, row_scale=gates.cpu())
+    assert_close(dy[:R], dyo, dtype, "unpermute_bwd dy")
+    dgo = OM.gate_grad(dout, y[:R], dest, offs, e_lo, e_hi, T, k)
+    assert_close(dg, dgo, torch.float32, "dgates", scale=10 if dtype == torch.float32 else 1e3)
+
+
+def test_permute_roundtrip_identity():
+    """top-1, gates 1, all experts local: unpermute(permute(x)) == x exactly."""
+    from dhellam_amd.operators import moe
+    T, H, E = 2048, 512, 8
+    lg = _logits(T, E, 7)
+    idx, gates, _ = moe.route_topk(lg.cuda(), 1)
+    plan, _ = moe.sort_assignments(idx, E)
+    x = randn((T, H), torch.bfloat16, 8).cuda()
+    xp, _ = moe.permute_fwd(x, plan, 0, E, T)
+    back, _ = moe.unpermute_fwd(xp, plan, torch.ones_like(gates), 0, E)
+    assert torch.equal(back, x)
+    assert int(plan.tokens_per_expert.sum()) == T
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,N,K", [([300, 212], 512, 256), ([1000, 0, 24], 1024, 520), ([2048, 2048], 2048, 1024),
+                                       ([5], 64, 64)])
+def test_grouped_gemm_variants(dtype, rows, N, K):
+    from dhellam_amd.operators import moe
+    G = len(rows)
+    offs = torch.tensor(np.concatenate(([7], 7 + np.cumsum(rows))), dtype=torch.int32)   # non-zero base on purpose
+    R = sum(rows)
+    a = randn((R, K), dtype, 1, std=0.5)
+    b = randn((G, N, K), dtype, 2, std=0.5)
+    c = moe.grouped_gemm_nt(a.cuda(), b.cuda(), offs.cuda())
+    ref = torch.cat([a[sum(rows[:g]):sum(rows[:g + 1])].double() @ b[g].double().T for g in range(G)])
+    assert_close(c, ref, dtype, "NT")
+    bt = b.transpose(1, 2).contiguous()   # [G, K, N]
+    c2 = moe.grouped_gemm_nn(a.cuda(), bt.cuda(), offs.cuda())
+    assert_close(c2, ref, dtype, "NN")
+    d = randn((R, N), dtype, 3, std=0.5)
+    w = moe.grouped_gemm_tn(d.cuda(), a.cuda(), offs.cuda())
+    wref = torch.stack([d[sum(rows[:g]):sum(rows[:g + 1])].double().T @ a[sum(rows[:g]):sum(rows[:g + 1])].double()
+                        for g in range(G)])
+    assert_close(w, wref, dtype, "TN")
+    acc0 = randn((G, N, K), dtype, 4)
+    acc = acc0.clone().cuda()
+    moe.grouped_gemm_tn(d.cuda(), a.cuda(), offs.cuda(), out=acc, accumulate=True)
+    assert_close(acc, wref + acc0.double(), dtype, "TN accumulate")
+
+
+def test_expert_ffn_fwd_bwd():
+    from dhellam_amd.operators import moe
+    dtype = torch.bfloat16
+    T, H, F, E, k = 1024, 512, 768, 8, 2
+    lg = _logits(T, E, 9)
+    idx, gates, _ = moe.route_topk(lg.cuda(), k)
+    plan, _ = moe.sort_assignments(idx, E)
+    offs_cpu = plan.expert_offsets.cpu().numpy()
+    e_lo, e_hi = 0, 2
+    R = int(offs_cpu[e_hi] - offs_cpu[e_lo])
+    x = randn((T, H), dtype, 10)
+    w1 = randn((2, 2 * F, H), dtype, 11, std=0.02)
+    w2 = randn((2, H, F), dtype, 12, std=0.02)
+    xp, _ = moe.permute_fwd(x.cuda(), plan, e_lo, e_hi, R)
+    offs = plan.expert_offsets[e_lo:e_hi + 1]
+    y, saved, _ = moe.expert_ffn_fwd(xp, w1.cuda(), w2.cuda(), offs)
+    yo, ho, ao = OM.grouped_ffn(xp.cpu(), w1, w2, offs_cpu[e_lo:e_hi + 1], round_to=dtype)
+    assert_close(saved[0], ho, dtype, "h")
+    assert_close(y, yo, dtype, "ffn out")
+    # backward against autograd of the fp64 oracle (no intermediate rounding there: tolerance 2x)
+    dy = randn((R, H), dtype, 13)
+    xr = xp.cpu().double().requires_grad_()
+    w1r, w2r = w1.double().requires_grad_(), w2.double().requires_grad_()
+    yr, _, _ = OM.grouped_ffn(xr, w1r, w2r, offs_cpu[e_lo:e_hi + 1])
+    (yr * dy.double()).sum().backward()
+    dxp, dw1, dw2, _ = moe.expert_ffn_bwd(dy.cuda(), xp, w1.cuda(), w2.cuda(), offs, saved)
+    assert_close(dxp, xr.grad, dtype, "dxp", scale=2)
+    assert_close(dw1, w1r.grad, dtype, "dw1", scale=2)
+    assert_close(dw2, w2r.grad, dtype, "dw2", scale=2)

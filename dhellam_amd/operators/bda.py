@@ -12,9 +12,10 @@ from .. import _lib
 from ._util import on_stream
 
 
-def bda_fwd(input, residual, stream=None, profiling=False, p: float = 0.0, return_mask: bool = False):
-    """In place on ``input`` like the reference.  Returns (output, mask, ms); mask is
-    None unless ``return_mask`` (then an int8 ones tensor)."""
+def bda_fwd(input, residual, stream=None, profiling=False, p: float = 0.0, return_mask: bool = False, out=None):
+    """In place on ``input`` like the reference, unless ``out`` (same numel/dtype) is given.
+    Returns (output, mask, ms); mask is None unless ``return_mask`` (then an int8 ones
+    tensor)."""
     if p != 0.0:
         raise NotImplementedError("bda_fwd: only p = 0 (no dropout) is implemented")
     assert input.is_cuda and input.is_contiguous() and residual.is_contiguous()
@@ -22,10 +23,12 @@ def bda_fwd(input, residual, stream=None, profiling=False, p: float = 0.0, retur
     lib = _lib.load()
     el: list = []
     with on_stream(stream, profiling, el) as st:
-        _lib.check(lib.dh_residual_add(input.data_ptr(), residual.data_ptr(), input.data_ptr(), input.numel(),
+        dst = input if out is None else out
+        assert dst.is_contiguous() and dst.numel() == input.numel() and dst.dtype == input.dtype
+        _lib.check(lib.dh_residual_add(input.data_ptr(), residual.data_ptr(), dst.data_ptr(), input.numel(),
                                        _lib.dt(input), st.cuda_stream))
         mask = torch.ones_like(input, dtype=torch.int8) if return_mask else None
-    return input, mask, el[0]
+    return dst, mask, el[0]
 
 
 def bda_bwd(dgrad, mask, output=None, stream=None, profiling=False):

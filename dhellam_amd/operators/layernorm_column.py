@@ -1,0 +1,101 @@
+"""Dense projection GEMMs with the reference's wrapper signatures.
+
+Mirrors dhellam/operators/layernorm_column.py:7-62 (``gemm_fwd``), :209-263
+(``dgrad_bwd``) and :265-323 (``wgrad_bwd``).  Weights are stored [out, in];
+the layout letters are the reference's: "TN" computes input @ weight.T, "NN"
+grad @ weight, "NT" grad.T @ input.  Dense GEMM is a library call on this path
+(hipBLASLt through ``torch.matmul``), exactly what every scheduler call site of
+the reference selects with ``is_matmul=True`` (dhellam/core/dstb.py:84-106,
+300-340); with ``is_matmul=False`` the same product goes through ``_Clib.pygemm``.
+Output dtype follows the inputs (the reference hard-codes fp16).  Elapsed time
+is in milliseconds, measured with events on the op's stream.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .._Clib import pygemm as gemm
+from ._util import on_stream
+
+
+def gemm_fwd(args, input: torch.Tensor, weight: torch.Tensor, output: Optional[torch.Tensor] = None,
+             layout: str = "TN", profiling: bool = False, math_sm_count: int = 0, is_matmul: bool = False,
+             stream=None):
+    transa = layout[0] == "T"
+    transb = layout[1] == "T"
+    el: list = []
+    with on_stream(stream, profiling, el):
+        if is_matmul:
+            w = weight.t() if transa else weight
+            x = input.t() if transb else input
+            output = torch.matmul(x, w) if output is None else torch.matmul(x, w, out=output)
+        else:
+            if output is None:
+                output = torch.empty(input.shape[1] if transb else input.shape[0],
+                                     weight.shape[0] if transa else weight.shape[1], dtype=input.dtype,
+                                     device=input.device)
+            gemm(weight, input, output, None, 0, transa, transb, False, math_sm_count, False)
+    return output, el[0]
+
+
+def dgrad_bwd(args, input_grad: torch.Tensor, weight: torch.Tensor, dgrad_output: Optional[torch.Tensor],
+              layout: str = "NN", profiling: bool = False, math_sm_count: int = 0, is_matmul: bool = False,
+              stream=None):
+    transa = layout[0] == "T"
+    transb = layout[1] == "T"
+    el: list = []
+    with on_stream(stream, profiling, el):
+        if dgrad_output is None:
+            dgrad_output = torch.empty(input_grad.shape[1] if transb else input_grad.shape[0],
+                                       weight.shape[0] if transa else weight.shape[1], dtype=input_grad.dtype,
+                                       device=input_grad.device)
+        if is_matmul:
+            w = weight.t() if transa else weight
+            g = input_grad.t() if transb else input_grad
+            torch.matmul(g, w, out=dgrad_output)
+        else:
+            gemm(weight, input_grad, dgrad_output, None, 0, transa, transb, False, math_sm_count, False)
+    return dgrad_output, el[0]
+
+
+def wgrad_bwd(args, input_grad: torch.Tensor, input_data: torch.Tensor, wgrad_output: Optional[torch.Tensor],
+              grad_accumulate: bool = False, layout: str = "NT", profiling: bool = False, math_sm_count: int = 0,
+              is_matmul: bool = False, stream=None):
+    """wgrad [out, in] = input_grad.T @ input_data.  As in the reference's matmul path
+    (layernorm_column.py:289-292) a given ``wgrad_output`` is ACCUMULATED into."""
+    transa = layout[0] == "T"
+    transb = layout[1] == "T"
+    el: list = []
+    with on_stream(stream, profiling, el):
+        if is_matmul:
+            d = input_data.t() if transa else input_data
+            g = input_grad.t() if transb else input_grad
+            if wgrad_output is None:
+                wgrad_output = torch.matmul(g, d)
+            elif wgrad_output.dtype == g.dtype:
+                wgrad_output.addmm_(g, d)
+            else:  # fp32 main_grad with 16-bit operands
+                wgrad_output.add_(torch.matmul(g, d))
+        else:
+            if wgrad_output is None:
+                wgrad_output = torch.empty(input_grad.shape[1] if transb else input_grad.shape[0],
+                                           input_data.shape[0] if transa else input_data.shape[1],
+                                           dtype=input_grad.dtype, device=input_grad.device)
+                grad_accumulate = False
+            gemm(input_data, input_grad, wgrad_output, None, 0, transa, transb, grad_accumulate, math_sm_count, False)
+    return wgrad_output, el[0]
+
+
+def gemm_bwd(args, input_grad, input_data, weight, dgrad_output=None, wgrad_output=None, grad_accumulate=False,
+             profiling=False, math_sm_count=0, is_matmul=True, stream=None):
+    """dgrad then wgrad of one projection (layernorm_column.py:121-207).
+    Returns (dgrad, wgrad, dgrad_ms, wgrad_ms)."""
+    dgrad_output, t1 = dgrad_bwd(args, input_grad, weight, dgrad_output, "NN", profiling, math_sm_count, is_matmul, stream)
+    wgrad_output, t2 = wgrad_bwd(args, input_grad, input_data, wgrad_output, grad_accumulate, "NT", profiling,
+                                 math_sm_count, is_matmul, stream)
+    return dgrad_output, wgrad_output, t1, t2
+
+
+gemm_fwd_event = gemm_fwd  # the reference's event-timed twin (layernorm_column.py:64-119); timing is always by event here

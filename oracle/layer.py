@@ -1,0 +1,113 @@
+"""Oracle for one pre-norm Llama decoder layer, forward and backward (autograd).
+
+Test infrastructure: eager PyTorch on the CPU.  This is also "the PyTorch CPU eager
+path" whose time is reported beside the GPU numbers.
+
+Layer (dropout 0, no biases), following the op chain of dhellam/core/dstb.py:700-757:
+  h1 = RMSNorm(x) -> [gather] -> qkv = X Wqkv^T -> RoPE(q, k) -> causal GQA attention
+  -> a = o Wo^T -> [scatter] -> x2 = x + a -> h2 = RMSNorm(x2) -> [gather]
+  -> u = X2 Wgu^T (gate | up) -> m = silu(gate) * up -> y = m Wd^T -> [scatter] -> out = x2 + y
+QKV packing per kv group g: [q heads of g | k_g | v_g].
+Sequence-parallel stand-ins (one rank's view, no cross-rank sum): gather(h, P) writes the
+rank's rows into the peer tensor P and returns it, its backward returns the rank's row
+slice of the incoming gradient; scatter(a, G) returns the rank's row slice, its backward
+writes the slice's gradient into the peer-gradient tensor G and returns that.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import ops as O
+
+
+class _Gather(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, h, peer, r0, r1):
+        ctx.r = (r0, r1)
+        out = peer.clone()
+        out[r0:r1] = h
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        r0, r1 = ctx.r
+        return g[r0:r1], None, None, None
+
+
+class _Scatter(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, peer_grad, r0, r1):
+        ctx.r = (r0, r1)
+        ctx.save_for_backward(peer_grad)
+        return a[r0:r1].clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        r0, r1 = ctx.r
+        (pg,) = ctx.saved_tensors
+        out = pg.clone()
+        out[r0:r1] = g
+        return out, None, None, None
+
+
+def _rms(x, gamma, eps):
+    return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * gamma
+
+
+def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=None):
+    """cfg: hidden, heads (q heads on this rank), groups (kv heads on this rank), head_dim,
+    ffn (per rank), seq, batch, tp, tp_rank, eps, theta.  w: column_attn_weight,
+    linear_attn_weight, column_mlp_weight, linear_mlp_weight, ln_attn_weight,
+    ln_mlp_weight.  mb: x, dy [b, seq/tp, hidden] (+ sp_peer_* [b*seq, hidden] when tp > 1).
+    ``round_to``: dtype every op's output is rounded to (models a 16-bit pipeline).
+    Returns (out, grads) with grads = {x, ln_attn_weight, ln_mlp_weight, column_attn_weight,
+    linear_attn_weight, column_mlp_weight, linear_mlp_weight}."""
+    rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
+    hq, hk, d, F = cfg["heads"], cfg["groups"], cfg["head_dim"], cfg["ffn"]
+    b, s, tp, rk = cfg["batch"], cfg["seq"], cfg["tp"], cfg["tp_rank"]
+    H = cfg["hidden"]
+    T = b * s
+    rows = T // tp
+    r0, r1 = rk * rows, (rk + 1) * rows
+    P = {k: v.to(dtype).requires_grad_() for k, v in w.items()}
+    x = mb["x"].to(dtype).reshape(rows, H).requires_grad_()
+    dy = mb["dy"].to(dtype).reshape(rows, H)
+
+    def gather(h, key):
+        return _Gather.apply(h, mb[key].to(dtype), r0, r1) if tp > 1 else h
+
+    def scatter(a, key):
+        return _Scatter.apply(a, mb[key].to(dtype), r0, r1) if tp > 1 else a
+
+    h1 = rnd(_rms(x, P["ln_attn_weight"], cfg["eps"]))
+    X = gather(h1, "sp_peer_attn")
+    qkv = rnd(X @ P["column_attn_weight"].T)                              # [T, (hq + 2 hk) d]
+    r = hq // hk
+    g = qkv.view(T, hk, (r + 2) * d)
+    q = g[:, :, : r * d].reshape(T, hq, d)
+    k = g[:, :, r * d:(r + 1) * d]
+    v = g[:, :, (r + 1) * d:]
+    pos = torch.arange(T) % s
+    if cfg.get("theta") is not None:
+        q = rnd(O.rope(q, pos, cfg["theta"], dtype=dtype))
+        k = rnd(O.rope(k, pos, cfg["theta"], dtype=dtype))
+    qh = q.view(b, s, hq, d).permute(0, 2, 1, 3)
+    kh = k.reshape(b, s, hk, d).repeat_interleave(r, dim=2).permute(0, 2, 1, 3)
+    vh = v.reshape(b, s, hk, d).repeat_interleave(r, dim=2).permute(0, 2, 1, 3)
+    sc = torch.matmul(qh, kh.transpose(2, 3)) / math.sqrt(d)
+    sc = sc.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+    o = rnd(torch.matmul(torch.softmax(sc, -1), vh).permute(0, 2, 1, 3).reshape(T, hq * d))
+    a = rnd(o @ P["linear_attn_weight"].T)
+    x2 = rnd(x + scatter(a, "sp_peer_attn_bwd"))
+    h2 = rnd(_rms(x2, P["ln_mlp_weight"], cfg["eps"]))
+    X2 = gather(h2, "sp_peer_mlp")
+    u = rnd(X2 @ P["column_mlp_weight"].T)
+    m = rnd(u[:, :F] * torch.sigmoid(u[:, :F]) * u[:, F:])
+    y = rnd(m @ P["linear_mlp_weight"].T)
+    out = rnd(x2 + scatter(y, "sp_peer_mlp_bwd"))
+    (out * dy).sum().backward()
+    grads = {k: v.grad for k, v in P.items()}
+    grads["x"] = x.grad.view(b, rows // b, H)
+    return out.detach().view(b, rows // b, H), grads

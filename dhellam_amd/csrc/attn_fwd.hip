@@ -195,6 +195,304 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Head dim 128, second-generation kernel.
+//
+// A workgroup is 8 wavefronts = RG row groups (32 query rows each) x SPLIT key/value
+// splits.  Every iteration SPLIT tiles of BN keys are resident; split s works on tile
+// it*SPLIT + s, so two wavefronts share each SIMD with independent instruction streams
+// (one in MFMA while the other is in the softmax), and they share every K/V tile through
+// LDS.  The partial (O, m, l) of the splits are combined through LDS at the end.
+// K/V tiles go global -> LDS directly (16 bytes per lane, no staging registers, two
+// stages); rows are unpadded 256 B and bank conflicts are avoided by an XOR swizzle of
+// the 16-byte chunk index, applied on the global-address side of the copy:
+//   K (read as 16 B row fragments):  chunk ^= row % 16
+//   V (read with transpose loads) :  chunk ^= 4 * (row % 4) + (row / 4) % 4
+// Causal work is made uniform by giving a workgroup the query tiles i and n-1-i.
+// Issue the copies of one pipeline stage: this wavefront's LD 1 KB blocks (4 rows of a K or V tile each).
+template <typename T, int SPLIT, int BN, int LD>
+__device__ __forceinline__ void fwd_issue_stage(T *stage, const T *kg, const T *vg, int k_stride, int v_stride, int it,
+                                                int ntiles, int sk, int w, int lrow, int l16) {
+  constexpr int TILE = BN * 128;
+#pragma unroll
+  for (int i = 0; i < LD; ++i) {
+    const int blk = w * LD + i;                  // 1 KB block inside the stage (wave-uniform)
+    const int tile = blk / (BN / 2);
+    const int kvsel = (blk % (BN / 2)) / (BN / 4);
+    const int rgp = blk % (BN / 4);
+    const int tile_g = it * SPLIT + tile;
+    if (tile_g < ntiles) {
+      const int row = 4 * rgp + lrow;
+      int kr = tile_g * BN + row;
+      kr = kr < sk ? kr : sk - 1;                // rows past the end are masked later; keep the read in bounds
+      const int f = kvsel ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
+      const T *src = (kvsel ? vg + (int64_t)kr * v_stride : kg + (int64_t)kr * k_stride) + ((l16 ^ f) * 8);
+      T *dst = stage + tile * 2 * TILE + kvsel * TILE + rgp * 512;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+    }
+  }
+}
+
+template <typename T, int RG, int SPLIT, int BN>
+__global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int D = 128, BM = 32 * RG, NB = BN / 32, NS = BN / 16;
+  static_assert(RG * SPLIT == 8, "8 wavefronts per workgroup");
+  constexpr int TILE = BN * D;                    // elements of one K (or V) tile
+  constexpr int STAGE = SPLIT * 2 * TILE;         // elements per pipeline stage
+  constexpr int BLK_PER_STAGE = STAGE * (int)sizeof(T) / 1024;  // 1 KB copy blocks per stage
+  constexpr int LD = BLK_PER_STAGE / 8;
+  static_assert(BLK_PER_STAGE % 8 == 0, "copy blocks must divide over the wavefronts");
+  // Two separate LDS objects, one per stage: reads of one stage are then known not to
+  // alias the copies in flight into the other, and need not wait for them.
+  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
+  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int nqt = (sq + BM - 1) / BM;
+  const int causal = p.causal;
+  const int k_stride = (int)p.k_stride, v_stride = (int)p.v_stride;
+  const float scale_log2 = p.scale_log2;
+  // causal: this workgroup owns query tiles (pair, nqt-1-pair); otherwise one tile
+  int qt[2], nq;
+  if (causal) {
+    const int pair = blockIdx.x;
+    if (2 * pair >= nqt) return;
+    qt[0] = nqt - 1 - pair;
+    qt[1] = pair;
+    nq = (qt[0] == qt[1]) ? 1 : 2;
+  } else {
+    if ((int)blockIdx.x >= nqt) return;
+    qt[0] = blockIdx.x; qt[1] = 0;
+    nq = 1;
+  }
+  const int hkv = h / (p.hq / p.hk);
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int rg = w % RG, sp = w / RG;
+  const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
+  const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
+
+  // ---- per-lane constants of the copy and of the fragment reads ---------------------------
+  const int l16 = lane & 15, lrow = lane >> 4;        // copy: chunk slot and row inside a 4-row block
+  const int xk = c & 15;                              // K row fragment: chunk ^= row % 16 (row = 32 nb + c)
+  const int r = lane & 15;
+  const int va_x = 4 * (r >> 2) + hh;                 // V transpose read, first four keys of a step
+  const int vb_x = va_x + 2;                          // second four keys (row + 8)
+  const int v_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  const int v_sub = (r & 3) & 1;
+
+  for (int qi = 0; qi < nq; ++qi) {
+    const int m0 = qt[qi] * BM;
+    const int wrow0 = m0 + rg * 32;
+    const int row_q = wrow0 + c;
+    const int row_ld = row_q < sq ? row_q : sq - 1;
+    const T *qp = reinterpret_cast<const T *>(p.q) + (int64_t)(q0 + row_ld) * p.q_stride + (int64_t)h * D;
+    Frag Qf[D / 16];
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) Qf[ks] = frag_ld<T>(qp + ks * 16 + 8 * hh);
+
+    int nk_end = sk;
+    if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
+    const int ntiles = (nk_end + BN - 1) / BN;
+    const int niter = (ntiles + SPLIT - 1) / SPLIT;
+
+    floatx16 O[D / 32];
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) O[t][v] = 0.f;
+    float m_run = -1e30f, l_run = 0.f;
+
+    // One tile of this wavefront's split, read from `stage`.
+    auto compute = [&](const T *stage, int it) {
+      const int tile_g = it * SPLIT + sp;
+      const int n0 = tile_g * BN;
+      if (tile_g >= ntiles || (causal && n0 > wrow0 + 31)) return;
+      const T *tK = stage + sp * 2 * TILE;
+      const T *tV = tK + TILE;
+      floatx16 S[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) S[nb][v] = 0.f;
+      {
+        // K fragments are fetched one step ahead of the MFMA that consumes them.
+        Frag a_cur = frag_ld<T>(tK + c * D + ((hh ^ xk) * 8));
+#pragma unroll
+        for (int i = 0; i < NB * (D / 16); ++i) {
+          const int nb = i / (D / 16), ks = i % (D / 16);
+          Frag a_nxt = a_cur;
+          if (i + 1 < NB * (D / 16)) {
+            const int nb2 = (i + 1) / (D / 16), ks2 = (i + 1) % (D / 16);
+            a_nxt = frag_ld<T>(tK + (nb2 * 32 + c) * D + (((2 * ks2 + hh) ^ xk) * 8));
+          }
+          S[nb] = M::mma(a_cur, Qf[ks], S[nb]);
+          a_cur = a_nxt;
+        }
+      }
+      const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+      if (need_mask) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int kv = n0 + nb * 32 + acc_row(v, hh);
+            if (kv >= sk || (causal && kv > row_q)) S[nb][v] = -INFINITY;
+          }
+      }
+      float mx = S[0][0];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      if (__any(m_new > m_run)) {
+        const float alpha = fast_exp2((m_run - m_new) * scale_log2);
+        l_run *= alpha;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) O[t][v] *= alpha;
+      }
+      m_run = m_new;
+      const float mc = m_new * scale_log2;
+      float ps = 0.f;
+      Frag Pb[NS];
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        float pv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          pv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
+          ps += pv[j];
+        }
+        Pb[s] = frag_pack<T>(pv);
+      }
+      l_run += ps;
+      // V^T fragments: transpose reads issued as one batch per 16-key step, consumed as they land.
+      // They are written in assembly so that they are not held back by the copies in flight
+      // into the OTHER stage (a transpose-read builtin would wait for every outstanding copy).
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const uint32_t ra = (uint32_t)(uintptr_t)(tV + (16 * s + 4 * hh + (r >> 2)) * D + v_sub * 4);
+        const uint32_t rb = ra + 8 * D * (uint32_t)sizeof(T);
+        uint32_t ad[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int lc = 4 * t + v_lc;
+          ad[2 * t] = ra + ((lc ^ va_x) * 16);
+          ad[2 * t + 1] = rb + ((lc ^ vb_x) * 16);
+        }
+        short4v f[8];
+        asm volatile("ds_read_b64_tr_b16 %0, %8\n\tds_read_b64_tr_b16 %1, %9\n\t"
+                     "ds_read_b64_tr_b16 %2, %10\n\tds_read_b64_tr_b16 %3, %11\n\t"
+                     "ds_read_b64_tr_b16 %4, %12\n\tds_read_b64_tr_b16 %5, %13\n\t"
+                     "ds_read_b64_tr_b16 %6, %14\n\tds_read_b64_tr_b16 %7, %15"
+                     : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&v"(f[4]), "=&v"(f[5]), "=&v"(f[6]), "=&v"(f[7])
+                     : "v"(ad[0]), "v"(ad[1]), "v"(ad[2]), "v"(ad[3]), "v"(ad[4]), "v"(ad[5]), "v"(ad[6]), "v"(ad[7])
+                     : "memory");
+#define DH_FWD_PV(t, cnt)                                                                  \
+        asm volatile("s_waitcnt lgkmcnt(" #cnt ")" : "+v"(f[2 * t]), "+v"(f[2 * t + 1]));  \
+        {                                                                                  \
+          short8v o8;                                                                      \
+          o8[0] = f[2 * t][0]; o8[1] = f[2 * t][1]; o8[2] = f[2 * t][2]; o8[3] = f[2 * t][3];              \
+          o8[4] = f[2 * t + 1][0]; o8[5] = f[2 * t + 1][1]; o8[6] = f[2 * t + 1][2]; o8[7] = f[2 * t + 1][3]; \
+          O[t] = M::mma(__builtin_bit_cast(Frag, o8), Pb[s], O[t]);                         \
+        }
+        DH_FWD_PV(0, 6)
+        DH_FWD_PV(1, 4)
+        DH_FWD_PV(2, 2)
+        DH_FWD_PV(3, 0)
+#undef DH_FWD_PV
+      }
+    };
+
+    if (niter > 0) fwd_issue_stage<T, SPLIT, BN, LD>(sStage0, kg, vg, k_stride, v_stride, 0, ntiles, sk, w, lrow, l16);
+    __syncthreads();
+    for (int it = 0; it < niter; it += 2) {
+      if (it + 1 < niter) fwd_issue_stage<T, SPLIT, BN, LD>(sStage1, kg, vg, k_stride, v_stride, it + 1, ntiles, sk, w, lrow, l16);
+      compute(sStage0, it);
+      __syncthreads();   // stage 1 has landed, and everyone is done with stage 0
+      if (it + 1 < niter) {
+        if (it + 2 < niter) fwd_issue_stage<T, SPLIT, BN, LD>(sStage0, kg, vg, k_stride, v_stride, it + 2, ntiles, sk, w, lrow, l16);
+        compute(sStage1, it + 1);
+        __syncthreads();
+      }
+    }
+
+    // ---- combine the key/value splits through LDS (fixed order: deterministic) --------------
+    // O of split s > 0, row group g -> slot x = (s-1)*RG + g: slots 0..3 in stage 0, the rest in stage 1;
+    // m and l after them in stage 1.
+    float *x0 = reinterpret_cast<float *>(sStage0);
+    float *x1 = reinterpret_cast<float *>(sStage1);
+    float *xml = x1 + 2 * 4096;
+    static_assert((SPLIT - 1) * RG <= 6, "exchange slots");
+    static_assert(STAGE * sizeof(T) >= 4 * 4096 * sizeof(float), "stage 0 holds four O slots");
+    static_assert(STAGE * sizeof(T) >= (2 * 4096 + 6 * 128) * sizeof(float), "stage 1 holds two O slots and m/l");
+    if (sp > 0) {
+      const int x = (sp - 1) * RG + rg;
+      float *dst = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(t * 16 + v) * 64 + lane] = O[t][v];
+      xml[x * 128 + lane] = m_run;
+      xml[x * 128 + 64 + lane] = l_run;
+    }
+    __syncthreads();
+    if (sp == 0) {
+#pragma unroll
+      for (int s2 = 1; s2 < SPLIT; ++s2) {
+        const int x = (s2 - 1) * RG + rg;
+        const float *src = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+        const float m_o = xml[x * 128 + lane], l_o = xml[x * 128 + 64 + lane];
+        const float m_new = fmaxf(m_run, m_o);
+        const float a_me = fast_exp2((m_run - m_new) * scale_log2);
+        const float a_o = fast_exp2((m_o - m_new) * scale_log2);
+        l_run = l_run * a_me + l_o * a_o;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) O[t][v] = O[t][v] * a_me + src[(t * 16 + v) * 64 + lane] * a_o;
+        m_run = m_new;
+      }
+      const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+      const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+      if (row_q < sq) {
+        T *op = reinterpret_cast<T *>(p.o) + (int64_t)(q0 + row_q) * p.o_stride + (int64_t)h * D;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int vb = 0; vb < 4; ++vb) {
+            struct alignas(8) { T v[4]; } o4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o4.v[j] = static_cast<T>(O[t][4 * vb + j] * inv);
+            *reinterpret_cast<decltype(o4) *>(op + 32 * t + 8 * vb + 4 * hh) = o4;
+          }
+        if (hh == 0)
+          p.lse[((int64_t)b * p.hq + h) * p.max_sq + row_q] = l_tot > 0.f ? m_run * p.scale + logf(l_tot) : -INFINITY;
+      }
+    }
+    __syncthreads();   // the exchange area is reused by the next query tile's copies
+  }
+}
+
+template <typename T, int RG, int SPLIT, int BN>
+static int launch_attn_fwd_d128(const AttnFwdParams &p, int batch, hipStream_t st) {
+  constexpr int BM = 32 * RG;
+  const int nqt = (int)cdiv(p.max_sq, BM);
+  dim3 grid((unsigned)(p.causal ? (nqt + 1) / 2 : nqt), (unsigned)p.hq, (unsigned)batch);
+  hipLaunchKernelGGL((attn_fwd_d128_kernel<T, RG, SPLIT, BN>), grid, dim3(512), 0, st, p);
+  return DH_OK;
+}
+
 template <typename T, int D, int NW>
 static int launch_attn_fwd(const AttnFwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * NW, BN = 64;
@@ -239,6 +537,7 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
   DH_CHECK(d == 64 || d == 128, "bf16/fp16 attention supports head dim 64 or 128 (got %d)", d);
   DH_CHECK(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && o_stride % 4 == 0,
            "token strides must keep rows 16-byte aligned");
+  DH_CHECK(k_stride < (1ll << 31) && v_stride < (1ll << 31), "token stride too large");
   DH_CHECK(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out), "q/k/v/out must be 16-byte aligned");
   AttnFwdParams p;
   p.q = q; p.k = k; p.v = v; p.o = out; p.lse = lse;
@@ -248,15 +547,18 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.causal = causal;
-  // Few query tiles (small batch*heads) -> smaller workgroups so the grid still covers the chip.
-  const int64_t blocks128 = cdiv(max_seqlen_q, 128) * hq * batch;
-  const bool small = blocks128 < 2 * 256;
   int rc;
-  if (dtype == DH_BF16) {
-    if (d == 128) rc = small ? launch_attn_fwd<bf16_t, 128, 2>(p, batch, st) : launch_attn_fwd<bf16_t, 128, 4>(p, batch, st);
-    else rc = small ? launch_attn_fwd<bf16_t, 64, 2>(p, batch, st) : launch_attn_fwd<bf16_t, 64, 4>(p, batch, st);
+  if (d == 128) {
+    // 128-row query tiles when that still gives every CU a workgroup, else 64-row tiles.
+    const int64_t wg128 = (causal ? (cdiv(max_seqlen_q, 128) + 1) / 2 : cdiv(max_seqlen_q, 128)) * hq * batch;
+    const bool big = wg128 >= 256;
+    if (dtype == DH_BF16) rc = big ? launch_attn_fwd_d128<bf16_t, 4, 2, 64>(p, batch, st) : launch_attn_fwd_d128<bf16_t, 2, 4, 32>(p, batch, st);
+    else rc = big ? launch_attn_fwd_d128<f16_t, 4, 2, 64>(p, batch, st) : launch_attn_fwd_d128<f16_t, 2, 4, 32>(p, batch, st);
   } else {
-    if (d == 128) rc = small ? launch_attn_fwd<f16_t, 128, 2>(p, batch, st) : launch_attn_fwd<f16_t, 128, 4>(p, batch, st);
+    // Few query tiles (small batch*heads) -> smaller workgroups so the grid still covers the chip.
+    const int64_t blocks128 = cdiv(max_seqlen_q, 128) * hq * batch;
+    const bool small = blocks128 < 2 * 256;
+    if (dtype == DH_BF16) rc = small ? launch_attn_fwd<bf16_t, 64, 2>(p, batch, st) : launch_attn_fwd<bf16_t, 64, 4>(p, batch, st);
     else rc = small ? launch_attn_fwd<f16_t, 64, 2>(p, batch, st) : launch_attn_fwd<f16_t, 64, 4>(p, batch, st);
   }
   if (rc != DH_OK) return rc;

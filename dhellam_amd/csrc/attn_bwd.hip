@@ -434,6 +434,468 @@ __global__ void __launch_bounds__(64 * NW) attn_bwd_dq_kernel(const AttnBwdParam
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Head dim 128, second-generation kernels: direct global->LDS copies into swizzled tiles
+// (no staging registers, no bank conflicts), two pipeline stages held in separate LDS
+// objects, causal work made uniform by pairing tile i with tile n-1-i.
+// ---------------------------------------------------------------------------------------------
+
+// dQ: 8 wavefronts = RG query row groups x SPLIT key splits (as the forward kernel); the
+// partial dQ of the splits are added through LDS in split order.
+template <typename T, int RG, int SPLIT, int BN>
+__global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int D = 128, BM = 32 * RG, NB = BN / 32, NS = BN / 16;
+  static_assert(RG * SPLIT == 8, "8 wavefronts per workgroup");
+  constexpr int TILE = BN * D;
+  constexpr int STAGE = SPLIT * 2 * TILE;                       // K and V tile per split
+  constexpr int BLK_PER_STAGE = STAGE * (int)sizeof(T) / 1024;
+  constexpr int LD = BLK_PER_STAGE / 8;
+  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
+  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int nqt = (sq + BM - 1) / BM;
+  const int causal = p.causal;
+  const int k_stride = (int)p.k_stride, v_stride = (int)p.v_stride;
+  const float scale_log2 = p.scale_log2;
+  int qt[2], nq;
+  if (causal) {
+    const int pair = blockIdx.x;
+    if (2 * pair >= nqt) return;
+    qt[0] = nqt - 1 - pair; qt[1] = pair;
+    nq = (qt[0] == qt[1]) ? 1 : 2;
+  } else {
+    if ((int)blockIdx.x >= nqt) return;
+    qt[0] = blockIdx.x; qt[1] = 0; nq = 1;
+  }
+  const int hkv = h / (p.hq / p.hk);
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int rg = w % RG, sp = w / RG;
+  const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
+  const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
+  const int lrow = lane >> 4;
+
+  for (int qi = 0; qi < nq; ++qi) {
+    const int m0 = qt[qi] * BM;
+    const int wrow0 = m0 + rg * 32;
+    const int row_q = wrow0 + c;
+    const bool row_ok = row_q < sq;
+    const int row_ld = row_ok ? row_q : sq - 1;
+    Frag Qf[D / 16], dOf[D / 16];
+    {
+      const T *qp = reinterpret_cast<const T *>(p.q) + (int64_t)(q0 + row_ld) * p.q_stride + (int64_t)h * D;
+      const T *dp = reinterpret_cast<const T *>(p.dout) + (int64_t)(q0 + row_ld) * p.do_stride + (int64_t)h * D;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        Qf[ks] = frag_ld<T>(qp + ks * 16 + 8 * hh);
+        dOf[ks] = frag_ld<T>(dp + ks * 16 + 8 * hh);
+      }
+    }
+    const float lse_c = row_ok ? p.lse[((int64_t)b * p.hq + h) * p.max_sq + row_q] * 1.4426950408889634f : INFINITY;
+    const float del_c = row_ok ? p.delta[((int64_t)b * p.hq + h) * p.max_sq + row_q] : 0.f;
+    int nk_end = sk;
+    if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
+    const int ntiles = (nk_end + BN - 1) / BN;
+    const int niter = (ntiles + SPLIT - 1) / SPLIT;
+
+    floatx16 dQt[D / 32];
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dQt[t][v] = 0.f;
+
+    auto issue = [&](T *stage, int it) {
+#pragma unroll
+      for (int i = 0; i < LD; ++i) {
+        const int blk = w * LD + i;
+        const int tile = blk / (BN / 2);
+        const int kvsel = (blk % (BN / 2)) / (BN / 4);
+        const int rgp = blk % (BN / 4);
+        const int tile_g = it * SPLIT + tile;
+        if (tile_g < ntiles) {
+          const int row = 4 * rgp + lrow;
+          int kr = tile_g * BN + row;
+          kr = kr < sk ? kr : sk - 1;
+          dma_rows4<T>(kvsel ? vg : kg, kr, kvsel ? v_stride : k_stride, row, lane,
+                       stage + tile * 2 * TILE + kvsel * TILE + rgp * 512);
+        }
+      }
+    };
+    auto compute = [&](const T *stage, int it) {
+      const int tile_g = it * SPLIT + sp;
+      const int n0 = tile_g * BN;
+      if (tile_g >= ntiles || (causal && n0 > wrow0 + 31)) return;
+      const T *tK = stage + sp * 2 * TILE;
+      const T *tV = tK + TILE;
+      floatx16 S[NB], dP[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          S[nb][v] = 0.f;
+          dP[nb][v] = 0.f;
+        }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        Frag ak = frag_ld_swz<T>(tK, nb * 32 + c, hh);
+        Frag av = frag_ld_swz<T>(tV, nb * 32 + c, hh);
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+          Frag ak2 = ak, av2 = av;
+          if (ks + 1 < D / 16) {
+            ak2 = frag_ld_swz<T>(tK, nb * 32 + c, 2 * (ks + 1) + hh);
+            av2 = frag_ld_swz<T>(tV, nb * 32 + c, 2 * (ks + 1) + hh);
+          }
+          S[nb] = M::mma(ak, Qf[ks], S[nb]);
+          dP[nb] = M::mma(av, dOf[ks], dP[nb]);
+          ak = ak2;
+          av = av2;
+        }
+      }
+      const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+      Frag dSb[NS];
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        float dsv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int nb = s >> 1, v = 8 * (s & 1) + j;
+          float pe = fast_exp2(S[nb][v] * scale_log2 - lse_c);
+          if (need_mask) {
+            const int kv = n0 + nb * 32 + acc_row(v, hh);
+            if (kv >= sk || (causal && kv > row_q)) pe = 0.f;
+          }
+          dsv[j] = pe * (dP[nb][v] - del_c);
+        }
+        dSb[s] = frag_pack<T>(dsv);
+      }
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        Tr4 kt;
+        tr4_issue<T>(kt, tK, 16 * s, lane);
+        dQt[0] = M::mma(tr4_get<T, 6>(kt, 0), dSb[s], dQt[0]);
+        dQt[1] = M::mma(tr4_get<T, 4>(kt, 1), dSb[s], dQt[1]);
+        dQt[2] = M::mma(tr4_get<T, 2>(kt, 2), dSb[s], dQt[2]);
+        dQt[3] = M::mma(tr4_get<T, 0>(kt, 3), dSb[s], dQt[3]);
+      }
+    };
+
+    if (niter > 0) issue(sStage0, 0);
+    __syncthreads();
+    for (int it = 0; it < niter; it += 2) {
+      if (it + 1 < niter) issue(sStage1, it + 1);
+      compute(sStage0, it);
+      __syncthreads();
+      if (it + 1 < niter) {
+        if (it + 2 < niter) issue(sStage0, it + 2);
+        compute(sStage1, it + 1);
+        __syncthreads();
+      }
+    }
+
+    // add the splits' partial dQ through LDS, in split order
+    float *x0 = reinterpret_cast<float *>(sStage0);
+    float *x1 = reinterpret_cast<float *>(sStage1);
+    static_assert((SPLIT - 1) * RG <= 6, "exchange slots");
+    if (sp > 0) {
+      const int x = (sp - 1) * RG + rg;
+      float *dst = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(t * 16 + v) * 64 + lane] = dQt[t][v];
+    }
+    __syncthreads();
+    if (sp == 0) {
+#pragma unroll
+      for (int s2 = 1; s2 < SPLIT; ++s2) {
+        const int x = (s2 - 1) * RG + rg;
+        const float *src = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) dQt[t][v] += src[(t * 16 + v) * 64 + lane];
+      }
+      if (row_ok) {
+        T *dqp = reinterpret_cast<T *>(p.dq) + (int64_t)(q0 + row_q) * p.dq_stride + (int64_t)h * D;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int vb = 0; vb < 4; ++vb) {
+            struct alignas(8) { T v[4]; } a;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+            *reinterpret_cast<decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh) = a;
+          }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T, int RG, int SPLIT, int BN>
+static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
+  constexpr int BM = 32 * RG;
+  const int nqt = (int)cdiv(p.max_sq, BM);
+  dim3 grid((unsigned)(p.causal ? (nqt + 1) / 2 : nqt), (unsigned)p.hq, (unsigned)batch);
+  hipLaunchKernelGGL((attn_bwd_dq_d128_kernel<T, RG, SPLIT, BN>), grid, dim3(512), 0, st, p);
+  return DH_OK;
+}
+
+// dK/dV: 4 wavefronts = 2 key row groups (32 rows each) x 2 query splits.  K and V
+// fragments of the group stay in registers; every iteration brings two 32-row query tiles
+// (Q, dO, lse, delta) of the current head into LDS, one per split.  The splits' partial
+// dK/dV are added through LDS in split order.  Causal: the workgroup owns key tiles j and
+// n-1-j, so every workgroup does the same amount of work.
+template <typename T>
+__global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int D = 128, KG = 2, QSPLIT = 2, BN = 32 * KG, BM = 32;
+  constexpr int QT = BM * D;                          // elements of one Q (or dO) tile
+  constexpr int SLOT = 2 * QT + 128;                  // Q tile, dO tile, 32 lse + 32 delta (as 256 bytes)
+  constexpr int STAGE = QSPLIT * SLOT;
+  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
+  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+
+  const int b = blockIdx.z;
+  const int hkv = blockIdx.y / p.hsplit, hs = blockIdx.y % p.hsplit;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int nkt = (sk + BN - 1) / BN;
+  const int causal = p.causal;
+  const int q_stride = (int)p.q_stride, do_stride = (int)p.do_stride;
+  const float scale_log2 = p.scale_log2;
+  int kt[2], nk;
+  if (causal) {
+    const int pair = blockIdx.x;
+    if (2 * pair >= nkt) return;
+    kt[0] = pair; kt[1] = nkt - 1 - pair;             // heavy (early keys) first
+    nk = (kt[0] == kt[1]) ? 1 : 2;
+  } else {
+    if ((int)blockIdx.x >= nkt) return;
+    kt[0] = blockIdx.x; kt[1] = 0; nk = 1;
+  }
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = lane & 31, hh = lane >> 5;
+  const int kg = w % KG, qs = w / KG;
+  const int ratio = p.hq / p.hk;
+  const int hper = ratio / p.hsplit;
+  const int lrow = lane >> 4;
+  const int64_t lse_stride = p.max_sq;
+
+  for (int ki = 0; ki < nk; ++ki) {
+    const int j0 = kt[ki] * BN;
+    const int jw0 = j0 + 32 * kg;
+    const int jrow = jw0 + c;
+    Frag Kf[D / 16], Vf[D / 16];
+    {
+      const int jl = jrow < sk ? jrow : sk - 1;
+      const T *kp = reinterpret_cast<const T *>(p.k) + (int64_t)(k0 + jl) * p.k_stride + (int64_t)hkv * D;
+      const T *vp = reinterpret_cast<const T *>(p.v) + (int64_t)(k0 + jl) * p.v_stride + (int64_t)hkv * D;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        Kf[ks] = frag_ld<T>(kp + ks * 16 + 8 * hh);
+        Vf[ks] = frag_ld<T>(vp + ks * 16 + 8 * hh);
+      }
+    }
+    floatx16 dKt[D / 32], dVt[D / 32];
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        dKt[t][v] = 0.f;
+        dVt[t][v] = 0.f;
+      }
+    const int i_begin = causal ? (j0 / BM) * BM : 0;
+    const int ntq = i_begin < sq ? (sq - i_begin + BM - 1) / BM : 0;
+    const int it_per_head = (ntq + QSPLIT - 1) / QSPLIT;
+    const int niter = it_per_head * hper;
+
+    // copies of one stage: 32 blocks of 1 KB (4 rows of a Q or dO tile) + one 256-byte lse/delta block per split
+    auto issue = [&](T *stage, int it) {
+      const int g = it / it_per_head, ti = it % it_per_head;
+      const int h = hkv * ratio + hs * hper + g;
+      const T *qg = reinterpret_cast<const T *>(p.q) + (int64_t)q0 * p.q_stride + (int64_t)h * D;
+      const T *dg = reinterpret_cast<const T *>(p.dout) + (int64_t)q0 * p.do_stride + (int64_t)h * D;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int blk = w * 8 + i;
+        const int slot = blk / 16, sel = (blk % 16) / 8, rgp = blk % 8;
+        const int tq = ti * QSPLIT + slot;
+        if (tq < ntq) {
+          const int row = 4 * rgp + lrow;
+          int ir = i_begin + tq * BM + row;
+          ir = ir < sq ? ir : sq - 1;
+          dma_rows4<T>(sel ? dg : qg, ir, sel ? do_stride : q_stride, row, lane, stage + slot * SLOT + sel * QT + rgp * 512);
+        }
+      }
+      if (w < QSPLIT) {
+        const int tq = ti * QSPLIT + w;
+        if (tq < ntq) {
+          int ir = i_begin + tq * BM + (lane & 31);
+          ir = ir < sq ? ir : sq - 1;
+          const float *src = (lane < 32 ? p.lse : p.delta) + ((int64_t)b * p.hq + h) * lse_stride + ir;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                           (__attribute__((address_space(3))) void *)(stage + w * SLOT + 2 * QT), 4, 0, 0);
+        }
+      }
+    };
+    auto compute = [&](const T *stage, int it) {
+      const int ti = it % it_per_head;
+      const int tq = ti * QSPLIT + qs;
+      const int i0 = i_begin + tq * BM;
+      if (tq >= ntq || (causal && i0 + BM - 1 < jw0)) return;
+      const T *tQ = stage + qs * SLOT;
+      const T *tdO = tQ + QT;
+      const float *tL = reinterpret_cast<const float *>(tQ + 2 * QT);   // [32 lse | 32 delta]
+      floatx16 S, dP;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        S[v] = 0.f;
+        dP[v] = 0.f;
+      }
+      {
+        Frag aq = frag_ld_swz<T>(tQ, c, hh);
+        Frag ad = frag_ld_swz<T>(tdO, c, hh);
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+          Frag aq2 = aq, ad2 = ad;
+          if (ks + 1 < D / 16) {
+            aq2 = frag_ld_swz<T>(tQ, c, 2 * (ks + 1) + hh);
+            ad2 = frag_ld_swz<T>(tdO, c, 2 * (ks + 1) + hh);
+          }
+          S = M::mma(aq, Kf[ks], S);
+          dP = M::mma(ad, Vf[ks], dP);
+          aq = aq2;
+          ad = ad2;
+        }
+      }
+      const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
+      float pv[16], dsv[16];
+#pragma unroll
+      for (int vb = 0; vb < 4; ++vb) {
+        const float4 l4 = *reinterpret_cast<const float4 *>(tL + 8 * vb + 4 * hh);
+        const float4 d4 = *reinterpret_cast<const float4 *>(tL + 32 + 8 * vb + 4 * hh);
+        const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
+        const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * vb + e;
+          float pe = fast_exp2(S[v] * scale_log2 - ls[e] * 1.4426950408889634f);
+          if (need_mask) {
+            const int i = i0 + acc_row(v, hh);
+            if (i >= sq || (causal && jrow > i)) pe = 0.f;
+          }
+          pv[v] = pe;
+          dsv[v] = pe * (dP[v] - dl[e]);
+        }
+      }
+      Frag Pb[2], dSb[2];
+      Pb[0] = frag_pack<T>(pv);
+      Pb[1] = frag_pack<T>(pv + 8);
+      dSb[0] = frag_pack<T>(dsv);
+      dSb[1] = frag_pack<T>(dsv + 8);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        Tr4 dot, qt;
+        tr4_issue<T>(dot, tdO, 16 * s, lane);
+        tr4_issue<T>(qt, tQ, 16 * s, lane);
+        dVt[0] = M::mma(tr4_get<T, 14>(dot, 0), Pb[s], dVt[0]);
+        dVt[1] = M::mma(tr4_get<T, 12>(dot, 1), Pb[s], dVt[1]);
+        dVt[2] = M::mma(tr4_get<T, 10>(dot, 2), Pb[s], dVt[2]);
+        dVt[3] = M::mma(tr4_get<T, 8>(dot, 3), Pb[s], dVt[3]);
+        dKt[0] = M::mma(tr4_get<T, 6>(qt, 0), dSb[s], dKt[0]);
+        dKt[1] = M::mma(tr4_get<T, 4>(qt, 1), dSb[s], dKt[1]);
+        dKt[2] = M::mma(tr4_get<T, 2>(qt, 2), dSb[s], dKt[2]);
+        dKt[3] = M::mma(tr4_get<T, 0>(qt, 3), dSb[s], dKt[3]);
+      }
+    };
+
+    if (niter > 0) issue(sStage0, 0);
+    __syncthreads();
+    for (int it = 0; it < niter; it += 2) {
+      if (it + 1 < niter) issue(sStage1, it + 1);
+      compute(sStage0, it);
+      __syncthreads();
+      if (it + 1 < niter) {
+        if (it + 2 < niter) issue(sStage0, it + 2);
+        compute(sStage1, it + 1);
+        __syncthreads();
+      }
+    }
+
+    // add the second split's partial sums through LDS: dK in stage 0, dV in stage 1
+    float *xk = reinterpret_cast<float *>(sStage0) + kg * 4096;
+    float *xv = reinterpret_cast<float *>(sStage1) + kg * 4096;
+    static_assert(STAGE * sizeof(T) >= KG * 4096 * sizeof(float), "exchange area");
+    if (qs == 1) {
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          xk[(t * 16 + v) * 64 + lane] = dKt[t][v];
+          xv[(t * 16 + v) * 64 + lane] = dVt[t][v];
+        }
+    }
+    __syncthreads();
+    if (qs == 0) {
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          dKt[t][v] += xk[(t * 16 + v) * 64 + lane];
+          dVt[t][v] += xv[(t * 16 + v) * 64 + lane];
+        }
+      if (jrow < sk) {
+        if (p.hsplit == 1) {
+          T *dkp = reinterpret_cast<T *>(p.dk) + (int64_t)(k0 + jrow) * p.dk_stride + (int64_t)hkv * D;
+          T *dvp = reinterpret_cast<T *>(p.dv) + (int64_t)(k0 + jrow) * p.dv_stride + (int64_t)hkv * D;
+#pragma unroll
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb) {
+              struct alignas(8) { T v[4]; } a, bq;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                a.v[e] = static_cast<T>(dKt[t][4 * vb + e] * p.scale);
+                bq.v[e] = static_cast<T>(dVt[t][4 * vb + e]);
+              }
+              *reinterpret_cast<decltype(a) *>(dkp + 32 * t + 8 * vb + 4 * hh) = a;
+              *reinterpret_cast<decltype(bq) *>(dvp + 32 * t + 8 * vb + 4 * hh) = bq;
+            }
+        } else {
+          const int64_t off = (((int64_t)hs * p.total_k + (k0 + jrow)) * p.hk + hkv) * D;
+#pragma unroll
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int vb = 0; vb < 4; ++vb) {
+              *reinterpret_cast<float4 *>(p.dk_part + off + 32 * t + 8 * vb + 4 * hh) =
+                  make_float4(dKt[t][4 * vb] * p.scale, dKt[t][4 * vb + 1] * p.scale, dKt[t][4 * vb + 2] * p.scale,
+                              dKt[t][4 * vb + 3] * p.scale);
+              *reinterpret_cast<float4 *>(p.dv_part + off + 32 * t + 8 * vb + 4 * hh) =
+                  make_float4(dVt[t][4 * vb], dVt[t][4 * vb + 1], dVt[t][4 * vb + 2], dVt[t][4 * vb + 3]);
+            }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+static int launch_dkv_d128(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
+  const int nkt = (int)cdiv(max_sk, 64);
+  dim3 grid((unsigned)(p.causal ? (nkt + 1) / 2 : nkt), (unsigned)(p.hk * p.hsplit), (unsigned)batch);
+  hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(256), 0, st, p);
+  return DH_OK;
+}
+
 // ---- host -------------------------------------------------------------------------------------
 static int pick_hsplit(int max_sk, int batch, int hq, int hk, int bn) {
   const int ratio = hq / hk;
@@ -563,7 +1025,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.causal = causal;
-  p.hsplit = pick_hsplit(max_seqlen_k, batch, hq, hk, 32 * DKV_NW);
+  p.hsplit = pick_hsplit(d == 128 && causal ? (max_seqlen_k + 1) / 2 : max_seqlen_k, batch, hq, hk, 32 * DKV_NW);
   p.dk_part = nullptr;
   p.dv_part = nullptr;
   if (p.hsplit > 1) {
@@ -572,18 +1034,24 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
     p.dv_part = (float *)(ws + part);
   }
   const bool small_q = cdiv(max_seqlen_q, 128) * hq * batch < 2 * 256;
+  const bool big_q = (causal ? (cdiv(max_seqlen_q, 128) + 1) / 2 : cdiv(max_seqlen_q, 128)) * hq * batch >= 256;
+  DH_CHECK(k_stride < (1ll << 31) && v_stride < (1ll << 31) && q_stride < (1ll << 31) && do_stride < (1ll << 31),
+           "token stride too large");
   int rc = DH_OK;
 #define DH_BWD(TT, DD)                                                                         \
   do {                                                                                         \
-    if (max_seqlen_k > 0) rc = launch_dkv<TT, DD, DKV_NW>(p, batch, max_seqlen_k, st);         \
+    if (max_seqlen_k > 0)                                                                      \
+      rc = DD == 128 ? launch_dkv_d128<TT>(p, batch, max_seqlen_k, st) : launch_dkv<TT, DD, DKV_NW>(p, batch, max_seqlen_k, st); \
     if (rc == DH_OK && p.hsplit > 1 && total_k > 0) {                                          \
       int64_t blocks = cdiv(total_k * hk * (DD / 4), 256);                                     \
       if (blocks > 256 * 16) blocks = 256 * 16;                                                \
       hipLaunchKernelGGL((attn_bwd_gqa_sum_kernel<TT>), dim3((unsigned)blocks), dim3(256), 0, st, p.dk_part, \
                          p.dv_part, (TT *)dk, (TT *)dv, total_k, hk, DD, p.hsplit, dk_stride, dv_stride);    \
     }                                                                                          \
-    if (rc == DH_OK && max_seqlen_q > 0)                                                       \
-      rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st);  \
+    if (rc == DH_OK && max_seqlen_q > 0) {                                                     \
+      if (DD == 128) rc = big_q ? launch_dq_d128<TT, 4, 2, 32>(p, batch, st) : launch_dq_d128<TT, 2, 4, 32>(p, batch, st); \
+      else rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st); \
+    }                                                                                          \
   } while (0)
   if (dtype == DH_BF16) {
     if (d == 128) DH_BWD(bf16_t, 128); else DH_BWD(bf16_t, 64);

@@ -76,6 +76,74 @@ template <typename T> __device__ __forceinline__ typename Mma<T>::Frag frag_pack
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// ---- swizzled 256-byte-row tiles in LDS (head dim 128, 16-bit elements) -------------------------
+// A tile is [rows][128] elements with NO padding; the 16-byte chunk index of a row is XORed
+// with swz(row), a bijection of row % 16 whose upper two bits enumerate row % 4.  That makes
+// both access patterns conflict-free: 16-byte row fragments (16 consecutive rows hit 16
+// different chunks) and transpose reads (the 4 rows a half-wave reads land in 4 different
+// 64-byte groups).  Tiles are filled by direct global->LDS copies of 1 KB (4 rows) per
+// wavefront instruction, the swizzle being applied to the GLOBAL chunk a lane fetches.
+__device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2) & 3); }
+
+// Copy 4 consecutive rows (row0 .. row0+3, each 128 elements) of a row-major global matrix
+// into the swizzled tile at `dst4` (wave-uniform LDS address of the 4-row block).  Lane l
+// handles row row0 + l/16 and LDS chunk l%16.  `row_g` is the lane's (clamped) global row.
+template <typename T>
+__device__ __forceinline__ void dma_rows4(const T *gbase, int64_t row_g, int ld, int row_in_tile, int lane, T *dst4) {
+  const T *src = gbase + row_g * ld + (((lane & 15) ^ swz(row_in_tile)) * 8);
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                   (__attribute__((address_space(3))) void *)dst4, 16, 0, 0);
+}
+
+// 16-byte row fragment (8 consecutive k of one row) from a swizzled tile: row, logical chunk.
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::Frag frag_ld_swz(const T *tile, int row, int chunk) {
+  return frag_ld<T>(tile + row * 128 + ((chunk ^ swz(row)) * 8));
+}
+
+// Four transposed fragments (the four 32-column blocks t = 0..3) of a swizzled tile for the
+// k rows {ka .. ka+3} u {ka+8 .. ka+11}, ka = k0 + 4*hh, issued as one batch of eight
+// transpose reads.  Written in assembly: a builtin would make the compiler wait for every
+// direct-to-LDS copy still in flight (it cannot tell the stages apart).  The caller must
+// order its uses after tr4_wait<N>().
+struct Tr4 { short4v f[8]; };
+template <typename T>
+__device__ __forceinline__ void tr4_issue(Tr4 &o, const T *tile, int k0, int lane) {
+  const int hh = lane >> 5, r = lane & 15;
+  const int rowa = k0 + 4 * hh + (r >> 2);
+  const int xa = swz(rowa), xb = swz(rowa + 8);
+  const uint32_t base = (uint32_t)(uintptr_t)(tile + rowa * 128 + ((r & 3) & 1) * 4);
+  const int lc0 = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  uint32_t ad[8];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    ad[2 * t] = base + (((4 * t + lc0) ^ xa) * 16);
+    ad[2 * t + 1] = base + 8 * 128 * (uint32_t)sizeof(T) + (((4 * t + lc0) ^ xb) * 16);
+  }
+  asm volatile("ds_read_b64_tr_b16 %0, %8\n\tds_read_b64_tr_b16 %1, %9\n\t"
+               "ds_read_b64_tr_b16 %2, %10\n\tds_read_b64_tr_b16 %3, %11\n\t"
+               "ds_read_b64_tr_b16 %4, %12\n\tds_read_b64_tr_b16 %5, %13\n\t"
+               "ds_read_b64_tr_b16 %6, %14\n\tds_read_b64_tr_b16 %7, %15"
+               : "=&v"(o.f[0]), "=&v"(o.f[1]), "=&v"(o.f[2]), "=&v"(o.f[3]), "=&v"(o.f[4]), "=&v"(o.f[5]),
+                 "=&v"(o.f[6]), "=&v"(o.f[7])
+               : "v"(ad[0]), "v"(ad[1]), "v"(ad[2]), "v"(ad[3]), "v"(ad[4]), "v"(ad[5]), "v"(ad[6]), "v"(ad[7])
+               : "memory");
+}
+// Wait until at most N LDS reads issued after fragment t of `o` are outstanding, then return fragment t.
+// (LDS reads complete in order, so "at most N outstanding" means everything older has landed.)
+template <typename T, int N>
+__device__ __forceinline__ typename Mma<T>::Frag tr4_get(Tr4 &o, int t) {
+  static_assert(N >= 0 && N <= 14 && N % 2 == 0, "even count up to 14");
+#define DH_W(n) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(o.f[2 * t]), "+v"(o.f[2 * t + 1]))
+  if (N == 14) DH_W(14); else if (N == 12) DH_W(12); else if (N == 10) DH_W(10); else if (N == 8) DH_W(8);
+  else if (N == 6) DH_W(6); else if (N == 4) DH_W(4); else if (N == 2) DH_W(2); else DH_W(0);
+#undef DH_W
+  short8v o8;
+  o8[0] = o.f[2 * t][0]; o8[1] = o.f[2 * t][1]; o8[2] = o.f[2 * t][2]; o8[3] = o.f[2 * t][3];
+  o8[4] = o.f[2 * t + 1][0]; o8[5] = o.f[2 * t + 1][1]; o8[6] = o.f[2 * t + 1][2]; o8[7] = o.f[2 * t + 1][3];
+  return __builtin_bit_cast(typename Mma<T>::Frag, o8);
+}
+
 // Row index inside a 32-row accumulator block held by register v of lane half h.
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 

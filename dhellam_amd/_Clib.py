@@ -108,6 +108,18 @@ def _attn_fwd_raw(q, k, v, out, lse, cu_q, cu_k, max_q, max_k, scale, causal, st
                                _tok_stride(out), float(scale), int(bool(causal)), _lib.dt(q), stream_ptr))
 
 
+_rng_zero: dict = {}
+
+
+def _zero_rng_state(device) -> torch.Tensor:
+    """The int64[2] seed/offset slot of the return list; always zero (no dropout), one per device."""
+    t = _rng_zero.get(device)
+    if t is None:
+        t = torch.zeros(2, dtype=torch.int64, device=device)
+        _rng_zero[device] = t
+    return t
+
+
 def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                      is_causal, return_softmax, math_sm_count, profiling):
     """ops.h:18-32 / flash_atten.cu:436-477.  Runs on the current stream.
@@ -134,8 +146,7 @@ def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
                                                         max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
                                                         stream.cuda_stream))
     p = torch.empty(0, dtype=q.dtype, device=q.device)
-    rng_state = torch.zeros(2, dtype=torch.int64, device=q.device)
-    res = [out, q, k, v, out, lse, p, rng_state]
+    res = [out, q, k, v, out, lse, p, _zero_rng_state(q.device)]
     if profiling:
         res.append(torch.tensor([ms], dtype=torch.float32))
     return res

@@ -1,0 +1,119 @@
+"""Plan search host logic (no GPU): record format, DP optimality against brute force, plan JSON."""
+import itertools
+import random
+
+from dhellam_amd.core import dstb
+from dhellam_amd.search import op_table, search
+
+
+def test_op_ids_and_candidates():
+    assert op_table.OP_TABLE_IDX["ln_attn"] == 24 and op_table.OP_TABLE_IDX["attn_bwd"] == 10      # search/op_table.py:1-37
+    assert op_table.OP_TABLE_IDX["gemm_wgrad_mlp_c_reduce_scatter_mlp_c_bwd"] == 9
+    fwd_c, bwd_c = op_table.get_candidate_operator_groups()
+    assert fwd_c[0] == [] and [24] in fwd_c and [16, 35, 11, 17] in fwd_c and [35, 11] in fwd_c
+    assert [16, 11] not in fwd_c                                   # not contiguous
+    assert [24, 16] not in fwd_c                                   # crosses a boundary
+    assert len(fwd_c) == 1 + 1 + 10 + 3 + 6 + 1 and len(bwd_c) == 1 + 1 + 10 + 1 + 3 + 15 + 1 + 1
+
+
+def test_record_format_roundtrip(tmp_path):
+    f = tmp_path / "op_profile_num.txt"
+    with open(f, "w") as fp:
+        fp.write(search.format_record([16, 35, 11], [19, 23], 1.25, 2.5, 2.0))
+        fp.write(search.format_record([], [26], 1.0, 0.5, 0.5))
+        fp.write(search.format_record([24], [], 1.0, 0.25, 0.25))
+        fp.write("garbage line\n")
+    assert open(f).readline() == "[[16, 35, 11],[19, 23]] speedup: 1.25 seq_time:2.5 para_time:2.0\n"   # profiler.py:179-180
+    prof = search.parse_op_file(str(f))
+    assert prof == {((16, 35, 11), (19, 23)): 2.0, ((), (26,)): 0.5, ((24,), ()): 0.25}
+
+
+def _brute(profile, fwd_groups, bwd_groups):
+    """Reference-style search: enumerate every refinement of the boundary groups, then the
+    classic 2-D DP over the two group sequences (search/search.py:77-143)."""
+    def refinements(groups):
+        per = []
+        for g in groups:
+            opts = []
+            for cuts in itertools.product([0, 1], repeat=len(g) - 1):
+                parts, cur = [], [g[0]]
+                for op, cut in zip(g[1:], cuts):
+                    if cut:
+                        parts.append(cur); cur = [op]
+                    else:
+                        cur.append(op)
+                parts.append(cur)
+                opts.append(parts)
+            per.append(opts)
+        for combo in itertools.product(*per):
+            yield [p for parts in combo for p in parts]
+    best = float("inf")
+    t = lambda f, b: profile[(tuple(f), tuple(b))]
+    for fr in refinements(fwd_groups):
+        for br in refinements(bwd_groups):
+            m, n = len(fr), len(br)
+            d = [[0.0] * (n + 1) for _ in range(m + 1)]
+            for i in range(1, m + 1):
+                d[i][0] = d[i - 1][0] + t(fr[i - 1], [])
+            for j in range(1, n + 1):
+                d[0][j] = d[0][j - 1] + t([], br[j - 1])
+            for i in range(1, m + 1):
+                for j in range(1, n + 1):
+                    d[i][j] = min(d[i - 1][j] + t(fr[i - 1], []), d[i][j - 1] + t([], br[j - 1]),
+                                  d[i - 1][j - 1] + t(fr[i - 1], br[j - 1]))
+            best = min(best, d[m][n])
+    return best
+
+
+def test_dp_matches_brute_force_enumeration():
+    rng = random.Random(0)
+    fwd_groups, bwd_groups = [[1], [2, 3, 4], [5, 6]], [[11, 12], [13], [14, 15, 16]]
+    for trial in range(5):
+        prof = {}
+        fc, bc = op_table.candidate_groups(fwd_groups), op_table.candidate_groups(bwd_groups)
+        solo = {}
+        for f in fc:
+            for b in bc:
+                if not f and not b:
+                    continue
+                base = sum(solo.setdefault(x, rng.uniform(0.1, 1.0)) for x in f + b)
+                # pairing saves a random share of the smaller side
+                save = rng.uniform(0, 0.9) * min(sum(solo[x] for x in f), sum(solo[x] for x in b)) if f and b else 0.0
+                prof[(tuple(f), tuple(b))] = base - save
+        cost, blocks = search.search_plan(prof, fwd_groups, bwd_groups)
+        assert abs(cost - _brute(prof, fwd_groups, bwd_groups)) < 1e-9
+        # the blocks cover both lists in order and their times add up to the cost
+        assert [x for f, _ in blocks for x in f] == [1, 2, 3, 4, 5, 6]
+        assert [x for _, b in blocks for x in b] == [11, 12, 13, 14, 15, 16]
+        assert abs(sum(prof[(tuple(f), tuple(b))] for f, b in blocks) - cost) < 1e-9
+
+
+def test_illegal_pairs_are_never_chosen():
+    fwd_groups, bwd_groups = [[1, 2]], [[11, 12]]
+    prof = {(tuple(f), tuple(b)): 1.0 for f in op_table.candidate_groups(fwd_groups)
+            for b in op_table.candidate_groups(bwd_groups) if f or b}
+    prof[((1, 2), (11, 12))] = 0.1
+    cost, blocks = search.search_plan(prof, fwd_groups, bwd_groups)
+    assert blocks == [([1, 2], [11, 12])] and cost == 0.1
+    cost, blocks = search.search_plan(prof, fwd_groups, bwd_groups, illegal=lambda f, b: len(f) == 2 and len(b) == 2)
+    assert cost == 1.0 + 1.0 - 0.0 or cost == 2.0
+    assert ([1, 2], [11, 12]) not in blocks
+
+
+def test_plan_json_is_loadable_and_complete(tmp_path):
+    (_, _, fwd), (_, _, bwd) = op_table.operator_list_prune()
+    # a plan that pairs group by group where possible
+    blocks = [(fwd[i] if i < len(fwd) else [], bwd[i] if i < len(bwd) else []) for i in range(max(len(fwd), len(bwd)))]
+    data = search.dump_plan(blocks, str(tmp_path / "best_result.json"))
+    assert set(data) == {"DCBlocks"} and all(len(b) == 3 for b in data["DCBlocks"])
+    assert data["DCBlocks"][0] == [["ln_attn"], ["bda_mlp_bwd"], "None"]
+    assert data["DCBlocks"][1][2] == ["allgather_attn", "allgather_mlp_bwd"]
+    assert data["DCBlocks"][2][1] == ["gemm_wgrad_mlp_c"]                      # fused search op written under its plan name
+    plan = dstb.init_DCBlocks(str(tmp_path / "best_result.json"))
+    named = [str(o) for blk in plan.dcblocks for col in (blk.stream1_op, blk.stream2_op, blk.stream3_op) for o in (col or [])]
+    graph_ops = [n for n, num, *_ in dstb._GRAPH if num < 100]
+    assert sorted(named) == sorted(graph_ops), "every op of the layer appears exactly once in the plan"
+    # a comm stand-in never precedes its producer's block and sits in its consumer's block
+    pos = {str(o): i for i, blk in enumerate(plan.dcblocks) for col in (blk.stream1_op, blk.stream2_op, blk.stream3_op) for o in (col or [])}
+    for comm, consumer in op_table.COMM_CONSUMER.items():
+        assert pos[comm] == pos[consumer] and pos[str(plan.ops[comm].pre)] < pos[comm]

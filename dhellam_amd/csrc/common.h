@@ -75,6 +75,19 @@ __device__ __forceinline__ float block256_sum(float v, float *red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
+// Sum over a block of BT threads (BT / 64 waves, BT in {256, 1024}); `red` holds BT / 64 floats.
+template <int BT> __device__ __forceinline__ float block_sum(float v, float *red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();  // protect `red` from the previous use
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < BT / 64; ++i) t += red[i];
+  return t;
+}
+
 // Dispatch a callable templated on the element type.
 #define DH_DISPATCH_DTYPE(dtype, ...)                                    \
   switch (dtype) {                                                       \

@@ -12,14 +12,14 @@
 
 namespace dh {
 
-template <typename T, int TPR, int VPT, bool LN>
-__global__ void __launch_bounds__(256)
+template <typename T, int BT, int TPR, int VPT, bool LN>
+__global__ void __launch_bounds__(BT)
 norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *__restrict__ beta,
                 T *__restrict__ y, float *__restrict__ mu_out, float *__restrict__ rs_out, int64_t rows,
                 int cols, float eps, float gamma_shift) {
   constexpr int N = Vec<T>::N;
-  constexpr int RPB = 256 / TPR;
-  __shared__ float red[4];
+  constexpr int RPB = BT / TPR;
+  __shared__ float red[BT / 64];
   const int nvec = cols / N;
   const int lane = threadIdx.x % TPR;
   const int sub = threadIdx.x / TPR;
@@ -55,7 +55,7 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
     }
     float mean = 0.f, var;
     if (LN) {
-      s = (TPR == 64) ? wave_sum(s) : block256_sum(s, red);
+      s = (TPR == 64) ? wave_sum(s) : block_sum<BT>(s, red);
       mean = s * inv_cols;
       float s2 = 0.f;
 #pragma unroll
@@ -69,10 +69,10 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
           }
         }
       }
-      s2 = (TPR == 64) ? wave_sum(s2) : block256_sum(s2, red);
+      s2 = (TPR == 64) ? wave_sum(s2) : block_sum<BT>(s2, red);
       var = s2 * inv_cols;
     } else {
-      s = (TPR == 64) ? wave_sum(s) : block256_sum(s, red);
+      s = (TPR == 64) ? wave_sum(s) : block_sum<BT>(s, red);
       var = s * inv_cols;
     }
     const float rs = 1.0f / sqrtf(var + eps);
@@ -137,14 +137,14 @@ norm_fwd_generic_kernel(const T *__restrict__ x, const T *__restrict__ gamma, co
 }
 
 // Backward main pass.  part: fp32 [2][gridDim.x][cols] (dgamma rows, then dbeta rows).
-template <typename T, int TPR, int VPT, bool LN>
-__global__ void __launch_bounds__(256)
+template <typename T, int BT, int TPR, int VPT, bool LN>
+__global__ void __launch_bounds__(BT)
 norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *__restrict__ mu,
                 const float *__restrict__ rsigma, const T *__restrict__ gamma, const T *__restrict__ add_to_dx,
                 T *__restrict__ dx, float *__restrict__ part, int64_t rows, int cols, float gamma_shift) {
   constexpr int N = Vec<T>::N;
-  constexpr int RPB = 256 / TPR;
-  __shared__ float red[4];
+  constexpr int RPB = BT / TPR;
+  __shared__ float red[BT / 64];
   extern __shared__ float stage[];  // TPR==64 only: [4 waves][TPR*VPT*N] floats
   const int nvec = cols / N;
   const int lane = threadIdx.x % TPR;
@@ -164,10 +164,30 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
     }
   }
 
+  // The next row's x and dy are requested before the current row's reduction, so that a block
+  // keeps two rows of loads in flight.
+  Vec<T> xn[VPT], dn[VPT];
+  auto fetch = [&](int64_t row) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int v = lane + i * TPR;
+      if (row < rows && v < nvec) {
+        xn[i] = ldg(x + row * cols + (int64_t)v * N);
+        dn[i] = ldg(dy + row * cols + (int64_t)v * N);
+      }
+    }
+  };
+  fetch((int64_t)blockIdx.x * RPB + sub);
   for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
     const int64_t row = row0 + sub;
     const bool active = row < rows;
     Vec<T> xv[VPT], dv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      xv[i] = xn[i];
+      dv[i] = dn[i];
+    }
+    fetch(row + (int64_t)gridDim.x * RPB);
     float rs = 0.f, mean = 0.f;
     if (active) {
       rs = rsigma[row];
@@ -178,8 +198,6 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
     for (int i = 0; i < VPT; ++i) {
       const int v = lane + i * TPR;
       if (active && v < nvec) {
-        xv[i] = ldg(x + row * cols + (int64_t)v * N);
-        dv[i] = ldg(dy + row * cols + (int64_t)v * N);
 #pragma unroll
         for (int j = 0; j < N; ++j) {
           const float xh = (to_f(xv[i].v[j]) - mean) * rs;
@@ -196,8 +214,8 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
       s1 = wave_sum(s1);
       if (LN) s2 = wave_sum(s2);
     } else {
-      s1 = block256_sum(s1, red);
-      if (LN) s2 = block256_sum(s2, red);
+      s1 = block_sum<BT>(s1, red);
+      if (LN) s2 = block_sum<BT>(s2, red);
     }
     const float c1 = s1 * inv_cols, c2 = s2 * inv_cols;
     if (active) {
@@ -325,11 +343,68 @@ norm_bwd_generic_wgrad_kernel(const T *__restrict__ dy, const T *__restrict__ x,
 }
 
 // Reduce partial rows: part [2][P][cols] -> dgamma (and dbeta) [cols].
-// Block = 32 columns x 8 row groups; row groups are combined through LDS in a fixed order.
+// Block = 16 float4 lanes (64 columns) x 16 row groups; each lane streams its rows with four
+// independent accumulators, the row groups are combined through LDS in a fixed order.
 template <typename T, bool LN>
 __global__ void __launch_bounds__(256)
 norm_bwd_finalize_kernel(const float *__restrict__ part, T *__restrict__ dgamma, T *__restrict__ dbeta, int P,
                          int64_t cols, int accumulate) {
+  __shared__ float4 sg[16][16], sb[16][16];
+  const int cx = threadIdx.x & 15, ry = threadIdx.x >> 4;
+  const int64_t c = (int64_t)blockIdx.x * 64 + cx * 4;
+  float4 ag[4], ab[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    ag[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    ab[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  if (c < cols) {   // cols is a multiple of 4 on this path
+    for (int p0 = ry; p0 < P; p0 += 64) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int p = p0 + 16 * u;
+        if (p < P) {
+          const float4 v = *reinterpret_cast<const float4 *>(part + (int64_t)p * cols + c);
+          ag[u].x += v.x; ag[u].y += v.y; ag[u].z += v.z; ag[u].w += v.w;
+          if (LN) {
+            const float4 w = *reinterpret_cast<const float4 *>(part + ((int64_t)P + p) * cols + c);
+            ab[u].x += w.x; ab[u].y += w.y; ab[u].z += w.z; ab[u].w += w.w;
+          }
+        }
+      }
+    }
+  }
+  auto fold = [](const float4 (&a)[4]) {
+    return make_float4((a[0].x + a[1].x) + (a[2].x + a[3].x), (a[0].y + a[1].y) + (a[2].y + a[3].y),
+                       (a[0].z + a[1].z) + (a[2].z + a[3].z), (a[0].w + a[1].w) + (a[2].w + a[3].w));
+  };
+  sg[ry][cx] = fold(ag);
+  sb[ry][cx] = fold(ab);
+  __syncthreads();
+  if (ry == 0 && c < cols) {
+    float tg[4] = {0.f, 0.f, 0.f, 0.f}, tb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      tg[0] += sg[r][cx].x; tg[1] += sg[r][cx].y; tg[2] += sg[r][cx].z; tg[3] += sg[r][cx].w;
+      tb[0] += sb[r][cx].x; tb[1] += sb[r][cx].y; tb[2] += sb[r][cx].z; tb[3] += sb[r][cx].w;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (accumulate) {
+        tg[e] += to_f(dgamma[c + e]);
+        if (LN) tb[e] += to_f(dbeta[c + e]);
+      }
+      dgamma[c + e] = from_f<T>(tg[e]);
+      if (LN) dbeta[c + e] = from_f<T>(tb[e]);
+    }
+  }
+}
+
+// Same reduction for column counts that are not a multiple of 4 (generic path).
+template <typename T, bool LN>
+__global__ void __launch_bounds__(256)
+norm_bwd_finalize_scalar_kernel(const float *__restrict__ part, T *__restrict__ dgamma, T *__restrict__ dbeta, int P,
+                                int64_t cols, int accumulate) {
   __shared__ float sg[8][33], sb[8][33];
   const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
   const int64_t c = (int64_t)blockIdx.x * 32 + cx;
@@ -362,10 +437,12 @@ norm_bwd_finalize_kernel(const float *__restrict__ part, T *__restrict__ dgamma,
 // ---- host side --------------------------------------------------------------------
 struct NormPlan {
   bool vec;   // vector path usable
-  int tpr;    // threads per row
+  int tpr;    // threads per row (64: one wave per row, 4 rows per 256-thread block; 256; 1024)
   int vpt;    // 16-byte vectors per thread
 };
 
+// Wide rows are spread over 1024 threads so that a thread keeps few columns: the backward's
+// per-column accumulators then fit in few registers and many waves stay resident.
 static NormPlan norm_plan(int64_t cols, int elt, bool all_aligned) {
   NormPlan p{false, 0, 0};
   const int n = 16 / elt;
@@ -374,9 +451,12 @@ static NormPlan norm_plan(int64_t cols, int elt, bool all_aligned) {
   if (nvec <= 64 * 4) {
     p.tpr = 64;
     p.vpt = nvec <= 64 ? 1 : (nvec <= 128 ? 2 : 4);
-  } else if (nvec <= 256 * 8) {
+  } else if (nvec <= 512) {
     p.tpr = 256;
-    p.vpt = nvec <= 512 ? 2 : (nvec <= 1024 ? 4 : 8);
+    p.vpt = 2;
+  } else if (nvec <= 2048) {
+    p.tpr = 1024;
+    p.vpt = nvec <= 1024 ? 1 : 2;
   } else {
     return p;
   }
@@ -391,12 +471,12 @@ static int64_t bwd_blocks(int64_t rows, int64_t cols, int elt) {
     int64_t chunks = cdiv(rows, 64);
     return chunks < 1 ? 1 : (chunks > 256 ? 256 : chunks);
   }
-  const int rpb = 256 / p.tpr;
+  const int rpb = p.tpr == 64 ? 4 : 1;
   const int64_t iters = cdiv(rows, rpb);
-  int64_t nb = iters / 4;
-  if (nb < 128) nb = 128;
-  if (nb > 1024) nb = 1024;
-  if (nb > iters) nb = iters;
+  // One row-iteration per block while that keeps the partial rows few (<= 512); the extra
+  // partial traffic is cheaper than walking rows one after another inside a block.
+  int64_t nb = iters;
+  if (nb > 512) nb = 512;
   if (nb < 1) nb = 1;
   return nb;
 }
@@ -410,16 +490,18 @@ static int launch_fwd(const NormPlan &p, const T *x, const T *gamma, const T *be
                        mu, rs, rows, cols, eps, shift);
     return 0;
   }
-  const int rpb = 256 / p.tpr;
+  const int rpb = p.tpr == 64 ? 4 : 1;
   int64_t nb = cdiv(rows, rpb);
   if (nb > 256 * 16) nb = 256 * 16;
-#define L(TPR, VPT)                                                                                       \
-  hipLaunchKernelGGL((norm_fwd_kernel<T, TPR, VPT, LN>), dim3((unsigned)nb), dim3(256), 0, st, x, gamma, beta, y, \
-                     mu, rs, rows, (int)cols, eps, shift)
+#define L(BT, TPR, VPT)                                                                                      \
+  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN>), dim3((unsigned)nb), dim3(BT), 0, st, x, gamma, beta, \
+                     y, mu, rs, rows, (int)cols, eps, shift)
   if (p.tpr == 64) {
-    if (p.vpt == 1) L(64, 1); else if (p.vpt == 2) L(64, 2); else L(64, 4);
+    if (p.vpt == 1) L(256, 64, 1); else if (p.vpt == 2) L(256, 64, 2); else L(256, 64, 4);
+  } else if (p.tpr == 256) {
+    L(256, 256, 2);
   } else {
-    if (p.vpt == 2) L(256, 2); else if (p.vpt == 4) L(256, 4); else L(256, 8);
+    if (p.vpt == 1) L(1024, 1024, 1); else L(1024, 1024, 2);
   }
 #undef L
   return 0;
@@ -438,19 +520,25 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
     hipLaunchKernelGGL((norm_bwd_generic_wgrad_kernel<T, LN>), dim3((unsigned)cdiv(cols, 64), (unsigned)nb),
                        dim3(256), 0, st, dy, x, mu, rs, part, rows, cols, rpc);
   } else {
-#define L(TPR, VPT)                                                                                          \
-  hipLaunchKernelGGL((norm_bwd_kernel<T, TPR, VPT, LN>), dim3((unsigned)nb), dim3(256),                       \
+#define L(BT, TPR, VPT)                                                                                      \
+  hipLaunchKernelGGL((norm_bwd_kernel<T, BT, TPR, VPT, LN>), dim3((unsigned)nb), dim3(BT),                        \
                      (TPR == 64 ? 4 * 64 * VPT * (16 / sizeof(T)) * sizeof(float) : 0), st, dy, x, mu, rs, gamma, \
                      add, dx, part, rows, (int)cols, shift)
     if (p.tpr == 64) {
-      if (p.vpt == 1) L(64, 1); else if (p.vpt == 2) L(64, 2); else L(64, 4);
+      if (p.vpt == 1) L(256, 64, 1); else if (p.vpt == 2) L(256, 64, 2); else L(256, 64, 4);
+    } else if (p.tpr == 256) {
+      L(256, 256, 2);
     } else {
-      if (p.vpt == 2) L(256, 2); else if (p.vpt == 4) L(256, 4); else L(256, 8);
+      if (p.vpt == 1) L(1024, 1024, 1); else L(1024, 1024, 2);
     }
 #undef L
   }
-  hipLaunchKernelGGL((norm_bwd_finalize_kernel<T, LN>), dim3((unsigned)cdiv(cols, 32)), dim3(256), 0, st, part,
-                     dgamma, dbeta, (int)nb, cols, accumulate);
+  if (cols % 4 == 0)
+    hipLaunchKernelGGL((norm_bwd_finalize_kernel<T, LN>), dim3((unsigned)cdiv(cols, 64)), dim3(256), 0, st, part,
+                       dgamma, dbeta, (int)nb, cols, accumulate);
+  else
+    hipLaunchKernelGGL((norm_bwd_finalize_scalar_kernel<T, LN>), dim3((unsigned)cdiv(cols, 32)), dim3(256), 0, st,
+                       part, dgamma, dbeta, (int)nb, cols, accumulate);
   return 0;
 }
 

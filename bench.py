@@ -56,6 +56,32 @@ def time_gpu(fn, iters=20, warmup=3, stream=None):
     return start.elapsed_time(end) / iters
 
 
+def time_gpu_graph(fn, iters=20):
+    """Mean ms per call with ``iters`` calls captured in one HIP graph and the replay bracketed by
+    HIP events on the replay stream: for kernels of a few microseconds this measures the kernels,
+    not the Python launch path."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            for _ in range(iters):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record(s)
+        g.replay()
+        end.record(s)
+        end.synchronize()
+    torch.cuda.current_stream().wait_stream(s)
+    return start.elapsed_time(end) / iters
+
+
 def kernel_rooflines(cfg):
     """Per-operator achieved rate against its roofline at the 70B-shard shapes (and the
     ring / MoE shapes).  Algorithmic work only: compulsory bytes, unmasked MACs."""
@@ -86,27 +112,27 @@ def kernel_rooflines(cfg):
     for rows in (R, 8 * R, 64 * R):
         x, gm, dy = rn(rows, H), torch.ones(H, device=dev, dtype=dt), rn(rows, H)
         y, _, rs, _ = pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None)
-        ms = time_gpu(lambda: pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None))
+        ms = time_gpu_graph(lambda: pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None))
         add(f"rmsnorm_fwd[{rows}x{H}]", "hbm", 2 * rows * H * e + H * e + 4 * rows, ms, "2RHe+He+4R bytes")
-        ms = time_gpu(lambda: pylayernorm_bwd(dy, x, None, rs, gm, 0, False, None))
+        ms = time_gpu_graph(lambda: pylayernorm_bwd(dy, x, None, rs, gm, 0, False, None))
         add(f"rmsnorm_bwd[{rows}x{H}]", "hbm", 3 * rows * H * e + 4 * rows + 2 * H * e, ms, "3RHe+4R+2He bytes")
         del x, dy, y
     # --- rope -----------------------------------------------------------------------------
     qkv = rn(T, cfg.qkv_per_rank)
     q = qkv[:, : hq * d].view(T, hq, d)
     k = qkv[:, hq * d:(hq + hk) * d].view(T, hk, d)
-    ms = time_gpu(lambda: rope_fwd(q, k, None, cfg.rope_theta, cfg.seq_length, None, False, inplace=True))
+    ms = time_gpu_graph(lambda: rope_fwd(q, k, None, cfg.rope_theta, cfg.seq_length, None, False, inplace=True))
     add(f"rope[{T}x({hq}+{hk})x{d}]", "hbm", 2 * T * (hq + hk) * d * e, ms, "2T(Hq+Hk)de bytes")
     # --- swiglu ---------------------------------------------------------------------------
     yy, gg = rn(T, 2 * F), rn(T, F)
-    ms = time_gpu(lambda: swiglu(yy))
+    ms = time_gpu_graph(lambda: swiglu(yy))
     add(f"swiglu_fwd[{T}x{2 * F}]", "hbm", 3 * T * F * e, ms, "3TFe bytes")
-    ms = time_gpu(lambda: swiglu_back(gg, yy))
+    ms = time_gpu_graph(lambda: swiglu_back(gg, yy))
     add(f"swiglu_bwd[{T}x{2 * F}]", "hbm", 5 * T * F * e, ms, "5TFe bytes")
     # --- residual add -----------------------------------------------------------------------
     a, b = rn(R, H), rn(R, H)
     o = torch.empty_like(a)
-    ms = time_gpu(lambda: bda_fwd(a, b, out=o))
+    ms = time_gpu_graph(lambda: bda_fwd(a, b, out=o))
     add(f"residual_add[{R}x{H}]", "hbm", 3 * R * H * e, ms, "3RHe bytes")
     del yy, gg
     # --- attention (70B shard: causal, S=4096, 8q/1kv, d=128) --------------------------------
@@ -141,7 +167,7 @@ def kernel_rooflines(cfg):
     outs = [rn(S1, hq1, d) for _ in range(4)]
     lses = [torch.randn(1, hq1, S1, generator=g, device=dev) for _ in range(4)]
     om, lm = torch.empty(S1, hq1, d, device=dev, dtype=dt), torch.empty(1, hq1, S1, device=dev)
-    ms = time_gpu(lambda: _Clib.pyattn_merge(outs, lses, [0] * 4, [S1] * 4, om, lm))
+    ms = time_gpu_graph(lambda: _Clib.pyattn_merge(outs, lses, [0] * 4, [S1] * 4, om, lm))
     add("attn_merge[4 steps x 4096x32x128]", "hbm", 5 * S1 * hq1 * d * e + 5 * 4 * S1 * hq1, ms, "(n+1)THde+(n+1)4TH bytes")
     del q1, k1, v1, do1, outs, lses, om, dq1, dk1, dv1, o1
     # --- MoE: 8192 tokens, 8 experts top-2, hidden 4096, expert FFN 14336, this rank holds experts 0,1 ----
@@ -151,10 +177,10 @@ def kernel_rooflines(cfg):
     idx, gates, _ = moe.route_topk(logits, K)
     plan, _ = moe.sort_assignments(idx, E)
     Rm = int(plan.expert_offsets[2].item())
-    ms = time_gpu(lambda: moe.permute_fwd(xm, plan, 0, 2, Rm))
+    ms = time_gpu_graph(lambda: moe.permute_fwd(xm, plan, 0, 2, Rm))
     add(f"moe_permute[R={Rm} H={Hm}]", "hbm", 2 * Rm * Hm * e + 8 * Rm, ms, "2RHe+8R bytes")
     xp, _ = moe.permute_fwd(xm, plan, 0, 2, Rm)
-    ms = time_gpu(lambda: moe.unpermute_fwd(xp, plan, gates, 0, 2))
+    ms = time_gpu_graph(lambda: moe.unpermute_fwd(xp, plan, gates, 0, 2))
     add(f"moe_unpermute[R={Rm} T={Tm} H={Hm}]", "hbm", Rm * Hm * e + Tm * Hm * e + 8 * Rm, ms, "RHe+THe+8R bytes")
     w1 = (torch.randn(2, 2 * Fm, Hm, generator=g, device=dev) * 0.02).to(dt)
     w2 = (torch.randn(2, Hm, Fm, generator=g, device=dev) * 0.02).to(dt)
@@ -194,6 +220,39 @@ def cpu_baseline(cfg):
                       f"fp32 eager PyTorch + autograd on the host (the oracle), after 1 warm-up"}
 
 
+def profile_op(name: str, iters: int = 5):
+    """Run one operator a few times and exit (target of `rocprofv3 --pmc ... -- python bench.py
+    --profile-op NAME`).  ``copy`` is the calibration kernel: a 1 GiB device-to-device copy whose
+    fetch and write sizes are known."""
+    from dhellam_amd import _Clib, _lib
+    dev, dt = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(s, generator=g, device=dev, dtype=torch.float32).to(dt)
+    if name == "copy":
+        n = 1 << 30
+        a = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        b = torch.empty_like(a)
+        lib = _lib.load()
+        fn = lambda: _lib.check(lib.dh_copy_bytes(a.data_ptr(), b.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+    elif name in ("attn_fwd", "attn_bwd", "ring_fwd", "ring_bwd"):
+        T, hq, hk, d = (4096, 8, 1, 128) if name.startswith("attn") else (4096, 32, 8, 128)
+        q, k, v, do = rn(T, hq, d), rn(T, hk, d), rn(T, hk, d), rn(T, hq, d)
+        cu = torch.tensor([0, T], dtype=torch.int32, device=dev)
+        sc = 1.0 / math.sqrt(d)
+        o = _Clib.pymha_varlen_fwd(q, k, v, cu, cu, T, T, 0.0, sc, True, False, 0, False)
+        if name.endswith("fwd"):
+            fn = lambda: _Clib.pymha_varlen_fwd(q, k, v, cu, cu, T, T, 0.0, sc, True, False, 0, False)
+        else:
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            sp = torch.cuda.current_stream().cuda_stream
+            fn = lambda: _Clib._attn_bwd_raw(do, q, k, v, o[0], o[5], dq, dk, dv, None, cu, cu, T, T, sc, True, sp)
+    else:
+        raise SystemExit(f"unknown --profile-op {name}")
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +262,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
+    ap.add_argument("--profile-op", default=None,
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, copy) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "
@@ -212,6 +273,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     _ensure_built()
+    if args.profile_op:
+        torch.cuda.set_device(0)
+        profile_op(args.profile_op)
+        return
     from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
     torch.cuda.set_device(0)
     cfg = llama70b_tp8_shard()

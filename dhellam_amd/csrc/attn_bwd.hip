@@ -455,7 +455,12 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
   __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
   __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
 
-  const int b = blockIdx.z, h = blockIdx.y;
+  const int b = blockIdx.y;
+  // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
+  const int ratio = p.hq / p.hk, P = gridDim.x / p.hq;
+  int hkv, item;
+  xcd_group_item(blockIdx.x, p.hk, ratio * P, hkv, item);
+  const int h = hkv * ratio + item / P, px = item % P;
   const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
   const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
   const int nqt = (sq + BM - 1) / BM;
@@ -464,15 +469,14 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
   const float scale_log2 = p.scale_log2;
   int qt[2], nq;
   if (causal) {
-    const int pair = blockIdx.x;
+    const int pair = px;
     if (2 * pair >= nqt) return;
     qt[0] = nqt - 1 - pair; qt[1] = pair;
     nq = (qt[0] == qt[1]) ? 1 : 2;
   } else {
-    if ((int)blockIdx.x >= nqt) return;
-    qt[0] = blockIdx.x; qt[1] = 0; nq = 1;
+    if (px >= nqt) return;
+    qt[0] = px; qt[1] = 0; nq = 1;
   }
-  const int hkv = h / (p.hq / p.hk);
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
   const int rg = w % RG, sp = w / RG;
@@ -642,7 +646,7 @@ template <typename T, int RG, int SPLIT, int BN>
 static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * RG;
   const int nqt = (int)cdiv(p.max_sq, BM);
-  dim3 grid((unsigned)(p.causal ? (nqt + 1) / 2 : nqt), (unsigned)p.hq, (unsigned)batch);
+  dim3 grid((unsigned)((p.causal ? (nqt + 1) / 2 : nqt) * p.hq), (unsigned)batch);
   hipLaunchKernelGGL((attn_bwd_dq_d128_kernel<T, RG, SPLIT, BN>), grid, dim3(512), 0, st, p);
   return DH_OK;
 }
@@ -663,8 +667,12 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
   __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
   __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
 
-  const int b = blockIdx.z;
-  const int hkv = blockIdx.y / p.hsplit, hs = blockIdx.y % p.hsplit;
+  const int b = blockIdx.y;
+  // all key tiles of one head group read the same Q / dO rows: keep a group on one XCD's L2
+  const int G = p.hk * p.hsplit;
+  int hg, px;
+  xcd_group_item(blockIdx.x, G, gridDim.x / G, hg, px);
+  const int hkv = hg / p.hsplit, hs = hg % p.hsplit;
   const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
   const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
   const int nkt = (sk + BN - 1) / BN;
@@ -673,13 +681,13 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
   const float scale_log2 = p.scale_log2;
   int kt[2], nk;
   if (causal) {
-    const int pair = blockIdx.x;
+    const int pair = px;
     if (2 * pair >= nkt) return;
     kt[0] = pair; kt[1] = nkt - 1 - pair;             // heavy (early keys) first
     nk = (kt[0] == kt[1]) ? 1 : 2;
   } else {
-    if ((int)blockIdx.x >= nkt) return;
-    kt[0] = blockIdx.x; kt[1] = 0; nk = 1;
+    if (px >= nkt) return;
+    kt[0] = px; kt[1] = 0; nk = 1;
   }
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
@@ -891,7 +899,7 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
 template <typename T>
 static int launch_dkv_d128(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
   const int nkt = (int)cdiv(max_sk, 64);
-  dim3 grid((unsigned)(p.causal ? (nkt + 1) / 2 : nkt), (unsigned)(p.hk * p.hsplit), (unsigned)batch);
+  dim3 grid((unsigned)((p.causal ? (nkt + 1) / 2 : nkt) * p.hk * p.hsplit), (unsigned)batch);
   hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(256), 0, st, p);
   return DH_OK;
 }

@@ -251,7 +251,12 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
   __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
 
-  const int b = blockIdx.z, h = blockIdx.y;
+  const int b = blockIdx.y;
+  // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
+  const int ratio = p.hq / p.hk, P = gridDim.x / p.hq;
+  int hkv, item;
+  xcd_group_item(blockIdx.x, p.hk, ratio * P, hkv, item);
+  const int h = hkv * ratio + item / P, px = item % P;
   const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
   const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
   const int nqt = (sq + BM - 1) / BM;
@@ -261,17 +266,16 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   // causal: this workgroup owns query tiles (pair, nqt-1-pair); otherwise one tile
   int qt[2], nq;
   if (causal) {
-    const int pair = blockIdx.x;
+    const int pair = px;
     if (2 * pair >= nqt) return;
     qt[0] = nqt - 1 - pair;
     qt[1] = pair;
     nq = (qt[0] == qt[1]) ? 1 : 2;
   } else {
-    if ((int)blockIdx.x >= nqt) return;
-    qt[0] = blockIdx.x; qt[1] = 0;
+    if (px >= nqt) return;
+    qt[0] = px; qt[1] = 0;
     nq = 1;
   }
-  const int hkv = h / (p.hq / p.hk);
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
   const int rg = w % RG, sp = w / RG;
@@ -488,7 +492,7 @@ template <typename T, int RG, int SPLIT, int BN>
 static int launch_attn_fwd_d128(const AttnFwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * RG;
   const int nqt = (int)cdiv(p.max_sq, BM);
-  dim3 grid((unsigned)(p.causal ? (nqt + 1) / 2 : nqt), (unsigned)p.hq, (unsigned)batch);
+  dim3 grid((unsigned)((p.causal ? (nqt + 1) / 2 : nqt) * p.hq), (unsigned)batch);
   hipLaunchKernelGGL((attn_fwd_d128_kernel<T, RG, SPLIT, BN>), grid, dim3(512), 0, st, p);
   return DH_OK;
 }

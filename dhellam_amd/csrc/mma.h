@@ -147,4 +147,21 @@ __device__ __forceinline__ typename Mma<T>::Frag tr4_get(Tr4 &o, int t) {
 // Row index inside a 32-row accumulator block held by register v of lane half h.
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 
+// Workgroups reach the 8 XCDs round-robin by linear id and each XCD has its own L2.  Split a linear id over
+// G groups of I items so that the workgroups of one group (which re-read the same rows) stay on as few XCDs
+// as possible: whole groups per XCD when G divides by 8, one group per 8 / G XCDs when G divides 8.
+__device__ __forceinline__ void xcd_group_item(int id, int G, int I, int &g, int &i) {
+  const int x = id & 7, n = id >> 3;
+  if ((G & 7) == 0) {
+    g = x + 8 * (n / I);
+    i = n % I;
+  } else if (8 % G == 0 && ((G * I) & 7) == 0) {
+    g = x % G;
+    i = x / G + (8 / G) * n;
+  } else {
+    g = id % G;
+    i = id / G;
+  }
+}
+
 }  // namespace dh

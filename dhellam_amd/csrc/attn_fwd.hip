@@ -210,28 +210,53 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
 //   K (read as 16 B row fragments):  chunk ^= row % 16
 //   V (read with transpose loads) :  chunk ^= 4 * (row % 4) + (row / 4) % 4
 // Causal work is made uniform by giving a workgroup the query tiles i and n-1-i.
-// Issue the copies of one pipeline stage: this wavefront's LD 1 KB blocks (4 rows of a K or V tile each).
+// All global->LDS copies and all LDS reads of the main loop are written in assembly: the
+// compiler then keeps no per-lane 64-bit pointers and inserts no waits of its own between
+// copies in flight and fragment reads, and the copies are spread between the MFMAs so
+// that they do not queue up behind each other.
+
+// Per-lane constants of the general (clamped) K/V tile copies.
+struct FwdCopyLane {
+  int lrow, l16;         // row inside a 4-row copy block, 16-byte chunk slot
+};
+
+// One 1 KB copy (4 rows of a K or V tile) in its fast form: wave-uniform 64-bit global base, the lane's
+// 32-bit byte offset, wave-uniform LDS byte address.  The compiler does not count these copies: the
+// kernel waits for them itself (dma_wait_all) before the barrier that publishes a stage.
+__device__ __forceinline__ void dma_block_fast(const char *base, uint32_t lane_off, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_off), "s"(base), "s"(lds_dst)
+               : "memory", "m0");
+}
+
+// All LD copy blocks of wavefront `w` for iteration `it`, general form: rows past the last key are
+// clamped per lane (they are masked in the scores, and their V rows meet zero probabilities).  Kept as
+// a rolled loop: it runs once per query tile, for tiles that reach past the keys, and for wavefronts
+// whose own tile is fully masked.
 template <typename T, int SPLIT, int BN, int LD>
 __device__ __forceinline__ void fwd_issue_stage(T *stage, const T *kg, const T *vg, int k_stride, int v_stride, int it,
-                                                int ntiles, int sk, int w, int lrow, int l16) {
+                                                int ntiles, int sk, int w, const FwdCopyLane &cl) {
   constexpr int TILE = BN * 128;
-#pragma unroll
+  asm volatile("" : "+s"(it));                   // keep the address arithmetic next to the copies
+#pragma unroll 1
   for (int i = 0; i < LD; ++i) {
-    const int blk = w * LD + i;                  // 1 KB block inside the stage (wave-uniform)
+    const int blk = w * LD + i;
     const int tile = blk / (BN / 2);
     const int kvsel = (blk % (BN / 2)) / (BN / 4);
     const int rgp = blk % (BN / 4);
     const int tile_g = it * SPLIT + tile;
-    if (tile_g < ntiles) {
-      const int row = 4 * rgp + lrow;
-      int kr = tile_g * BN + row;
-      kr = kr < sk ? kr : sk - 1;                // rows past the end are masked later; keep the read in bounds
-      const int f = kvsel ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
-      const T *src = (kvsel ? vg + (int64_t)kr * v_stride : kg + (int64_t)kr * k_stride) + ((l16 ^ f) * 8);
-      T *dst = stage + tile * 2 * TILE + kvsel * TILE + rgp * 512;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
-    }
+    if (tile_g >= ntiles) continue;
+    T *dst = stage + tile * 2 * TILE + kvsel * TILE + rgp * 512;
+    int kr = tile_g * BN + 4 * rgp + cl.lrow;
+    kr = kr < sk ? kr : sk - 1;
+    const int row = 4 * rgp + cl.lrow;
+    const T *gsel = kvsel ? vg : kg;
+    const int stride = kvsel ? v_stride : k_stride;
+    const int f = kvsel ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
+    const T *src = gsel + (int64_t)kr * stride + ((cl.l16 ^ f) * 8);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                     (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
   }
 }
 
@@ -245,11 +270,8 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   constexpr int STAGE = SPLIT * 2 * TILE;         // elements per pipeline stage
   constexpr int BLK_PER_STAGE = STAGE * (int)sizeof(T) / 1024;  // 1 KB copy blocks per stage
   constexpr int LD = BLK_PER_STAGE / 8;
-  static_assert(BLK_PER_STAGE % 8 == 0, "copy blocks must divide over the wavefronts");
-  // Two separate LDS objects, one per stage: reads of one stage are then known not to
-  // alias the copies in flight into the other, and need not wait for them.
-  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
-  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+  static_assert(BLK_PER_STAGE % 8 == 0 && LD == 8, "eight copy blocks per wavefront and stage");
+  __shared__ __attribute__((aligned(1024))) T sStage[2 * STAGE];
 
   const int b = blockIdx.y;
   // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
@@ -276,20 +298,46 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
     qt[0] = px; qt[1] = 0;
     nq = 1;
   }
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
   const int c = lane & 31, hh = lane >> 5;
   const int rg = w % RG, sp = w / RG;
   const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
   const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)sStage;
 
   // ---- per-lane constants of the copy and of the fragment reads ---------------------------
-  const int l16 = lane & 15, lrow = lane >> 4;        // copy: chunk slot and row inside a 4-row block
-  const int xk = c & 15;                              // K row fragment: chunk ^= row % 16 (row = 32 nb + c)
+  FwdCopyLane cl0;                                    // copy: chunk slot and row inside a 4-row block
+  cl0.l16 = lane & 15;
+  cl0.lrow = lane >> 4;
+  // Fast copies: the 8 copy blocks of a wavefront are 32 consecutive rows of ONE tile (K or V), so per
+  // iteration they share a base that advances by 4 rows per block, and the lane offset only depends on
+  // block % 4 (through the swizzle).
+  constexpr int BPT = BN / 4;                         // copy blocks per K (or V) tile
+  const int cp_tile = (w * LD) / (2 * BPT);           // which of the SPLIT resident tiles
+  const int cp_v = ((w * LD) % (2 * BPT)) / BPT;      // 0: K, 1: V
+  const int cp_r0 = 4 * ((w * LD) % BPT);             // first row inside the tile
+  const int cp_stride = cp_v ? v_stride : k_stride;
+  const char *cp_g = reinterpret_cast<const char *>(cp_v ? vg : kg);
+  const uint32_t cp_dst0 = (uint32_t)((cp_tile * 2 * TILE + cp_v * TILE) * (int)sizeof(T) + cp_r0 * 256);
+  const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
+  uint32_t cp_off[4];
+  {
+    const uint32_t rowb = (uint32_t)(cl0.lrow * cp_stride) * (uint32_t)sizeof(T);
+    const uint32_t chunk = (uint32_t)(cp_v ? (cl0.l16 ^ (4 * cl0.lrow)) : (cl0.l16 ^ cl0.lrow)) << 4;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << (cp_v ? 4 : 6)));
+  }
+  // Fragment reads: byte offsets of the lane inside a K / V tile.  The swizzle XORs only bits 4..7 of an
+  // address whose other low bits are fixed, so the remaining fragments of a tile are reached by XORing a
+  // constant into these (K: 32 * ks; V: 64 * t) plus an immediate offset (K: 8 KB per 32 keys; V: 4 KB per 16).
   const int r = lane & 15;
+  const uint32_t kb_lane = (uint32_t)(sp * 2 * TILE * (int)sizeof(T) + c * 256 + ((hh ^ (c & 15)) << 4));
   const int va_x = 4 * (r >> 2) + hh;                 // V transpose read, first four keys of a step
-  const int vb_x = va_x + 2;                          // second four keys (row + 8)
   const int v_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
-  const int v_sub = (r & 3) & 1;
+  const uint32_t v_row = (uint32_t)((sp * 2 * TILE + TILE) * (int)sizeof(T) + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t va_lane = v_row + (uint32_t)((v_lc ^ va_x) << 4);
+  const uint32_t vb_lane = v_row + 8 * 256 + (uint32_t)((v_lc ^ (va_x + 2)) << 4);   // second four keys (row + 8)
 
   for (int qi = 0; qi < nq; ++qi) {
     const int m0 = qt[qi] * BM;
@@ -305,6 +353,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
     if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
     const int ntiles = (nk_end + BN - 1) / BN;
     const int niter = (ntiles + SPLIT - 1) / SPLIT;
+    const int n_fast = sk / (SPLIT * BN);          // iterations whose tiles lie wholly inside the keys
 
     floatx16 O[D / 32];
 #pragma unroll
@@ -313,129 +362,148 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       for (int v = 0; v < 16; ++v) O[t][v] = 0.f;
     float m_run = -1e30f, l_run = 0.f;
 
-    // One tile of this wavefront's split, read from `stage`.
-    auto compute = [&](const T *stage, int it) {
+    if (niter > 0) fwd_issue_stage<T, SPLIT, BN, LD>(sStage, kg, vg, k_stride, v_stride, 0, ntiles, sk, w, cl0);
+    dma_wait_all();
+    __syncthreads();
+
+#pragma unroll 1
+    for (int it = 0; it < niter; ++it) {
+      // This iteration reads stage it % 2; the copies of iteration it + 1 go to the other stage.
+      const uint32_t cur = lds0 + (uint32_t)((it & 1) * STAGE * (int)sizeof(T));
+      const uint32_t nxt = lds0 + (uint32_t)(((it + 1) & 1) * STAGE * (int)sizeof(T));
+      const int nit = it + 1;
+      const bool copy = nit < niter;
+      const bool fast = copy && nit < n_fast;
+      const bool fcopy = fast && nit * SPLIT + cp_tile < ntiles;   // this wavefront's tile of the next stage exists
+      const char *cp_src = cp_g + (int64_t)((nit * SPLIT + cp_tile) * BN + cp_r0) * cp_stride * (int)sizeof(T);
+      uint32_t cp_dst = nxt + cp_dst0;
       const int tile_g = it * SPLIT + sp;
       const int n0 = tile_g * BN;
-      if (tile_g >= ntiles || (causal && n0 > wrow0 + 31)) return;
-      const T *tK = stage + sp * 2 * TILE;
-      const T *tV = tK + TILE;
-      floatx16 S[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) S[nb][v] = 0.f;
-      {
-        // K fragments are fetched one step ahead of the MFMA that consumes them.
-        Frag a_cur = frag_ld<T>(tK + c * D + ((hh ^ xk) * 8));
-#pragma unroll
-        for (int i = 0; i < NB * (D / 16); ++i) {
-          const int nb = i / (D / 16), ks = i % (D / 16);
-          Frag a_nxt = a_cur;
-          if (i + 1 < NB * (D / 16)) {
-            const int nb2 = (i + 1) / (D / 16), ks2 = (i + 1) % (D / 16);
-            a_nxt = frag_ld<T>(tK + (nb2 * 32 + c) * D + (((2 * ks2 + hh) ^ xk) * 8));
-          }
-          S[nb] = M::mma(a_cur, Qf[ks], S[nb]);
-          a_cur = a_nxt;
-        }
-      }
-      const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
-      if (need_mask) {
+      const bool idle = tile_g >= ntiles || (causal && n0 > wrow0 + 31);
+      if (copy && (idle || !fast))
+        fwd_issue_stage<T, SPLIT, BN, LD>(sStage + ((it + 1) & 1) * STAGE, kg, vg, k_stride, v_stride, nit, ntiles, sk, w, cl0);
+      if (!idle) {
+        uint32_t kb = cur + kb_lane, va = cur + va_lane, vb = cur + vb_lane;
+        // derive the other addresses inside the loop, not ahead of it
+        asm volatile("" : "+v"(kb), "+v"(va), "+v"(vb));
+#define DH_FWD_COPY(i)                                                                                  \
+        do {                                                                                            \
+          if (fcopy) {                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                          \
+            dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                            \
+            cp_src += cp_step;                                                                          \
+            cp_dst += 1024;                                                                             \
+            __builtin_amdgcn_sched_barrier(0);                                                          \
+          }                                                                                             \
+        } while (0)
+        floatx16 S[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int kv = n0 + nb * 32 + acc_row(v, hh);
-            if (kv >= sk || (causal && kv > row_q)) S[nb][v] = -INFINITY;
+          for (int v = 0; v < 16; ++v) S[nb][v] = 0.f;
+        {
+          // K fragments are fetched in pairs, one pair ahead of the MFMAs that consume them.
+          constexpr int NP = NB * (D / 16) / 2;
+          int4v ka[4];
+          lds_read128<0>(ka[0], kb);
+          lds_read128<0>(ka[1], kb ^ 32u);
+#pragma unroll
+          for (int pr = 0; pr < NP; ++pr) {
+            const int i = 2 * pr, nb = i / (D / 16), ks = i % (D / 16);
+            const int a = 2 * (pr & 1), bq = 2 * ((pr + 1) & 1);
+            if (pr + 1 < NP) {
+              const int i2 = i + 2, nb2 = i2 / (D / 16), ks2 = i2 % (D / 16);
+              if (nb2 == 0) {
+                lds_read128<0>(ka[bq], kb ^ (uint32_t)(ks2 << 5));
+                lds_read128<0>(ka[bq + 1], kb ^ (uint32_t)((ks2 + 1) << 5));
+              } else {
+                lds_read128<32 * 256>(ka[bq], kb ^ (uint32_t)(ks2 << 5));
+                lds_read128<32 * 256>(ka[bq + 1], kb ^ (uint32_t)((ks2 + 1) << 5));
+              }
+              lds_wait<2>(ka[a], ka[a + 1]);
+            } else {
+              lds_wait<0>(ka[a], ka[a + 1]);
+            }
+            S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a]), Qf[ks], S[nb]);
+            S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a + 1]), Qf[ks + 1], S[nb]);
+            if (pr % NB == NB - 1) DH_FWD_COPY(pr / NB);      // copy blocks 0..3
           }
-      }
-      float mx = S[0][0];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      if (__any(m_new > m_run)) {
-        const float alpha = fast_exp2((m_run - m_new) * scale_log2);
-        l_run *= alpha;
-#pragma unroll
-        for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) O[t][v] *= alpha;
-      }
-      m_run = m_new;
-      const float mc = m_new * scale_log2;
-      float ps = 0.f;
-      Frag Pb[NS];
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        float pv[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          pv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
-          ps += pv[j];
         }
-        Pb[s] = frag_pack<T>(pv);
-      }
-      l_run += ps;
-      // V^T fragments: transpose reads issued as one batch per 16-key step, consumed as they land.
-      // They are written in assembly so that they are not held back by the copies in flight
-      // into the OTHER stage (a transpose-read builtin would wait for every outstanding copy).
+        const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+        if (need_mask) {
 #pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        const uint32_t ra = (uint32_t)(uintptr_t)(tV + (16 * s + 4 * hh + (r >> 2)) * D + v_sub * 4);
-        const uint32_t rb = ra + 8 * D * (uint32_t)sizeof(T);
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int kv = n0 + nb * 32 + acc_row(v, hh);
+              if (kv >= sk || (causal && kv > row_q)) S[nb][v] = -INFINITY;
+            }
+        }
+        float mx = S[0][0];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        if (__any(m_new > m_run)) {
+          const float alpha = fast_exp2((m_run - m_new) * scale_log2);
+          l_run *= alpha;
+#pragma unroll
+          for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) O[t][v] *= alpha;
+        }
+        m_run = m_new;
+        const float mc = m_new * scale_log2;
+        float ps = 0.f;
+        Frag Pb[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          float pv[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            pv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
+            ps += pv[j];
+          }
+          Pb[s] = frag_pack<T>(pv);
+        }
+        l_run += ps;
+        // V^T fragments: eight transpose reads per 16-key step, consumed as they land.
         uint32_t ad[8];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const int lc = 4 * t + v_lc;
-          ad[2 * t] = ra + ((lc ^ va_x) * 16);
-          ad[2 * t + 1] = rb + ((lc ^ vb_x) * 16);
+          ad[2 * t] = va ^ (uint32_t)(t << 6);
+          ad[2 * t + 1] = vb ^ (uint32_t)(t << 6);
         }
-        short4v f[8];
-        asm volatile("ds_read_b64_tr_b16 %0, %8\n\tds_read_b64_tr_b16 %1, %9\n\t"
-                     "ds_read_b64_tr_b16 %2, %10\n\tds_read_b64_tr_b16 %3, %11\n\t"
-                     "ds_read_b64_tr_b16 %4, %12\n\tds_read_b64_tr_b16 %5, %13\n\t"
-                     "ds_read_b64_tr_b16 %6, %14\n\tds_read_b64_tr_b16 %7, %15"
-                     : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&v"(f[4]), "=&v"(f[5]), "=&v"(f[6]), "=&v"(f[7])
-                     : "v"(ad[0]), "v"(ad[1]), "v"(ad[2]), "v"(ad[3]), "v"(ad[4]), "v"(ad[5]), "v"(ad[6]), "v"(ad[7])
-                     : "memory");
-#define DH_FWD_PV(t, cnt)                                                                  \
-        asm volatile("s_waitcnt lgkmcnt(" #cnt ")" : "+v"(f[2 * t]), "+v"(f[2 * t + 1]));  \
-        {                                                                                  \
-          short8v o8;                                                                      \
-          o8[0] = f[2 * t][0]; o8[1] = f[2 * t][1]; o8[2] = f[2 * t][2]; o8[3] = f[2 * t][3];              \
-          o8[4] = f[2 * t + 1][0]; o8[5] = f[2 * t + 1][1]; o8[6] = f[2 * t + 1][2]; o8[7] = f[2 * t + 1][3]; \
-          O[t] = M::mma(__builtin_bit_cast(Frag, o8), Pb[s], O[t]);                         \
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          short4v f[8];
+          if (s == 0) lds_read_tr8<0>(f, ad);
+          else if (s == 1) lds_read_tr8<16 * 256>(f, ad);
+          else if (s == 2) lds_read_tr8<32 * 256>(f, ad);
+          else lds_read_tr8<48 * 256>(f, ad);
+          lds_wait<4>(f[0], f[1], f[2], f[3]);
+          O[0] = M::mma(frag_join<T>(f[0], f[1]), Pb[s], O[0]);
+          O[1] = M::mma(frag_join<T>(f[2], f[3]), Pb[s], O[1]);
+          if (NS == 2) DH_FWD_COPY(4 + 2 * s);
+          lds_wait<0>(f[4], f[5], f[6], f[7]);
+          O[2] = M::mma(frag_join<T>(f[4], f[5]), Pb[s], O[2]);
+          O[3] = M::mma(frag_join<T>(f[6], f[7]), Pb[s], O[3]);
+          if (NS == 2) DH_FWD_COPY(5 + 2 * s);
+          else DH_FWD_COPY(4 + s);                                        // copy blocks 4..7
         }
-        DH_FWD_PV(0, 6)
-        DH_FWD_PV(1, 4)
-        DH_FWD_PV(2, 2)
-        DH_FWD_PV(3, 0)
-#undef DH_FWD_PV
+#undef DH_FWD_COPY
       }
-    };
-
-    if (niter > 0) fwd_issue_stage<T, SPLIT, BN, LD>(sStage0, kg, vg, k_stride, v_stride, 0, ntiles, sk, w, lrow, l16);
-    __syncthreads();
-    for (int it = 0; it < niter; it += 2) {
-      if (it + 1 < niter) fwd_issue_stage<T, SPLIT, BN, LD>(sStage1, kg, vg, k_stride, v_stride, it + 1, ntiles, sk, w, lrow, l16);
-      compute(sStage0, it);
-      __syncthreads();   // stage 1 has landed, and everyone is done with stage 0
-      if (it + 1 < niter) {
-        if (it + 2 < niter) fwd_issue_stage<T, SPLIT, BN, LD>(sStage0, kg, vg, k_stride, v_stride, it + 2, ntiles, sk, w, lrow, l16);
-        compute(sStage1, it + 1);
-        __syncthreads();
-      }
+      dma_wait_all();
+      __syncthreads();   // the next stage has landed, and everyone is done with this one
     }
 
     // ---- combine the key/value splits through LDS (fixed order: deterministic) --------------
     // O of split s > 0, row group g -> slot x = (s-1)*RG + g: slots 0..3 in stage 0, the rest in stage 1;
     // m and l after them in stage 1.
-    float *x0 = reinterpret_cast<float *>(sStage0);
-    float *x1 = reinterpret_cast<float *>(sStage1);
+    float *x0 = reinterpret_cast<float *>(sStage);
+    float *x1 = reinterpret_cast<float *>(sStage + STAGE);
     float *xml = x1 + 2 * 4096;
     static_assert((SPLIT - 1) * RG <= 6, "exchange slots");
     static_assert(STAGE * sizeof(T) >= 4 * 4096 * sizeof(float), "stage 0 holds four O slots");

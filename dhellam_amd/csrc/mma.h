@@ -144,6 +144,49 @@ __device__ __forceinline__ typename Mma<T>::Frag tr4_get(Tr4 &o, int t) {
   return __builtin_bit_cast(typename Mma<T>::Frag, o8);
 }
 
+// ---- LDS reads in assembly ------------------------------------------------------------------------
+// The kernels that fill LDS with direct global->LDS copies read it back through these helpers: the
+// compiler cannot tell which pipeline stage a read touches and would otherwise wait for every copy in
+// flight.  The caller orders each use after lds_wait<N>() on the destination registers (LDS reads
+// complete in order: "at most N outstanding" means everything issued earlier has landed).
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+// Wait for every global->LDS copy this wavefront has issued (the ones issued in assembly are not
+// counted by the compiler).
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <int OFF> __device__ __forceinline__ void lds_read128(int4v &d, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(d) : "v"(addr), "n"(OFF) : "memory");
+}
+// Eight transpose reads (b64, 16-bit elements) from eight lane addresses plus a common byte offset.
+template <int OFF> __device__ __forceinline__ void lds_read_tr8(short4v (&f)[8], const uint32_t (&ad)[8]) {
+  asm volatile("ds_read_b64_tr_b16 %0, %8 offset:%16\n\tds_read_b64_tr_b16 %1, %9 offset:%16\n\t"
+               "ds_read_b64_tr_b16 %2, %10 offset:%16\n\tds_read_b64_tr_b16 %3, %11 offset:%16\n\t"
+               "ds_read_b64_tr_b16 %4, %12 offset:%16\n\tds_read_b64_tr_b16 %5, %13 offset:%16\n\t"
+               "ds_read_b64_tr_b16 %6, %14 offset:%16\n\tds_read_b64_tr_b16 %7, %15 offset:%16"
+               : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&v"(f[4]), "=&v"(f[5]), "=&v"(f[6]), "=&v"(f[7])
+               : "v"(ad[0]), "v"(ad[1]), "v"(ad[2]), "v"(ad[3]), "v"(ad[4]), "v"(ad[5]), "v"(ad[6]), "v"(ad[7]), "n"(OFF)
+               : "memory");
+}
+template <int N> __device__ __forceinline__ void lds_wait(int4v &d) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(d) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(int4v &a, int4v &b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(short4v &a, short4v &b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void lds_wait(short4v &a, short4v &b, short4v &c, short4v &d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <typename T> __device__ __forceinline__ typename Mma<T>::Frag frag_join(const short4v &a, const short4v &b) {
+  short8v o8;
+  o8[0] = a[0]; o8[1] = a[1]; o8[2] = a[2]; o8[3] = a[3];
+  o8[4] = b[0]; o8[5] = b[1]; o8[6] = b[2]; o8[7] = b[3];
+  return __builtin_bit_cast(typename Mma<T>::Frag, o8);
+}
+
 // Row index inside a 32-row accumulator block held by register v of lane half h.
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 

@@ -11,6 +11,9 @@
 // tile.  fp32 scores are scaled inside the exp2 argument (one FMA), the running
 // output is rescaled only when some row's maximum actually moved.
 #include "mma.h"
+#ifndef DH_FWD_LAG
+#define DH_FWD_LAG true
+#endif
 
 namespace dh {
 
@@ -230,48 +233,42 @@ __device__ __forceinline__ void dma_block_fast(const char *base, uint32_t lane_o
                : "memory", "m0");
 }
 
-// All LD copy blocks of wavefront `w` for iteration `it`, general form: rows past the last key are
-// clamped per lane (they are masked in the scores, and their V rows meet zero probabilities).  Kept as
-// a rolled loop: it runs once per query tile, for tiles that reach past the keys, and for wavefronts
-// whose own tile is fully masked.
-template <typename T, int SPLIT, int BN, int LD>
-__device__ __forceinline__ void fwd_issue_stage(T *stage, const T *kg, const T *vg, int k_stride, int v_stride, int it,
-                                                int ntiles, int sk, int w, const FwdCopyLane &cl) {
-  constexpr int TILE = BN * 128;
-  asm volatile("" : "+s"(it));                   // keep the address arithmetic next to the copies
+// The 8 copy blocks (32 rows of one K or V tile) of a wavefront in general form: rows past the last key
+// are clamped per lane (they are masked in the scores, and their V rows meet zero probabilities).  Kept
+// as a rolled loop: it runs once per query tile and for tiles that reach past the keys.
+template <typename T>
+__device__ __forceinline__ void fwd_issue_general(T *dst, const T *g, int stride, int is_v, int row0_g, int row0_t, int sk,
+                                                  const FwdCopyLane &cl) {
+  asm volatile("" : "+s"(row0_g));               // keep the address arithmetic next to the copies
 #pragma unroll 1
-  for (int i = 0; i < LD; ++i) {
-    const int blk = w * LD + i;
-    const int tile = blk / (BN / 2);
-    const int kvsel = (blk % (BN / 2)) / (BN / 4);
-    const int rgp = blk % (BN / 4);
-    const int tile_g = it * SPLIT + tile;
-    if (tile_g >= ntiles) continue;
-    T *dst = stage + tile * 2 * TILE + kvsel * TILE + rgp * 512;
-    int kr = tile_g * BN + 4 * rgp + cl.lrow;
+  for (int i = 0; i < 8; ++i) {
+    int kr = row0_g + 4 * i + cl.lrow;
     kr = kr < sk ? kr : sk - 1;
-    const int row = 4 * rgp + cl.lrow;
-    const T *gsel = kvsel ? vg : kg;
-    const int stride = kvsel ? v_stride : k_stride;
-    const int f = kvsel ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
-    const T *src = gsel + (int64_t)kr * stride + ((cl.l16 ^ f) * 8);
+    const int row = row0_t + 4 * i + cl.lrow;
+    const int f = is_v ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
+    const T *src = g + (int64_t)kr * stride + ((cl.l16 ^ f) * 8);
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                     (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+                                     (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
   }
 }
 
-template <typename T, int RG, int SPLIT, int BN>
+// LAG: the wavefronts of the upper half of the workgroup (the second wavefront of every SIMD) run their
+// P V products one iteration late.  In each half of an iteration one wavefront of a SIMD is then in its
+// matrix phase while the other is in its softmax, instead of both competing for the same unit.  V tiles
+// live one iteration longer for that (three V slots against two K slots).
+template <typename T, int RG, int SPLIT, int BN, bool LAG>
 __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int D = 128, BM = 32 * RG, NB = BN / 32, NS = BN / 16;
   static_assert(RG * SPLIT == 8, "8 wavefronts per workgroup");
   constexpr int TILE = BN * D;                    // elements of one K (or V) tile
-  constexpr int STAGE = SPLIT * 2 * TILE;         // elements per pipeline stage
-  constexpr int BLK_PER_STAGE = STAGE * (int)sizeof(T) / 1024;  // 1 KB copy blocks per stage
-  constexpr int LD = BLK_PER_STAGE / 8;
-  static_assert(BLK_PER_STAGE % 8 == 0 && LD == 8, "eight copy blocks per wavefront and stage");
-  __shared__ __attribute__((aligned(1024))) T sStage[2 * STAGE];
+  constexpr int SLOT = SPLIT * TILE;              // elements of one K (or V) slot: the tiles of all splits
+  constexpr int SLOTB = SLOT * (int)sizeof(T);
+  constexpr int BPT = BN / 4;                     // 1 KB copy blocks per tile
+  static_assert(SPLIT * 2 * BPT == 64, "eight copy blocks per wavefront and iteration");
+  constexpr int NV = LAG ? 3 : 2;                 // V slots
+  __shared__ __attribute__((aligned(1024))) T sAll[(2 + NV) * SLOT];   // K slots 0..1, then the V slots
 
   const int b = blockIdx.y;
   // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
@@ -302,24 +299,25 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
   const int c = lane & 31, hh = lane >> 5;
   const int rg = w % RG, sp = w / RG;
+  const bool lag = LAG && w >= 4;
   const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
   const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)sStage;
+  const uint32_t ldsK = (uint32_t)(uintptr_t)sAll, ldsV = ldsK + 2 * SLOTB;
 
   // ---- per-lane constants of the copy and of the fragment reads ---------------------------
   FwdCopyLane cl0;                                    // copy: chunk slot and row inside a 4-row block
   cl0.l16 = lane & 15;
   cl0.lrow = lane >> 4;
-  // Fast copies: the 8 copy blocks of a wavefront are 32 consecutive rows of ONE tile (K or V), so per
-  // iteration they share a base that advances by 4 rows per block, and the lane offset only depends on
-  // block % 4 (through the swizzle).
-  constexpr int BPT = BN / 4;                         // copy blocks per K (or V) tile
-  const int cp_tile = (w * LD) / (2 * BPT);           // which of the SPLIT resident tiles
-  const int cp_v = ((w * LD) % (2 * BPT)) / BPT;      // 0: K, 1: V
-  const int cp_r0 = 4 * ((w * LD) % BPT);             // first row inside the tile
+  // The 8 copy blocks of a wavefront are 32 consecutive rows of ONE tile (K or V), so per iteration they
+  // share a base that advances by 4 rows per block, and the lane offset only depends on block % 4
+  // (through the swizzle).
+  const int cp_tile = (w * 8) / (2 * BPT);            // which of the SPLIT resident tiles
+  const int cp_v = ((w * 8) % (2 * BPT)) / BPT;       // 0: K, 1: V
+  const int cp_r0 = 4 * ((w * 8) % BPT);              // first row inside the tile
   const int cp_stride = cp_v ? v_stride : k_stride;
-  const char *cp_g = reinterpret_cast<const char *>(cp_v ? vg : kg);
-  const uint32_t cp_dst0 = (uint32_t)((cp_tile * 2 * TILE + cp_v * TILE) * (int)sizeof(T) + cp_r0 * 256);
+  const T *cp_gt = cp_v ? vg : kg;
+  const char *cp_g = reinterpret_cast<const char *>(cp_gt);
+  const int cp_dst0 = cp_tile * TILE + cp_r0 * D;     // elements inside a slot
   const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
   uint32_t cp_off[4];
   {
@@ -328,14 +326,14 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
 #pragma unroll
     for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << (cp_v ? 4 : 6)));
   }
-  // Fragment reads: byte offsets of the lane inside a K / V tile.  The swizzle XORs only bits 4..7 of an
+  // Fragment reads: byte offsets of the lane inside a K / V slot.  The swizzle XORs only bits 4..7 of an
   // address whose other low bits are fixed, so the remaining fragments of a tile are reached by XORing a
   // constant into these (K: 32 * ks; V: 64 * t) plus an immediate offset (K: 8 KB per 32 keys; V: 4 KB per 16).
   const int r = lane & 15;
-  const uint32_t kb_lane = (uint32_t)(sp * 2 * TILE * (int)sizeof(T) + c * 256 + ((hh ^ (c & 15)) << 4));
+  const uint32_t kb_lane = (uint32_t)(sp * TILE * (int)sizeof(T) + c * 256 + ((hh ^ (c & 15)) << 4));
   const int va_x = 4 * (r >> 2) + hh;                 // V transpose read, first four keys of a step
   const int v_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
-  const uint32_t v_row = (uint32_t)((sp * 2 * TILE + TILE) * (int)sizeof(T) + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t v_row = (uint32_t)(sp * TILE * (int)sizeof(T) + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
   const uint32_t va_lane = v_row + (uint32_t)((v_lc ^ va_x) << 4);
   const uint32_t vb_lane = v_row + 8 * 256 + (uint32_t)((v_lc ^ (va_x + 2)) << 4);   // second four keys (row + 8)
 
@@ -361,41 +359,88 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
 #pragma unroll
       for (int v = 0; v < 16; ++v) O[t][v] = 0.f;
     float m_run = -1e30f, l_run = 0.f;
+    Frag Pb[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Pb[s][j] = static_cast<T>(0.f);
 
-    if (niter > 0) fwd_issue_stage<T, SPLIT, BN, LD>(sStage, kg, vg, k_stride, v_stride, 0, ntiles, sk, w, cl0);
+    if (niter > 0 && cp_tile < ntiles)
+      fwd_issue_general<T>(sAll + (cp_v ? 2 * SLOT : 0) + cp_dst0, cp_gt, cp_stride, cp_v, cp_tile * BN + cp_r0, cp_r0, sk, cl0);
     dma_wait_all();
     __syncthreads();
 
+    // slots of iteration it: K it % 2, V it % NV
+    uint32_t k_cur = ldsK, k_nxt = ldsK + SLOTB;
+    int v_cur = 0, v_prev = NV - 1;
+    bool act_prev = false;
+    const char *cp_src = nullptr;
+    uint32_t cp_dst = 0;
+    bool fcopy = false;
+
+#define DH_FWD_COPY(i)                                                                                  \
+    do {                                                                                                \
+      if (fcopy) {                                                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+        dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                                \
+        cp_src += cp_step;                                                                              \
+        cp_dst += 1024;                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+      }                                                                                                 \
+    } while (0)
+
+    // O^T += V^T P^T for the tile in V slot `vs`; copy blocks 4..7 go out between the MFMAs.
+    auto pv = [&](int vs) {
+      uint32_t va = ldsV + (uint32_t)(vs * SLOTB) + va_lane, vb = ldsV + (uint32_t)(vs * SLOTB) + vb_lane;
+      asm volatile("" : "+v"(va), "+v"(vb));     // derive the other addresses here, not ahead of the loop
+      uint32_t ad[8];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        ad[2 * t] = va ^ (uint32_t)(t << 6);
+        ad[2 * t + 1] = vb ^ (uint32_t)(t << 6);
+      }
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        short4v f[8];
+        if (s == 0) lds_read_tr8<0>(f, ad);
+        else if (s == 1) lds_read_tr8<16 * 256>(f, ad);
+        else if (s == 2) lds_read_tr8<32 * 256>(f, ad);
+        else lds_read_tr8<48 * 256>(f, ad);
+        lds_wait<4>(f[0], f[1], f[2], f[3]);
+        O[0] = M::mma(frag_join<T>(f[0], f[1]), Pb[s], O[0]);
+        O[1] = M::mma(frag_join<T>(f[2], f[3]), Pb[s], O[1]);
+        if (NS == 2) DH_FWD_COPY(4 + 2 * s);
+        lds_wait<0>(f[4], f[5], f[6], f[7]);
+        O[2] = M::mma(frag_join<T>(f[4], f[5]), Pb[s], O[2]);
+        O[3] = M::mma(frag_join<T>(f[6], f[7]), Pb[s], O[3]);
+        if (NS == 2) DH_FWD_COPY(5 + 2 * s);
+        else DH_FWD_COPY(4 + s);
+      }
+    };
+
 #pragma unroll 1
     for (int it = 0; it < niter; ++it) {
-      // This iteration reads stage it % 2; the copies of iteration it + 1 go to the other stage.
-      const uint32_t cur = lds0 + (uint32_t)((it & 1) * STAGE * (int)sizeof(T));
-      const uint32_t nxt = lds0 + (uint32_t)(((it + 1) & 1) * STAGE * (int)sizeof(T));
       const int nit = it + 1;
-      const bool copy = nit < niter;
-      const bool fast = copy && nit < n_fast;
-      const bool fcopy = fast && nit * SPLIT + cp_tile < ntiles;   // this wavefront's tile of the next stage exists
-      const char *cp_src = cp_g + (int64_t)((nit * SPLIT + cp_tile) * BN + cp_r0) * cp_stride * (int)sizeof(T);
-      uint32_t cp_dst = nxt + cp_dst0;
+      const bool copy = nit < niter && nit * SPLIT + cp_tile < ntiles;   // this wavefront's tile of the next iteration exists
+      const int v_nxt = v_cur + 1 == NV ? 0 : v_cur + 1;
+      fcopy = copy && nit < n_fast;
+      cp_src = cp_g + (int64_t)((nit * SPLIT + cp_tile) * BN + cp_r0) * cp_stride * (int)sizeof(T);
+      cp_dst = (cp_v ? ldsV + (uint32_t)(v_nxt * SLOTB) : k_nxt) + (uint32_t)(cp_dst0 * (int)sizeof(T));
+      if (copy && !fcopy)
+        fwd_issue_general<T>(sAll + (cp_v ? (2 + v_nxt) * SLOT : (nit & 1) * SLOT) + cp_dst0, cp_gt, cp_stride, cp_v,
+                             (nit * SPLIT + cp_tile) * BN + cp_r0, cp_r0, sk, cl0);
       const int tile_g = it * SPLIT + sp;
       const int n0 = tile_g * BN;
-      const bool idle = tile_g >= ntiles || (causal && n0 > wrow0 + 31);
-      if (copy && (idle || !fast))
-        fwd_issue_stage<T, SPLIT, BN, LD>(sStage + ((it + 1) & 1) * STAGE, kg, vg, k_stride, v_stride, nit, ntiles, sk, w, cl0);
-      if (!idle) {
-        uint32_t kb = cur + kb_lane, va = cur + va_lane, vb = cur + vb_lane;
-        // derive the other addresses inside the loop, not ahead of it
-        asm volatile("" : "+v"(kb), "+v"(va), "+v"(vb));
-#define DH_FWD_COPY(i)                                                                                  \
-        do {                                                                                            \
-          if (fcopy) {                                                                                  \
-            __builtin_amdgcn_sched_barrier(0);                                                          \
-            dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                            \
-            cp_src += cp_step;                                                                          \
-            cp_dst += 1024;                                                                             \
-            __builtin_amdgcn_sched_barrier(0);                                                          \
-          }                                                                                             \
-        } while (0)
+      const bool act = tile_g < ntiles && !(causal && n0 > wrow0 + 31);
+
+      // lagging wavefronts: last iteration's P V first; their copy blocks 4..7 go out there
+      if (lag) {
+        if (act_prev) pv(v_prev);
+        else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
+      }
+      if (act) {
+        uint32_t kb = k_cur + kb_lane;
+        asm volatile("" : "+v"(kb));
         floatx16 S[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -457,60 +502,45 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
         m_run = m_new;
         const float mc = m_new * scale_log2;
         float ps = 0.f;
-        Frag Pb[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-          float pv[8];
+          float pvv[8];
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            pv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
-            ps += pv[j];
+            pvv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
+            ps += pvv[j];
           }
-          Pb[s] = frag_pack<T>(pv);
+          Pb[s] = frag_pack<T>(pvv);
         }
         l_run += ps;
-        // V^T fragments: eight transpose reads per 16-key step, consumed as they land.
-        uint32_t ad[8];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          ad[2 * t] = va ^ (uint32_t)(t << 6);
-          ad[2 * t + 1] = vb ^ (uint32_t)(t << 6);
-        }
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-          short4v f[8];
-          if (s == 0) lds_read_tr8<0>(f, ad);
-          else if (s == 1) lds_read_tr8<16 * 256>(f, ad);
-          else if (s == 2) lds_read_tr8<32 * 256>(f, ad);
-          else lds_read_tr8<48 * 256>(f, ad);
-          lds_wait<4>(f[0], f[1], f[2], f[3]);
-          O[0] = M::mma(frag_join<T>(f[0], f[1]), Pb[s], O[0]);
-          O[1] = M::mma(frag_join<T>(f[2], f[3]), Pb[s], O[1]);
-          if (NS == 2) DH_FWD_COPY(4 + 2 * s);
-          lds_wait<0>(f[4], f[5], f[6], f[7]);
-          O[2] = M::mma(frag_join<T>(f[4], f[5]), Pb[s], O[2]);
-          O[3] = M::mma(frag_join<T>(f[6], f[7]), Pb[s], O[3]);
-          if (NS == 2) DH_FWD_COPY(5 + 2 * s);
-          else DH_FWD_COPY(4 + s);                                        // copy blocks 4..7
-        }
-#undef DH_FWD_COPY
+      } else {
+        DH_FWD_COPY(0); DH_FWD_COPY(1); DH_FWD_COPY(2); DH_FWD_COPY(3);
       }
+      if (!lag) {
+        if (act) pv(v_cur);
+        else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
+      }
+      act_prev = act;
+      v_prev = v_cur;
+      v_cur = v_nxt;
+      { const uint32_t t = k_cur; k_cur = k_nxt; k_nxt = t; }
       dma_wait_all();
-      __syncthreads();   // the next stage has landed, and everyone is done with this one
+      __syncthreads();   // the next slots have landed, and everyone is done with the ones they replace next
     }
+    fcopy = false;
+    if (lag && act_prev) pv(v_prev);
+#undef DH_FWD_COPY
+    __syncthreads();     // everyone is done with the tiles: the area is reused for the exchange below
 
     // ---- combine the key/value splits through LDS (fixed order: deterministic) --------------
-    // O of split s > 0, row group g -> slot x = (s-1)*RG + g: slots 0..3 in stage 0, the rest in stage 1;
-    // m and l after them in stage 1.
-    float *x0 = reinterpret_cast<float *>(sStage);
-    float *x1 = reinterpret_cast<float *>(sStage + STAGE);
-    float *xml = x1 + 2 * 4096;
+    // O of split s > 0, row group g -> slot x = (s-1)*RG + g (16 KB each), then m and l of every slot.
+    float *xo = reinterpret_cast<float *>(sAll);
+    float *xml = xo + 6 * 4096;
     static_assert((SPLIT - 1) * RG <= 6, "exchange slots");
-    static_assert(STAGE * sizeof(T) >= 4 * 4096 * sizeof(float), "stage 0 holds four O slots");
-    static_assert(STAGE * sizeof(T) >= (2 * 4096 + 6 * 128) * sizeof(float), "stage 1 holds two O slots and m/l");
+    static_assert((2 + NV) * SLOT * sizeof(T) >= (6 * 4096 + 6 * 128) * sizeof(float), "exchange area");
     if (sp > 0) {
       const int x = (sp - 1) * RG + rg;
-      float *dst = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+      float *dst = xo + x * 4096;
 #pragma unroll
       for (int t = 0; t < D / 32; ++t)
 #pragma unroll
@@ -523,7 +553,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
 #pragma unroll
       for (int s2 = 1; s2 < SPLIT; ++s2) {
         const int x = (s2 - 1) * RG + rg;
-        const float *src = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+        const float *src = xo + x * 4096;
         const float m_o = xml[x * 128 + lane], l_o = xml[x * 128 + 64 + lane];
         const float m_new = fmaxf(m_run, m_o);
         const float a_me = fast_exp2((m_run - m_new) * scale_log2);
@@ -556,12 +586,12 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   }
 }
 
-template <typename T, int RG, int SPLIT, int BN>
+template <typename T, int RG, int SPLIT, int BN, bool LAG>
 static int launch_attn_fwd_d128(const AttnFwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * RG;
   const int nqt = (int)cdiv(p.max_sq, BM);
   dim3 grid((unsigned)((p.causal ? (nqt + 1) / 2 : nqt) * p.hq), (unsigned)batch);
-  hipLaunchKernelGGL((attn_fwd_d128_kernel<T, RG, SPLIT, BN>), grid, dim3(512), 0, st, p);
+  hipLaunchKernelGGL((attn_fwd_d128_kernel<T, RG, SPLIT, BN, LAG>), grid, dim3(512), 0, st, p);
   return DH_OK;
 }
 
@@ -624,8 +654,8 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
     // 128-row query tiles when that still gives every CU a workgroup, else 64-row tiles.
     const int64_t wg128 = (causal ? (cdiv(max_seqlen_q, 128) + 1) / 2 : cdiv(max_seqlen_q, 128)) * hq * batch;
     const bool big = wg128 >= 256;
-    if (dtype == DH_BF16) rc = big ? launch_attn_fwd_d128<bf16_t, 4, 2, 64>(p, batch, st) : launch_attn_fwd_d128<bf16_t, 2, 4, 32>(p, batch, st);
-    else rc = big ? launch_attn_fwd_d128<f16_t, 4, 2, 64>(p, batch, st) : launch_attn_fwd_d128<f16_t, 2, 4, 32>(p, batch, st);
+    if (dtype == DH_BF16) rc = big ? launch_attn_fwd_d128<bf16_t, 4, 2, 64, DH_FWD_LAG>(p, batch, st) : launch_attn_fwd_d128<bf16_t, 2, 4, 32, DH_FWD_LAG>(p, batch, st);
+    else rc = big ? launch_attn_fwd_d128<f16_t, 4, 2, 64, DH_FWD_LAG>(p, batch, st) : launch_attn_fwd_d128<f16_t, 2, 4, 32, DH_FWD_LAG>(p, batch, st);
   } else {
     // Few query tiles (small batch*heads) -> smaller workgroups so the grid still covers the chip.
     const int64_t blocks128 = cdiv(max_seqlen_q, 128) * hq * batch;

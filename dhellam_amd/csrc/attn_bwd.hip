@@ -441,19 +441,24 @@ __global__ void __launch_bounds__(64 * NW) attn_bwd_dq_kernel(const AttnBwdParam
 // ---------------------------------------------------------------------------------------------
 
 // dQ: 8 wavefronts = RG query row groups x SPLIT key splits (as the forward kernel); the
-// partial dQ of the splits are added through LDS in split order.
+// partial dQ of the splits are added through LDS in split order.  As in the forward kernel
+// the main loop is one rolled body whose global->LDS copies and LDS reads are written in
+// assembly (scalar copy bases, XOR-derived fragment addresses, no compiler waits between
+// copies in flight and reads); the copies are spread between the MFMAs.
 template <typename T, int RG, int SPLIT, int BN>
 __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
-  constexpr int D = 128, BM = 32 * RG, NB = BN / 32, NS = BN / 16;
+  static_assert(BN == 32, "32-key tiles");
+  constexpr int D = 128, BM = 32 * RG, NS = BN / 16;
   static_assert(RG * SPLIT == 8, "8 wavefronts per workgroup");
   constexpr int TILE = BN * D;
-  constexpr int STAGE = SPLIT * 2 * TILE;                       // K and V tile per split
-  constexpr int BLK_PER_STAGE = STAGE * (int)sizeof(T) / 1024;
-  constexpr int LD = BLK_PER_STAGE / 8;
-  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
-  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+  constexpr int SLOT = SPLIT * TILE;              // elements of one K (or V) slot: the tiles of all splits
+  constexpr int SLOTB = SLOT * (int)sizeof(T);
+  constexpr int BPT = BN / 4;                     // 1 KB copy blocks per tile
+  constexpr int CPW = SPLIT * 2 * BPT / 8;        // copy blocks per wavefront and iteration (4 or 8)
+  static_assert(CPW == 4 || CPW == 8, "copy blocks per wavefront");
+  __shared__ __attribute__((aligned(1024))) T sAll[4 * SLOT];   // K slots 0..1, V slots 0..1
 
   const int b = blockIdx.y;
   // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
@@ -477,12 +482,41 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
     if (px >= nqt) return;
     qt[0] = px; qt[1] = 0; nq = 1;
   }
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
   const int c = lane & 31, hh = lane >> 5;
   const int rg = w % RG, sp = w / RG;
   const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
   const T *vg = reinterpret_cast<const T *>(p.v) + (int64_t)k0 * p.v_stride + (int64_t)hkv * D;
-  const int lrow = lane >> 4;
+  const uint32_t ldsK = (uint32_t)(uintptr_t)sAll, ldsV = ldsK + 2 * SLOTB;
+
+  // ---- copies: the CPW blocks of a wavefront are consecutive rows of ONE tile (K or V) -------------
+  CopyLane cl0;
+  cl0.l16 = lane & 15;
+  cl0.lrow = lane >> 4;
+  const int cp_tile = (w * CPW) / (2 * BPT);
+  const int cp_v = ((w * CPW) % (2 * BPT)) / BPT;
+  const int cp_r0 = 4 * ((w * CPW) % BPT);
+  const int cp_stride = cp_v ? v_stride : k_stride;
+  const T *cp_gt = cp_v ? vg : kg;
+  const char *cp_g = reinterpret_cast<const char *>(cp_gt);
+  const int cp_dst0 = cp_tile * TILE + cp_r0 * D;
+  const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
+  uint32_t cp_off[4];                                 // both tiles use swz(row): chunk ^= 4 * (row % 4) + (row / 4) % 4
+  {
+    const uint32_t rowb = (uint32_t)(cl0.lrow * cp_stride) * (uint32_t)sizeof(T);
+    const uint32_t chunk = (uint32_t)(cl0.l16 ^ (4 * cl0.lrow)) << 4;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
+  }
+  // ---- fragment reads: lane byte offsets inside a slot; other fragments by XOR / immediate offset ----
+  const int r = lane & 15;
+  const uint32_t rf_lane = (uint32_t)(sp * TILE * (int)sizeof(T) + c * 256 + ((hh ^ swz(c)) << 4));   // row c, chunk hh
+  const int ta_x = 4 * (r >> 2) + hh;                 // transpose read of K: swz of rows 4*hh + r/4 (+8)
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  const uint32_t t_row = (uint32_t)(sp * TILE * (int)sizeof(T) + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
+  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
 
   for (int qi = 0; qi < nq; ++qi) {
     const int m0 = qt[qi] * BM;
@@ -506,6 +540,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
     if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
     const int ntiles = (nk_end + BN - 1) / BN;
     const int niter = (ntiles + SPLIT - 1) / SPLIT;
+    const int n_fast = sk / (SPLIT * BN);          // iterations whose tiles lie wholly inside the keys
 
     floatx16 dQt[D / 32];
 #pragma unroll
@@ -513,102 +548,124 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
 #pragma unroll
       for (int v = 0; v < 16; ++v) dQt[t][v] = 0.f;
 
-    auto issue = [&](T *stage, int it) {
-#pragma unroll
-      for (int i = 0; i < LD; ++i) {
-        const int blk = w * LD + i;
-        const int tile = blk / (BN / 2);
-        const int kvsel = (blk % (BN / 2)) / (BN / 4);
-        const int rgp = blk % (BN / 4);
-        const int tile_g = it * SPLIT + tile;
-        if (tile_g < ntiles) {
-          const int row = 4 * rgp + lrow;
-          int kr = tile_g * BN + row;
-          kr = kr < sk ? kr : sk - 1;
-          dma_rows4<T>(kvsel ? vg : kg, kr, kvsel ? v_stride : k_stride, row, lane,
-                       stage + tile * 2 * TILE + kvsel * TILE + rgp * 512);
-        }
-      }
-    };
-    auto compute = [&](const T *stage, int it) {
+    if (niter > 0 && cp_tile < ntiles)
+      dma_tile32_general<T, CPW>(sAll + (cp_v ? 2 * SLOT : 0) + cp_dst0, cp_gt, cp_stride, 1, cp_tile * BN + cp_r0, cp_r0, sk, cl0);
+    dma_wait_all();
+    __syncthreads();
+
+    const char *cp_src = nullptr;
+    uint32_t cp_dst = 0;
+    bool fcopy = false;
+#define DH_DQ_COPY(i)                                                                                   \
+    do {                                                                                                \
+      if ((i) < CPW && fcopy) {                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+        dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                                \
+        cp_src += cp_step;                                                                              \
+        cp_dst += 1024;                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+      }                                                                                                 \
+    } while (0)
+
+#pragma unroll 1
+    for (int it = 0; it < niter; ++it) {
+      const int nit = it + 1;
+      const uint32_t cur = (uint32_t)((it & 1) * SLOTB), nxt = (uint32_t)((nit & 1) * SLOTB);
+      const bool copy = nit < niter && nit * SPLIT + cp_tile < ntiles;
+      fcopy = copy && nit < n_fast;
+      cp_src = cp_g + (int64_t)((nit * SPLIT + cp_tile) * BN + cp_r0) * cp_stride * (int)sizeof(T);
+      cp_dst = (cp_v ? ldsV : ldsK) + nxt + (uint32_t)(cp_dst0 * (int)sizeof(T));
+      if (copy && !fcopy)
+        dma_tile32_general<T, CPW>(sAll + (cp_v ? 2 * SLOT : 0) + (nit & 1) * SLOT + cp_dst0, cp_gt, cp_stride, 1,
+                                   (nit * SPLIT + cp_tile) * BN + cp_r0, cp_r0, sk, cl0);
       const int tile_g = it * SPLIT + sp;
       const int n0 = tile_g * BN;
-      if (tile_g >= ntiles || (causal && n0 > wrow0 + 31)) return;
-      const T *tK = stage + sp * 2 * TILE;
-      const T *tV = tK + TILE;
-      floatx16 S[NB], dP[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+      const bool act = tile_g < ntiles && !(causal && n0 > wrow0 + 31);
+      if (act) {
+        uint32_t kb = ldsK + cur + rf_lane, vb = ldsV + cur + rf_lane;
+        uint32_t ta = ldsK + cur + ta_lane, tb = ldsK + cur + tb_lane;
+        asm volatile("" : "+v"(kb), "+v"(vb), "+v"(ta), "+v"(tb));   // derive the other addresses here, not ahead of the loop
+        floatx16 S, dP;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          S[nb][v] = 0.f;
-          dP[nb][v] = 0.f;
+          S[v] = 0.f;
+          dP[v] = 0.f;
         }
+        {
+          // K and V row fragments are fetched one step ahead of the MFMAs that consume them.
+          int4v fk[2], fv[2];
+          lds_read128<0>(fk[0], kb);
+          lds_read128<0>(fv[0], vb);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        Frag ak = frag_ld_swz<T>(tK, nb * 32 + c, hh);
-        Frag av = frag_ld_swz<T>(tV, nb * 32 + c, hh);
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          Frag ak2 = ak, av2 = av;
-          if (ks + 1 < D / 16) {
-            ak2 = frag_ld_swz<T>(tK, nb * 32 + c, 2 * (ks + 1) + hh);
-            av2 = frag_ld_swz<T>(tV, nb * 32 + c, 2 * (ks + 1) + hh);
+          for (int ks = 0; ks < D / 16; ++ks) {
+            const int a = ks & 1, nx = (ks + 1) & 1;
+            if (ks + 1 < D / 16) {
+              lds_read128<0>(fk[nx], kb ^ (uint32_t)((ks + 1) << 5));
+              lds_read128<0>(fv[nx], vb ^ (uint32_t)((ks + 1) << 5));
+              lds_wait<2>(fk[a], fv[a]);
+            } else {
+              lds_wait<0>(fk[a], fv[a]);
+            }
+            S = M::mma(__builtin_bit_cast(Frag, fk[a]), Qf[ks], S);
+            dP = M::mma(__builtin_bit_cast(Frag, fv[a]), dOf[ks], dP);
+            if (CPW == 8 && (ks & 1)) DH_DQ_COPY(ks >> 1);           // copy blocks 0..3
+            if (CPW == 4 && (ks & 3) == 3) DH_DQ_COPY(ks >> 2);      // copy blocks 0..1
           }
-          S[nb] = M::mma(ak, Qf[ks], S[nb]);
-          dP[nb] = M::mma(av, dOf[ks], dP[nb]);
-          ak = ak2;
-          av = av2;
         }
-      }
-      const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
-      Frag dSb[NS];
+        const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+        Frag dSb[NS];
 #pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        float dsv[8];
+        for (int s = 0; s < NS; ++s) {
+          float dsv[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int nb = s >> 1, v = 8 * (s & 1) + j;
-          float pe = fast_exp2(S[nb][v] * scale_log2 - lse_c);
-          if (need_mask) {
-            const int kv = n0 + nb * 32 + acc_row(v, hh);
-            if (kv >= sk || (causal && kv > row_q)) pe = 0.f;
+          for (int j = 0; j < 8; ++j) {
+            const int v = 8 * s + j;
+            float pe = fast_exp2(S[v] * scale_log2 - lse_c);
+            if (need_mask) {
+              const int kv = n0 + acc_row(v, hh);
+              if (kv >= sk || (causal && kv > row_q)) pe = 0.f;
+            }
+            dsv[j] = pe * (dP[v] - del_c);
           }
-          dsv[j] = pe * (dP[nb][v] - del_c);
+          dSb[s] = frag_pack<T>(dsv);
         }
-        dSb[s] = frag_pack<T>(dsv);
-      }
+        // dQ^T += K^T dS^T: K^T fragments by transpose reads of the K tile
+        uint32_t ad[8];
 #pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        Tr4 kt;
-        tr4_issue<T>(kt, tK, 16 * s, lane);
-        dQt[0] = M::mma(tr4_get<T, 6>(kt, 0), dSb[s], dQt[0]);
-        dQt[1] = M::mma(tr4_get<T, 4>(kt, 1), dSb[s], dQt[1]);
-        dQt[2] = M::mma(tr4_get<T, 2>(kt, 2), dSb[s], dQt[2]);
-        dQt[3] = M::mma(tr4_get<T, 0>(kt, 3), dSb[s], dQt[3]);
+        for (int t = 0; t < 4; ++t) {
+          ad[2 * t] = ta ^ (uint32_t)(t << 6);
+          ad[2 * t + 1] = tb ^ (uint32_t)(t << 6);
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          short4v f[8];
+          if (s == 0) lds_read_tr8<0>(f, ad);
+          else lds_read_tr8<16 * 256>(f, ad);
+          lds_wait<4>(f[0], f[1], f[2], f[3]);
+          dQt[0] = M::mma(frag_join<T>(f[0], f[1]), dSb[s], dQt[0]);
+          dQt[1] = M::mma(frag_join<T>(f[2], f[3]), dSb[s], dQt[1]);
+          if (CPW == 8) DH_DQ_COPY(4 + 2 * s);
+          lds_wait<0>(f[4], f[5], f[6], f[7]);
+          dQt[2] = M::mma(frag_join<T>(f[4], f[5]), dSb[s], dQt[2]);
+          dQt[3] = M::mma(frag_join<T>(f[6], f[7]), dSb[s], dQt[3]);
+          if (CPW == 8) DH_DQ_COPY(5 + 2 * s);
+          else DH_DQ_COPY(2 + s);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < CPW; ++i) DH_DQ_COPY(i);
       }
-    };
-
-    if (niter > 0) issue(sStage0, 0);
-    __syncthreads();
-    for (int it = 0; it < niter; it += 2) {
-      if (it + 1 < niter) issue(sStage1, it + 1);
-      compute(sStage0, it);
-      __syncthreads();
-      if (it + 1 < niter) {
-        if (it + 2 < niter) issue(sStage0, it + 2);
-        compute(sStage1, it + 1);
-        __syncthreads();
-      }
+      dma_wait_all();
+      __syncthreads();   // the next slots have landed, and everyone is done with the current ones
     }
+#undef DH_DQ_COPY
 
-    // add the splits' partial dQ through LDS, in split order
-    float *x0 = reinterpret_cast<float *>(sStage0);
-    float *x1 = reinterpret_cast<float *>(sStage1);
+    // add the splits' partial dQ through LDS, in split order: slot x = (s-1)*RG + g, 16 KB each
+    float *xo = reinterpret_cast<float *>(sAll);
     static_assert((SPLIT - 1) * RG <= 6, "exchange slots");
+    static_assert(4 * SLOT * sizeof(T) >= (size_t)(SPLIT - 1) * RG * 4096 * sizeof(float), "exchange area");
     if (sp > 0) {
-      const int x = (sp - 1) * RG + rg;
-      float *dst = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+      float *dst = xo + ((sp - 1) * RG + rg) * 4096;
 #pragma unroll
       for (int t = 0; t < D / 32; ++t)
 #pragma unroll
@@ -618,8 +675,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
     if (sp == 0) {
 #pragma unroll
       for (int s2 = 1; s2 < SPLIT; ++s2) {
-        const int x = (s2 - 1) * RG + rg;
-        const float *src = x < 4 ? x0 + x * 4096 : x1 + (x - 4) * 4096;
+        const float *src = xo + ((s2 - 1) * RG + rg) * 4096;
 #pragma unroll
         for (int t = 0; t < D / 32; ++t)
 #pragma unroll

@@ -218,40 +218,6 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
 // copies in flight and fragment reads, and the copies are spread between the MFMAs so
 // that they do not queue up behind each other.
 
-// Per-lane constants of the general (clamped) K/V tile copies.
-struct FwdCopyLane {
-  int lrow, l16;         // row inside a 4-row copy block, 16-byte chunk slot
-};
-
-// One 1 KB copy (4 rows of a K or V tile) in its fast form: wave-uniform 64-bit global base, the lane's
-// 32-bit byte offset, wave-uniform LDS byte address.  The compiler does not count these copies: the
-// kernel waits for them itself (dma_wait_all) before the barrier that publishes a stage.
-__device__ __forceinline__ void dma_block_fast(const char *base, uint32_t lane_off, uint32_t lds_dst) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(lane_off), "s"(base), "s"(lds_dst)
-               : "memory", "m0");
-}
-
-// The 8 copy blocks (32 rows of one K or V tile) of a wavefront in general form: rows past the last key
-// are clamped per lane (they are masked in the scores, and their V rows meet zero probabilities).  Kept
-// as a rolled loop: it runs once per query tile and for tiles that reach past the keys.
-template <typename T>
-__device__ __forceinline__ void fwd_issue_general(T *dst, const T *g, int stride, int is_v, int row0_g, int row0_t, int sk,
-                                                  const FwdCopyLane &cl) {
-  asm volatile("" : "+s"(row0_g));               // keep the address arithmetic next to the copies
-#pragma unroll 1
-  for (int i = 0; i < 8; ++i) {
-    int kr = row0_g + 4 * i + cl.lrow;
-    kr = kr < sk ? kr : sk - 1;
-    const int row = row0_t + 4 * i + cl.lrow;
-    const int f = is_v ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
-    const T *src = g + (int64_t)kr * stride + ((cl.l16 ^ f) * 8);
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                     (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
-  }
-}
-
 // LAG: the wavefronts of the upper half of the workgroup (the second wavefront of every SIMD) run their
 // P V products one iteration late.  In each half of an iteration one wavefront of a SIMD is then in its
 // matrix phase while the other is in its softmax, instead of both competing for the same unit.  V tiles
@@ -305,7 +271,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   const uint32_t ldsK = (uint32_t)(uintptr_t)sAll, ldsV = ldsK + 2 * SLOTB;
 
   // ---- per-lane constants of the copy and of the fragment reads ---------------------------
-  FwdCopyLane cl0;                                    // copy: chunk slot and row inside a 4-row block
+  CopyLane cl0;                                    // copy: chunk slot and row inside a 4-row block
   cl0.l16 = lane & 15;
   cl0.lrow = lane >> 4;
   // The 8 copy blocks of a wavefront are 32 consecutive rows of ONE tile (K or V), so per iteration they
@@ -366,7 +332,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       for (int j = 0; j < 8; ++j) Pb[s][j] = static_cast<T>(0.f);
 
     if (niter > 0 && cp_tile < ntiles)
-      fwd_issue_general<T>(sAll + (cp_v ? 2 * SLOT : 0) + cp_dst0, cp_gt, cp_stride, cp_v, cp_tile * BN + cp_r0, cp_r0, sk, cl0);
+      dma_tile32_general<T>(sAll + (cp_v ? 2 * SLOT : 0) + cp_dst0, cp_gt, cp_stride, cp_v, cp_tile * BN + cp_r0, cp_r0, sk, cl0);
     dma_wait_all();
     __syncthreads();
 
@@ -427,7 +393,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       cp_src = cp_g + (int64_t)((nit * SPLIT + cp_tile) * BN + cp_r0) * cp_stride * (int)sizeof(T);
       cp_dst = (cp_v ? ldsV + (uint32_t)(v_nxt * SLOTB) : k_nxt) + (uint32_t)(cp_dst0 * (int)sizeof(T));
       if (copy && !fcopy)
-        fwd_issue_general<T>(sAll + (cp_v ? (2 + v_nxt) * SLOT : (nit & 1) * SLOT) + cp_dst0, cp_gt, cp_stride, cp_v,
+        dma_tile32_general<T>(sAll + (cp_v ? (2 + v_nxt) * SLOT : (nit & 1) * SLOT) + cp_dst0, cp_gt, cp_stride, cp_v,
                              (nit * SPLIT + cp_tile) * BN + cp_r0, cp_r0, sk, cl0);
       const int tile_g = it * SPLIT + sp;
       const int n0 = tile_g * BN;

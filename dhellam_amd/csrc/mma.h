@@ -187,6 +187,42 @@ template <typename T> __device__ __forceinline__ typename Mma<T>::Frag frag_join
   return __builtin_bit_cast(typename Mma<T>::Frag, o8);
 }
 
+// ---- global -> LDS tile copies of the d = 128 attention kernels ----------------------------------
+// Per-lane constants of the general (clamped) K/V tile copies.
+struct CopyLane {
+  int lrow, l16;         // row inside a 4-row copy block, 16-byte chunk slot
+};
+
+// One 1 KB copy (4 rows of a K or V tile) in its fast form: wave-uniform 64-bit global base, the lane's
+// 32-bit byte offset, wave-uniform LDS byte address.  The compiler does not count these copies: the
+// kernel waits for them itself (dma_wait_all) before the barrier that publishes a stage.
+__device__ __forceinline__ void dma_block_fast(const char *base, uint32_t lane_off, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_off), "s"(base), "s"(lds_dst)
+               : "memory", "m0");
+}
+
+// NBLK copy blocks (4 rows each, consecutive rows of one tile) of a wavefront in general form: rows past the last key
+// are clamped per lane (they are masked in the scores, and their V rows meet zero probabilities).  Kept
+// as a rolled loop: it runs once per query tile and for tiles that reach past the keys.
+// `swz_v`: the tile uses swz(row) (transpose-read tiles) instead of row % 16 (row-fragment tiles).
+template <typename T, int NBLK = 8>
+__device__ __forceinline__ void dma_tile32_general(T *dst, const T *g, int stride, int swz_v, int row0_g, int row0_t, int sk,
+                                                  const CopyLane &cl) {
+  asm volatile("" : "+s"(row0_g));               // keep the address arithmetic next to the copies
+#pragma unroll 1
+  for (int i = 0; i < NBLK; ++i) {
+    int kr = row0_g + 4 * i + cl.lrow;
+    kr = kr < sk ? kr : sk - 1;
+    const int row = row0_t + 4 * i + cl.lrow;
+    const int f = swz_v ? (4 * (row & 3) + ((row >> 2) & 3)) : (row & 15);
+    const T *src = g + (int64_t)kr * stride + ((cl.l16 ^ f) * 8);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                     (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
+  }
+}
+
 // Row index inside a 32-row accumulator block held by register v of lane half h.
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 

@@ -24,6 +24,8 @@ namespace dh {
 struct AttnBwdParams {
   const void *dout, *q, *k, *v;
   const float *lse, *delta;
+  const float *ld2;          // fp32 [2][plane]: lse * log2(e), then delta, each [batch][hq][max_sq] (d = 128 kernels)
+  int64_t ld2_plane;         // elements between the two planes
   void *dq, *dk, *dv;
   float *dk_part, *dv_part;  // fp32 [hsplit][total_k][hk][d] when hsplit > 1
   const int32_t *cu_q, *cu_k;
@@ -38,6 +40,7 @@ struct AttnBwdParams {
 template <typename T>
 __global__ void __launch_bounds__(256)
 attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *__restrict__ delta,
+                  const float *__restrict__ lse, float *__restrict__ ld2, int64_t ld2_plane,
                   const int32_t *__restrict__ cu_q, int max_sq, int hq, int d, int lanes_per, int64_t do_stride,
                   int64_t o_stride) {
   constexpr int N = Vec<T>::N;
@@ -57,7 +60,14 @@ attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *
       for (int j = 0; j < N; ++j) s += to_f(a.v[j]) * to_f(o.v[j]);
     }
     for (int o = lanes_per >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-    if (ln == 0) delta[((int64_t)b * hq + h) * max_sq + i] = s;
+    if (ln == 0) {
+      const int64_t at = ((int64_t)b * hq + h) * max_sq + i;
+      delta[at] = s;
+      if (ld2) {             // the copy the d = 128 kernels stream: lse in exp2 units next to delta
+        ld2[at] = lse[at] * 1.4426950408889634f;
+        ld2[ld2_plane + at] = s;
+      }
+    }
   }
 }
 
@@ -711,7 +721,8 @@ static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
 // fragments of the group stay in registers; every iteration brings two 32-row query tiles
 // (Q, dO, lse, delta) of the current head into LDS, one per split.  The splits' partial
 // dK/dV are added through LDS in split order.  Causal: the workgroup owns key tiles j and
-// n-1-j, so every workgroup does the same amount of work.
+// n-1-j, so every workgroup does the same amount of work.  The main loop is one rolled body
+// with assembly copies (scalar bases) and assembly LDS reads, as in the forward kernel.
 template <typename T>
 __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdParams p) {
   using M = Mma<T>;
@@ -719,9 +730,10 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
   constexpr int D = 128, KG = 2, QSPLIT = 2, BN = 32 * KG, BM = 32;
   constexpr int QT = BM * D;                          // elements of one Q (or dO) tile
   constexpr int SLOT = 2 * QT + 128;                  // Q tile, dO tile, 32 lse + 32 delta (as 256 bytes)
+  constexpr int SLOTB = SLOT * (int)sizeof(T);
   constexpr int STAGE = QSPLIT * SLOT;
-  __shared__ __attribute__((aligned(16))) T sStage0[STAGE];
-  __shared__ __attribute__((aligned(16))) T sStage1[STAGE];
+  constexpr int STAGEB = STAGE * (int)sizeof(T);
+  __shared__ __attribute__((aligned(1024))) T sAll[2 * STAGE];
 
   const int b = blockIdx.y;
   // all key tiles of one head group read the same Q / dO rows: keep a group on one XCD's L2
@@ -745,158 +757,258 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
     if (px >= nkt) return;
     kt[0] = px; kt[1] = 0; nk = 1;
   }
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  agpr_reserve_192();
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
   const int c = lane & 31, hh = lane >> 5;
   const int kg = w % KG, qs = w / KG;
   const int ratio = p.hq / p.hk;
   const int hper = ratio / p.hsplit;
-  const int lrow = lane >> 4;
-  const int64_t lse_stride = p.max_sq;
+  const int h_first = hkv * ratio + hs * hper;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)sAll;
+
+  // ---- copies: wavefront w brings one whole tile per iteration: Q (w even) or dO (w odd) of split w / 2;
+  // wavefronts 0 and 1 also bring the 64 lse/delta values of split w ----------------------------------
+  CopyLane cl0;
+  cl0.l16 = lane & 15;
+  cl0.lrow = lane >> 4;
+  const int cp_slot = w >> 1, cp_do = w & 1;
+  const int cp_stride = cp_do ? do_stride : q_stride;
+  const T *cp_gt = reinterpret_cast<const T *>(cp_do ? p.dout : p.q) + (int64_t)q0 * cp_stride;
+  const char *cp_g = reinterpret_cast<const char *>(cp_gt);
+  const int cp_dst0 = cp_slot * SLOT + cp_do * QT;    // elements inside a stage
+  const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
+  uint32_t cp_off[4];                                 // tiles use swz(row): chunk ^= 4 * (row % 4) + (row / 4) % 4
+  {
+    const uint32_t rowb = (uint32_t)(cl0.lrow * cp_stride) * (uint32_t)sizeof(T);
+    const uint32_t chunk = (uint32_t)(cl0.l16 ^ (4 * cl0.lrow)) << 4;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
+  }
+  const uint32_t ld_off = (uint32_t)((lane & 31) * 4) + (lane < 32 ? 0u : (uint32_t)p.ld2_plane * 4u);
+  const char *ld_g = reinterpret_cast<const char *>(p.ld2);
+  // ---- fragment reads: lane byte offsets inside a slot; other fragments by XOR / immediate offset ----
+  const int r = lane & 15;
+  const uint32_t rf_lane = (uint32_t)(qs * SLOTB + c * 256 + ((hh ^ swz(c)) << 4));   // row c, chunk hh
+  const int ta_x = 4 * (r >> 2) + hh;                 // transpose reads: swz of rows 4*hh + r/4 (+8)
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  const uint32_t t_row = (uint32_t)(qs * SLOTB + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
+  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
+  const uint32_t tl_lane = (uint32_t)(qs * SLOTB + 2 * QT * (int)sizeof(T) + 16 * hh);  // lse of rows 4*hh + 8*vb + e
 
   for (int ki = 0; ki < nk; ++ki) {
     const int j0 = kt[ki] * BN;
     const int jw0 = j0 + 32 * kg;
     const int jrow = jw0 + c;
-    Frag Kf[D / 16], Vf[D / 16];
+    // Fixed accumulation registers of this kernel: dV^T tiles in a[0:63], dK^T tiles in a[64:127],
+    // this wavefront's K fragments in a[128:159], its V fragments in a[160:191].
     {
       const int jl = jrow < sk ? jrow : sk - 1;
       const T *kp = reinterpret_cast<const T *>(p.k) + (int64_t)(k0 + jl) * p.k_stride + (int64_t)hkv * D;
       const T *vp = reinterpret_cast<const T *>(p.v) + (int64_t)(k0 + jl) * p.v_stride + (int64_t)hkv * D;
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        Kf[ks] = frag_ld<T>(kp + ks * 16 + 8 * hh);
-        Vf[ks] = frag_ld<T>(vp + ks * 16 + 8 * hh);
-      }
+#define DH_KV(ks)                                                        \
+      agpr_write_frag<T, 128 + 4 * ks>(frag_ld<T>(kp + ks * 16 + 8 * hh)); \
+      agpr_write_frag<T, 160 + 4 * ks>(frag_ld<T>(vp + ks * 16 + 8 * hh))
+      DH_KV(0); DH_KV(1); DH_KV(2); DH_KV(3); DH_KV(4); DH_KV(5); DH_KV(6); DH_KV(7);
+#undef DH_KV
     }
-    floatx16 dKt[D / 32], dVt[D / 32];
-#pragma unroll
-    for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        dKt[t][v] = 0.f;
-        dVt[t][v] = 0.f;
-      }
+    agpr_zero16<0>(); agpr_zero16<16>(); agpr_zero16<32>(); agpr_zero16<48>();
+    agpr_zero16<64>(); agpr_zero16<80>(); agpr_zero16<96>(); agpr_zero16<112>();
     const int i_begin = causal ? (j0 / BM) * BM : 0;
     const int ntq = i_begin < sq ? (sq - i_begin + BM - 1) / BM : 0;
     const int it_per_head = (ntq + QSPLIT - 1) / QSPLIT;
     const int niter = it_per_head * hper;
 
-    // copies of one stage: 32 blocks of 1 KB (4 rows of a Q or dO tile) + one 256-byte lse/delta block per split
-    auto issue = [&](T *stage, int it) {
-      const int g = it / it_per_head, ti = it % it_per_head;
-      const int h = hkv * ratio + hs * hper + g;
-      const T *qg = reinterpret_cast<const T *>(p.q) + (int64_t)q0 * p.q_stride + (int64_t)h * D;
-      const T *dg = reinterpret_cast<const T *>(p.dout) + (int64_t)q0 * p.do_stride + (int64_t)h * D;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int blk = w * 8 + i;
-        const int slot = blk / 16, sel = (blk % 16) / 8, rgp = blk % 8;
-        const int tq = ti * QSPLIT + slot;
-        if (tq < ntq) {
-          const int row = 4 * rgp + lrow;
-          int ir = i_begin + tq * BM + row;
-          ir = ir < sq ? ir : sq - 1;
-          dma_rows4<T>(sel ? dg : qg, ir, sel ? do_stride : q_stride, row, lane, stage + slot * SLOT + sel * QT + rgp * 512);
-        }
-      }
+    // The copies of iteration (head g, step ti) into the stage at element offset `st`:
+    // general form (any tile, rows clamped per lane), used for the first stage and for tail tiles.
+    auto issue_general = [&](int st, int g, int ti) {
+      const int h = h_first + g;
+      const int tq = ti * QSPLIT + cp_slot;
+      if (tq < ntq)
+        dma_tile32_general<T, 8>(sAll + st + cp_dst0, cp_gt + (int64_t)h * D, cp_stride, 1, i_begin + tq * BM, 0, sq, cl0);
       if (w < QSPLIT) {
-        const int tq = ti * QSPLIT + w;
-        if (tq < ntq) {
-          int ir = i_begin + tq * BM + (lane & 31);
+        const int tl = ti * QSPLIT + w;
+        if (tl < ntq) {
+          int ir = i_begin + tl * BM + (lane & 31);
           ir = ir < sq ? ir : sq - 1;
-          const float *src = (lane < 32 ? p.lse : p.delta) + ((int64_t)b * p.hq + h) * lse_stride + ir;
+          const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + h) * p.max_sq + ir;
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                           (__attribute__((address_space(3))) void *)(stage + w * SLOT + 2 * QT), 4, 0, 0);
+                                           (__attribute__((address_space(3))) void *)(sAll + st + w * SLOT + 2 * QT), 4, 0, 0);
         }
       }
     };
-    auto compute = [&](const T *stage, int it) {
-      const int ti = it % it_per_head;
+
+    if (niter > 0) issue_general(0, 0, 0);
+    dma_wait_all();
+    __syncthreads();
+
+    const char *cp_src = nullptr;
+    uint32_t cp_dst = 0;
+    bool fcopy = false;
+#define DH_DKV_COPY(i)                                                                                  \
+    do {                                                                                                \
+      if (fcopy) {                                                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+        dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                                \
+        cp_src += cp_step;                                                                              \
+        cp_dst += 1024;                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+      }                                                                                                 \
+    } while (0)
+
+    int g = 0, ti = 0;                                // head and step of iteration it
+#pragma unroll 1
+    for (int it = 0; it < niter; ++it) {
+      int gn = g, tn = ti + 1;                        // ... and of iteration it + 1
+      if (tn == it_per_head) { tn = 0; ++gn; }
+      const bool have_next = it + 1 < niter;
+      const uint32_t cur = lds0 + (uint32_t)((it & 1) * STAGEB);
+      const int nxt_el = ((it + 1) & 1) * STAGE;
+      {
+        const int hn = h_first + gn;
+        const int tq = tn * QSPLIT + cp_slot;
+        const int row0 = i_begin + tq * BM;
+        const bool copy = have_next && tq < ntq;
+        fcopy = copy && row0 + BM <= sq;
+        cp_src = cp_g + ((int64_t)row0 * cp_stride + (int64_t)hn * D) * (int)sizeof(T);
+        cp_dst = lds0 + (uint32_t)((nxt_el + cp_dst0) * (int)sizeof(T));
+        if (copy && !fcopy)
+          dma_tile32_general<T, 8>(sAll + nxt_el + cp_dst0, cp_gt + (int64_t)hn * D, cp_stride, 1, row0, 0, sq, cl0);
+        if (w < QSPLIT && have_next) {
+          const int tl = tn * QSPLIT + w;
+          const int rl = i_begin + tl * BM;
+          if (tl < ntq) {
+            if (rl + BM <= sq) {
+              const char *src = ld_g + (((int64_t)b * p.hq + hn) * p.max_sq + rl) * 4;
+              const uint32_t dst = lds0 + (uint32_t)((nxt_el + w * SLOT + 2 * QT) * (int)sizeof(T));
+              asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                           :
+                           : "v"(ld_off), "s"(src), "s"(dst)
+                           : "memory", "m0");
+            } else {
+              int ir = rl + (lane & 31);
+              ir = ir < sq ? ir : sq - 1;
+              const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + hn) * p.max_sq + ir;
+              __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                               (__attribute__((address_space(3))) void *)(sAll + nxt_el + w * SLOT + 2 * QT), 4, 0, 0);
+            }
+          }
+        }
+      }
       const int tq = ti * QSPLIT + qs;
       const int i0 = i_begin + tq * BM;
-      if (tq >= ntq || (causal && i0 + BM - 1 < jw0)) return;
-      const T *tQ = stage + qs * SLOT;
-      const T *tdO = tQ + QT;
-      const float *tL = reinterpret_cast<const float *>(tQ + 2 * QT);   // [32 lse | 32 delta]
-      floatx16 S, dP;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        S[v] = 0.f;
-        dP[v] = 0.f;
-      }
-      {
-        Frag aq = frag_ld_swz<T>(tQ, c, hh);
-        Frag ad = frag_ld_swz<T>(tdO, c, hh);
+      const bool act = tq < ntq && !(causal && i0 + BM - 1 < jw0);
+      if (act) {
+        // The LDS reads below are ordinary loads: the compiler does not know about the assembly copies,
+        // so it orders them only against other LDS traffic, and it places the partial waits itself.
+        // One wavefront per SIMD has nobody to hide its LDS latency behind, so all reads of a phase are
+        // issued in one batch ahead of the matrix instructions that consume them (the scheduling
+        // barriers keep the batches where they are written).
+        uint32_t qb = cur + rf_lane, ta = cur + ta_lane, tb = cur + tb_lane, tl = cur + tl_lane;
+        asm volatile("" : "+v"(qb), "+v"(ta), "+v"(tb), "+v"(tl));   // derive the other addresses here
+        typedef __attribute__((address_space(3))) const Frag *lds_frag;
+        typedef __attribute__((address_space(3))) const floatx4 *lds_f4;
+        typedef short4v __attribute__((address_space(3))) *lds_tr;
+        Frag fq[D / 16], fo[D / 16];
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) {
-          Frag aq2 = aq, ad2 = ad;
-          if (ks + 1 < D / 16) {
-            aq2 = frag_ld_swz<T>(tQ, c, 2 * (ks + 1) + hh);
-            ad2 = frag_ld_swz<T>(tdO, c, 2 * (ks + 1) + hh);
-          }
-          S = M::mma(aq, Kf[ks], S);
-          dP = M::mma(ad, Vf[ks], dP);
-          aq = aq2;
-          ad = ad2;
+          const uint32_t a = qb ^ (uint32_t)(ks << 5);
+          fq[ks] = *(lds_frag)(a);
+          fo[ks] = *(lds_frag)(a + QT * (uint32_t)sizeof(T));
         }
-      }
-      const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
-      float pv[16], dsv[16];
+        floatx4 l4[4], d4[4];                               // lse (exp2 units) and delta of rows 8*vb + 4*hh + e
 #pragma unroll
-      for (int vb = 0; vb < 4; ++vb) {
-        const float4 l4 = *reinterpret_cast<const float4 *>(tL + 8 * vb + 4 * hh);
-        const float4 d4 = *reinterpret_cast<const float4 *>(tL + 32 + 8 * vb + 4 * hh);
-        const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
-        const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int v = 4 * vb + e;
-          float pe = fast_exp2(S[v] * scale_log2 - ls[e] * 1.4426950408889634f);
-          if (need_mask) {
-            const int i = i0 + acc_row(v, hh);
-            if (i >= sq || (causal && jrow > i)) pe = 0.f;
-          }
-          pv[v] = pe;
-          dsv[v] = pe * (dP[v] - dl[e]);
+        for (int vb = 0; vb < 4; ++vb) {
+          l4[vb] = *(lds_f4)(tl + 32 * vb);
+          d4[vb] = *(lds_f4)(tl + 128 + 32 * vb);
         }
-      }
-      Frag Pb[2], dSb[2];
-      Pb[0] = frag_pack<T>(pv);
-      Pb[1] = frag_pack<T>(pv + 8);
-      dSb[0] = frag_pack<T>(dsv);
-      dSb[1] = frag_pack<T>(dsv + 8);
+        floatx16 S, dP;
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        Tr4 dot, qt;
-        tr4_issue<T>(dot, tdO, 16 * s, lane);
-        tr4_issue<T>(qt, tQ, 16 * s, lane);
-        dVt[0] = M::mma(tr4_get<T, 14>(dot, 0), Pb[s], dVt[0]);
-        dVt[1] = M::mma(tr4_get<T, 12>(dot, 1), Pb[s], dVt[1]);
-        dVt[2] = M::mma(tr4_get<T, 10>(dot, 2), Pb[s], dVt[2]);
-        dVt[3] = M::mma(tr4_get<T, 8>(dot, 3), Pb[s], dVt[3]);
-        dKt[0] = M::mma(tr4_get<T, 6>(qt, 0), dSb[s], dKt[0]);
-        dKt[1] = M::mma(tr4_get<T, 4>(qt, 1), dSb[s], dKt[1]);
-        dKt[2] = M::mma(tr4_get<T, 2>(qt, 2), dSb[s], dKt[2]);
-        dKt[3] = M::mma(tr4_get<T, 0>(qt, 3), dSb[s], dKt[3]);
+        for (int v = 0; v < 16; ++v) {
+          S[v] = 0.f;
+          dP[v] = 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+          switch (ks) {
+            case 0: mfma_b_fixed<T, 128, true>(S, fq[0]); mfma_b_fixed<T, 160, true>(dP, fo[0]); break;
+            case 1: mfma_b_fixed<T, 132>(S, fq[1]); mfma_b_fixed<T, 164>(dP, fo[1]); break;
+            case 2: mfma_b_fixed<T, 136>(S, fq[2]); mfma_b_fixed<T, 168>(dP, fo[2]); break;
+            case 3: mfma_b_fixed<T, 140>(S, fq[3]); mfma_b_fixed<T, 172>(dP, fo[3]); break;
+            case 4: mfma_b_fixed<T, 144>(S, fq[4]); mfma_b_fixed<T, 176>(dP, fo[4]); break;
+            case 5: mfma_b_fixed<T, 148>(S, fq[5]); mfma_b_fixed<T, 180>(dP, fo[5]); break;
+            case 6: mfma_b_fixed<T, 152>(S, fq[6]); mfma_b_fixed<T, 184>(dP, fo[6]); break;
+            default: mfma_b_fixed<T, 156>(S, fq[7]); mfma_b_fixed<T, 188>(dP, fo[7]); break;
+          }
+          if (ks & 1) DH_DKV_COPY(ks >> 1);                            // copy blocks 0..3
+        }
+        // transposed fragments of the dO and Q tiles for dV^T += dO^T P and dK^T += Q^T dS: all 32
+        // transpose reads go out now and land while S and dP finish and the softmax part runs
+        short4v to[2][4][2], tq[2][4][2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
+            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
+            to[s][t][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0 + QT * (uint32_t)sizeof(T)));
+            to[s][t][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1 + QT * (uint32_t)sizeof(T)));
+            tq[s][t][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
+            tq[s][t][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
+          }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_drain();                                                  // S and dP are read by ordinary code next
+        const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          float pv[8], dsv[8];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int vb = 2 * s + u;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int v = 4 * vb + e;
+              float pe = fast_exp2(S[v] * scale_log2 - l4[vb][e]);
+              if (need_mask) {
+                const int i = i0 + acc_row(v, hh);
+                if (i >= sq || (causal && jrow > i)) pe = 0.f;
+              }
+              pv[4 * u + e] = pe;
+              dsv[4 * u + e] = pe * (dP[v] - d4[vb][e]);
+            }
+          }
+          const Frag Pb = frag_pack<T>(pv), dSb = frag_pack<T>(dsv);
+          mfma_acc_fixed<T, 0, true>(frag_join<T>(to[s][0][0], to[s][0][1]), Pb);
+          mfma_acc_fixed<T, 16>(frag_join<T>(to[s][1][0], to[s][1][1]), Pb);
+          mfma_acc_fixed<T, 32>(frag_join<T>(to[s][2][0], to[s][2][1]), Pb);
+          mfma_acc_fixed<T, 48>(frag_join<T>(to[s][3][0], to[s][3][1]), Pb);
+          DH_DKV_COPY(4 + 2 * s);
+          mfma_acc_fixed<T, 64, true>(frag_join<T>(tq[s][0][0], tq[s][0][1]), dSb);
+          mfma_acc_fixed<T, 80>(frag_join<T>(tq[s][1][0], tq[s][1][1]), dSb);
+          mfma_acc_fixed<T, 96>(frag_join<T>(tq[s][2][0], tq[s][2][1]), dSb);
+          mfma_acc_fixed<T, 112>(frag_join<T>(tq[s][3][0], tq[s][3][1]), dSb);
+          DH_DKV_COPY(5 + 2 * s);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) DH_DKV_COPY(i);
       }
-    };
-
-    if (niter > 0) issue(sStage0, 0);
-    __syncthreads();
-    for (int it = 0; it < niter; it += 2) {
-      if (it + 1 < niter) issue(sStage1, it + 1);
-      compute(sStage0, it);
-      __syncthreads();
-      if (it + 1 < niter) {
-        if (it + 2 < niter) issue(sStage0, it + 2);
-        compute(sStage1, it + 1);
-        __syncthreads();
-      }
+      g = gn;
+      ti = tn;
+      dma_wait_all();
+      __syncthreads();   // the next stage has landed, and everyone is done with the current one
     }
+#undef DH_DKV_COPY
+    mfma_drain();                                     // the accumulators are read next
+    floatx16 dKt[D / 32], dVt[D / 32];
+    dVt[0] = agpr_read16<0>(); dVt[1] = agpr_read16<16>(); dVt[2] = agpr_read16<32>(); dVt[3] = agpr_read16<48>();
+    dKt[0] = agpr_read16<64>(); dKt[1] = agpr_read16<80>(); dKt[2] = agpr_read16<96>(); dKt[3] = agpr_read16<112>();
 
     // add the second split's partial sums through LDS: dK in stage 0, dV in stage 1
-    float *xk = reinterpret_cast<float *>(sStage0) + kg * 4096;
-    float *xv = reinterpret_cast<float *>(sStage1) + kg * 4096;
+    float *xk = reinterpret_cast<float *>(sAll) + kg * 4096;
+    float *xv = reinterpret_cast<float *>(sAll + STAGE) + kg * 4096;
     static_assert(STAGE * sizeof(T) >= KG * 4096 * sizeof(float), "exchange area");
     if (qs == 1) {
 #pragma unroll
@@ -1004,8 +1116,9 @@ static int launch_dq(const AttnBwdParams &p, int batch, hipStream_t st) {
 }
 
 template <typename T>
-static int launch_delta(const void *dout, const void *out, float *delta, const int32_t *cu_q, int batch, int max_sq,
-                        int hq, int d, int64_t do_stride, int64_t o_stride, hipStream_t st) {
+static int launch_delta(const void *dout, const void *out, float *delta, const float *lse, float *ld2, int64_t ld2_plane,
+                        const int32_t *cu_q, int batch, int max_sq, int hq, int d, int64_t do_stride, int64_t o_stride,
+                        hipStream_t st) {
   const int nvec = d / Vec<T>::N;
   int lanes_per = 1;
   while (lanes_per < nvec && lanes_per < 64) lanes_per <<= 1;
@@ -1014,7 +1127,8 @@ static int launch_delta(const void *dout, const void *out, float *delta, const i
   if (blocks > 256 * 16) blocks = 256 * 16;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL((attn_delta_kernel<T>), dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, st,
-                     (const T *)dout, (const T *)out, delta, cu_q, max_sq, hq, d, lanes_per, do_stride, o_stride);
+                     (const T *)dout, (const T *)out, delta, lse, ld2, ld2_plane, cu_q, max_sq, hq, d, lanes_per, do_stride,
+                     o_stride);
   return DH_OK;
 }
 
@@ -1032,7 +1146,9 @@ extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, 
                                               int hk, int d, int dtype) {
   using namespace dh;
   (void)total_q;
-  size_t n = align256((size_t)batch * hq * (max_seqlen_q > 0 ? max_seqlen_q : 0) * sizeof(float));
+  const size_t plane = align256((size_t)batch * hq * (max_seqlen_q > 0 ? max_seqlen_q : 0) * sizeof(float));
+  size_t n = plane;                               // delta
+  if (dtype != DH_F32 && d == 128) n += 2 * plane;  // lse (exp2 units) and delta side by side for the d = 128 kernels
   if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
     n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
   return n + 256;
@@ -1054,8 +1170,15 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   DH_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   uint8_t *ws = (uint8_t *)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  const size_t plane = align256((size_t)batch * hq * max_seqlen_q * sizeof(float));
   float *delta = delta_out ? delta_out : (float *)ws;
-  ws += align256((size_t)batch * hq * max_seqlen_q * sizeof(float));
+  ws += plane;
+  float *ld2 = nullptr;
+  if (dtype != DH_F32 && d == 128) {
+    ld2 = (float *)ws;
+    ws += 2 * plane;
+    DH_CHECK(plane < (1ull << 31), "batch * heads * max_seqlen_q too large");
+  }
 
   const int n = 16 / (int)dtype_size(dtype);
   DH_CHECK(d % n == 0 || dtype == DH_F32, "head dim %d must be a multiple of %d", d, n);
@@ -1063,7 +1186,8 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
            "dout/out rows must be 16-byte aligned");
   if (max_seqlen_q > 0) {
     DH_DISPATCH_DTYPE(dtype, {
-      launch_delta<T>(dout, out, delta, cu_seqlens_q, batch, max_seqlen_q, hq, d, do_stride, o_stride, st);
+      launch_delta<T>(dout, out, delta, lse, ld2, (int64_t)(plane / sizeof(float)), cu_seqlens_q, batch, max_seqlen_q, hq, d,
+                      do_stride, o_stride, st);
     });
   }
   if (dtype == DH_F32) {
@@ -1080,6 +1204,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
            "pointers must be 16-byte aligned");
   AttnBwdParams p;
   p.dout = dout; p.q = q; p.k = k; p.v = v; p.lse = lse; p.delta = delta;
+  p.ld2 = ld2; p.ld2_plane = (int64_t)(plane / sizeof(float));
   p.dq = dq; p.dk = dk; p.dv = dv;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
   p.max_sq = max_seqlen_q; p.hq = hq; p.hk = hk;

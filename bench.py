@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+ATTN_BWD_TRAFFIC_BYTES = 164.2e6   # measured; see profiles/attn_70b_shard_hbm_traffic.md
 
 
 def _ensure_built():
@@ -305,8 +306,11 @@ def main():
     dom = next((k for k in kernels if k["kernel"].startswith("attn_bwd")), None)
     roofline = None
     if dom is not None:
+        # HBM bytes per launch of the backward (its four kernels), from two rocprofv3 --pmc runs
+        # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000: factors from the 1 GiB copy kernel) at this exact shape.
         roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"],
-                    "unit": dom["unit"], "frac": dom["frac"], "traffic": None}
+                    "unit": dom["unit"], "frac": dom["frac"], "traffic": ATTN_BWD_TRAFFIC_BYTES,
+                    "traffic_unit": "bytes/launch (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, calibrated)"}
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg)
 
     line = {

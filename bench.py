@@ -247,6 +247,24 @@ def profile_op(name: str, iters: int = 5):
             dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
             sp = torch.cuda.current_stream().cuda_stream
             fn = lambda: _Clib._attn_bwd_raw(do, q, k, v, o[0], o[5], dq, dk, dv, None, cu, cu, T, T, sc, True, sp)
+    elif name in ("moe_ffn_fwd", "moe_ffn_bwd"):
+        from dhellam_amd.operators import moe
+        Tm, Hm, E, K, Fm = 8192, 4096, 8, 2, 14336
+        logits = torch.randn(Tm, E, generator=g, device=dev)
+        xm = rn(Tm, Hm)
+        idx, gates, _ = moe.route_topk(logits, K)
+        plan, _ = moe.sort_assignments(idx, E)
+        Rm = int(plan.expert_offsets[2].item())
+        xp, _ = moe.permute_fwd(xm, plan, 0, 2, Rm)
+        w1 = (torch.randn(2, 2 * Fm, Hm, generator=g, device=dev) * 0.02).to(dt)
+        w2 = (torch.randn(2, Hm, Fm, generator=g, device=dev) * 0.02).to(dt)
+        offs = plan.expert_offsets[0:3]
+        if name.endswith("fwd"):
+            fn = lambda: moe.expert_ffn_fwd(xp, w1, w2, offs)
+        else:
+            y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
+            dyp = rn(Rm, Hm)
+            fn = lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved)
     else:
         raise SystemExit(f"unknown --profile-op {name}")
     for _ in range(iters):
@@ -264,7 +282,7 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
-                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, copy) and exit")
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, copy) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "

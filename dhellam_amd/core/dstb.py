@@ -334,8 +334,12 @@ class DCFunc:
         if peer is None:
             raise RuntimeError("sequence-parallel gather stand-in needs the micro-batch's peer buffer")
         rows = input.numel() // input.shape[-1]
-        with torch.cuda.stream(stream):
-            peer[config.tp_rank * rows:(config.tp_rank + 1) * rows].copy_(input.view(rows, -1))
+        dst = peer[config.tp_rank * rows:(config.tp_rank + 1) * rows]
+        src = input.view(rows, -1)
+        assert dst.is_contiguous() and src.is_contiguous() and dst.dtype == src.dtype and dst.shape == src.shape
+        st = stream if stream is not None else torch.cuda.current_stream()
+        _lib.check(_lib.load().dh_copy_bytes(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(),
+                                             st.cuda_stream))
         return peer, None
 
     @staticmethod

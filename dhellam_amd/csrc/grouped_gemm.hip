@@ -6,8 +6,11 @@
 //   NT  c[r, n]  = sum_k a[r, k] * w[g][n, k]      forward  (both k-contiguous)
 //   NN  c[r, n]  = sum_k a[r, k] * w[g][k, n]      dgrad    (w strided in k)
 //   TN  c[g][m,n] = sum_r a[r, m] * b[r, n]        wgrad    (both strided in k = r)
-// A workgroup is 2x2 wavefronts, each owning a (32*WM) x (32*WN) output block
-// kept in accumulators; 64-deep k slices of both operands are staged in LDS
+// A workgroup is 2 x WVN wavefronts, each owning a (32*WM) x (32*WN) output block
+// kept in accumulators (256x256 tiles: 2x4 wavefronts of 128x64, two wavefronts per
+// SIMD, so that one wavefront's loads, LDS stores and barrier waits overlap the other's
+// MFMAs; with one wavefront per SIMD those phases simply added up); 64-deep k slices of
+// both operands are staged in LDS
 // (two stages, one barrier per slice).  k-contiguous operands are read from LDS
 // as 16-byte row fragments; k-strided operands stay row-major in LDS and are
 // read with transpose loads, so no operand is ever transposed in memory.
@@ -38,25 +41,27 @@ struct GGParams {
 // Load one 64-deep k slice of an operand into registers.
 //   KC (k-contiguous): tile [R rows][64 k]; element (row, k) at src[row * ld + k]
 //   KS (k-strided)   : tile [64 k][R cols]; element (k, col) at src[k * ld + col]
-template <typename T, int R, bool KSTRIDED>
+template <typename T, int R, bool KSTRIDED, int NT>
 struct TileLoader {
   static constexpr int VECS = R * GG_BK / 8;
-  static constexpr int LPT = VECS / 256;
-  static_assert(VECS % 256 == 0, "tile must divide over 256 threads");
+  static constexpr int LPT = VECS / NT;
+  static_assert(VECS % NT == 0, "tile must divide over the workgroup's threads");
   // rows: extent along the R dimension still valid (from tile origin); kext: valid k extent from this slice's origin
+  // FULL: the whole slice lies inside the operand (no predication: straight-line loads).
+  template <bool FULL>
   static __device__ __forceinline__ void gload(uint4 (&reg)[LPT], const T *src, int64_t ld, int rext, int kext, int tid) {
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
-      const int idx = tid + i * 256;
+      const int idx = tid + i * NT;
       int r, k;
       if (KSTRIDED) {
         k = idx / (R / 8);
         r = (idx % (R / 8)) * 8;
-        reg[i] = (k < kext && r < rext) ? *reinterpret_cast<const uint4 *>(src + (int64_t)k * ld + r) : make_uint4(0, 0, 0, 0);
+        reg[i] = (FULL || (k < kext && r < rext)) ? *reinterpret_cast<const uint4 *>(src + (int64_t)k * ld + r) : make_uint4(0, 0, 0, 0);
       } else {
         r = idx / (GG_BK / 8);
         k = (idx % (GG_BK / 8)) * 8;
-        reg[i] = (r < rext && k < kext) ? *reinterpret_cast<const uint4 *>(src + (int64_t)r * ld + k) : make_uint4(0, 0, 0, 0);
+        reg[i] = (FULL || (r < rext && k < kext)) ? *reinterpret_cast<const uint4 *>(src + (int64_t)r * ld + k) : make_uint4(0, 0, 0, 0);
       }
     }
   }
@@ -65,7 +70,7 @@ struct TileLoader {
   static __device__ __forceinline__ void sstore(const uint4 (&reg)[LPT], T *dst, int tid) {
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
-      const int idx = tid + i * 256;
+      const int idx = tid + i * NT;
       if (KSTRIDED) {
         const int k = idx / (R / 8), r = (idx % (R / 8)) * 8;
         *reinterpret_cast<uint4 *>(dst + k * LD + r) = reg[i];
@@ -83,13 +88,14 @@ struct TileLoader {
   }
 };
 
-template <typename T, bool TA, bool TB, int WM, int WN, bool GROUPED_OUT>
-__global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
+// WM x WN: 32x32 accumulator blocks per wavefront; the workgroup is 2 x WVN wavefronts.
+template <typename T, bool TA, bool TB, int WM, int WN, int WVN, bool GROUPED_OUT>
+__global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
-  constexpr int BM = 64 * WM, BN = 64 * WN;
-  using LA = TileLoader<T, BM, TA>;
-  using LB = TileLoader<T, BN, TB>;
+  constexpr int BM = 64 * WM, BN = 32 * WN * WVN, NT = 128 * WVN;
+  using LA = TileLoader<T, BM, TA, NT>;
+  using LB = TileLoader<T, BN, TB, NT>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T *sA = reinterpret_cast<T *>(smem_raw);   // [2][LA::ELEMS]
   T *sB = sA + 2 * LA::ELEMS;                // [2][LB::ELEMS]
@@ -126,7 +132,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
-  const int wm = w >> 1, wn = w & 1;
+  const int wm = w / WVN, wn = w % WVN;
   const int n0 = tn * BN;
 
   // Operand origins and extents.
@@ -163,8 +169,13 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
   auto gload = [&](int s) {
     const int64_t k0 = (int64_t)s * GG_BK;
     const int kext = (int)(k_total - k0 < GG_BK ? k_total - k0 : GG_BK);
-    LA::gload(ra, TA ? ag + k0 * p.lda : ag + k0, p.lda, a_rext, kext, tid);
-    LB::gload(rb, TB ? bg + k0 * p.ldb : bg + k0, p.ldb, b_rext, kext, tid);
+    if (a_rext >= BM && b_rext >= BN && kext == GG_BK) {     // interior slice (wave-uniform test)
+      LA::template gload<true>(ra, TA ? ag + k0 * p.lda : ag + k0, p.lda, a_rext, kext, tid);
+      LB::template gload<true>(rb, TB ? bg + k0 * p.ldb : bg + k0, p.ldb, b_rext, kext, tid);
+    } else {
+      LA::template gload<false>(ra, TA ? ag + k0 * p.lda : ag + k0, p.lda, a_rext, kext, tid);
+      LB::template gload<false>(rb, TB ? bg + k0 * p.ldb : bg + k0, p.ldb, b_rext, kext, tid);
+    }
   };
   if (nslices > 0) {
     gload(0);
@@ -178,17 +189,25 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
     if (s + 1 < nslices) gload(s + 1);
     const T *tA = sA + st * LA::ELEMS;
     const T *tB = sB + st * LB::ELEMS;
+    // operand fragments are read one k step ahead of the MFMAs that use them
+    Frag fa[2][WM], fb[2][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[0][i] = LA::frag(tA, wm * 32 * WM + 32 * i, 0, lane);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[0][j] = LB::frag(tB, wn * 32 * WN + 32 * j, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < GG_BK / 16; ++ks) {
-      Frag fa[WM], fb[WN];
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < GG_BK / 16) {
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[i] = LA::frag(tA, wm * 32 * WM + 32 * i, ks, lane);
+        for (int i = 0; i < WM; ++i) fa[nxt][i] = LA::frag(tA, wm * 32 * WM + 32 * i, ks + 1, lane);
 #pragma unroll
-      for (int j = 0; j < WN; ++j) fb[j] = LB::frag(tB, wn * 32 * WN + 32 * j, ks, lane);
+        for (int j = 0; j < WN; ++j) fb[nxt][j] = LB::frag(tB, wn * 32 * WN + 32 * j, ks + 1, lane);
+      }
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = M::mma(fb[j], fa[i], acc[i][j]);  // C^T block: rows n, cols m
+        for (int j = 0; j < WN; ++j) acc[i][j] = M::mma(fb[cur][j], fa[cur][i], acc[i][j]);  // C^T block: rows n, cols m
     }
     if (s + 1 < nslices) {
       LA::sstore(ra, sA + (st ^ 1) * LA::ELEMS, tid);
@@ -210,9 +229,10 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     const int m = wm * 32 * WM + 32 * i + c;
-    if (m < m_lim) {
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
+    for (int j = 0; j < WN; ++j) {
+      const floatx16 av = acc[i][j];
+      if (m < m_lim) {
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {
           const int n = wn * 32 * WN + 32 * j + 8 * vb + 4 * hh;
@@ -223,28 +243,200 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(const GGParams p) {
             if (p.accumulate) {
               const Q4 old = *dst;
 #pragma unroll
-              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e] + static_cast<float>(old.v[e]));
+              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e] + static_cast<float>(old.v[e]));
             } else {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e]);
+              for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
             }
             *dst = o;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---- NT with direct global->LDS copies --------------------------------------------------------------
+// The forward product at 256x256 tiles when K is a multiple of 64.  The register-staged kernel above
+// runs its phases one after the other (wait for the global loads, store them to LDS, barrier, MFMAs):
+// switching off one phase at a time showed their times simply add up.  Here the next k slice goes
+// global -> LDS by assembly copies issued between the MFMAs of the current slice (no staging registers,
+// no LDS stores, the wavefront never waits for its own loads before the end of the slice).
+// Tiles are [256 rows][64 k] with unpadded 128-byte rows; the 16-byte chunk index is XORed with
+// (row / 2) % 8, applied on the global side of the copy, which makes the 16-byte row-fragment reads
+// conflict-free.  8 wavefronts = 2 (m) x 4 (n), 128x64 outputs each; wavefronts 0-3 copy the A tile
+// (64 rows each), wavefronts 4-7 the B tile.
+template <typename T>
+__global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int BM = 256, BN = 256, WM = 4, WN = 2, WVN = 4;
+  constexpr int TILEB = 256 * GG_BK * (int)sizeof(T);   // one operand tile: 32 KB
+  constexpr int STAGEB = 2 * TILEB;                     // A tile, then B tile
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
+
+  // A contiguous run of tiles per XCD, m fastest (tiles that share a weight panel run together).
+  // Cutting the grid into 4 x 8 super-tiles per XCD instead lowers the L2 miss traffic by a third
+  // (measured) but is slower: the bound is not the fabric.
+  const int ntiles = p.tiles_m * p.tiles_n;
+  int pid = blockIdx.x;
+  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  int tm = pid % p.tiles_m;
+  const int tn = pid / p.tiles_m;
+  const int base = p.offs[0];
+  int g = 0, row_begin = 0, row_end = 0;
+  {
+    bool found = false;
+    for (int gi = 0; gi < p.groups; ++gi) {
+      const int rb = p.offs[gi] - base, re = p.offs[gi + 1] - base;
+      const int t = (re - rb + BM - 1) / BM;
+      if (!found && tm < t) {
+        g = gi; row_begin = rb; row_end = re; found = true;
+      } else if (!found) {
+        tm -= t;
+      }
+    }
+    if (!found) return;
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, hh = lane >> 5;
+  const int wm = w / WVN, wn = w % WVN;
+  const int n0 = tn * BN, m0 = row_begin + tm * BM;
+  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
+  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
+  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (int64_t)n0 * p.ldb;
+  const int nslices = (int)(p.k_dim / GG_BK);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+
+  // ---- copies ------------------------------------------------------------------------------------
+  const int cp_b = w >> 2;                              // 0: A tile, 1: B tile
+  const int cp_row0 = 64 * (w & 3);
+  const int cp_ld = (int)(cp_b ? p.ldb : p.lda);
+  const int cp_ext = cp_b ? b_rext : a_rext;            // valid rows of the tile
+  const T *cp_t = cp_b ? bg : ag;
+  const char *cp_g = reinterpret_cast<const char *>(cp_t + (int64_t)cp_row0 * cp_ld);
+  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * 128);
+  const uint32_t cp_step = (uint32_t)(8 * cp_ld) * (uint32_t)sizeof(T);
+  const bool cp_fast = cp_row0 + 64 <= cp_ext;          // every row this wavefront copies exists
+  const int lr = lane >> 3, lc = lane & 7;
+  uint32_t cp_off[2];                                   // block i of 8 rows: swizzle (row / 2) % 8 = (4 * (i % 2) + lr / 2) % 8
+#pragma unroll
+  for (int x = 0; x < 2; ++x)
+    cp_off[x] = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)((lc ^ ((4 * x + (lr >> 1)) & 7)) << 4);
+  // general form (tiles at the edge of a group or of n): rows past the end re-read the last valid row
+  auto copy_general = [&](uint32_t stage, int slice) {
+#pragma unroll 1
+    for (int i = 0; i < 8; ++i) {
+      int row = cp_row0 + 8 * i + lr;
+      const int f = (row >> 1) & 7;
+      row = row < cp_ext ? row : cp_ext - 1;
+      const T *src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * GG_BK + ((lc ^ f) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)(smem + stage + cp_dst0 + i * 1024), 16, 0, 0);
+    }
+  };
+  // ---- fragment reads: byte offsets inside a stage; other k steps by XOR, other 32-row blocks by +4 KB ----
+  const uint32_t sw = (uint32_t)((hh ^ ((c >> 1) & 7)) << 4);
+  const uint32_t fa_lane = (uint32_t)((wm * 32 * WM + c) * 128) + sw;             // A tile rows (m)
+  const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * 128) + sw;     // B tile rows (n)
+  typedef __attribute__((address_space(3))) const Frag *lds_frag;
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  if (nslices > 0 && cp_ext > 0) copy_general(0, 0);
+  dma_wait_all();
+  __syncthreads();
+
+#pragma unroll 1
+  for (int s = 0; s < nslices; ++s) {
+    const uint32_t cur = (uint32_t)((s & 1) * STAGEB), nxt = (uint32_t)(((s + 1) & 1) * STAGEB);
+    const bool copy = s + 1 < nslices && cp_ext > 0;
+    const bool fcopy = copy && cp_fast;
+    const char *cp_src = cp_g + (int64_t)(s + 1) * GG_BK * (int)sizeof(T);
+    uint32_t cp_dst = lds0 + nxt + cp_dst0;
+    if (copy && !fcopy) copy_general(nxt, s + 1);
+    uint32_t fa0 = lds0 + cur + fa_lane, fb0 = lds0 + cur + fb_lane;
+    asm volatile("" : "+v"(fa0), "+v"(fb0));            // derive the other addresses here, not ahead of the loop
+    Frag fa[2][WM], fb[2][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(fa0 + i * 4096);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(fb0 + j * 4096);
+#pragma unroll
+    for (int ks = 0; ks < GG_BK / 16; ++ks) {
+      const int cu = ks & 1, nx = cu ^ 1;
+      if (ks + 1 < GG_BK / 16) {
+#pragma unroll
+        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)((fa0 ^ (uint32_t)((ks + 1) << 5)) + i * 4096);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)((fb0 ^ (uint32_t)((ks + 1) << 5)) + j * 4096);
+      }
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);  // C^T block: rows n, cols m
+        if ((i & 1) && fcopy) {                       // one 1 KB copy block after every 4 MFMAs
+          __builtin_amdgcn_sched_barrier(0);
+          dma_block_fast(cp_src, cp_off[(2 * ks + (i >> 1)) & 1], cp_dst);
+          cp_src += cp_step;
+          cp_dst += 1024;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    dma_wait_all();
+    __syncthreads();   // the next stage has landed, and everyone is done with the current one
+  }
+
+  // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
+  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int m = wm * 32 * WM + 32 * i + c;
+    if (m < a_rext) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          const int n = wn * 32 * WN + 32 * j + 8 * vb + 4 * hh;
+          if (n < b_rext) {
+            struct alignas(8) Q4 { T v[4]; };
+            Q4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e]);
+            *reinterpret_cast<Q4 *>(cg + (int64_t)m * p.ldc + n) = o;
           }
         }
     }
   }
 }
 
-template <typename T, bool TA, bool TB, int WM, int WN, bool GROUPED_OUT>
+template <typename T>
+static int launch_gg_nt_dma(GGParams p, int64_t m_extent, hipStream_t st) {
+  p.tiles_n = (int)cdiv(p.n_dim, 256);
+  p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
+  if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
+  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(512), 0, st, p);
+  return DH_OK;
+}
+
+template <typename T, bool TA, bool TB, int WM, int WN, int WVN, bool GROUPED_OUT>
 static int launch_gg(GGParams p, int64_t m_extent, hipStream_t st) {
-  constexpr int BM = 64 * WM, BN = 64 * WN;
-  using LA = TileLoader<T, BM, TA>;
-  using LB = TileLoader<T, BN, TB>;
+  constexpr int BM = 64 * WM, BN = 32 * WN * WVN, NT = 128 * WVN;
+  using LA = TileLoader<T, BM, TA, NT>;
+  using LB = TileLoader<T, BN, TB, NT>;
   constexpr size_t smem = 2 * (LA::ELEMS + LB::ELEMS) * sizeof(T);
   static_assert(smem <= 160 * 1024, "LDS budget");
   static bool attr_set = false;
   if (!attr_set) {
-    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&grouped_gemm_kernel<T, TA, TB, WM, WN, GROUPED_OUT>),
+    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&grouped_gemm_kernel<T, TA, TB, WM, WN, WVN, GROUPED_OUT>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     attr_set = true;
   }
@@ -252,7 +444,7 @@ static int launch_gg(GGParams p, int64_t m_extent, hipStream_t st) {
   p.tiles_m = GROUPED_OUT ? (int)cdiv(m_extent, BM) : (int)(cdiv(m_extent, BM) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), GROUPED_OUT ? (unsigned)p.groups : 1u);
-  hipLaunchKernelGGL((grouped_gemm_kernel<T, TA, TB, WM, WN, GROUPED_OUT>), grid, dim3(256), smem, st, p);
+  hipLaunchKernelGGL((grouped_gemm_kernel<T, TA, TB, WM, WN, WVN, GROUPED_OUT>), grid, dim3(NT), smem, st, p);
   return DH_OK;
 }
 
@@ -262,10 +454,10 @@ static int dispatch_gg(const GGParams &p, int64_t m_extent, int dtype, hipStream
   const int64_t big_tiles = cdiv(m_extent, 256) * cdiv(p.n_dim, 256) * (GROUPED_OUT ? p.groups : 1);
   const bool big = big_tiles >= 256;
   if (dtype == DH_BF16)
-    return big ? launch_gg<bf16_t, TA, TB, 4, 4, GROUPED_OUT>(p, m_extent, st)
-               : launch_gg<bf16_t, TA, TB, 2, 2, GROUPED_OUT>(p, m_extent, st);
-  return big ? launch_gg<f16_t, TA, TB, 4, 4, GROUPED_OUT>(p, m_extent, st)
-             : launch_gg<f16_t, TA, TB, 2, 2, GROUPED_OUT>(p, m_extent, st);
+    return big ? launch_gg<bf16_t, TA, TB, 4, 2, 4, GROUPED_OUT>(p, m_extent, st)
+               : launch_gg<bf16_t, TA, TB, 2, 2, 2, GROUPED_OUT>(p, m_extent, st);
+  return big ? launch_gg<f16_t, TA, TB, 4, 2, 4, GROUPED_OUT>(p, m_extent, st)
+             : launch_gg<f16_t, TA, TB, 2, 2, 2, GROUPED_OUT>(p, m_extent, st);
 }
 
 static int gg_common_checks(const void *a, const void *b, void *c, const int32_t *offs, int groups, int dtype) {
@@ -290,7 +482,12 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0;
-  rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
+  const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
+  if (big && k % GG_BK == 0 && k < (1ll << 30))
+    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_nt_dma<f16_t>(p, max_rows, (hipStream_t)stream);
+  else
+    rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;

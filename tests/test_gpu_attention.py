@@ -76,6 +76,8 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     ([128, 77], [640, 33], 6, 3, 64, False),
     ([2048], [1024], 8, 2, 128, False),          # ring 'lower' shape
     ([1024], [2048], 8, 2, 128, False),          # ring 'upper' shape
+    ([384, 129], [384, 129], 4, 4, 128, True),   # MHA at d 128: dK/dV written directly (no head split)
+    ([128] * 4, [512] * 4, 64, 16, 128, False),  # many kv heads: two query heads per dK/dV workgroup
 ])
 def test_attention_16bit(dtype, lens_q, lens_k, hq, hk, d, causal):
     _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal)

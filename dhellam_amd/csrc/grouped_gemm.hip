@@ -18,6 +18,12 @@
 // ends up with runs of 4 consecutive output columns of one row: 8-byte stores.
 // Group row ranges are read on the device from the offsets table.
 #include "mma.h"
+#ifndef DH_GG_WVN
+#define DH_GG_WVN 4
+#endif
+#ifndef DH_GG_CPI
+#define DH_GG_CPI 2
+#endif
 
 namespace dh {
 
@@ -266,11 +272,19 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 // (row / 2) % 8, applied on the global side of the copy, which makes the 16-byte row-fragment reads
 // conflict-free.  8 wavefronts = 2 (m) x 4 (n), 128x64 outputs each; wavefronts 0-3 copy the A tile
 // (64 rows each), wavefronts 4-7 the B tile.
-template <typename T>
-__global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams p) {
+// WVN = 4: 8 wavefronts of 128x64 (two per SIMD, accumulators in VGPRs).
+// WVN = 2: 4 wavefronts of 128x128 (one per SIMD): half the LDS fragment traffic per MFMA (the 128x64 form
+// moves 1 KB through the LDS per MFMA, reads plus copy writes, which is the whole LDS bandwidth at full MFMA
+// rate: there copies and MFMAs did not overlap at all).  Its 256 accumulator registers live in the fixed
+// AGPRs a[0:255], block (i, j) at a[16 * (i * WN + j)], named only by assembly MFMAs (as ordinary variables
+// the register allocator moves all of them between the register files around every k slice).
+template <typename T, int WVN>
+__global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GGParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
-  constexpr int BM = 256, BN = 256, WM = 4, WN = 2, WVN = 4;
+  constexpr int BM = 256, BN = 256, WM = 4, WN = 8 / WVN, NW = 2 * WVN;
+  constexpr bool FIXED = (WVN == 2);
+  constexpr int CPB = 64 / NW;                          // 1 KB copy blocks per wavefront and slice
   constexpr int TILEB = 256 * GG_BK * (int)sizeof(T);   // one operand tile: 32 KB
   constexpr int STAGEB = 2 * TILEB;                     // A tile, then B tile
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
@@ -301,7 +315,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hh = lane >> 5;
-  const int wm = w / WVN, wn = w % WVN;
+  const int wm = w / WVN, wn = w % WVN;   // 2 x WVN wavefronts
   const int n0 = tn * BN, m0 = row_begin + tm * BM;
   const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
   const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
@@ -310,15 +324,15 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
   // ---- copies ------------------------------------------------------------------------------------
-  const int cp_b = w >> 2;                              // 0: A tile, 1: B tile
-  const int cp_row0 = 64 * (w & 3);
+  const int cp_b = w / (NW / 2);                        // 0: A tile, 1: B tile
+  const int cp_row0 = 8 * CPB * (w % (NW / 2));
   const int cp_ld = (int)(cp_b ? p.ldb : p.lda);
   const int cp_ext = cp_b ? b_rext : a_rext;            // valid rows of the tile
   const T *cp_t = cp_b ? bg : ag;
   const char *cp_g = reinterpret_cast<const char *>(cp_t + (int64_t)cp_row0 * cp_ld);
   const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * 128);
   const uint32_t cp_step = (uint32_t)(8 * cp_ld) * (uint32_t)sizeof(T);
-  const bool cp_fast = cp_row0 + 64 <= cp_ext;          // every row this wavefront copies exists
+  const bool cp_fast = cp_row0 + 8 * CPB <= cp_ext;     // every row this wavefront copies exists
   const int lr = lane >> 3, lc = lane & 7;
   uint32_t cp_off[2];                                   // block i of 8 rows: swizzle (row / 2) % 8 = (4 * (i % 2) + lr / 2) % 8
 #pragma unroll
@@ -327,7 +341,7 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
   // general form (tiles at the edge of a group or of n): rows past the end re-read the last valid row
   auto copy_general = [&](uint32_t stage, int slice) {
 #pragma unroll 1
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < CPB; ++i) {
       int row = cp_row0 + 8 * i + lr;
       const int f = (row >> 1) & 7;
       row = row < cp_ext ? row : cp_ext - 1;
@@ -342,13 +356,18 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
   const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * 128) + sw;     // B tile rows (n)
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
 
-  floatx16 acc[WM][WN];
+  floatx16 acc[FIXED ? 1 : WM][FIXED ? 1 : WN];
+  if constexpr (FIXED) {
+    agpr_reserve_256();
+    agpr_zero256();
+  } else {
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < WN; ++j)
+      for (int j = 0; j < WN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  }
 
   if (nslices > 0 && cp_ext > 0) copy_general(0, 0);
   dma_wait_all();
@@ -378,16 +397,22 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
 #pragma unroll
         for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)((fb0 ^ (uint32_t)((ks + 1) << 5)) + j * 4096);
       }
+      if constexpr (FIXED) __builtin_amdgcn_sched_barrier(0);   // the next fragments are requested before these MFMAs
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
 #pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);  // C^T block: rows n, cols m
-        if ((i & 1) && fcopy) {                       // one 1 KB copy block after every 4 MFMAs
-          __builtin_amdgcn_sched_barrier(0);
-          dma_block_fast(cp_src, cp_off[(2 * ks + (i >> 1)) & 1], cp_dst);
-          cp_src += cp_step;
-          cp_dst += 1024;
-          __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < WN; ++j) {  // C^T block: rows n, cols m
+          if constexpr (FIXED) mfma_acc_fixed_idx<T>(i * WN + j, fb[cu][j], fa[cu][i]);
+          else acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
+          // one 1 KB copy block after every DH_GG_CPI MFMAs until the slice's CPB blocks are out
+          const int mi = (ks * WM + i) * WN + j;
+          if (mi % DH_GG_CPI == DH_GG_CPI - 1 && mi / DH_GG_CPI < CPB && fcopy) {
+            __builtin_amdgcn_sched_barrier(0);
+            dma_block_fast(cp_src, cp_off[(mi / DH_GG_CPI) & 1], cp_dst);
+            cp_src += cp_step;
+            cp_dst += 1024;
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
@@ -397,12 +422,16 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
 
   // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
   T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0;
+  if constexpr (FIXED) mfma_drain();
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     const int m = wm * 32 * WM + 32 * i + c;
-    if (m < a_rext) {
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
+    for (int j = 0; j < WN; ++j) {
+      floatx16 av;
+      if constexpr (FIXED) av = agpr_read16_idx(i * WN + j);   // read by every lane (EXEC is full here)
+      else av = acc[i][j];
+      if (m < a_rext) {
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {
           const int n = wn * 32 * WN + 32 * j + 8 * vb + 4 * hh;
@@ -410,20 +439,21 @@ __global__ void __launch_bounds__(512) grouped_gemm_nt_dma_kernel(const GGParams
             struct alignas(8) Q4 { T v[4]; };
             Q4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e]);
+            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
             *reinterpret_cast<Q4 *>(cg + (int64_t)m * p.ldc + n) = o;
           }
         }
+      }
     }
   }
 }
 
-template <typename T>
+template <typename T, int WVN>
 static int launch_gg_nt_dma(GGParams p, int64_t m_extent, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
   p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
-  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(512), 0, st, p);
+  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T, WVN>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
   return DH_OK;
 }
 
@@ -484,8 +514,8 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.b_group_stride = n * k; p.accumulate = 0;
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % GG_BK == 0 && k < (1ll << 30))
-    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_nt_dma<f16_t>(p, max_rows, (hipStream_t)stream);
+    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t, DH_GG_WVN>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_nt_dma<f16_t, DH_GG_WVN>(p, max_rows, (hipStream_t)stream);
   else
     rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;

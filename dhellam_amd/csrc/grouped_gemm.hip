@@ -24,6 +24,12 @@
 #ifndef DH_GG_CPI
 #define DH_GG_CPI 2
 #endif
+#ifndef DH_GG_BKT
+#define DH_GG_BKT 64
+#endif
+#ifndef DH_GG_NST
+#define DH_GG_NST 2
+#endif
 
 namespace dh {
 
@@ -278,16 +284,31 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 // rate: there copies and MFMAs did not overlap at all).  Its 256 accumulator registers live in the fixed
 // AGPRs a[0:255], block (i, j) at a[16 * (i * WN + j)], named only by assembly MFMAs (as ordinary variables
 // the register allocator moves all of them between the register files around every k slice).
-template <typename T, int WVN>
+// BKT: k depth of a slice (64 or 32); NST: LDS stages.  The copies of slice s + NST - 1 are issued during
+// slice s, so with NST > 2 a copy has more than a whole slice to land before anyone waits for it (with two
+// stages the copies issued late in a slice are waited for almost at once: their latency is exposed).
+template <typename T, int WVN, int BKT, int NST>
 __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GGParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int BM = 256, BN = 256, WM = 4, WN = 8 / WVN, NW = 2 * WVN;
   constexpr bool FIXED = (WVN == 2);
-  constexpr int CPB = 64 / NW;                          // 1 KB copy blocks per wavefront and slice
-  constexpr int TILEB = 256 * GG_BK * (int)sizeof(T);   // one operand tile: 32 KB
+  constexpr int ROWB = BKT * (int)sizeof(T);            // bytes of a tile row (128 or 64)
+  constexpr int CHUNKS = ROWB / 16;                     // 16-byte chunks per row
+  constexpr int RP = 256 / ROWB;                        // rows per 256 bytes: the swizzle is (row / RP) % CHUNKS
+  constexpr int RPB = 1024 / ROWB;                      // rows per 1 KB copy block
+  constexpr int CPB = 2 * 256 / RPB / NW;               // copy blocks per wavefront and slice
+  constexpr int KS = BKT / 16;                          // MFMA k steps per slice
+  constexpr int DIST = NST - 1;                         // copies run this many slices ahead
+  // With four stages a slice is published one slice BEFORE it is used, so its first fragments are
+  // requested before the barrier that ends the previous slice (no LDS latency at the start of a slice).
+  constexpr bool CROSS = NST >= 4;
+  constexpr int WAITD = CROSS ? 2 : 1;                  // the barrier at the end of slice s publishes slice s + WAITD
+  static_assert(!CROSS || KS % 2 == 0, "fragment sets alternate across slices");
+  constexpr int TILEB = 256 * ROWB;                     // one operand tile
   constexpr int STAGEB = 2 * TILEB;                     // A tile, then B tile
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
+  static_assert(NST * STAGEB <= 160 * 1024 && (DIST - 1) * CPB < 64, "LDS budget / wait counter range");
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[NST * STAGEB];
 
   // A contiguous run of tiles per XCD, m fastest (tiles that share a weight panel run together).
   // Cutting the grid into 4 x 8 super-tiles per XCD instead lowers the L2 miss traffic by a third
@@ -320,40 +341,40 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
   const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
   const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (int64_t)n0 * p.ldb;
-  const int nslices = (int)(p.k_dim / GG_BK);
+  const int nslices = (int)(p.k_dim / BKT);
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
   // ---- copies ------------------------------------------------------------------------------------
   const int cp_b = w / (NW / 2);                        // 0: A tile, 1: B tile
-  const int cp_row0 = 8 * CPB * (w % (NW / 2));
+  const int cp_row0 = RPB * CPB * (w % (NW / 2));
   const int cp_ld = (int)(cp_b ? p.ldb : p.lda);
   const int cp_ext = cp_b ? b_rext : a_rext;            // valid rows of the tile
   const T *cp_t = cp_b ? bg : ag;
   const char *cp_g = reinterpret_cast<const char *>(cp_t + (int64_t)cp_row0 * cp_ld);
-  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * 128);
-  const uint32_t cp_step = (uint32_t)(8 * cp_ld) * (uint32_t)sizeof(T);
-  const bool cp_fast = cp_row0 + 8 * CPB <= cp_ext;     // every row this wavefront copies exists
-  const int lr = lane >> 3, lc = lane & 7;
-  uint32_t cp_off[2];                                   // block i of 8 rows: swizzle (row / 2) % 8 = (4 * (i % 2) + lr / 2) % 8
+  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * ROWB);
+  const uint32_t cp_step = (uint32_t)(RPB * cp_ld) * (uint32_t)sizeof(T);
+  const bool cp_fast = cp_row0 + RPB * CPB <= cp_ext;   // every row this wavefront copies exists
+  const int lr = lane / CHUNKS, lc = lane % CHUNKS;
+  uint32_t cp_off[2];                                   // block i: swizzle (row / RP) % CHUNKS = (RPB / RP * (i % 2) + lr / RP) % CHUNKS
 #pragma unroll
   for (int x = 0; x < 2; ++x)
-    cp_off[x] = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)((lc ^ ((4 * x + (lr >> 1)) & 7)) << 4);
+    cp_off[x] = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)((lc ^ ((RPB / RP * x + lr / RP) % CHUNKS)) << 4);
   // general form (tiles at the edge of a group or of n): rows past the end re-read the last valid row
   auto copy_general = [&](uint32_t stage, int slice) {
 #pragma unroll 1
     for (int i = 0; i < CPB; ++i) {
-      int row = cp_row0 + 8 * i + lr;
-      const int f = (row >> 1) & 7;
+      int row = cp_row0 + RPB * i + lr;
+      const int f = (row / RP) % CHUNKS;
       row = row < cp_ext ? row : cp_ext - 1;
-      const T *src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * GG_BK + ((lc ^ f) * 8);
+      const T *src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * BKT + ((lc ^ f) * 8);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                        (__attribute__((address_space(3))) void *)(smem + stage + cp_dst0 + i * 1024), 16, 0, 0);
     }
   };
-  // ---- fragment reads: byte offsets inside a stage; other k steps by XOR, other 32-row blocks by +4 KB ----
-  const uint32_t sw = (uint32_t)((hh ^ ((c >> 1) & 7)) << 4);
-  const uint32_t fa_lane = (uint32_t)((wm * 32 * WM + c) * 128) + sw;             // A tile rows (m)
-  const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * 128) + sw;     // B tile rows (n)
+  // ---- fragment reads: byte offsets inside a stage; other k steps by XOR, other 32-row blocks by + 32 rows ----
+  const uint32_t sw = (uint32_t)((hh ^ ((c / RP) % CHUNKS)) << 4);
+  const uint32_t fa_lane = (uint32_t)((wm * 32 * WM + c) * ROWB) + sw;            // A tile rows (m)
+  const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * ROWB) + sw;    // B tile rows (n)
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
 
   floatx16 acc[FIXED ? 1 : WM][FIXED ? 1 : WN];
@@ -369,33 +390,52 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   }
 
-  if (nslices > 0 && cp_ext > 0) copy_general(0, 0);
+  for (int s = 0; s < DIST; ++s)
+    if (s < nslices && cp_ext > 0) copy_general((uint32_t)(s * STAGEB), s);
   dma_wait_all();
   __syncthreads();
 
+  Frag fa[2][WM], fb[2][WN];
+  if constexpr (CROSS) {
+    if (nslices > 0) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(lds0 + fa_lane + i * 32 * ROWB);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(lds0 + fb_lane + j * 32 * ROWB);
+    }
+  }
+  int st_cur = 0, st_nxt = DIST % NST;                  // stage of slice s, stage of slice s + DIST
 #pragma unroll 1
   for (int s = 0; s < nslices; ++s) {
-    const uint32_t cur = (uint32_t)((s & 1) * STAGEB), nxt = (uint32_t)(((s + 1) & 1) * STAGEB);
-    const bool copy = s + 1 < nslices && cp_ext > 0;
+    const uint32_t cur = (uint32_t)(st_cur * STAGEB), nxt = (uint32_t)(st_nxt * STAGEB);
+    const bool copy = s + DIST < nslices && cp_ext > 0;
     const bool fcopy = copy && cp_fast;
-    const char *cp_src = cp_g + (int64_t)(s + 1) * GG_BK * (int)sizeof(T);
+    const char *cp_src = cp_g + (int64_t)(s + DIST) * ROWB;
     uint32_t cp_dst = lds0 + nxt + cp_dst0;
-    if (copy && !fcopy) copy_general(nxt, s + 1);
+    if (copy && !fcopy) copy_general(nxt, s + DIST);
     uint32_t fa0 = lds0 + cur + fa_lane, fb0 = lds0 + cur + fb_lane;
-    asm volatile("" : "+v"(fa0), "+v"(fb0));            // derive the other addresses here, not ahead of the loop
-    Frag fa[2][WM], fb[2][WN];
+    const uint32_t nst1 = (uint32_t)((st_cur + 1 == NST ? 0 : st_cur + 1) * STAGEB);   // stage of slice s + 1
+    uint32_t fa1 = lds0 + nst1 + fa_lane, fb1 = lds0 + nst1 + fb_lane;
+    asm volatile("" : "+v"(fa0), "+v"(fb0), "+v"(fa1), "+v"(fb1));   // derive the other addresses here, not ahead of the loop
+    if constexpr (!CROSS) {
 #pragma unroll
-    for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(fa0 + i * 4096);
+      for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(fa0 + i * 32 * ROWB);
 #pragma unroll
-    for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(fb0 + j * 4096);
+      for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(fb0 + j * 32 * ROWB);
+    }
 #pragma unroll
-    for (int ks = 0; ks < GG_BK / 16; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
       const int cu = ks & 1, nx = cu ^ 1;
-      if (ks + 1 < GG_BK / 16) {
+      if (ks + 1 < KS) {
 #pragma unroll
-        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)((fa0 ^ (uint32_t)((ks + 1) << 5)) + i * 4096);
+        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)((fa0 ^ (uint32_t)((ks + 1) << 5)) + i * 32 * ROWB);
 #pragma unroll
-        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)((fb0 ^ (uint32_t)((ks + 1) << 5)) + j * 4096);
+        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)((fb0 ^ (uint32_t)((ks + 1) << 5)) + j * 32 * ROWB);
+      } else if (CROSS && s + 1 < nslices) {            // first fragments of the next slice (already published)
+#pragma unroll
+        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)(fa1 + i * 32 * ROWB);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)(fb1 + j * 32 * ROWB);
       }
       if constexpr (FIXED) __builtin_amdgcn_sched_barrier(0);   // the next fragments are requested before these MFMAs
 #pragma unroll
@@ -416,8 +456,18 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
         }
       }
     }
-    dma_wait_all();
-    __syncthreads();   // the next stage has landed, and everyone is done with the current one
+    // slice s + WAITD must have landed; the copies of the DIST - WAITD slices after it may still be in
+    // flight (copies complete in order), unless fewer were issued (tail of k) or this wavefront uses
+    // the general copies
+    if (DIST > WAITD && fcopy) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DIST - WAITD) * CPB) : "memory");
+    else dma_wait_all();
+    st_cur = st_cur + 1 == NST ? 0 : st_cur + 1;
+    st_nxt = st_nxt + 1 == NST ? 0 : st_nxt + 1;
+    // A bare barrier: __syncthreads() would also wait for EVERY outstanding memory operation, i.e. drain
+    // the copies that are meant to stay in flight across it.  What the barrier has to order is covered by
+    // the waits above (this wavefront's copies of the slice being published) and by the fact that a
+    // wavefront's fragment reads of slice s have returned before its last MFMAs of slice s were issued.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
 
   // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
@@ -448,12 +498,12 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   }
 }
 
-template <typename T, int WVN>
+template <typename T, int WVN, int BKT, int NST>
 static int launch_gg_nt_dma(GGParams p, int64_t m_extent, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
   p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
-  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T, WVN>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
+  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T, WVN, BKT, NST>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
   return DH_OK;
 }
 
@@ -513,9 +563,9 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0;
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
-  if (big && k % GG_BK == 0 && k < (1ll << 30))
-    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t, DH_GG_WVN>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_nt_dma<f16_t, DH_GG_WVN>(p, max_rows, (hipStream_t)stream);
+  if (big && k % 64 == 0 && k < (1ll << 30))
+    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_nt_dma<f16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST>(p, max_rows, (hipStream_t)stream);
   else
     rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;

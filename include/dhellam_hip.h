@@ -231,8 +231,11 @@ int dh_grouped_gemm_tn(const void *a, const void *b, void *c,
                        int64_t m, int64_t n, int accumulate, int dtype,
                        void *stream);
 
-/* Plain device-to-device copy kernel (a known-size streaming kernel used to
- * calibrate the profiler's HBM byte counters). */
+/* Plain device-to-device copy kernel: a known-size streaming kernel used to
+ * calibrate the profiler's HBM byte counters, and the local stand-in for the
+ * sequence-parallel all-gather of the reference's communication operator
+ * (dhellam/operators/comm.py, all_gather_into_tensor call sites in
+ * dhellam/core/dstb.py) when one GPU holds the whole sequence. */
 int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
 
 #ifdef __cplusplus

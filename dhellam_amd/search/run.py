@@ -40,7 +40,7 @@ def validate(cfg, weights, mbs, plan_path, steps=10, warmup=3):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--out-dir", default="gpurun_out/search")
+    ap.add_argument("--out-dir", default="search_out")
     ap.add_argument("--seq", type=int, default=4096)
     ap.add_argument("--repeat", type=int, default=5)
     ap.add_argument("--micro-batches", type=int, default=4)

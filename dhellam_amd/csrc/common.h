@@ -53,6 +53,32 @@ template <typename T> __device__ __forceinline__ void stg(T *p, const Vec<T> &x)
   *reinterpret_cast<Vec<T> *>(p) = x;
 }
 
+// Streaming variants for data touched once per kernel.  With NT the access carries the
+// non-temporal hint: such lines do not displace reusable ones in L2 and the HBM rate of a pure
+// streaming kernel rises by 10-30 % once its working set exceeds the 256 MB last-level cache;
+// below that size the hint loses the cache hits a consumer kernel would get, so callers pass
+// NT = stream_hint(bytes touched).
+typedef uint32_t dh_u32x4 __attribute__((ext_vector_type(4)));
+template <bool NT, typename T> __device__ __forceinline__ Vec<T> ldg_s(const T *p) {
+  if constexpr (NT) {
+    const dh_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const dh_u32x4 *>(p));
+    return __builtin_bit_cast(Vec<T>, r);
+  } else {
+    return ldg(p);
+  }
+}
+template <bool NT, typename T> __device__ __forceinline__ void stg_s(T *p, const Vec<T> &x) {
+  if constexpr (NT) {
+    __builtin_nontemporal_store(__builtin_bit_cast(dh_u32x4, x), reinterpret_cast<dh_u32x4 *>(p));
+  } else {
+    stg(p, x);
+  }
+}
+#ifndef DH_STREAM_HINT_BYTES
+#define DH_STREAM_HINT_BYTES (256ll << 20)
+#endif
+static inline bool stream_hint(int64_t bytes_touched) { return bytes_touched > DH_STREAM_HINT_BYTES; }
+
 // ---- wave64 reductions --------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -24,12 +24,24 @@ extern "C" int dh_version(void) { return 100; }
 extern "C" const char *dh_last_error(void) { return dh::g_err; }
 
 // Grid-stride 16-byte copy; the tail (nbytes % 16) is copied bytewise by block 0.
+template <bool NT>
 __global__ void __launch_bounds__(256) copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
                                                    int64_t nvec, const uint8_t *src_tail, uint8_t *dst_tail,
                                                    int ntail) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (; i < nvec; i += stride) dst[i] = src[i];
+  // Each trip a workgroup moves one contiguous 16 KB run: four 16-byte vectors per lane, 4 KB apart.
+  using V = dh::Vec<uint32_t>;
+  const uint32_t *s = reinterpret_cast<const uint32_t *>(src);
+  uint32_t *d = reinterpret_cast<uint32_t *>(dst);
+  const int64_t step = (int64_t)gridDim.x * 1024;
+  for (int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x; i < nvec; i += step) {
+    V v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * 256 < nvec) v[u] = dh::ldg_s<NT>(s + (i + u * 256) * 4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * 256 < nvec) dh::stg_s<NT>(d + (i + u * 256) * 4, v[u]);
+  }
   if (blockIdx.x == 0 && (int)threadIdx.x < ntail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
@@ -42,10 +54,15 @@ extern "C" int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *s
   const int ntail = (int)(nbytes % 16);
   int64_t blocks = dh::cdiv(nvec, 256 * 4);
   if (blocks < 1) blocks = 1;
-  if (blocks > 256 * 16) blocks = 256 * 16;
-  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4 *)src, (uint4 *)dst, nvec, (const uint8_t *)src + nvec * 16,
-                     (uint8_t *)dst + nvec * 16, ntail);
+  if (blocks > 65536) blocks = 65536;
+  if (dh::stream_hint(2 * nbytes))
+    hipLaunchKernelGGL(copy_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, (uint4 *)dst, nvec, (const uint8_t *)src + nvec * 16,
+                       (uint8_t *)dst + nvec * 16, ntail);
+  else
+    hipLaunchKernelGGL(copy_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, (uint4 *)dst, nvec, (const uint8_t *)src + nvec * 16,
+                       (uint8_t *)dst + nvec * 16, ntail);
   DH_LAUNCH_CHECK();
   return DH_OK;
 }

@@ -9,28 +9,38 @@ namespace dh {
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 // One "item" = one 16-byte vector of the output row; rows x fv items in total.
-template <typename T, int UNROLL>
+// Item mapping of the streaming kernels: blocked = a workgroup's UNROLL vectors per lane are 256
+// apart (one contiguous 4 KB * UNROLL run per workgroup per trip); otherwise a grid stride apart.
+#ifndef DH_EW_BLOCKED
+#define DH_EW_BLOCKED 1
+#endif
+#ifndef DH_EW_MAXGRID
+#define DH_EW_MAXGRID 65536
+#endif
+
+template <typename T, int UNROLL, bool NT>
 __global__ void __launch_bounds__(256)
 swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems, int fv) {
   constexpr int N = Vec<T>::N;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t ustride = DH_EW_BLOCKED ? 256 : stride;
+  int64_t it = (int64_t)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
   for (; it < nitems; it += stride * UNROLL) {
     Vec<T> a[UNROLL], b[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nitems) {
         const int64_t r = id / fv;
         const int c = (int)(id - r * fv);
         const T *row = y + r * (2 * (int64_t)fv * N);
-        a[u] = ldg(row + (int64_t)c * N);
-        b[u] = ldg(row + ((int64_t)fv + c) * N);
+        a[u] = ldg_s<NT>(row + (int64_t)c * N);
+        b[u] = ldg_s<NT>(row + ((int64_t)fv + c) * N);
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nitems) {
         Vec<T> o;
 #pragma unroll
@@ -38,35 +48,36 @@ swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems, 
           const float g = to_f(a[u].v[j]);
           o.v[j] = from_f<T>(g * sigmoidf_(g) * to_f(b[u].v[j]));
         }
-        stg(out + id * N, o);
+        stg_s<NT>(out + id * N, o);
       }
     }
   }
 }
 
-template <typename T, int UNROLL>
+template <typename T, int UNROLL, bool NT>
 __global__ void __launch_bounds__(256)
 swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, int64_t nitems, int fv) {
   constexpr int N = Vec<T>::N;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t ustride = DH_EW_BLOCKED ? 256 : stride;
+  int64_t it = (int64_t)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
   for (; it < nitems; it += stride * UNROLL) {
     Vec<T> a[UNROLL], b[UNROLL], gv[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nitems) {
         const int64_t r = id / fv;
         const int c = (int)(id - r * fv);
         const T *row = y + r * (2 * (int64_t)fv * N);
-        a[u] = ldg(row + (int64_t)c * N);
-        b[u] = ldg(row + ((int64_t)fv + c) * N);
-        gv[u] = ldg(g + id * N);
+        a[u] = ldg_s<NT>(row + (int64_t)c * N);
+        b[u] = ldg_s<NT>(row + ((int64_t)fv + c) * N);
+        gv[u] = ldg_s<NT>(g + id * N);
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nitems) {
         const int64_t r = id / fv;
         const int c = (int)(id - r * fv);
@@ -79,8 +90,8 @@ swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restric
           d2.v[j] = from_f<T>(gg * (y1 * s));
         }
         T *row = dy + r * (2 * (int64_t)fv * N);
-        stg(row + (int64_t)c * N, d1);
-        stg(row + ((int64_t)fv + c) * N, d2);
+        stg_s<NT>(row + (int64_t)c * N, d1);
+        stg_s<NT>(row + ((int64_t)fv + c) * N, d2);
       }
     }
   }
@@ -118,30 +129,31 @@ __device__ __forceinline__ float ew_apply(float x, float b, float r, float m) {
   return m * (x + b) + r;
 }
 
-template <typename T, int OP, int UNROLL>
+template <typename T, int OP, int UNROLL, bool NT>
 __global__ void __launch_bounds__(256)
 ew_kernel(const T *__restrict__ x, const T *__restrict__ bias, const T *__restrict__ res, const T *__restrict__ mask,
           T *__restrict__ out, int64_t nvec, int64_t n) {
   constexpr int N = Vec<T>::N;
   const int64_t stride = (int64_t)gridDim.x * 256;
-  int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t ustride = DH_EW_BLOCKED ? 256 : stride;
+  int64_t it = (int64_t)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
   for (; it < nvec; it += stride * UNROLL) {
     Vec<T> xv[UNROLL], bv[UNROLL], rv[UNROLL], mv[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nvec) {
-        xv[u] = ldg(x + id * N);
-        if (OP != EW_GELU) rv[u] = ldg(res + id * N);
+        xv[u] = ldg_s<NT>(x + id * N);
+        if (OP != EW_GELU) rv[u] = ldg_s<NT>(res + id * N);
         if (OP == EW_BMA) {
-          bv[u] = ldg(bias + id * N);
-          if (mask) mv[u] = ldg(mask + id * N);
+          bv[u] = ldg_s<NT>(bias + id * N);
+          if (mask) mv[u] = ldg_s<NT>(mask + id * N);
         }
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * stride;
+      const int64_t id = it + u * ustride;
       if (id < nvec) {
         Vec<T> o;
 #pragma unroll
@@ -150,7 +162,7 @@ ew_kernel(const T *__restrict__ x, const T *__restrict__ bias, const T *__restri
           o.v[j] = from_f<T>(ew_apply<T, OP>(to_f(xv[u].v[j]), OP == EW_BMA ? to_f(bv[u].v[j]) : 0.f,
                                              OP != EW_GELU ? to_f(rv[u].v[j]) : 0.f, m));
         }
-        stg(out + id * N, o);
+        stg_s<NT>(out + id * N, o);
       }
     }
   }
@@ -168,7 +180,7 @@ ew_kernel(const T *__restrict__ x, const T *__restrict__ bias, const T *__restri
 static inline unsigned stream_grid(int64_t items, int per_thread) {
   int64_t b = cdiv(items, 256ll * per_thread);
   if (b < 1) b = 1;
-  if (b > 256 * 32) b = 256 * 32;
+  if (b > DH_EW_MAXGRID) b = DH_EW_MAXGRID;
   return (unsigned)b;
 }
 
@@ -179,9 +191,31 @@ static int launch_ew(const void *x, const void *bias, const void *res, const voi
   bool al = aligned16(x) && aligned16(out) && (!bias || aligned16(bias)) && (!res || aligned16(res)) &&
             (!mask || aligned16(mask));
   const int64_t nvec = al ? n / N : 0;
-  hipLaunchKernelGGL((ew_kernel<T, OP, 4>), dim3(stream_grid(nvec, 4)), dim3(256), 0, st, (const T *)x,
-                     (const T *)bias, (const T *)res, (const T *)mask, (T *)out, nvec, n);
+  const int streams = 2 + (bias ? 1 : 0) + (res ? 1 : 0) + (mask ? 1 : 0);
+#define L(NT)                                                                                                 \
+  hipLaunchKernelGGL((ew_kernel<T, OP, 4, NT>), dim3(stream_grid(nvec, 4)), dim3(256), 0, st, (const T *)x,     \
+                     (const T *)bias, (const T *)res, (const T *)mask, (T *)out, nvec, n)
+  if (stream_hint(n * (int64_t)sizeof(T) * streams)) L(true); else L(false);
+#undef L
   return 0;
+}
+
+// nitems 16-byte output vectors; the forward touches 3 of them per item, the backward 5.
+template <typename T>
+static void launch_swiglu_fwd(const T *y, T *out, int64_t nitems, int fv, hipStream_t st) {
+  const dim3 grid(stream_grid(nitems, 4));
+  if (stream_hint(3 * 16 * nitems))
+    hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4, true>), grid, dim3(256), 0, st, y, out, nitems, fv);
+  else
+    hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4, false>), grid, dim3(256), 0, st, y, out, nitems, fv);
+}
+template <typename T>
+static void launch_swiglu_bwd(const T *g, const T *y, T *dy, int64_t nitems, int fv, hipStream_t st) {
+  const dim3 grid(stream_grid(nitems, 2));
+  if (stream_hint(5 * 16 * nitems))
+    hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2, true>), grid, dim3(256), 0, st, g, y, dy, nitems, fv);
+  else
+    hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2, false>), grid, dim3(256), 0, st, g, y, dy, nitems, fv);
 }
 
 }  // namespace dh
@@ -196,8 +230,7 @@ extern "C" int dh_swiglu_fwd(const void *y, void *out, int64_t rows, int64_t f, 
     constexpr int N = Vec<T>::N;
     if (f % N == 0 && aligned16(y) && aligned16(out) && f / N < (1ll << 31)) {
       const int64_t nitems = rows * (f / N);
-      hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4>), dim3(stream_grid(nitems, 4)), dim3(256), 0, st, (const T *)y,
-                         (T *)out, nitems, (int)(f / N));
+      launch_swiglu_fwd<T>((const T *)y, (T *)out, nitems, (int)(f / N), st);
     } else {
       hipLaunchKernelGGL((swiglu_fwd_scalar_kernel<T>), dim3(stream_grid(rows * f, 4)), dim3(256), 0, st,
                          (const T *)y, (T *)out, rows * f, f);
@@ -218,8 +251,7 @@ extern "C" int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t row
     constexpr int N = Vec<T>::N;
     if (f % N == 0 && aligned16(y) && aligned16(g) && aligned16(dy) && f / N < (1ll << 31)) {
       const int64_t nitems = rows * (f / N);
-      hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2>), dim3(stream_grid(nitems, 2)), dim3(256), 0, st, (const T *)g,
-                         (const T *)y, (T *)dy, nitems, (int)(f / N));
+      launch_swiglu_bwd<T>((const T *)g, (const T *)y, (T *)dy, nitems, (int)(f / N), st);
     } else {
       hipLaunchKernelGGL((swiglu_bwd_scalar_kernel<T>), dim3(stream_grid(rows * f, 4)), dim3(256), 0, st,
                          (const T *)g, (const T *)y, (T *)dy, rows * f, f);

@@ -12,7 +12,7 @@
 
 namespace dh {
 
-template <typename T, int BT, int TPR, int VPT, bool LN>
+template <typename T, int BT, int TPR, int VPT, bool LN, bool NT>
 __global__ void __launch_bounds__(BT)
 norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *__restrict__ beta,
                 T *__restrict__ y, float *__restrict__ mu_out, float *__restrict__ rs_out, int64_t rows,
@@ -45,7 +45,7 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
     for (int i = 0; i < VPT; ++i) {
       const int v = lane + i * TPR;
       if (active && v < nvec) {
-        xv[i] = ldg(xr + (int64_t)v * N);
+        xv[i] = ldg_s<NT>(xr + (int64_t)v * N);
 #pragma unroll
         for (int j = 0; j < N; ++j) {
           const float f = to_f(xv[i].v[j]);
@@ -90,7 +90,7 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
             if (LN) f += to_f(b[i].v[j]);
             o.v[j] = from_f<T>(f);
           }
-          stg(yr + (int64_t)v * N, o);
+          stg_s<NT>(yr + (int64_t)v * N, o);
         }
       }
       if (lane == 0) {
@@ -137,7 +137,7 @@ norm_fwd_generic_kernel(const T *__restrict__ x, const T *__restrict__ gamma, co
 }
 
 // Backward main pass.  part: fp32 [2][gridDim.x][cols] (dgamma rows, then dbeta rows).
-template <typename T, int BT, int TPR, int VPT, bool LN>
+template <typename T, int BT, int TPR, int VPT, bool LN, bool NT>
 __global__ void __launch_bounds__(BT)
 norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *__restrict__ mu,
                 const float *__restrict__ rsigma, const T *__restrict__ gamma, const T *__restrict__ add_to_dx,
@@ -172,8 +172,8 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
     for (int i = 0; i < VPT; ++i) {
       const int v = lane + i * TPR;
       if (row < rows && v < nvec) {
-        xn[i] = ldg(x + row * cols + (int64_t)v * N);
-        dn[i] = ldg(dy + row * cols + (int64_t)v * N);
+        xn[i] = ldg_s<NT>(x + row * cols + (int64_t)v * N);
+        dn[i] = ldg_s<NT>(dy + row * cols + (int64_t)v * N);
       }
     }
   };
@@ -224,7 +224,7 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
         const int v = lane + i * TPR;
         if (v < nvec) {
           Vec<T> o, r;
-          if (add_to_dx) r = ldg(add_to_dx + row * cols + (int64_t)v * N);
+          if (add_to_dx) r = ldg_s<NT>(add_to_dx + row * cols + (int64_t)v * N);
 #pragma unroll
           for (int j = 0; j < N; ++j) {
             const float xh = (to_f(xv[i].v[j]) - mean) * rs;
@@ -233,7 +233,7 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
             if (add_to_dx) f += to_f(r.v[j]);
             o.v[j] = from_f<T>(f);
           }
-          stg(dx + row * cols + (int64_t)v * N, o);
+          stg_s<NT>(dx + row * cols + (int64_t)v * N, o);
         }
       }
     }
@@ -493,9 +493,14 @@ static int launch_fwd(const NormPlan &p, const T *x, const T *gamma, const T *be
   const int rpb = p.tpr == 64 ? 4 : 1;
   int64_t nb = cdiv(rows, rpb);
   if (nb > 256 * 16) nb = 256 * 16;
+  const bool nt = stream_hint(2 * rows * cols * (int64_t)sizeof(T));
+#define L2(BT, TPR, VPT, NT)                                                                                 \
+  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT), 0, st, x, gamma,  \
+                     beta, y, mu, rs, rows, (int)cols, eps, shift)
 #define L(BT, TPR, VPT)                                                                                      \
-  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN>), dim3((unsigned)nb), dim3(BT), 0, st, x, gamma, beta, \
-                     y, mu, rs, rows, (int)cols, eps, shift)
+  do {                                                                                                       \
+    if (nt) L2(BT, TPR, VPT, true); else L2(BT, TPR, VPT, false);                                             \
+  } while (0)
   if (p.tpr == 64) {
     if (p.vpt == 1) L(256, 64, 1); else if (p.vpt == 2) L(256, 64, 2); else L(256, 64, 4);
   } else if (p.tpr == 256) {
@@ -504,6 +509,7 @@ static int launch_fwd(const NormPlan &p, const T *x, const T *gamma, const T *be
     if (p.vpt == 1) L(1024, 1024, 1); else L(1024, 1024, 2);
   }
 #undef L
+#undef L2
   return 0;
 }
 
@@ -520,10 +526,15 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
     hipLaunchKernelGGL((norm_bwd_generic_wgrad_kernel<T, LN>), dim3((unsigned)cdiv(cols, 64), (unsigned)nb),
                        dim3(256), 0, st, dy, x, mu, rs, part, rows, cols, rpc);
   } else {
-#define L(BT, TPR, VPT)                                                                                      \
-  hipLaunchKernelGGL((norm_bwd_kernel<T, BT, TPR, VPT, LN>), dim3((unsigned)nb), dim3(BT),                        \
+    const bool nt = stream_hint((add ? 4 : 3) * rows * cols * (int64_t)sizeof(T));
+#define L2(BT, TPR, VPT, NT)                                                                                 \
+  hipLaunchKernelGGL((norm_bwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT),                    \
                      (TPR == 64 ? 4 * 64 * VPT * (16 / sizeof(T)) * sizeof(float) : 0), st, dy, x, mu, rs, gamma, \
                      add, dx, part, rows, (int)cols, shift)
+#define L(BT, TPR, VPT)                                                                                      \
+  do {                                                                                                       \
+    if (nt) L2(BT, TPR, VPT, true); else L2(BT, TPR, VPT, false);                                             \
+  } while (0)
     if (p.tpr == 64) {
       if (p.vpt == 1) L(256, 64, 1); else if (p.vpt == 2) L(256, 64, 2); else L(256, 64, 4);
     } else if (p.tpr == 256) {
@@ -532,6 +543,7 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
       if (p.vpt == 1) L(1024, 1024, 1); else L(1024, 1024, 2);
     }
 #undef L
+#undef L2
   }
   if (cols % 4 == 0)
     hipLaunchKernelGGL((norm_bwd_finalize_kernel<T, LN>), dim3((unsigned)cdiv(cols, 64)), dim3(256), 0, st, part,

@@ -11,6 +11,12 @@
 // tile.  fp32 scores are scaled inside the exp2 argument (one FMA), the running
 // output is rescaled only when some row's maximum actually moved.
 #include "mma.h"
+#ifndef DH_FWD_RESCALE_LOG2
+#define DH_FWD_RESCALE_LOG2 8
+#endif
+#ifndef DH_FWD_KAHEAD
+#define DH_FWD_KAHEAD 2
+#endif
 #ifndef DH_FWD_LAG
 #define DH_FWD_LAG true
 #endif
@@ -233,7 +239,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
   constexpr int SLOTB = SLOT * (int)sizeof(T);
   constexpr int BPT = BN / 4;                     // 1 KB copy blocks per tile
   static_assert(SPLIT * 2 * BPT == 64, "eight copy blocks per wavefront and iteration");
-  constexpr int NV = LAG ? 3 : 2;                 // V slots
+  constexpr int NV = 3;                           // V slots: read one iteration late, copied one ahead
   __shared__ __attribute__((aligned(1024))) T sAll[(2 + NV) * SLOT];   // K slots 0..1, then the V slots
 
   const int b = blockIdx.y;
@@ -365,25 +371,127 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
         ad[2 * t] = va ^ (uint32_t)(t << 6);
         ad[2 * t + 1] = vb ^ (uint32_t)(t << 6);
       }
+      short4v f[2][8];
+      auto rd = [&](int st) {
+        if (st == 0) lds_read_tr8<0>(f[st & 1], ad);
+        else if (st == 1) lds_read_tr8<16 * 256>(f[st & 1], ad);
+        else if (st == 2) lds_read_tr8<32 * 256>(f[st & 1], ad);
+        else lds_read_tr8<48 * 256>(f[st & 1], ad);
+      };
+      rd(0);
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
-        short4v f[8];
-        if (s == 0) lds_read_tr8<0>(f, ad);
-        else if (s == 1) lds_read_tr8<16 * 256>(f, ad);
-        else if (s == 2) lds_read_tr8<32 * 256>(f, ad);
-        else lds_read_tr8<48 * 256>(f, ad);
-        lds_wait<4>(f[0], f[1], f[2], f[3]);
-        O[0] = M::mma(frag_join<T>(f[0], f[1]), Pb[s], O[0]);
-        O[1] = M::mma(frag_join<T>(f[2], f[3]), Pb[s], O[1]);
+        short4v(&g)[8] = f[s & 1];
+        if (s + 1 < NS) {
+          rd(s + 1);
+          lds_wait<12>(g[0], g[1], g[2], g[3]);
+        } else {
+          lds_wait<4>(g[0], g[1], g[2], g[3]);
+        }
+        O[0] = M::mma(frag_join<T>(g[0], g[1]), Pb[s], O[0]);
+        O[1] = M::mma(frag_join<T>(g[2], g[3]), Pb[s], O[1]);
         if (NS == 2) DH_FWD_COPY(4 + 2 * s);
-        lds_wait<0>(f[4], f[5], f[6], f[7]);
-        O[2] = M::mma(frag_join<T>(f[4], f[5]), Pb[s], O[2]);
-        O[3] = M::mma(frag_join<T>(f[6], f[7]), Pb[s], O[3]);
+        if (s + 1 < NS) lds_wait<8>(g[4], g[5], g[6], g[7]);
+        else lds_wait<0>(g[4], g[5], g[6], g[7]);
+        O[2] = M::mma(frag_join<T>(g[4], g[5]), Pb[s], O[2]);
+        O[3] = M::mma(frag_join<T>(g[6], g[7]), Pb[s], O[3]);
         if (NS == 2) DH_FWD_COPY(5 + 2 * s);
         else DH_FWD_COPY(4 + s);
       }
     };
 
+    // S^T = K Q^T for this wavefront's tile of the current iteration; copy blocks 0..3 go out between the MFMAs.
+    floatx16 S[NB];
+    auto qk = [&](uint32_t k_slot) {
+      uint32_t kb = k_slot + kb_lane;
+      asm volatile("" : "+v"(kb));
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) S[nb][v] = 0.f;
+      // K fragments are fetched in pairs, DH_FWD_KAHEAD pairs ahead of the MFMAs that consume them.
+      constexpr int NP = NB * (D / 16) / 2, AH = DH_FWD_KAHEAD;
+      int4v ka[2 * (AH + 1)];
+      auto issue = [&](int pr) {
+        const int i = 2 * pr, nb = i / (D / 16), ks = i % (D / 16), q = 2 * (pr % (AH + 1));
+        if (nb == 0) {
+          lds_read128<0>(ka[q], kb ^ (uint32_t)(ks << 5));
+          lds_read128<0>(ka[q + 1], kb ^ (uint32_t)((ks + 1) << 5));
+        } else {
+          lds_read128<32 * 256>(ka[q], kb ^ (uint32_t)(ks << 5));
+          lds_read128<32 * 256>(ka[q + 1], kb ^ (uint32_t)((ks + 1) << 5));
+        }
+      };
+#pragma unroll
+      for (int pr = 0; pr < AH; ++pr) issue(pr);
+#pragma unroll
+      for (int pr = 0; pr < NP; ++pr) {
+        const int i = 2 * pr, nb = i / (D / 16), ks = i % (D / 16), a = 2 * (pr % (AH + 1));
+        if (pr + AH < NP) issue(pr + AH);
+        const int newer = (pr + AH < NP ? AH : NP - 1 - pr) * 2;     // reads issued after this pair
+        if (newer == 0) lds_wait<0>(ka[a], ka[a + 1]);
+        else if (newer == 2) lds_wait<2>(ka[a], ka[a + 1]);
+        else if (newer == 4) lds_wait<4>(ka[a], ka[a + 1]);
+        else lds_wait<6>(ka[a], ka[a + 1]);
+        S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a]), Qf[ks], S[nb]);
+        S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a + 1]), Qf[ks + 1], S[nb]);
+        if (pr % NB == NB - 1) DH_FWD_COPY(pr / NB);      // copy blocks 0..3
+      }
+    };
+
+    // Online softmax of S (tile starting at key n0): masks, moves the running maximum when needed, leaves
+    // P^T in Pb.
+    auto softmax = [&](int n0) {
+      const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+      if (need_mask) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int kv = n0 + nb * 32 + acc_row(v, hh);
+            if (kv >= sk || (causal && kv > row_q)) S[nb][v] = -INFINITY;
+          }
+      }
+      float mx = S[0][0];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      // Lazy rescale: the running maximum is only a reference point for the exponentials, so it may lag
+      // the true maximum.  It is moved (and O, l rescaled) only when some row of the wavefront has grown
+      // past it by more than DH_FWD_RESCALE_LOG2 binades; until then P <= 2^DH_FWD_RESCALE_LOG2, which
+      // fp32 sums and 16-bit P hold without loss, and out = O / l and lse = m + log l are unchanged.
+      const float m_new = fmaxf(m_run, mx);
+      if (__any((m_new - m_run) * scale_log2 > (float)DH_FWD_RESCALE_LOG2)) {
+        const float alpha = fast_exp2((m_run - m_new) * scale_log2);
+        l_run *= alpha;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) O[t][v] *= alpha;
+        m_run = m_new;
+      }
+      const float mc = m_run * scale_log2;
+      float ps = 0.f;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        float pvv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          pvv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
+          ps += pvv[j];
+        }
+        Pb[s] = frag_pack<T>(pvv);
+      }
+      l_run += ps;
+    };
+
+    // Every wavefront runs P V one iteration late.  The first wavefront of a SIMD orders an iteration as
+    // [P V of the previous tile, S of this tile | softmax of this tile], the second one (lag) as
+    // [softmax of the previous tile | P V of the previous tile, S of this tile]: whenever one of them is in
+    // its matrix phase the other is in its softmax.
+    int n0_prev = 0;
 #pragma unroll 1
     for (int it = 0; it < niter; ++it) {
       const int nit = it + 1;
@@ -399,94 +507,15 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       const int n0 = tile_g * BN;
       const bool act = tile_g < ntiles && !(causal && n0 > wrow0 + 31);
 
-      // lagging wavefronts: last iteration's P V first; their copy blocks 4..7 go out there
-      if (lag) {
-        if (act_prev) pv(v_prev);
-        else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
-      }
-      if (act) {
-        uint32_t kb = k_cur + kb_lane;
-        asm volatile("" : "+v"(kb));
-        floatx16 S[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) S[nb][v] = 0.f;
-        {
-          // K fragments are fetched in pairs, one pair ahead of the MFMAs that consume them.
-          constexpr int NP = NB * (D / 16) / 2;
-          int4v ka[4];
-          lds_read128<0>(ka[0], kb);
-          lds_read128<0>(ka[1], kb ^ 32u);
-#pragma unroll
-          for (int pr = 0; pr < NP; ++pr) {
-            const int i = 2 * pr, nb = i / (D / 16), ks = i % (D / 16);
-            const int a = 2 * (pr & 1), bq = 2 * ((pr + 1) & 1);
-            if (pr + 1 < NP) {
-              const int i2 = i + 2, nb2 = i2 / (D / 16), ks2 = i2 % (D / 16);
-              if (nb2 == 0) {
-                lds_read128<0>(ka[bq], kb ^ (uint32_t)(ks2 << 5));
-                lds_read128<0>(ka[bq + 1], kb ^ (uint32_t)((ks2 + 1) << 5));
-              } else {
-                lds_read128<32 * 256>(ka[bq], kb ^ (uint32_t)(ks2 << 5));
-                lds_read128<32 * 256>(ka[bq + 1], kb ^ (uint32_t)((ks2 + 1) << 5));
-              }
-              lds_wait<2>(ka[a], ka[a + 1]);
-            } else {
-              lds_wait<0>(ka[a], ka[a + 1]);
-            }
-            S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a]), Qf[ks], S[nb]);
-            S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a + 1]), Qf[ks + 1], S[nb]);
-            if (pr % NB == NB - 1) DH_FWD_COPY(pr / NB);      // copy blocks 0..3
-          }
-        }
-        const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
-        if (need_mask) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              const int kv = n0 + nb * 32 + acc_row(v, hh);
-              if (kv >= sk || (causal && kv > row_q)) S[nb][v] = -INFINITY;
-            }
-        }
-        float mx = S[0][0];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        if (__any(m_new > m_run)) {
-          const float alpha = fast_exp2((m_run - m_new) * scale_log2);
-          l_run *= alpha;
-#pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) O[t][v] *= alpha;
-        }
-        m_run = m_new;
-        const float mc = m_new * scale_log2;
-        float ps = 0.f;
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-          float pvv[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            pvv[j] = fast_exp2(S[s >> 1][8 * (s & 1) + j] * scale_log2 - mc);
-            ps += pvv[j];
-          }
-          Pb[s] = frag_pack<T>(pvv);
-        }
-        l_run += ps;
-      } else {
-        DH_FWD_COPY(0); DH_FWD_COPY(1); DH_FWD_COPY(2); DH_FWD_COPY(3);
-      }
-      if (!lag) {
-        if (act) pv(v_cur);
-        else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
-      }
+      if (lag && act_prev) softmax(n0_prev);
+      if (act_prev) pv(v_prev);
+      else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
+      if (act) qk(k_cur);
+      else { DH_FWD_COPY(0); DH_FWD_COPY(1); DH_FWD_COPY(2); DH_FWD_COPY(3); }
+      if (!lag && act) softmax(n0);
+
       act_prev = act;
+      n0_prev = n0;
       v_prev = v_cur;
       v_cur = v_nxt;
       { const uint32_t t = k_cur; k_cur = k_nxt; k_nxt = t; }
@@ -494,7 +523,8 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       __syncthreads();   // the next slots have landed, and everyone is done with the ones they replace next
     }
     fcopy = false;
-    if (lag && act_prev) pv(v_prev);
+    if (lag && act_prev) softmax(n0_prev);
+    if (act_prev) pv(v_prev);
 #undef DH_FWD_COPY
     __syncthreads();     // everyone is done with the tiles: the area is reused for the exchange below
 

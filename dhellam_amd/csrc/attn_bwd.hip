@@ -19,13 +19,21 @@
 // needs no fp32 dQ accumulator in memory and no atomics.
 #include "mma.h"
 
+#ifndef DH_DKV8
+#define DH_DKV8 1
+#endif
+#ifndef DH_DKV8_GROUP
+#define DH_DKV8_GROUP 2
+#endif
+
 namespace dh {
 
 struct AttnBwdParams {
   const void *dout, *q, *k, *v;
   const float *lse, *delta;
-  const float *ld2;          // fp32 [2][plane]: lse * log2(e), then delta, each [batch][hq][max_sq] (d = 128 kernels)
+  const float *ld2;          // fp32 [2][plane]: lse * log2(e), then delta, each [batch][hq][ld2_pitch] (d = 128 kernels)
   int64_t ld2_plane;         // elements between the two planes
+  int ld2_pitch;             // max_sq rounded up to 32: every 32-row query tile of a head is one aligned 128-byte run
   void *dq, *dk, *dv;
   float *dk_part, *dv_part;  // fp32 [hsplit][total_k][hk][d] when hsplit > 1
   const int32_t *cu_q, *cu_k;
@@ -40,7 +48,7 @@ struct AttnBwdParams {
 template <typename T>
 __global__ void __launch_bounds__(256)
 attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *__restrict__ delta,
-                  const float *__restrict__ lse, float *__restrict__ ld2, int64_t ld2_plane,
+                  const float *__restrict__ lse, float *__restrict__ ld2, int64_t ld2_plane, int ld2_pitch,
                   const int32_t *__restrict__ cu_q, int max_sq, int hq, int d, int lanes_per, int64_t do_stride,
                   int64_t o_stride) {
   constexpr int N = Vec<T>::N;
@@ -64,8 +72,9 @@ attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *
       const int64_t at = ((int64_t)b * hq + h) * max_sq + i;
       delta[at] = s;
       if (ld2) {             // the copy the d = 128 kernels stream: lse in exp2 units next to delta
-        ld2[at] = lse[at] * 1.4426950408889634f;
-        ld2[ld2_plane + at] = s;
+        const int64_t a2 = ((int64_t)b * hq + h) * ld2_pitch + i;
+        ld2[a2] = lse[at] * 1.4426950408889634f;
+        ld2[ld2_plane + a2] = s;
       }
     }
   }
@@ -832,7 +841,7 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
         if (tl < ntq) {
           int ir = i_begin + tl * BM + (lane & 31);
           ir = ir < sq ? ir : sq - 1;
-          const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + h) * p.max_sq + ir;
+          const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + h) * p.ld2_pitch + ir;
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                            (__attribute__((address_space(3))) void *)(sAll + st + w * SLOT + 2 * QT), 4, 0, 0);
         }
@@ -880,7 +889,7 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
           const int rl = i_begin + tl * BM;
           if (tl < ntq) {
             if (rl + BM <= sq) {
-              const char *src = ld_g + (((int64_t)b * p.hq + hn) * p.max_sq + rl) * 4;
+              const char *src = ld_g + (((int64_t)b * p.hq + hn) * p.ld2_pitch + rl) * 4;
               const uint32_t dst = lds0 + (uint32_t)((nxt_el + w * SLOT + 2 * QT) * (int)sizeof(T));
               asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
                            :
@@ -889,7 +898,7 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
             } else {
               int ir = rl + (lane & 31);
               ir = ir < sq ? ir : sq - 1;
-              const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + hn) * p.max_sq + ir;
+              const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + hn) * p.ld2_pitch + ir;
               __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                                (__attribute__((address_space(3))) void *)(sAll + nxt_el + w * SLOT + 2 * QT), 4, 0, 0);
             }
@@ -1064,11 +1073,338 @@ __global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdPar
   }
 }
 
+// dK/dV with eight wavefronts: 2 key row groups (32 rows each) x 4 query splits, i.e. two wavefronts per
+// SIMD whose matrix and softmax phases interleave.  To fit that into 256 registers per wavefront the K / V
+// tiles of the workgroup live in LDS (read as row fragments every iteration) instead of registers, the
+// accumulators are ordinary variables, and lse / delta of a query tile come straight from memory (one
+// aligned 128-byte run per tile and plane), loaded one iteration ahead.  LDS: two stages of four Q + dO tile
+// pairs (128 KB) + the K and V tiles (32 KB).  The splits' partial dK/dV are added through LDS in a fixed
+// order.  Causal pairing of key tiles, head-group splitting and the copy scheme are those of the
+// four-wavefront kernel above.
+template <typename T>
+__global__ void __launch_bounds__(512) attn_bwd_dkv8_d128_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int D = 128, KG = 2, QSPLIT = 4, BN = 32 * KG, BM = 32;
+  constexpr int QT = BM * D;                          // elements of one Q (or dO) tile
+  constexpr int QTB = QT * (int)sizeof(T);
+  constexpr int SLOT = 2 * QT;                        // Q tile, dO tile
+  constexpr int SLOTB = SLOT * (int)sizeof(T);
+  constexpr int STAGE = QSPLIT * SLOT;
+  constexpr int STAGEB = STAGE * (int)sizeof(T);
+  constexpr int KVT = BN * D;                         // elements of the K (or V) tile
+  constexpr int KVTB = KVT * (int)sizeof(T);
+  __shared__ __attribute__((aligned(1024))) T sAll[2 * STAGE + 2 * KVT];
+
+  const int b = blockIdx.y;
+  const int G = p.hk * p.hsplit;
+  int hg, px;
+  xcd_group_item(blockIdx.x, G, gridDim.x / G, hg, px);
+  const int hkv = hg / p.hsplit, hs = hg % p.hsplit;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int nkt = (sk + BN - 1) / BN;
+  const int causal = p.causal;
+  const int q_stride = (int)p.q_stride, do_stride = (int)p.do_stride;
+  const float scale_log2 = p.scale_log2;
+  int kt[2], nk;
+  if (causal) {
+    const int pair = px;
+    if (2 * pair >= nkt) return;
+    kt[0] = pair; kt[1] = nkt - 1 - pair;             // heavy (early keys) first
+    nk = (kt[0] == kt[1]) ? 1 : 2;
+  } else {
+    if (px >= nkt) return;
+    kt[0] = px; kt[1] = 0; nk = 1;
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
+  const int c = lane & 31, hh = lane >> 5;
+  const int kg = w % KG, qs = w / KG;
+  const int ratio = p.hq / p.hk;
+  const int hper = ratio / p.hsplit;
+  const int h_first = hkv * ratio + hs * hper;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)sAll;
+  const uint32_t ldsKV = lds0 + 2u * STAGEB;
+
+  // ---- copies: wavefront w brings one whole tile per iteration: Q (w even) or dO (w odd) of split w / 2 ----
+  CopyLane cl0;
+  cl0.l16 = lane & 15;
+  cl0.lrow = lane >> 4;
+  const int cp_slot = w >> 1, cp_do = w & 1;
+  const int cp_stride = cp_do ? do_stride : q_stride;
+  const T *cp_gt = reinterpret_cast<const T *>(cp_do ? p.dout : p.q) + (int64_t)q0 * cp_stride;
+  const char *cp_g = reinterpret_cast<const char *>(cp_gt);
+  const int cp_dst0 = cp_slot * SLOT + cp_do * QT;    // elements inside a stage
+  const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
+  uint32_t cp_off[4];                                 // tiles use swz(row): chunk ^= 4 * (row % 4) + (row / 4) % 4
+  {
+    const uint32_t rowb = (uint32_t)(cl0.lrow * cp_stride) * (uint32_t)sizeof(T);
+    const uint32_t chunk = (uint32_t)(cl0.l16 ^ (4 * cl0.lrow)) << 4;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
+  }
+  // ---- fragment reads: lane byte offsets inside a slot; other fragments by XOR / immediate offset ----
+  const int r = lane & 15;
+  const uint32_t rf_lane = (uint32_t)(qs * SLOTB + c * 256 + ((hh ^ swz(c)) << 4));   // row c, chunk hh
+  const uint32_t kv_lane = (uint32_t)((kg * 32 + c) * 256 + ((hh ^ swz(c)) << 4));    // K / V row of this lane
+  const int ta_x = 4 * (r >> 2) + hh;                 // transpose reads: swz of rows 4*hh + r/4 (+8)
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  const uint32_t t_row = (uint32_t)(qs * SLOTB + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
+  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
+  typedef __attribute__((address_space(3))) const Frag *lds_frag;
+  typedef short4v __attribute__((address_space(3))) *lds_tr;
+
+  for (int ki = 0; ki < nk; ++ki) {
+    const int j0 = kt[ki] * BN;
+    const int jw0 = j0 + 32 * kg;
+    const int jrow = jw0 + c;
+    // this workgroup's K and V tiles -> LDS: wavefronts 0, 1 bring the two halves of K, wavefronts 2, 3 of V
+    if (w < 4) {
+      const int half = w & 1, isv = w >> 1;
+      const T *gsrc = reinterpret_cast<const T *>(isv ? p.v : p.k) + (int64_t)k0 * (isv ? p.v_stride : p.k_stride) +
+                      (int64_t)hkv * D;
+      dma_tile32_general<T, 8>(sAll + 2 * STAGE + isv * KVT + half * 32 * D, gsrc, (int)(isv ? p.v_stride : p.k_stride), 1,
+                               j0 + 32 * half, 0, sk, cl0);
+    }
+    floatx16 dKt[D / 32], dVt[D / 32];
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        dKt[t][v] = 0.f;
+        dVt[t][v] = 0.f;
+      }
+    const int i_begin = causal ? (j0 / BM) * BM : 0;
+    const int ntq = i_begin < sq ? (sq - i_begin + BM - 1) / BM : 0;
+    const int it_per_head = (ntq + QSPLIT - 1) / QSPLIT;
+    const int niter = it_per_head * hper;
+
+    auto issue_general = [&](int st, int g, int ti) {
+      const int h = h_first + g;
+      const int tq = ti * QSPLIT + cp_slot;
+      if (tq < ntq)
+        dma_tile32_general<T, 8>(sAll + st + cp_dst0, cp_gt + (int64_t)h * D, cp_stride, 1, i_begin + tq * BM, 0, sq, cl0);
+    };
+    // lse (exp2 units) and delta of the rows 8*vb + 4*hh + e of this wavefront's query tile in iteration (g, ti)
+    floatx4 l4[4], d4[4];
+    auto load_ld = [&](int g, int ti) {
+      const int tq = ti * QSPLIT + qs;
+      if (tq < ntq) {
+        const float *src = p.ld2 + ((int64_t)b * p.hq + (h_first + g)) * p.ld2_pitch + (i_begin + tq * BM) + 4 * hh;
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          l4[vb] = *reinterpret_cast<const floatx4 *>(src + 8 * vb);
+          d4[vb] = *reinterpret_cast<const floatx4 *>(src + p.ld2_plane + 8 * vb);
+        }
+      }
+    };
+#pragma unroll
+    for (int vb = 0; vb < 4; ++vb)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        l4[vb][e] = 0.f;
+        d4[vb][e] = 0.f;
+      }
+
+    if (niter > 0) {
+      issue_general(0, 0, 0);
+      load_ld(0, 0);
+    }
+    dma_wait_all();
+    __syncthreads();
+
+    const char *cp_src = nullptr;
+    uint32_t cp_dst = 0;
+    bool fcopy = false;
+#define DH_DKV_COPY(i)                                                                                  \
+    do {                                                                                                \
+      if (fcopy) {                                                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+        dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                                \
+        cp_src += cp_step;                                                                              \
+        cp_dst += 1024;                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                              \
+      }                                                                                                 \
+    } while (0)
+
+    int g = 0, ti = 0;                                // head and step of iteration it
+#pragma unroll 1
+    for (int it = 0; it < niter; ++it) {
+      int gn = g, tn = ti + 1;                        // ... and of iteration it + 1
+      if (tn == it_per_head) { tn = 0; ++gn; }
+      const bool have_next = it + 1 < niter;
+      const uint32_t cur = lds0 + (uint32_t)((it & 1) * STAGEB);
+      const int nxt_el = ((it + 1) & 1) * STAGE;
+      {
+        const int hn = h_first + gn;
+        const int tq = tn * QSPLIT + cp_slot;
+        const int row0 = i_begin + tq * BM;
+        const bool copy = have_next && tq < ntq;
+        fcopy = copy && row0 + BM <= sq;
+        cp_src = cp_g + ((int64_t)row0 * cp_stride + (int64_t)hn * D) * (int)sizeof(T);
+        cp_dst = lds0 + (uint32_t)((nxt_el + cp_dst0) * (int)sizeof(T));
+        if (copy && !fcopy)
+          dma_tile32_general<T, 8>(sAll + nxt_el + cp_dst0, cp_gt + (int64_t)hn * D, cp_stride, 1, row0, 0, sq, cl0);
+      }
+      const int tq = ti * QSPLIT + qs;
+      const int i0 = i_begin + tq * BM;
+      const bool act = tq < ntq && !(causal && i0 + BM - 1 < jw0);
+      if (act) {
+        uint32_t qb = cur + rf_lane, ta = cur + ta_lane, tb = cur + tb_lane, kb = ldsKV + kv_lane;
+        asm volatile("" : "+v"(qb), "+v"(ta), "+v"(tb), "+v"(kb));   // derive the other addresses here
+        floatx16 S, dP;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          S[v] = 0.f;
+          dP[v] = 0.f;
+        }
+        // S = Q K^T and dP = dO V^T with the key index on lanes
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+          const uint32_t aq = qb ^ (uint32_t)(ks << 5), ak = kb ^ (uint32_t)(ks << 5);
+          S = M::mma(*(lds_frag)(aq), *(lds_frag)(ak), S);
+          dP = M::mma(*(lds_frag)(aq + QTB), *(lds_frag)(ak + KVTB), dP);
+          if (ks % DH_DKV8_GROUP == DH_DKV8_GROUP - 1) __builtin_amdgcn_sched_barrier(0);   // bounds the fragments in flight
+        }
+        const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
+        Frag Pb[2], dSb[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          float pv[8], dsv[8];
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int vb = 2 * s + u;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int v = 4 * vb + e;
+              float pe = fast_exp2(S[v] * scale_log2 - l4[vb][e]);
+              float de = pe * (dP[v] - d4[vb][e]);
+              if (need_mask) {
+                const int i = i0 + acc_row(v, hh);
+                if (i >= sq || (causal && jrow > i)) {
+                  pe = 0.f;
+                  de = 0.f;          // rows past the sequence end carry unwritten lse / delta
+                }
+              }
+              pv[4 * u + e] = pe;
+              dsv[4 * u + e] = de;
+            }
+          }
+          Pb[s] = frag_pack<T>(pv);
+          dSb[s] = frag_pack<T>(dsv);
+        }
+        if (have_next) load_ld(gn, tn);               // next tile's lse / delta, in flight across the barrier
+        // dV^T += dO^T P and dK^T += Q^T dS; the eight copy blocks of this wavefront go out in between
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256) + QTB;
+            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256) + QTB;
+            const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
+            const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
+            dVt[t] = M::mma(frag_join<T>(x0, x1), Pb[s], dVt[t]);
+            if (t & 1) DH_DKV_COPY(4 * s + (t >> 1));
+          }
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
+            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
+            const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
+            const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
+            dKt[t] = M::mma(frag_join<T>(x0, x1), dSb[s], dKt[t]);
+            if (t & 1) DH_DKV_COPY(4 * s + 2 + (t >> 1));
+          }
+        }
+      } else {
+        if (have_next) load_ld(gn, tn);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) DH_DKV_COPY(i);
+      }
+      g = gn;
+      ti = tn;
+      dma_wait_all();
+      __syncthreads();   // the next stage has landed, and everyone is done with the current one
+    }
+#undef DH_DKV_COPY
+
+    // add the splits' partial sums through LDS in a fixed order: (0 += 2, 1 += 3), then 0 += 1.
+    // Slot (split, key group) holds dK then dV, 16 KB each, in the stage area.
+    static_assert(2 * STAGE * sizeof(T) >= (size_t)2 * KG * 2 * 4096 * sizeof(float), "exchange area");
+    typedef __attribute__((address_space(3))) float *lds_f;
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+      const int senders_from = round == 0 ? 2 : 1, senders_to = round == 0 ? 4 : 2;
+      if (qs >= senders_from && qs < senders_to) {
+        uint32_t xb = lds0 + (uint32_t)((((qs - senders_from) * KG + kg) * 2 * 4096 + lane) * 4);
+        asm volatile("" : "+v"(xb));       // one base register + immediate offsets, computed here
+        lds_f dst = (lds_f)(xb);
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            dst[(t * 16 + v) * 64] = dKt[t][v];
+            dst[4096 + (t * 16 + v) * 64] = dVt[t][v];
+          }
+      }
+      __syncthreads();
+      if (qs < senders_from) {
+        uint32_t xb = lds0 + (uint32_t)(((qs * KG + kg) * 2 * 4096 + lane) * 4);
+        asm volatile("" : "+v"(xb));
+        lds_f src = (lds_f)(xb);
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            dKt[t][v] += src[(t * 16 + v) * 64];
+            dVt[t][v] += src[4096 + (t * 16 + v) * 64];
+          }
+      }
+      __syncthreads();
+    }
+    if (qs == 0 && jrow < sk) {
+      if (p.hsplit == 1) {
+        T *dkp = reinterpret_cast<T *>(p.dk) + (int64_t)(k0 + jrow) * p.dk_stride + (int64_t)hkv * D;
+        T *dvp = reinterpret_cast<T *>(p.dv) + (int64_t)(k0 + jrow) * p.dv_stride + (int64_t)hkv * D;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int vb = 0; vb < 4; ++vb) {
+            struct alignas(8) { T v[4]; } a, bq;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              a.v[e] = static_cast<T>(dKt[t][4 * vb + e] * p.scale);
+              bq.v[e] = static_cast<T>(dVt[t][4 * vb + e]);
+            }
+            *reinterpret_cast<decltype(a) *>(dkp + 32 * t + 8 * vb + 4 * hh) = a;
+            *reinterpret_cast<decltype(bq) *>(dvp + 32 * t + 8 * vb + 4 * hh) = bq;
+          }
+      } else {
+        const int64_t off = (((int64_t)hs * p.total_k + (k0 + jrow)) * p.hk + hkv) * D;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int vb = 0; vb < 4; ++vb) {
+            *reinterpret_cast<float4 *>(p.dk_part + off + 32 * t + 8 * vb + 4 * hh) =
+                make_float4(dKt[t][4 * vb] * p.scale, dKt[t][4 * vb + 1] * p.scale, dKt[t][4 * vb + 2] * p.scale,
+                            dKt[t][4 * vb + 3] * p.scale);
+            *reinterpret_cast<float4 *>(p.dv_part + off + 32 * t + 8 * vb + 4 * hh) =
+                make_float4(dVt[t][4 * vb], dVt[t][4 * vb + 1], dVt[t][4 * vb + 2], dVt[t][4 * vb + 3]);
+          }
+      }
+    }
+    __syncthreads();   // the K / V tiles and the exchange area are rewritten by the next key tile
+  }
+}
+
 template <typename T>
 static int launch_dkv_d128(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
   const int nkt = (int)cdiv(max_sk, 64);
   dim3 grid((unsigned)((p.causal ? (nkt + 1) / 2 : nkt) * p.hk * p.hsplit), (unsigned)batch);
-  hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(256), 0, st, p);
+  if (DH_DKV8) hipLaunchKernelGGL((attn_bwd_dkv8_d128_kernel<T>), grid, dim3(512), 0, st, p);
+  else hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(256), 0, st, p);
   return DH_OK;
 }
 
@@ -1117,7 +1453,7 @@ static int launch_dq(const AttnBwdParams &p, int batch, hipStream_t st) {
 
 template <typename T>
 static int launch_delta(const void *dout, const void *out, float *delta, const float *lse, float *ld2, int64_t ld2_plane,
-                        const int32_t *cu_q, int batch, int max_sq, int hq, int d, int64_t do_stride, int64_t o_stride,
+                        int ld2_pitch, const int32_t *cu_q, int batch, int max_sq, int hq, int d, int64_t do_stride, int64_t o_stride,
                         hipStream_t st) {
   const int nvec = d / Vec<T>::N;
   int lanes_per = 1;
@@ -1127,7 +1463,7 @@ static int launch_delta(const void *dout, const void *out, float *delta, const f
   if (blocks > 256 * 16) blocks = 256 * 16;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL((attn_delta_kernel<T>), dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, st,
-                     (const T *)dout, (const T *)out, delta, lse, ld2, ld2_plane, cu_q, max_sq, hq, d, lanes_per, do_stride,
+                     (const T *)dout, (const T *)out, delta, lse, ld2, ld2_plane, ld2_pitch, cu_q, max_sq, hq, d, lanes_per, do_stride,
                      o_stride);
   return DH_OK;
 }
@@ -1148,7 +1484,8 @@ extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, 
   (void)total_q;
   const size_t plane = align256((size_t)batch * hq * (max_seqlen_q > 0 ? max_seqlen_q : 0) * sizeof(float));
   size_t n = plane;                               // delta
-  if (dtype != DH_F32 && d == 128) n += 2 * plane;  // lse (exp2 units) and delta side by side for the d = 128 kernels
+  const size_t plane2 = align256((size_t)batch * hq * (size_t)(((max_seqlen_q > 0 ? max_seqlen_q : 0) + 31) / 32 * 32) * sizeof(float));
+  if (dtype != DH_F32 && d == 128) n += 2 * plane2;  // lse (exp2 units) and delta side by side for the d = 128 kernels
   if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
     n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
   return n + 256;
@@ -1174,10 +1511,12 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   float *delta = delta_out ? delta_out : (float *)ws;
   ws += plane;
   float *ld2 = nullptr;
+  const int ld2_pitch = (max_seqlen_q + 31) / 32 * 32;
+  const size_t plane2 = align256((size_t)batch * hq * (size_t)ld2_pitch * sizeof(float));
   if (dtype != DH_F32 && d == 128) {
     ld2 = (float *)ws;
-    ws += 2 * plane;
-    DH_CHECK(plane < (1ull << 31), "batch * heads * max_seqlen_q too large");
+    ws += 2 * plane2;
+    DH_CHECK(plane2 < (1ull << 31), "batch * heads * max_seqlen_q too large");
   }
 
   const int n = 16 / (int)dtype_size(dtype);
@@ -1186,7 +1525,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
            "dout/out rows must be 16-byte aligned");
   if (max_seqlen_q > 0) {
     DH_DISPATCH_DTYPE(dtype, {
-      launch_delta<T>(dout, out, delta, lse, ld2, (int64_t)(plane / sizeof(float)), cu_seqlens_q, batch, max_seqlen_q, hq, d,
+      launch_delta<T>(dout, out, delta, lse, ld2, (int64_t)(plane2 / sizeof(float)), ld2_pitch, cu_seqlens_q, batch, max_seqlen_q, hq, d,
                       do_stride, o_stride, st);
     });
   }
@@ -1204,7 +1543,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
            "pointers must be 16-byte aligned");
   AttnBwdParams p;
   p.dout = dout; p.q = q; p.k = k; p.v = v; p.lse = lse; p.delta = delta;
-  p.ld2 = ld2; p.ld2_plane = (int64_t)(plane / sizeof(float));
+  p.ld2 = ld2; p.ld2_plane = (int64_t)(plane2 / sizeof(float)); p.ld2_pitch = ld2_pitch;
   p.dq = dq; p.dk = dk; p.dv = dv;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
   p.max_sq = max_seqlen_q; p.hq = hq; p.hk = hk;

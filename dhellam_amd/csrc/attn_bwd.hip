@@ -3,9 +3,10 @@
 //
 // Three kernels:
 //   delta   : delta_i = sum_d dO[i,d] * O[i,d]                      (streaming)
-//   dK/dV   : a workgroup owns 32*NW key/value rows (K, V fragments stay in
-//             registers), walks the query heads of its GQA group and the query
-//             tiles that attend to it; S = Q K^T and dP = dO V^T are computed
+//   dK/dV   : a workgroup owns 64 key/value rows (K, V fragments stay in
+//             registers for head dim 64, in LDS for head dim 128), walks the
+//             query heads of its GQA group and the query tiles that attend to
+//             it; S = Q K^T and dP = dO V^T are computed
 //             with the key index on lanes so that P and dS feed dV^T += dO^T P
 //             and dK^T += Q^T dS straight from their accumulators, with the
 //             transposed Q / dO fragments coming from LDS transpose reads.
@@ -19,12 +20,6 @@
 // needs no fp32 dQ accumulator in memory and no atomics.
 #include "mma.h"
 
-#ifndef DH_DKV8
-#define DH_DKV8 1
-#endif
-#ifndef DH_DKV8_GROUP
-#define DH_DKV8_GROUP 2
-#endif
 
 namespace dh {
 
@@ -726,363 +721,17 @@ static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
   return DH_OK;
 }
 
-// dK/dV: 4 wavefronts = 2 key row groups (32 rows each) x 2 query splits.  K and V
-// fragments of the group stay in registers; every iteration brings two 32-row query tiles
-// (Q, dO, lse, delta) of the current head into LDS, one per split.  The splits' partial
-// dK/dV are added through LDS in split order.  Causal: the workgroup owns key tiles j and
-// n-1-j, so every workgroup does the same amount of work.  The main loop is one rolled body
-// with assembly copies (scalar bases) and assembly LDS reads, as in the forward kernel.
-template <typename T>
-__global__ void __launch_bounds__(256) attn_bwd_dkv_d128_kernel(const AttnBwdParams p) {
-  using M = Mma<T>;
-  using Frag = typename M::Frag;
-  constexpr int D = 128, KG = 2, QSPLIT = 2, BN = 32 * KG, BM = 32;
-  constexpr int QT = BM * D;                          // elements of one Q (or dO) tile
-  constexpr int SLOT = 2 * QT + 128;                  // Q tile, dO tile, 32 lse + 32 delta (as 256 bytes)
-  constexpr int SLOTB = SLOT * (int)sizeof(T);
-  constexpr int STAGE = QSPLIT * SLOT;
-  constexpr int STAGEB = STAGE * (int)sizeof(T);
-  __shared__ __attribute__((aligned(1024))) T sAll[2 * STAGE];
-
-  const int b = blockIdx.y;
-  // all key tiles of one head group read the same Q / dO rows: keep a group on one XCD's L2
-  const int G = p.hk * p.hsplit;
-  int hg, px;
-  xcd_group_item(blockIdx.x, G, gridDim.x / G, hg, px);
-  const int hkv = hg / p.hsplit, hs = hg % p.hsplit;
-  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
-  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
-  const int nkt = (sk + BN - 1) / BN;
-  const int causal = p.causal;
-  const int q_stride = (int)p.q_stride, do_stride = (int)p.do_stride;
-  const float scale_log2 = p.scale_log2;
-  int kt[2], nk;
-  if (causal) {
-    const int pair = px;
-    if (2 * pair >= nkt) return;
-    kt[0] = pair; kt[1] = nkt - 1 - pair;             // heavy (early keys) first
-    nk = (kt[0] == kt[1]) ? 1 : 2;
-  } else {
-    if (px >= nkt) return;
-    kt[0] = px; kt[1] = 0; nk = 1;
-  }
-  agpr_reserve_192();
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: copy bookkeeping stays scalar
-  const int c = lane & 31, hh = lane >> 5;
-  const int kg = w % KG, qs = w / KG;
-  const int ratio = p.hq / p.hk;
-  const int hper = ratio / p.hsplit;
-  const int h_first = hkv * ratio + hs * hper;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)sAll;
-
-  // ---- copies: wavefront w brings one whole tile per iteration: Q (w even) or dO (w odd) of split w / 2;
-  // wavefronts 0 and 1 also bring the 64 lse/delta values of split w ----------------------------------
-  CopyLane cl0;
-  cl0.l16 = lane & 15;
-  cl0.lrow = lane >> 4;
-  const int cp_slot = w >> 1, cp_do = w & 1;
-  const int cp_stride = cp_do ? do_stride : q_stride;
-  const T *cp_gt = reinterpret_cast<const T *>(cp_do ? p.dout : p.q) + (int64_t)q0 * cp_stride;
-  const char *cp_g = reinterpret_cast<const char *>(cp_gt);
-  const int cp_dst0 = cp_slot * SLOT + cp_do * QT;    // elements inside a stage
-  const uint32_t cp_step = (uint32_t)(4 * cp_stride) * (uint32_t)sizeof(T);
-  uint32_t cp_off[4];                                 // tiles use swz(row): chunk ^= 4 * (row % 4) + (row / 4) % 4
-  {
-    const uint32_t rowb = (uint32_t)(cl0.lrow * cp_stride) * (uint32_t)sizeof(T);
-    const uint32_t chunk = (uint32_t)(cl0.l16 ^ (4 * cl0.lrow)) << 4;
-#pragma unroll
-    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
-  }
-  const uint32_t ld_off = (uint32_t)((lane & 31) * 4) + (lane < 32 ? 0u : (uint32_t)p.ld2_plane * 4u);
-  const char *ld_g = reinterpret_cast<const char *>(p.ld2);
-  // ---- fragment reads: lane byte offsets inside a slot; other fragments by XOR / immediate offset ----
-  const int r = lane & 15;
-  const uint32_t rf_lane = (uint32_t)(qs * SLOTB + c * 256 + ((hh ^ swz(c)) << 4));   // row c, chunk hh
-  const int ta_x = 4 * (r >> 2) + hh;                 // transpose reads: swz of rows 4*hh + r/4 (+8)
-  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
-  const uint32_t t_row = (uint32_t)(qs * SLOTB + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
-  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
-  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
-  const uint32_t tl_lane = (uint32_t)(qs * SLOTB + 2 * QT * (int)sizeof(T) + 16 * hh);  // lse of rows 4*hh + 8*vb + e
-
-  for (int ki = 0; ki < nk; ++ki) {
-    const int j0 = kt[ki] * BN;
-    const int jw0 = j0 + 32 * kg;
-    const int jrow = jw0 + c;
-    // Fixed accumulation registers of this kernel: dV^T tiles in a[0:63], dK^T tiles in a[64:127],
-    // this wavefront's K fragments in a[128:159], its V fragments in a[160:191].
-    {
-      const int jl = jrow < sk ? jrow : sk - 1;
-      const T *kp = reinterpret_cast<const T *>(p.k) + (int64_t)(k0 + jl) * p.k_stride + (int64_t)hkv * D;
-      const T *vp = reinterpret_cast<const T *>(p.v) + (int64_t)(k0 + jl) * p.v_stride + (int64_t)hkv * D;
-#define DH_KV(ks)                                                        \
-      agpr_write_frag<T, 128 + 4 * ks>(frag_ld<T>(kp + ks * 16 + 8 * hh)); \
-      agpr_write_frag<T, 160 + 4 * ks>(frag_ld<T>(vp + ks * 16 + 8 * hh))
-      DH_KV(0); DH_KV(1); DH_KV(2); DH_KV(3); DH_KV(4); DH_KV(5); DH_KV(6); DH_KV(7);
-#undef DH_KV
-    }
-    agpr_zero16<0>(); agpr_zero16<16>(); agpr_zero16<32>(); agpr_zero16<48>();
-    agpr_zero16<64>(); agpr_zero16<80>(); agpr_zero16<96>(); agpr_zero16<112>();
-    const int i_begin = causal ? (j0 / BM) * BM : 0;
-    const int ntq = i_begin < sq ? (sq - i_begin + BM - 1) / BM : 0;
-    const int it_per_head = (ntq + QSPLIT - 1) / QSPLIT;
-    const int niter = it_per_head * hper;
-
-    // The copies of iteration (head g, step ti) into the stage at element offset `st`:
-    // general form (any tile, rows clamped per lane), used for the first stage and for tail tiles.
-    auto issue_general = [&](int st, int g, int ti) {
-      const int h = h_first + g;
-      const int tq = ti * QSPLIT + cp_slot;
-      if (tq < ntq)
-        dma_tile32_general<T, 8>(sAll + st + cp_dst0, cp_gt + (int64_t)h * D, cp_stride, 1, i_begin + tq * BM, 0, sq, cl0);
-      if (w < QSPLIT) {
-        const int tl = ti * QSPLIT + w;
-        if (tl < ntq) {
-          int ir = i_begin + tl * BM + (lane & 31);
-          ir = ir < sq ? ir : sq - 1;
-          const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + h) * p.ld2_pitch + ir;
-          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                           (__attribute__((address_space(3))) void *)(sAll + st + w * SLOT + 2 * QT), 4, 0, 0);
-        }
-      }
-    };
-
-    if (niter > 0) issue_general(0, 0, 0);
-    dma_wait_all();
-    __syncthreads();
-
-    const char *cp_src = nullptr;
-    uint32_t cp_dst = 0;
-    bool fcopy = false;
-#define DH_DKV_COPY(i)                                                                                  \
-    do {                                                                                                \
-      if (fcopy) {                                                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                              \
-        dma_block_fast(cp_src, cp_off[(i) & 3], cp_dst);                                                \
-        cp_src += cp_step;                                                                              \
-        cp_dst += 1024;                                                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                              \
-      }                                                                                                 \
-    } while (0)
-
-    int g = 0, ti = 0;                                // head and step of iteration it
-#pragma unroll 1
-    for (int it = 0; it < niter; ++it) {
-      int gn = g, tn = ti + 1;                        // ... and of iteration it + 1
-      if (tn == it_per_head) { tn = 0; ++gn; }
-      const bool have_next = it + 1 < niter;
-      const uint32_t cur = lds0 + (uint32_t)((it & 1) * STAGEB);
-      const int nxt_el = ((it + 1) & 1) * STAGE;
-      {
-        const int hn = h_first + gn;
-        const int tq = tn * QSPLIT + cp_slot;
-        const int row0 = i_begin + tq * BM;
-        const bool copy = have_next && tq < ntq;
-        fcopy = copy && row0 + BM <= sq;
-        cp_src = cp_g + ((int64_t)row0 * cp_stride + (int64_t)hn * D) * (int)sizeof(T);
-        cp_dst = lds0 + (uint32_t)((nxt_el + cp_dst0) * (int)sizeof(T));
-        if (copy && !fcopy)
-          dma_tile32_general<T, 8>(sAll + nxt_el + cp_dst0, cp_gt + (int64_t)hn * D, cp_stride, 1, row0, 0, sq, cl0);
-        if (w < QSPLIT && have_next) {
-          const int tl = tn * QSPLIT + w;
-          const int rl = i_begin + tl * BM;
-          if (tl < ntq) {
-            if (rl + BM <= sq) {
-              const char *src = ld_g + (((int64_t)b * p.hq + hn) * p.ld2_pitch + rl) * 4;
-              const uint32_t dst = lds0 + (uint32_t)((nxt_el + w * SLOT + 2 * QT) * (int)sizeof(T));
-              asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                           :
-                           : "v"(ld_off), "s"(src), "s"(dst)
-                           : "memory", "m0");
-            } else {
-              int ir = rl + (lane & 31);
-              ir = ir < sq ? ir : sq - 1;
-              const float *src = p.ld2 + (lane < 32 ? 0 : p.ld2_plane) + ((int64_t)b * p.hq + hn) * p.ld2_pitch + ir;
-              __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                               (__attribute__((address_space(3))) void *)(sAll + nxt_el + w * SLOT + 2 * QT), 4, 0, 0);
-            }
-          }
-        }
-      }
-      const int tq = ti * QSPLIT + qs;
-      const int i0 = i_begin + tq * BM;
-      const bool act = tq < ntq && !(causal && i0 + BM - 1 < jw0);
-      if (act) {
-        // The LDS reads below are ordinary loads: the compiler does not know about the assembly copies,
-        // so it orders them only against other LDS traffic, and it places the partial waits itself.
-        // One wavefront per SIMD has nobody to hide its LDS latency behind, so all reads of a phase are
-        // issued in one batch ahead of the matrix instructions that consume them (the scheduling
-        // barriers keep the batches where they are written).
-        uint32_t qb = cur + rf_lane, ta = cur + ta_lane, tb = cur + tb_lane, tl = cur + tl_lane;
-        asm volatile("" : "+v"(qb), "+v"(ta), "+v"(tb), "+v"(tl));   // derive the other addresses here
-        typedef __attribute__((address_space(3))) const Frag *lds_frag;
-        typedef __attribute__((address_space(3))) const floatx4 *lds_f4;
-        typedef short4v __attribute__((address_space(3))) *lds_tr;
-        Frag fq[D / 16], fo[D / 16];
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          const uint32_t a = qb ^ (uint32_t)(ks << 5);
-          fq[ks] = *(lds_frag)(a);
-          fo[ks] = *(lds_frag)(a + QT * (uint32_t)sizeof(T));
-        }
-        floatx4 l4[4], d4[4];                               // lse (exp2 units) and delta of rows 8*vb + 4*hh + e
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb) {
-          l4[vb] = *(lds_f4)(tl + 32 * vb);
-          d4[vb] = *(lds_f4)(tl + 128 + 32 * vb);
-        }
-        floatx16 S, dP;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          S[v] = 0.f;
-          dP[v] = 0.f;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          switch (ks) {
-            case 0: mfma_b_fixed<T, 128, true>(S, fq[0]); mfma_b_fixed<T, 160, true>(dP, fo[0]); break;
-            case 1: mfma_b_fixed<T, 132>(S, fq[1]); mfma_b_fixed<T, 164>(dP, fo[1]); break;
-            case 2: mfma_b_fixed<T, 136>(S, fq[2]); mfma_b_fixed<T, 168>(dP, fo[2]); break;
-            case 3: mfma_b_fixed<T, 140>(S, fq[3]); mfma_b_fixed<T, 172>(dP, fo[3]); break;
-            case 4: mfma_b_fixed<T, 144>(S, fq[4]); mfma_b_fixed<T, 176>(dP, fo[4]); break;
-            case 5: mfma_b_fixed<T, 148>(S, fq[5]); mfma_b_fixed<T, 180>(dP, fo[5]); break;
-            case 6: mfma_b_fixed<T, 152>(S, fq[6]); mfma_b_fixed<T, 184>(dP, fo[6]); break;
-            default: mfma_b_fixed<T, 156>(S, fq[7]); mfma_b_fixed<T, 188>(dP, fo[7]); break;
-          }
-          if (ks & 1) DH_DKV_COPY(ks >> 1);                            // copy blocks 0..3
-        }
-        // transposed fragments of the dO and Q tiles for dV^T += dO^T P and dK^T += Q^T dS: all 32
-        // transpose reads go out now and land while S and dP finish and the softmax part runs
-        short4v to[2][4][2], tq[2][4][2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
-            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
-            to[s][t][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0 + QT * (uint32_t)sizeof(T)));
-            to[s][t][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1 + QT * (uint32_t)sizeof(T)));
-            tq[s][t][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
-            tq[s][t][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
-          }
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_drain();                                                  // S and dP are read by ordinary code next
-        const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          float pv[8], dsv[8];
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const int vb = 2 * s + u;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int v = 4 * vb + e;
-              float pe = fast_exp2(S[v] * scale_log2 - l4[vb][e]);
-              if (need_mask) {
-                const int i = i0 + acc_row(v, hh);
-                if (i >= sq || (causal && jrow > i)) pe = 0.f;
-              }
-              pv[4 * u + e] = pe;
-              dsv[4 * u + e] = pe * (dP[v] - d4[vb][e]);
-            }
-          }
-          const Frag Pb = frag_pack<T>(pv), dSb = frag_pack<T>(dsv);
-          mfma_acc_fixed<T, 0, true>(frag_join<T>(to[s][0][0], to[s][0][1]), Pb);
-          mfma_acc_fixed<T, 16>(frag_join<T>(to[s][1][0], to[s][1][1]), Pb);
-          mfma_acc_fixed<T, 32>(frag_join<T>(to[s][2][0], to[s][2][1]), Pb);
-          mfma_acc_fixed<T, 48>(frag_join<T>(to[s][3][0], to[s][3][1]), Pb);
-          DH_DKV_COPY(4 + 2 * s);
-          mfma_acc_fixed<T, 64, true>(frag_join<T>(tq[s][0][0], tq[s][0][1]), dSb);
-          mfma_acc_fixed<T, 80>(frag_join<T>(tq[s][1][0], tq[s][1][1]), dSb);
-          mfma_acc_fixed<T, 96>(frag_join<T>(tq[s][2][0], tq[s][2][1]), dSb);
-          mfma_acc_fixed<T, 112>(frag_join<T>(tq[s][3][0], tq[s][3][1]), dSb);
-          DH_DKV_COPY(5 + 2 * s);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) DH_DKV_COPY(i);
-      }
-      g = gn;
-      ti = tn;
-      dma_wait_all();
-      __syncthreads();   // the next stage has landed, and everyone is done with the current one
-    }
-#undef DH_DKV_COPY
-    mfma_drain();                                     // the accumulators are read next
-    floatx16 dKt[D / 32], dVt[D / 32];
-    dVt[0] = agpr_read16<0>(); dVt[1] = agpr_read16<16>(); dVt[2] = agpr_read16<32>(); dVt[3] = agpr_read16<48>();
-    dKt[0] = agpr_read16<64>(); dKt[1] = agpr_read16<80>(); dKt[2] = agpr_read16<96>(); dKt[3] = agpr_read16<112>();
-
-    // add the second split's partial sums through LDS: dK in stage 0, dV in stage 1
-    float *xk = reinterpret_cast<float *>(sAll) + kg * 4096;
-    float *xv = reinterpret_cast<float *>(sAll + STAGE) + kg * 4096;
-    static_assert(STAGE * sizeof(T) >= KG * 4096 * sizeof(float), "exchange area");
-    if (qs == 1) {
-#pragma unroll
-      for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          xk[(t * 16 + v) * 64 + lane] = dKt[t][v];
-          xv[(t * 16 + v) * 64 + lane] = dVt[t][v];
-        }
-    }
-    __syncthreads();
-    if (qs == 0) {
-#pragma unroll
-      for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          dKt[t][v] += xk[(t * 16 + v) * 64 + lane];
-          dVt[t][v] += xv[(t * 16 + v) * 64 + lane];
-        }
-      if (jrow < sk) {
-        if (p.hsplit == 1) {
-          T *dkp = reinterpret_cast<T *>(p.dk) + (int64_t)(k0 + jrow) * p.dk_stride + (int64_t)hkv * D;
-          T *dvp = reinterpret_cast<T *>(p.dv) + (int64_t)(k0 + jrow) * p.dv_stride + (int64_t)hkv * D;
-#pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb) {
-              struct alignas(8) { T v[4]; } a, bq;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                a.v[e] = static_cast<T>(dKt[t][4 * vb + e] * p.scale);
-                bq.v[e] = static_cast<T>(dVt[t][4 * vb + e]);
-              }
-              *reinterpret_cast<decltype(a) *>(dkp + 32 * t + 8 * vb + 4 * hh) = a;
-              *reinterpret_cast<decltype(bq) *>(dvp + 32 * t + 8 * vb + 4 * hh) = bq;
-            }
-        } else {
-          const int64_t off = (((int64_t)hs * p.total_k + (k0 + jrow)) * p.hk + hkv) * D;
-#pragma unroll
-          for (int t = 0; t < D / 32; ++t)
-#pragma unroll
-            for (int vb = 0; vb < 4; ++vb) {
-              *reinterpret_cast<float4 *>(p.dk_part + off + 32 * t + 8 * vb + 4 * hh) =
-                  make_float4(dKt[t][4 * vb] * p.scale, dKt[t][4 * vb + 1] * p.scale, dKt[t][4 * vb + 2] * p.scale,
-                              dKt[t][4 * vb + 3] * p.scale);
-              *reinterpret_cast<float4 *>(p.dv_part + off + 32 * t + 8 * vb + 4 * hh) =
-                  make_float4(dVt[t][4 * vb], dVt[t][4 * vb + 1], dVt[t][4 * vb + 2], dVt[t][4 * vb + 3]);
-            }
-        }
-      }
-    }
-    __syncthreads();
-  }
-}
-
 // dK/dV with eight wavefronts: 2 key row groups (32 rows each) x 4 query splits, i.e. two wavefronts per
 // SIMD whose matrix and softmax phases interleave.  To fit that into 256 registers per wavefront the K / V
 // tiles of the workgroup live in LDS (read as row fragments every iteration) instead of registers, the
 // accumulators are ordinary variables, and lse / delta of a query tile come straight from memory (one
 // aligned 128-byte run per tile and plane), loaded one iteration ahead.  LDS: two stages of four Q + dO tile
 // pairs (128 KB) + the K and V tiles (32 KB).  The splits' partial dK/dV are added through LDS in a fixed
-// order.  Causal pairing of key tiles, head-group splitting and the copy scheme are those of the
-// four-wavefront kernel above.
+// order.  Causal: the workgroup owns key tiles j and n-1-j, so every workgroup does the same amount of
+// work.  The main loop is one rolled body; the Q / dO tiles of the next iteration come in with assembly
+// copies (scalar bases) issued between the matrix instructions.
 template <typename T>
-__global__ void __launch_bounds__(512) attn_bwd_dkv8_d128_kernel(const AttnBwdParams p) {
+__global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int D = 128, KG = 2, QSPLIT = 4, BN = 32 * KG, BM = 32;
@@ -1260,13 +909,29 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv8_d128_kernel(const AttnBwdPa
           S[v] = 0.f;
           dP[v] = 0.f;
         }
-        // S = Q K^T and dP = dO V^T with the key index on lanes
+        // S = Q K^T and dP = dO V^T with the key index on lanes; the four fragments of step ks + 1 are
+        // requested before the matrix instructions of step ks (the scheduling barriers pin that order)
+        {
+          Frag fq[2], fk[2], fo[2], fv[2];
+          fq[0] = *(lds_frag)(qb);
+          fk[0] = *(lds_frag)(kb);
+          fo[0] = *(lds_frag)(qb + QTB);
+          fv[0] = *(lds_frag)(kb + KVTB);
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          const uint32_t aq = qb ^ (uint32_t)(ks << 5), ak = kb ^ (uint32_t)(ks << 5);
-          S = M::mma(*(lds_frag)(aq), *(lds_frag)(ak), S);
-          dP = M::mma(*(lds_frag)(aq + QTB), *(lds_frag)(ak + KVTB), dP);
-          if (ks % DH_DKV8_GROUP == DH_DKV8_GROUP - 1) __builtin_amdgcn_sched_barrier(0);   // bounds the fragments in flight
+          for (int ks = 0; ks < D / 16; ++ks) {
+            const int cb = ks & 1, nb = cb ^ 1;
+            if (ks + 1 < D / 16) {
+              const uint32_t aq = qb ^ (uint32_t)((ks + 1) << 5), ak = kb ^ (uint32_t)((ks + 1) << 5);
+              fq[nb] = *(lds_frag)(aq);
+              fk[nb] = *(lds_frag)(ak);
+              fo[nb] = *(lds_frag)(aq + QTB);
+              fv[nb] = *(lds_frag)(ak + KVTB);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            S = M::mma(fq[cb], fk[cb], S);
+            dP = M::mma(fo[cb], fv[cb], dP);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
         const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
         Frag Pb[2], dSb[2];
@@ -1296,26 +961,28 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv8_d128_kernel(const AttnBwdPa
           dSb[s] = frag_pack<T>(dsv);
         }
         if (have_next) load_ld(gn, tn);               // next tile's lse / delta, in flight across the barrier
-        // dV^T += dO^T P and dK^T += Q^T dS; the eight copy blocks of this wavefront go out in between
+        // dV^T += dO^T P and dK^T += Q^T dS; the eight copy blocks of this wavefront go out in between.
+        // Step u = (s, which, t): which = 0 reads dO^T (for dV), 1 reads Q^T (for dK); the fragments of
+        // step u + 1 are requested before the matrix instruction of step u.
+        {
+          short4v x0[2], x1[2];
+          auto rd = [&](int u, int bsel) {
+            const int sx = u >> 3, which = (u >> 2) & 1, t = u & 3;
+            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(sx * 16 * 256) + (which ? 0u : (uint32_t)QTB);
+            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(sx * 16 * 256) + (which ? 0u : (uint32_t)QTB);
+            x0[bsel] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
+            x1[bsel] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
+          };
+          rd(0, 0);
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256) + QTB;
-            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256) + QTB;
-            const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
-            const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
-            dVt[t] = M::mma(frag_join<T>(x0, x1), Pb[s], dVt[t]);
-            if (t & 1) DH_DKV_COPY(4 * s + (t >> 1));
-          }
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
-            const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(s * 16 * 256);
-            const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
-            const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
-            dKt[t] = M::mma(frag_join<T>(x0, x1), dSb[s], dKt[t]);
-            if (t & 1) DH_DKV_COPY(4 * s + 2 + (t >> 1));
+          for (int u = 0; u < 16; ++u) {
+            const int sx = u >> 3, which = (u >> 2) & 1, t = u & 3, cb = u & 1;
+            if (u + 1 < 16) rd(u + 1, cb ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (which == 0) dVt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), Pb[sx], dVt[t]);
+            else dKt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), dSb[sx], dKt[t]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (u & 1) DH_DKV_COPY(u >> 1);
           }
         }
       } else {
@@ -1403,8 +1070,7 @@ template <typename T>
 static int launch_dkv_d128(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
   const int nkt = (int)cdiv(max_sk, 64);
   dim3 grid((unsigned)((p.causal ? (nkt + 1) / 2 : nkt) * p.hk * p.hsplit), (unsigned)batch);
-  if (DH_DKV8) hipLaunchKernelGGL((attn_bwd_dkv8_d128_kernel<T>), grid, dim3(512), 0, st, p);
-  else hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(256), 0, st, p);
+  hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(512), 0, st, p);
   return DH_OK;
 }
 

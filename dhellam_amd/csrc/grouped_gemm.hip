@@ -279,11 +279,6 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 // conflict-free.  8 wavefronts = 2 (m) x 4 (n), 128x64 outputs each; wavefronts 0-3 copy the A tile
 // (64 rows each), wavefronts 4-7 the B tile.
 // WVN = 4: 8 wavefronts of 128x64 (two per SIMD, accumulators in VGPRs).
-// WVN = 2: 4 wavefronts of 128x128 (one per SIMD): half the LDS fragment traffic per MFMA (the 128x64 form
-// moves 1 KB through the LDS per MFMA, reads plus copy writes, which is the whole LDS bandwidth at full MFMA
-// rate: there copies and MFMAs did not overlap at all).  Its 256 accumulator registers live in the fixed
-// AGPRs a[0:255], block (i, j) at a[16 * (i * WN + j)], named only by assembly MFMAs (as ordinary variables
-// the register allocator moves all of them between the register files around every k slice).
 // BKT: k depth of a slice (64 or 32); NST: LDS stages.  The copies of slice s + NST - 1 are issued during
 // slice s, so with NST > 2 a copy has more than a whole slice to land before anyone waits for it (with two
 // stages the copies issued late in a slice are waited for almost at once: their latency is exposed).
@@ -292,7 +287,7 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int BM = 256, BN = 256, WM = 4, WN = 8 / WVN, NW = 2 * WVN;
-  constexpr bool FIXED = (WVN == 2);
+  static_assert(WVN == 4, "eight wavefronts of 128x64");
   constexpr int ROWB = BKT * (int)sizeof(T);            // bytes of a tile row (128 or 64)
   constexpr int CHUNKS = ROWB / 16;                     // 16-byte chunks per row
   constexpr int RP = 256 / ROWB;                        // rows per 256 bytes: the swizzle is (row / RP) % CHUNKS
@@ -377,18 +372,13 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * ROWB) + sw;    // B tile rows (n)
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
 
-  floatx16 acc[FIXED ? 1 : WM][FIXED ? 1 : WN];
-  if constexpr (FIXED) {
-    agpr_reserve_256();
-    agpr_zero256();
-  } else {
+  floatx16 acc[WM][WN];
 #pragma unroll
-    for (int i = 0; i < WM; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  }
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   for (int s = 0; s < DIST; ++s)
     if (s < nslices && cp_ext > 0) copy_general((uint32_t)(s * STAGEB), s);
@@ -437,13 +427,11 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
 #pragma unroll
         for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)(fb1 + j * 32 * ROWB);
       }
-      if constexpr (FIXED) __builtin_amdgcn_sched_barrier(0);   // the next fragments are requested before these MFMAs
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
 #pragma unroll
         for (int j = 0; j < WN; ++j) {  // C^T block: rows n, cols m
-          if constexpr (FIXED) mfma_acc_fixed_idx<T>(i * WN + j, fb[cu][j], fa[cu][i]);
-          else acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
+          acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
           // one 1 KB copy block after every DH_GG_CPI MFMAs until the slice's CPB blocks are out
           const int mi = (ks * WM + i) * WN + j;
           if (mi % DH_GG_CPI == DH_GG_CPI - 1 && mi / DH_GG_CPI < CPB && fcopy) {
@@ -472,15 +460,12 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
 
   // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
   T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0;
-  if constexpr (FIXED) mfma_drain();
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     const int m = wm * 32 * WM + 32 * i + c;
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
-      floatx16 av;
-      if constexpr (FIXED) av = agpr_read16_idx(i * WN + j);   // read by every lane (EXEC is full here)
-      else av = acc[i][j];
+      const floatx16 av = acc[i][j];
       if (m < a_rext) {
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {

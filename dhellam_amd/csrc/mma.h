@@ -17,7 +17,6 @@
 // S[k0 + e][n0 + i]: four consecutive rows of ONE column -- an MFMA operand
 // fragment along the strided dimension, with no transpose in memory.
 #pragma once
-#include <type_traits>
 #include "common.h"
 
 namespace dh {
@@ -222,104 +221,6 @@ __device__ __forceinline__ void dma_tile32_general(T *dst, const T *g, int strid
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                      (__attribute__((address_space(3))) void *)(dst + i * 512), 16, 0, 0);
   }
-}
-
-// ---- MFMA with hand-assigned accumulation registers (one wavefront per SIMD: 256 VGPRs + 256 AGPRs) ---
-// Long-lived matrix operands (accumulators, stationary fragments) are kept in FIXED AGPRs that only the
-// assembly below names; the compiler never sees them as values, so it cannot shuffle them through
-// VGPRs around every matrix instruction (which it does when they are ordinary variables).  A kernel
-// using these helpers calls agpr_reserve_192() once: that makes the register count of the kernel
-// cover a0..a191.  The kernel must keep its own VGPR demand well under 256 so that the compiler has no
-// reason to use AGPRs itself.  The compiler does not see these as matrix instructions either: before
-// ordinary code reads a VGPR result, and before agpr_read16, the caller places mfma_drain().
-__device__ __forceinline__ void agpr_reserve_192() { asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191"); }
-__device__ __forceinline__ void agpr_reserve_256() { asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"); }
-
-// GAP: the instruction is preceded by idle cycles.  An ordinary vector instruction that produces an
-// operand (packing, zeroing) must not be followed at once by the matrix instruction that reads it; the
-// compiler keeps that distance for its own matrix instructions but cannot for these, and it is free to
-// move the producers right in front of them.  Use GAP on the first instruction that reads a fresh operand.
-// acc a[BASE : BASE+15] += a (VGPR) * b (VGPR)
-template <typename T, int BASE, bool GAP = false>
-__device__ __forceinline__ void mfma_acc_fixed(typename Mma<T>::Frag a, typename Mma<T>::Frag b) {
-  if constexpr (std::is_same<T, bf16_t>::value) {
-    if constexpr (GAP) asm volatile("s_nop 7\n\tv_mfma_f32_32x32x16_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(BASE), "n"(BASE + 15));
-    else asm volatile("v_mfma_f32_32x32x16_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(BASE), "n"(BASE + 15));
-  } else {
-    if constexpr (GAP) asm volatile("s_nop 7\n\tv_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(BASE), "n"(BASE + 15));
-    else asm volatile("v_mfma_f32_32x32x16_f16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(a), "v"(b), "n"(BASE), "n"(BASE + 15));
-  }
-}
-// c (VGPR) += a (VGPR) * fragment held in a[BREG : BREG+3]
-template <typename T, int BREG, bool GAP = false>
-__device__ __forceinline__ void mfma_b_fixed(floatx16 &c, typename Mma<T>::Frag a) {
-  if constexpr (std::is_same<T, bf16_t>::value) {
-    if constexpr (GAP) asm volatile("s_nop 7\n\tv_mfma_f32_32x32x16_bf16 %0, %1, a[%2:%3], %0" : "+v"(c) : "v"(a), "n"(BREG), "n"(BREG + 3));
-    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, a[%2:%3], %0" : "+v"(c) : "v"(a), "n"(BREG), "n"(BREG + 3));
-  } else {
-    if constexpr (GAP) asm volatile("s_nop 7\n\tv_mfma_f32_32x32x16_f16 %0, %1, a[%2:%3], %0" : "+v"(c) : "v"(a), "n"(BREG), "n"(BREG + 3));
-    else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, a[%2:%3], %0" : "+v"(c) : "v"(a), "n"(BREG), "n"(BREG + 3));
-  }
-}
-// a[BASE : BASE+3] = fragment
-template <typename T, int BASE> __device__ __forceinline__ void agpr_write_frag(typename Mma<T>::Frag f) {
-  const int4v x = __builtin_bit_cast(int4v, f);
-  asm volatile("v_accvgpr_write_b32 a[%4], %0\n\tv_accvgpr_write_b32 a[%5], %1\n\t"
-               "v_accvgpr_write_b32 a[%6], %2\n\tv_accvgpr_write_b32 a[%7], %3"
-               ::"v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "n"(BASE), "n"(BASE + 1), "n"(BASE + 2), "n"(BASE + 3));
-}
-// a[BASE : BASE+15] = 0
-template <int BASE> __device__ __forceinline__ void agpr_zero16() {
-  asm volatile("v_accvgpr_write_b32 a[%0], 0\n\tv_accvgpr_write_b32 a[%1], 0\n\tv_accvgpr_write_b32 a[%2], 0\n\tv_accvgpr_write_b32 a[%3], 0\n\t"
-               "v_accvgpr_write_b32 a[%4], 0\n\tv_accvgpr_write_b32 a[%5], 0\n\tv_accvgpr_write_b32 a[%6], 0\n\tv_accvgpr_write_b32 a[%7], 0\n\t"
-               "v_accvgpr_write_b32 a[%8], 0\n\tv_accvgpr_write_b32 a[%9], 0\n\tv_accvgpr_write_b32 a[%10], 0\n\tv_accvgpr_write_b32 a[%11], 0\n\t"
-               "v_accvgpr_write_b32 a[%12], 0\n\tv_accvgpr_write_b32 a[%13], 0\n\tv_accvgpr_write_b32 a[%14], 0\n\tv_accvgpr_write_b32 a[%15], 0"
-               ::"n"(BASE), "n"(BASE + 1), "n"(BASE + 2), "n"(BASE + 3), "n"(BASE + 4), "n"(BASE + 5), "n"(BASE + 6), "n"(BASE + 7),
-               "n"(BASE + 8), "n"(BASE + 9), "n"(BASE + 10), "n"(BASE + 11), "n"(BASE + 12), "n"(BASE + 13), "n"(BASE + 14), "n"(BASE + 15));
-}
-// result = a[BASE : BASE+15]
-template <int BASE> __device__ __forceinline__ floatx16 agpr_read16() {
-  float r[16];
-#define DH_RD(i) asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(r[i]) : "n"(BASE + i))
-  DH_RD(0); DH_RD(1); DH_RD(2); DH_RD(3); DH_RD(4); DH_RD(5); DH_RD(6); DH_RD(7);
-  DH_RD(8); DH_RD(9); DH_RD(10); DH_RD(11); DH_RD(12); DH_RD(13); DH_RD(14); DH_RD(15);
-#undef DH_RD
-  floatx16 o;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) o[i] = r[i];
-  return o;
-}
-// The same with the accumulator chosen by an index that is a constant after unrolling (block idx of 16).
-template <typename T> __device__ __forceinline__ void mfma_acc_fixed_idx(int idx, typename Mma<T>::Frag a, typename Mma<T>::Frag b) {
-  switch (idx) {
-    case 0: mfma_acc_fixed<T, 0>(a, b); break;     case 1: mfma_acc_fixed<T, 16>(a, b); break;
-    case 2: mfma_acc_fixed<T, 32>(a, b); break;    case 3: mfma_acc_fixed<T, 48>(a, b); break;
-    case 4: mfma_acc_fixed<T, 64>(a, b); break;    case 5: mfma_acc_fixed<T, 80>(a, b); break;
-    case 6: mfma_acc_fixed<T, 96>(a, b); break;    case 7: mfma_acc_fixed<T, 112>(a, b); break;
-    case 8: mfma_acc_fixed<T, 128>(a, b); break;   case 9: mfma_acc_fixed<T, 144>(a, b); break;
-    case 10: mfma_acc_fixed<T, 160>(a, b); break;  case 11: mfma_acc_fixed<T, 176>(a, b); break;
-    case 12: mfma_acc_fixed<T, 192>(a, b); break;  case 13: mfma_acc_fixed<T, 208>(a, b); break;
-    case 14: mfma_acc_fixed<T, 224>(a, b); break;  default: mfma_acc_fixed<T, 240>(a, b); break;
-  }
-}
-__device__ __forceinline__ floatx16 agpr_read16_idx(int idx) {
-  switch (idx) {
-    case 0: return agpr_read16<0>();     case 1: return agpr_read16<16>();   case 2: return agpr_read16<32>();
-    case 3: return agpr_read16<48>();    case 4: return agpr_read16<64>();   case 5: return agpr_read16<80>();
-    case 6: return agpr_read16<96>();    case 7: return agpr_read16<112>();  case 8: return agpr_read16<128>();
-    case 9: return agpr_read16<144>();   case 10: return agpr_read16<160>(); case 11: return agpr_read16<176>();
-    case 12: return agpr_read16<192>();  case 13: return agpr_read16<208>(); case 14: return agpr_read16<224>();
-    default: return agpr_read16<240>();
-  }
-}
-__device__ __forceinline__ void agpr_zero256() {
-  agpr_zero16<0>(); agpr_zero16<16>(); agpr_zero16<32>(); agpr_zero16<48>(); agpr_zero16<64>(); agpr_zero16<80>();
-  agpr_zero16<96>(); agpr_zero16<112>(); agpr_zero16<128>(); agpr_zero16<144>(); agpr_zero16<160>(); agpr_zero16<176>();
-  agpr_zero16<192>(); agpr_zero16<208>(); agpr_zero16<224>(); agpr_zero16<240>();
-}
-// Idle long enough for every matrix instruction issued above to have written its result.
-__device__ __forceinline__ void mfma_drain() {
-  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 }
 
 // Row index inside a 32-row accumulator block held by register v of lane half h.

@@ -52,9 +52,18 @@ attn_delta_kernel(const T *__restrict__ dout, const T *__restrict__ out, float *
   const int per_block = 256 / lanes_per;
   const int sub = threadIdx.x / lanes_per, ln = threadIdx.x % lanes_per;
   const int nvec = d / N;
-  for (int64_t item = (int64_t)blockIdx.x * per_block + sub; item < (int64_t)sq * hq;
+  const int rows = ld2 ? ((sq + 31) / 32) * 32 : sq;   // the side-by-side planes are written in whole 32-row tiles
+  for (int64_t item = (int64_t)blockIdx.x * per_block + sub; item < (int64_t)rows * hq;
        item += (int64_t)gridDim.x * per_block) {
     const int i = (int)(item / hq), h = (int)(item % hq);
+    if (i >= sq) {           // padding rows of the last tile: zeros, so that masked scores stay finite
+      if (ln == 0) {
+        const int64_t a2 = ((int64_t)b * hq + h) * ld2_pitch + i;
+        ld2[a2] = 0.f;
+        ld2[ld2_plane + a2] = 0.f;
+      }
+      continue;
+    }
     float s = 0.f;
     for (int c = ln; c < nvec; c += lanes_per) {
       const Vec<T> a = ldg(dout + (int64_t)(q0 + i) * do_stride + (int64_t)h * d + c * N);
@@ -793,15 +802,6 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
 #pragma unroll
     for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
   }
-  // ---- fragment reads: lane byte offsets inside a slot; other fragments by XOR / immediate offset ----
-  const int r = lane & 15;
-  const uint32_t rf_lane = (uint32_t)(qs * SLOTB + c * 256 + ((hh ^ swz(c)) << 4));   // row c, chunk hh
-  const uint32_t kv_lane = (uint32_t)((kg * 32 + c) * 256 + ((hh ^ swz(c)) << 4));    // K / V row of this lane
-  const int ta_x = 4 * (r >> 2) + hh;                 // transpose reads: swz of rows 4*hh + r/4 (+8)
-  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
-  const uint32_t t_row = (uint32_t)(qs * SLOTB + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
-  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
-  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
   typedef short4v __attribute__((address_space(3))) *lds_tr;
 
@@ -901,7 +901,20 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
       const int i0 = i_begin + tq * BM;
       const bool act = tq < ntq && !(causal && i0 + BM - 1 < jw0);
       if (act) {
-        uint32_t qb = cur + rf_lane, ta = cur + ta_lane, tb = cur + tb_lane, kb = ldsKV + kv_lane;
+        // Fragment reads: lane byte offsets inside a slot; the other fragments are reached by XOR / immediate
+        // offsets.  They are recomputed from the lane id here (a dozen instructions) rather than kept in
+        // registers across the loop, which has none to spare.
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int lc = ln & 31, lh = ln >> 5, r = ln & 15;
+        const uint32_t rowsw = (uint32_t)(lc * 256 + ((lh ^ swz(lc)) << 4));            // row lc, chunk lh
+        const int ta_x = 4 * (r >> 2) + lh;                 // transpose reads: swz of rows 4*lh + r/4 (+8)
+        const int t_lc = 2 * ((ln >> 4) & 1) + ((r & 3) >> 1);
+        const uint32_t t_row = (uint32_t)((4 * lh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+        const uint32_t slot = cur + (uint32_t)(qs * SLOTB);
+        uint32_t qb = slot + rowsw, kb = ldsKV + (uint32_t)(kg * 32 * 256) + rowsw;
+        uint32_t ta = slot + t_row + (uint32_t)((t_lc ^ ta_x) << 4);
+        uint32_t tb = slot + t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
         asm volatile("" : "+v"(qb), "+v"(ta), "+v"(tb), "+v"(kb));   // derive the other addresses here
         floatx16 S, dP;
 #pragma unroll
@@ -933,7 +946,14 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        const bool need_mask = (causal && i0 < jw0 + 31) || (i0 + BM > sq);
+        if ((causal && i0 < jw0 + 31) || (i0 + BM > sq)) {
+          // masked scores become -inf, i.e. P = dS = 0 (lse and delta of rows past the sequence end are zeros)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int i = i0 + acc_row(v, hh);
+            if (i >= sq || (causal && jrow > i)) S[v] = -INFINITY;
+          }
+        }
         Frag Pb[2], dSb[2];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
@@ -944,17 +964,9 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int v = 4 * vb + e;
-              float pe = fast_exp2(S[v] * scale_log2 - l4[vb][e]);
-              float de = pe * (dP[v] - d4[vb][e]);
-              if (need_mask) {
-                const int i = i0 + acc_row(v, hh);
-                if (i >= sq || (causal && jrow > i)) {
-                  pe = 0.f;
-                  de = 0.f;          // rows past the sequence end carry unwritten lse / delta
-                }
-              }
+              const float pe = fast_exp2(S[v] * scale_log2 - l4[vb][e]);
               pv[4 * u + e] = pe;
-              dsv[4 * u + e] = de;
+              dsv[4 * u + e] = pe * (dP[v] - d4[vb][e]);
             }
           }
           Pb[s] = frag_pack<T>(pv);
@@ -965,19 +977,21 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
         // Step u = (s, which, t): which = 0 reads dO^T (for dV), 1 reads Q^T (for dK); the fragments of
         // step u + 1 are requested before the matrix instruction of step u.
         {
-          short4v x0[2], x1[2];
-          auto rd = [&](int u, int bsel) {
+          constexpr int AH = 2;                      // steps requested ahead
+          short4v x0[AH + 1], x1[AH + 1];
+          auto rd = [&](int u) {
             const int sx = u >> 3, which = (u >> 2) & 1, t = u & 3;
             const uint32_t a0 = (ta ^ (uint32_t)(t << 6)) + (uint32_t)(sx * 16 * 256) + (which ? 0u : (uint32_t)QTB);
             const uint32_t a1 = (tb ^ (uint32_t)(t << 6)) + (uint32_t)(sx * 16 * 256) + (which ? 0u : (uint32_t)QTB);
-            x0[bsel] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
-            x1[bsel] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
+            x0[u % (AH + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0));
+            x1[u % (AH + 1)] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1));
           };
-          rd(0, 0);
+#pragma unroll
+          for (int u = 0; u < AH; ++u) rd(u);
 #pragma unroll
           for (int u = 0; u < 16; ++u) {
-            const int sx = u >> 3, which = (u >> 2) & 1, t = u & 3, cb = u & 1;
-            if (u + 1 < 16) rd(u + 1, cb ^ 1);
+            const int sx = u >> 3, which = (u >> 2) & 1, t = u & 3, cb = u % (AH + 1);
+            if (u + AH < 16) rd(u + AH);
             __builtin_amdgcn_sched_barrier(0);
             if (which == 0) dVt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), Pb[sx], dVt[t]);
             else dKt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), dSb[sx], dKt[t]);
@@ -1125,7 +1139,7 @@ static int launch_delta(const void *dout, const void *out, float *delta, const f
   int lanes_per = 1;
   while (lanes_per < nvec && lanes_per < 64) lanes_per <<= 1;
   const int per_block = 256 / lanes_per;
-  int64_t blocks = cdiv((int64_t)max_sq * hq, per_block);
+  int64_t blocks = cdiv((int64_t)(ld2 ? ld2_pitch : max_sq) * hq, per_block);
   if (blocks > 256 * 16) blocks = 256 * 16;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL((attn_delta_kernel<T>), dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, st,

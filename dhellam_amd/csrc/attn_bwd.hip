@@ -841,7 +841,9 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
     auto load_ld = [&](int g, int ti) {
       const int tq = ti * QSPLIT + qs;
       if (tq < ntq) {
-        const float *src = p.ld2 + ((int64_t)b * p.hq + (h_first + g)) * p.ld2_pitch + (i_begin + tq * BM) + 4 * hh;
+        int lx = lane;
+        asm volatile("" : "+v"(lx));       // the address is formed here, not kept across the loop
+        const float *src = p.ld2 + ((int64_t)b * p.hq + (h_first + g)) * p.ld2_pitch + (i_begin + tq * BM) + 4 * (lx >> 5);
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {
           l4[vb] = *reinterpret_cast<const floatx4 *>(src + 8 * vb);
@@ -1019,8 +1021,9 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
     for (int round = 0; round < 2; ++round) {
       const int senders_from = round == 0 ? 2 : 1, senders_to = round == 0 ? 4 : 2;
       if (qs >= senders_from && qs < senders_to) {
-        uint32_t xb = lds0 + (uint32_t)((((qs - senders_from) * KG + kg) * 2 * 4096 + lane) * 4);
-        asm volatile("" : "+v"(xb));       // one base register + immediate offsets, computed here
+        int lx = lane;
+        asm volatile("" : "+v"(lx));       // one base register + immediate offsets, computed here
+        const uint32_t xb = lds0 + (uint32_t)((((qs - senders_from) * KG + kg) * 2 * 4096 + lx) * 4);
         lds_f dst = (lds_f)(xb);
 #pragma unroll
         for (int t = 0; t < D / 32; ++t)
@@ -1032,8 +1035,9 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
       }
       __syncthreads();
       if (qs < senders_from) {
-        uint32_t xb = lds0 + (uint32_t)(((qs * KG + kg) * 2 * 4096 + lane) * 4);
-        asm volatile("" : "+v"(xb));
+        int lx = lane;
+        asm volatile("" : "+v"(lx));
+        const uint32_t xb = lds0 + (uint32_t)(((qs * KG + kg) * 2 * 4096 + lx) * 4);
         lds_f src = (lds_f)(xb);
 #pragma unroll
         for (int t = 0; t < D / 32; ++t)
@@ -1045,7 +1049,11 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
       }
       __syncthreads();
     }
-    if (qs == 0 && jrow < sk) {
+    // the store addresses are derived from the lane id here, so that nothing but the id lives through the loop
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    if (qs == 0 && jw0 + (ln & 31) < sk) {
+      const int hh = ln >> 5, jrow = jw0 + (ln & 31);
       if (p.hsplit == 1) {
         T *dkp = reinterpret_cast<T *>(p.dk) + (int64_t)(k0 + jrow) * p.dk_stride + (int64_t)hkv * D;
         T *dvp = reinterpret_cast<T *>(p.dv) + (int64_t)(k0 + jrow) * p.dv_stride + (int64_t)hkv * D;

@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
-ATTN_BWD_TRAFFIC_BYTES = 164.2e6   # measured; see profiles/attn_70b_shard_hbm_traffic.md
+ATTN_BWD_TRAFFIC_BYTES = 167.8e6   # measured; see profiles/attn_70b_shard_hbm_traffic.md
 
 
 def _ensure_built():

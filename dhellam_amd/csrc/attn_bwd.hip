@@ -635,7 +635,24 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
             if (CPW == 4 && (ks & 3) == 3) DH_DQ_COPY(ks >> 2);      // copy blocks 0..1
           }
         }
-        const bool need_mask = (causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk);
+        // dQ^T += K^T dS^T needs K^T fragments (transpose reads of the K tile): those of the first 16-key
+        // step are requested now and land during the softmax part, those of the next step while the
+        // current one multiplies.
+        uint32_t ad[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          ad[2 * t] = ta ^ (uint32_t)(t << 6);
+          ad[2 * t + 1] = tb ^ (uint32_t)(t << 6);
+        }
+        short4v f[2][8];
+        lds_read_tr8<0>(f[0], ad);
+        if ((causal && n0 + BN - 1 > wrow0) || (n0 + BN > sk)) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int kv = n0 + acc_row(v, hh);
+            if (kv >= sk || (causal && kv > row_q)) S[v] = -INFINITY;     // P = dS = 0
+          }
+        }
         Frag dSb[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
@@ -643,34 +660,27 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int v = 8 * s + j;
-            float pe = fast_exp2(S[v] * scale_log2 - lse_c);
-            if (need_mask) {
-              const int kv = n0 + acc_row(v, hh);
-              if (kv >= sk || (causal && kv > row_q)) pe = 0.f;
-            }
+            const float pe = fast_exp2(S[v] * scale_log2 - lse_c);
             dsv[j] = pe * (dP[v] - del_c);
           }
           dSb[s] = frag_pack<T>(dsv);
         }
-        // dQ^T += K^T dS^T: K^T fragments by transpose reads of the K tile
-        uint32_t ad[8];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          ad[2 * t] = ta ^ (uint32_t)(t << 6);
-          ad[2 * t + 1] = tb ^ (uint32_t)(t << 6);
-        }
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-          short4v f[8];
-          if (s == 0) lds_read_tr8<0>(f, ad);
-          else lds_read_tr8<16 * 256>(f, ad);
-          lds_wait<4>(f[0], f[1], f[2], f[3]);
-          dQt[0] = M::mma(frag_join<T>(f[0], f[1]), dSb[s], dQt[0]);
-          dQt[1] = M::mma(frag_join<T>(f[2], f[3]), dSb[s], dQt[1]);
+          short4v(&g)[8] = f[s & 1];
+          if (s + 1 < NS) {
+            lds_read_tr8<16 * 256>(f[(s + 1) & 1], ad);
+            lds_wait<12>(g[0], g[1], g[2], g[3]);
+          } else {
+            lds_wait<4>(g[0], g[1], g[2], g[3]);
+          }
+          dQt[0] = M::mma(frag_join<T>(g[0], g[1]), dSb[s], dQt[0]);
+          dQt[1] = M::mma(frag_join<T>(g[2], g[3]), dSb[s], dQt[1]);
           if (CPW == 8) DH_DQ_COPY(4 + 2 * s);
-          lds_wait<0>(f[4], f[5], f[6], f[7]);
-          dQt[2] = M::mma(frag_join<T>(f[4], f[5]), dSb[s], dQt[2]);
-          dQt[3] = M::mma(frag_join<T>(f[6], f[7]), dSb[s], dQt[3]);
+          if (s + 1 < NS) lds_wait<8>(g[4], g[5], g[6], g[7]);
+          else lds_wait<0>(g[4], g[5], g[6], g[7]);
+          dQt[2] = M::mma(frag_join<T>(g[4], g[5]), dSb[s], dQt[2]);
+          dQt[3] = M::mma(frag_join<T>(g[6], g[7]), dSb[s], dQt[3]);
           if (CPW == 8) DH_DQ_COPY(5 + 2 * s);
           else DH_DQ_COPY(2 + s);
         }

@@ -224,10 +224,10 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
 // copies in flight and fragment reads, and the copies are spread between the MFMAs so
 // that they do not queue up behind each other.
 
-// LAG: the wavefronts of the upper half of the workgroup (the second wavefront of every SIMD) run their
-// P V products one iteration late.  In each half of an iteration one wavefront of a SIMD is then in its
-// matrix phase while the other is in its softmax, instead of both competing for the same unit.  V tiles
-// live one iteration longer for that (three V slots against two K slots).
+// Every wavefront runs its P V products one tile late (V tiles live one iteration longer: three V slots
+// against two K slots).  LAG: the second wavefront of every SIMD (the upper half of the workgroup) also
+// delays its softmax to the start of the next iteration, so that one wavefront of a SIMD is in its
+// matrix phase while the other is in its softmax instead of both competing for the same unit.
 template <typename T, int RG, int SPLIT, int BN, bool LAG>
 __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams p) {
   using M = Mma<T>;

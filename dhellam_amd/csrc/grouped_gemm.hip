@@ -282,12 +282,17 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 // BKT: k depth of a slice (64 or 32); NST: LDS stages.  The copies of slice s + NST - 1 are issued during
 // slice s, so with NST > 2 a copy has more than a whole slice to land before anyone waits for it (with two
 // stages the copies issued late in a slice are waited for almost at once: their latency is exposed).
-template <typename T, int WVN, int BKT, int NST>
-__global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GGParams p) {
+// BKS: the B operand is k-strided ([k][n] row-major, the NN product).  Its tile is then [64 k][256 n] with
+// 512-byte rows, copied two k rows per block with the transpose-read swizzle (chunk ^= 4 * (k % 4) +
+// (k / 4) % 4 inside each 256-byte half row), and its fragments come from LDS transpose reads.
+template <typename T, int WVN, int BKT, int NST, bool BKS>
+__global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int BM = 256, BN = 256, WM = 4, WN = 8 / WVN, NW = 2 * WVN;
   static_assert(WVN == 4, "eight wavefronts of 128x64");
+  static_assert(!BKS || BKT == 64, "the k-strided B tile is 64 k rows of 512 bytes");
+  constexpr int BROWB = 256 * (int)sizeof(T);           // bytes of a row of the k-strided B tile
   constexpr int ROWB = BKT * (int)sizeof(T);            // bytes of a tile row (128 or 64)
   constexpr int CHUNKS = ROWB / 16;                     // 16-byte chunks per row
   constexpr int RP = 256 / ROWB;                        // rows per 256 bytes: the swizzle is (row / RP) % CHUNKS
@@ -335,33 +340,51 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   const int n0 = tn * BN, m0 = row_begin + tm * BM;
   const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
   const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
-  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (int64_t)n0 * p.ldb;
+  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
   const int nslices = (int)(p.k_dim / BKT);
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
   // ---- copies ------------------------------------------------------------------------------------
   const int cp_b = w / (NW / 2);                        // 0: A tile, 1: B tile
-  const int cp_row0 = RPB * CPB * (w % (NW / 2));
+  const bool cp_ks = BKS && cp_b;                       // this wavefront copies rows of the k-strided tile
+  const int cp_row0 = cp_ks ? (64 / (NW / 2)) * (w % (NW / 2)) : RPB * CPB * (w % (NW / 2));
   const int cp_ld = (int)(cp_b ? p.ldb : p.lda);
-  const int cp_ext = cp_b ? b_rext : a_rext;            // valid rows of the tile
+  const int cp_ext = cp_ks ? 64 : (cp_b ? b_rext : a_rext);   // valid rows of the tile
   const T *cp_t = cp_b ? bg : ag;
   const char *cp_g = reinterpret_cast<const char *>(cp_t + (int64_t)cp_row0 * cp_ld);
-  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * ROWB);
-  const uint32_t cp_step = (uint32_t)(RPB * cp_ld) * (uint32_t)sizeof(T);
-  const bool cp_fast = cp_row0 + RPB * CPB <= cp_ext;   // every row this wavefront copies exists
-  const int lr = lane / CHUNKS, lc = lane % CHUNKS;
-  uint32_t cp_off[2];                                   // block i: swizzle (row / RP) % CHUNKS = (RPB / RP * (i % 2) + lr / RP) % CHUNKS
+  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * (cp_ks ? BROWB : ROWB));
+  const uint32_t cp_step = (uint32_t)((cp_ks ? 2 : RPB) * cp_ld) * (uint32_t)sizeof(T);
+  const int64_t cp_slice = cp_ks ? (int64_t)64 * cp_ld * (int)sizeof(T) : (int64_t)ROWB;   // bytes from one k slice to the next
+  const bool cp_fast = cp_ks || cp_row0 + RPB * CPB <= cp_ext;   // every row this wavefront copies exists
+  const int lr = cp_ks ? lane >> 5 : lane / CHUNKS, lc = cp_ks ? lane & 15 : lane % CHUNKS;
+  // row-fragment tiles: block i has swizzle (row / RP) % CHUNKS = (RPB / RP * (i % 2) + lr / RP) % CHUNKS (two values).
+  // k-strided tile: block i holds k rows 2 i + lr, swizzle 4 * ((2 i + lr) % 4) + (i / 2) % 4, i.e. the lane part
+  // lc ^ (4 lr) XOR the block constant ((i & 1) << 3) | ((i >> 1) & 3).
+  uint32_t cp_off[2];
 #pragma unroll
   for (int x = 0; x < 2; ++x)
     cp_off[x] = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)((lc ^ ((RPB / RP * x + lr / RP) % CHUNKS)) << 4);
+  const uint32_t ks_base = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)(((lane >> 4) & 1) * 256);
+  const uint32_t ks_chunk = (uint32_t)(lc ^ (4 * lr));
+  auto block_off = [&](int i) -> uint32_t {
+    if (cp_ks) return ks_base + ((ks_chunk ^ (uint32_t)(((i & 1) << 3) | ((i >> 1) & 3))) << 4);
+    return cp_off[i & 1];
+  };
   // general form (tiles at the edge of a group or of n): rows past the end re-read the last valid row
   auto copy_general = [&](uint32_t stage, int slice) {
 #pragma unroll 1
     for (int i = 0; i < CPB; ++i) {
-      int row = cp_row0 + RPB * i + lr;
-      const int f = (row / RP) % CHUNKS;
-      row = row < cp_ext ? row : cp_ext - 1;
-      const T *src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * BKT + ((lc ^ f) * 8);
+      const T *src;
+      if (cp_ks) {
+        const int row = cp_row0 + 2 * i + lr;
+        const int f = 4 * (row & 3) + ((row >> 2) & 3);
+        src = cp_t + ((int64_t)slice * 64 + row) * cp_ld + ((lane >> 4) & 1) * 128 + ((lc ^ f) * 8);
+      } else {
+        int row = cp_row0 + RPB * i + lr;
+        const int f = (row / RP) % CHUNKS;
+        row = row < cp_ext ? row : cp_ext - 1;
+        src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * BKT + ((lc ^ f) * 8);
+      }
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                        (__attribute__((address_space(3))) void *)(smem + stage + cp_dst0 + i * 1024), 16, 0, 0);
     }
@@ -370,7 +393,27 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   const uint32_t sw = (uint32_t)((hh ^ ((c / RP) % CHUNKS)) << 4);
   const uint32_t fa_lane = (uint32_t)((wm * 32 * WM + c) * ROWB) + sw;            // A tile rows (m)
   const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * ROWB) + sw;    // B tile rows (n)
+  // k-strided B tile: transpose reads.  A read with the lane address &tile[k0 + r / 4][n0 + 4 * (r % 4)]
+  // (r = lane % 16) returns tile[k0 + 0..3][n0 + r] to the lane, so the fragment's k values 8 hh + 0..3 come
+  // from a read at k0 = 8 hh and 8 hh + 4..7 from one at k0 = 8 hh + 4: the natural k order, matching the
+  // row fragments of A.  t_lc: 16-byte chunk inside the 64-byte run of the 32-column block.
+  const int r16 = lane & 15;
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r16 & 3) >> 1);
+  const int tx = 4 * (r16 >> 2) + 2 * hh;              // swizzle of k row 8 hh + r / 4; the row 4 further down has tx + 1
+  const uint32_t t_row = (uint32_t)(TILEB + (8 * hh + (r16 >> 2)) * BROWB + ((r16 & 3) & 1) * 8);
+  const uint32_t tb_a = t_row + (uint32_t)((t_lc ^ tx) << 4);
+  const uint32_t tb_b = t_row + 4 * BROWB + (uint32_t)((t_lc ^ (tx + 1)) << 4);
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
+  typedef short4v __attribute__((address_space(3))) *lds_tr;
+  // B fragment j of k step ks in the stage at byte offset `stage` (BKS form): the k step is an immediate offset
+  auto ld_b_tr = [&](uint32_t stage, int ks, int j) -> Frag {
+    const int nb = wn * WN + j;                         // 32-column block of the tile
+    const uint32_t o = stage + (uint32_t)((nb >> 2) * 256);
+    const uint32_t a0 = (tb_a ^ (uint32_t)((nb & 3) << 6)) + o, a1 = (tb_b ^ (uint32_t)((nb & 3) << 6)) + o;
+    const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0 + (uint32_t)(ks * 16 * BROWB)));
+    const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1 + (uint32_t)(ks * 16 * BROWB)));
+    return frag_join<T>(x0, x1);
+  };
 
   floatx16 acc[WM][WN];
 #pragma unroll
@@ -386,13 +429,18 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   __syncthreads();
 
   Frag fa[2][WM], fb[2][WN];
-  if constexpr (CROSS) {
-    if (nslices > 0) {
+  // fragments of k step ks of the stage whose row-fragment bases are fa_/fb_ (byte offset stage_ for the BKS form)
+  auto load_frags = [&](int buf, uint32_t fa_, uint32_t fb_, uint32_t stage_, int ks) {
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(lds0 + fa_lane + i * 32 * ROWB);
+    for (int i = 0; i < WM; ++i) fa[buf][i] = *(lds_frag)((fa_ ^ (uint32_t)(ks << 5)) + i * 32 * ROWB);
 #pragma unroll
-      for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(lds0 + fb_lane + j * 32 * ROWB);
+    for (int j = 0; j < WN; ++j) {
+      if constexpr (BKS) fb[buf][j] = ld_b_tr(stage_, ks, j);
+      else fb[buf][j] = *(lds_frag)((fb_ ^ (uint32_t)(ks << 5)) + j * 32 * ROWB);
     }
+  };
+  if constexpr (CROSS) {
+    if (nslices > 0) load_frags(0, lds0 + fa_lane, lds0 + fb_lane, lds0, 0);
   }
   int st_cur = 0, st_nxt = DIST % NST;                  // stage of slice s, stage of slice s + DIST
 #pragma unroll 1
@@ -400,33 +448,20 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
     const uint32_t cur = (uint32_t)(st_cur * STAGEB), nxt = (uint32_t)(st_nxt * STAGEB);
     const bool copy = s + DIST < nslices && cp_ext > 0;
     const bool fcopy = copy && cp_fast;
-    const char *cp_src = cp_g + (int64_t)(s + DIST) * ROWB;
+    const char *cp_src = cp_g + (int64_t)(s + DIST) * cp_slice;
     uint32_t cp_dst = lds0 + nxt + cp_dst0;
     if (copy && !fcopy) copy_general(nxt, s + DIST);
     uint32_t fa0 = lds0 + cur + fa_lane, fb0 = lds0 + cur + fb_lane;
     const uint32_t nst1 = (uint32_t)((st_cur + 1 == NST ? 0 : st_cur + 1) * STAGEB);   // stage of slice s + 1
     uint32_t fa1 = lds0 + nst1 + fa_lane, fb1 = lds0 + nst1 + fb_lane;
-    asm volatile("" : "+v"(fa0), "+v"(fb0), "+v"(fa1), "+v"(fb1));   // derive the other addresses here, not ahead of the loop
-    if constexpr (!CROSS) {
-#pragma unroll
-      for (int i = 0; i < WM; ++i) fa[0][i] = *(lds_frag)(fa0 + i * 32 * ROWB);
-#pragma unroll
-      for (int j = 0; j < WN; ++j) fb[0][j] = *(lds_frag)(fb0 + j * 32 * ROWB);
-    }
+    uint32_t sg0 = lds0 + cur, sg1 = lds0 + nst1;
+    asm volatile("" : "+v"(fa0), "+v"(fb0), "+v"(fa1), "+v"(fb1), "+v"(sg0), "+v"(sg1));   // derive the other addresses here, not ahead of the loop
+    if constexpr (!CROSS) load_frags(0, fa0, fb0, sg0, 0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int cu = ks & 1, nx = cu ^ 1;
-      if (ks + 1 < KS) {
-#pragma unroll
-        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)((fa0 ^ (uint32_t)((ks + 1) << 5)) + i * 32 * ROWB);
-#pragma unroll
-        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)((fb0 ^ (uint32_t)((ks + 1) << 5)) + j * 32 * ROWB);
-      } else if (CROSS && s + 1 < nslices) {            // first fragments of the next slice (already published)
-#pragma unroll
-        for (int i = 0; i < WM; ++i) fa[nx][i] = *(lds_frag)(fa1 + i * 32 * ROWB);
-#pragma unroll
-        for (int j = 0; j < WN; ++j) fb[nx][j] = *(lds_frag)(fb1 + j * 32 * ROWB);
-      }
+      if (ks + 1 < KS) load_frags(nx, fa0, fb0, sg0, ks + 1);
+      else if (CROSS && s + 1 < nslices) load_frags(nx, fa1, fb1, sg1, 0);   // first fragments of the next slice (already published)
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
 #pragma unroll
@@ -436,7 +471,7 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
           const int mi = (ks * WM + i) * WN + j;
           if (mi % DH_GG_CPI == DH_GG_CPI - 1 && mi / DH_GG_CPI < CPB && fcopy) {
             __builtin_amdgcn_sched_barrier(0);
-            dma_block_fast(cp_src, cp_off[(mi / DH_GG_CPI) & 1], cp_dst);
+            dma_block_fast(cp_src, block_off(mi / DH_GG_CPI), cp_dst);
             cp_src += cp_step;
             cp_dst += 1024;
             __builtin_amdgcn_sched_barrier(0);
@@ -483,12 +518,12 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_nt_dma_kernel(const GG
   }
 }
 
-template <typename T, int WVN, int BKT, int NST>
-static int launch_gg_nt_dma(GGParams p, int64_t m_extent, hipStream_t st) {
+template <typename T, int WVN, int BKT, int NST, bool BKS>
+static int launch_gg_dma(GGParams p, int64_t m_extent, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
   p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
-  hipLaunchKernelGGL((grouped_gemm_nt_dma_kernel<T, WVN, BKT, NST>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
+  hipLaunchKernelGGL((grouped_gemm_dma_kernel<T, WVN, BKT, NST, BKS>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
   return DH_OK;
 }
 
@@ -549,8 +584,8 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.b_group_stride = n * k; p.accumulate = 0;
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && k < (1ll << 30))
-    rc = dtype == DH_BF16 ? launch_gg_nt_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_nt_dma<f16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST>(p, max_rows, (hipStream_t)stream);
+    rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_dma<f16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream);
   else
     rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;
@@ -570,7 +605,12 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = n; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0;
-  rc = dispatch_gg<false, true, false>(p, max_rows, dtype, (hipStream_t)stream);
+  const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
+  if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
+    rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_dma<f16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream);
+  else
+    rc = dispatch_gg<false, true, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;

@@ -102,7 +102,10 @@ def test_permute_roundtrip_identity():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,N,K", [([300, 212], 512, 256), ([1000, 0, 24], 1024, 520), ([2048, 2048], 2048, 1024),
-                                       ([5], 64, 64)])
+                                       ([5], 64, 64),
+                                       # enough 256x256 tiles for the direct global->LDS kernels (NT and NN), with an
+                                       # empty group, a 37-row group and three k slices
+                                       ([2100, 0, 1990, 37], 4096, 192)])
 def test_grouped_gemm_variants(dtype, rows, N, K):
     from dhellam_amd.operators import moe
     G = len(rows)

@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = pair32_max(mx);
       const float m_new = fmaxf(m_run, mx);
       if (__any(m_new > m_run)) {
         const float alpha = fast_exp2((m_run - m_new) * p.scale_log2);
@@ -186,7 +186,7 @@ __global__ void __launch_bounds__(64 * NW) attn_fwd_kernel(const AttnFwdParams p
     __syncthreads();
   }
 
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float l_tot = pair32_sum(l_run);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   if (row_q < sq) {
     T *op = reinterpret_cast<T *>(p.o) + (int64_t)(q0 + row_q) * p.o_stride + (int64_t)h * D;
@@ -457,7 +457,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, S[nb][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = pair32_max(mx);
       // Lazy rescale: the running maximum is only a reference point for the exponentials, so it may lag
       // the true maximum.  It is moved (and O, l rescaled) only when some row of the wavefront has grown
       // past it by more than DH_FWD_RESCALE_LOG2 binades; until then P <= 2^DH_FWD_RESCALE_LOG2, which
@@ -561,7 +561,7 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
           for (int v = 0; v < 16; ++v) O[t][v] = O[t][v] * a_me + src[(t * 16 + v) * 64 + lane] * a_o;
         m_run = m_new;
       }
-      const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+      const float l_tot = pair32_sum(l_run);
       const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
       if (row_q < sq) {
         T *op = reinterpret_cast<T *>(p.o) + (int64_t)(q0 + row_q) * p.o_stride + (int64_t)h * D;

@@ -223,6 +223,18 @@ __device__ __forceinline__ void dma_tile32_general(T *dst, const T *g, int strid
   }
 }
 
+// Reductions over the lane pair (l, l ^ 32) with v_permlane32_swap (VALU) instead of a shuffle through the
+// LDS crossbar: swapping the upper half of one copy of x with the lower half of another leaves, in every
+// lane, its own value in one result and its partner's in the other.
+__device__ __forceinline__ float pair32_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair32_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Row index inside a 32-row accumulator block held by register v of lane half h.
 __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 

@@ -78,6 +78,7 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     ([1024], [2048], 8, 2, 128, False),          # ring 'upper' shape
     ([384, 129], [384, 129], 4, 4, 128, True),   # MHA at d 128: dK/dV written directly (no head split)
     ([128] * 4, [512] * 4, 64, 16, 128, False),  # many kv heads: two query heads per dK/dV workgroup
+    ([0, 65, 33], [0, 65, 33], 4, 2, 128, True),   # an empty sequence in the batch
 ])
 def test_attention_16bit(dtype, lens_q, lens_k, hq, hk, d, causal):
     _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal)

@@ -196,10 +196,15 @@ def fa_cp_block_bwd(dout, out, q, dq, kv, dkv_, softmax_lse, rng_states, cu_seql
             cq, mq, ck, mk, cz = cu_seqlens_q, max_seqlen_q, cu_seqlens_k, max_seqlen_k, False
             first_touch_all = i == 0
             dq_rows = dq
-        if b != 1 and (dk_.data_ptr() != dkv[0].data_ptr() or not dk_.is_contiguous()):
-            raise RuntimeError("ring backward with batch > 1 needs contiguous dK/dV views")
+        # With batch > 1 the first-half views of an 'L' step are not contiguous: _rows() then hands out
+        # packed temporaries, and the results are copied back into the views.
+        dkv_is_temp = dk_.data_ptr() != dkv[0].data_ptr()
         dq_step = torch.empty(q_.shape, dtype=q.dtype, device=q.device)
         _Clib._attn_bwd_raw(do_, q_, k_, v_, o_, lse_, dq_step, dk_, dv_, None, cq, ck, mq, mk, scale, cz, sp)
+        if dkv_is_temp:
+            assert causal and case == "L"
+            dkv[0][:, 0].copy_(dk_.view(b, c, hk, d))
+            dkv[1][:, 0].copy_(dv_.view(b, c, hk, d))
         dq_step = dq_step.view(dq_rows.shape)
         # dq: the first contribution to a row is a copy, later ones add (ring_attn.py:391-408).
         if first_touch_all:

@@ -182,7 +182,7 @@ def _ring_gpu(q, chunks, dout, rank, cp):
 
 
 @pytest.mark.parametrize("dtype,b,c,hq,hk,d", [(torch.bfloat16, 1, 128, 4, 2, 128), (torch.bfloat16, 1, 96, 2, 2, 64),
-                                                 (torch.float32, 1, 48, 2, 1, 32)])
+                                                 (torch.float32, 1, 48, 2, 1, 32), (torch.bfloat16, 2, 64, 4, 2, 128)])
 @pytest.mark.parametrize("rank", [0, 1, 3])
 def test_ring_step_matches_oracle_and_dense(dtype, b, c, hq, hk, d, rank):
     cp = 4

@@ -265,6 +265,13 @@ def profile_op(name: str, iters: int = 5):
             y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
             dyp = rn(Rm, Hm)
             fn = lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved)
+    elif name == "layer":
+        # the serial schedule alone: four micro-batches of the 70B-shard layer, forward + backward
+        from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
+        cfg = llama70b_tp8_shard()
+        runner = LayerRunner(cfg, make_weights(cfg, 0, gen_device="cuda"))
+        mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(4)]
+        fn = lambda: runner.run_serial(mbs)
     else:
         raise SystemExit(f"unknown --profile-op {name}")
     for _ in range(iters):
@@ -282,7 +289,7 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
-                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, copy) and exit")
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, layer, copy) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "

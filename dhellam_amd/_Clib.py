@@ -10,6 +10,7 @@ merge, MoE, grouped GEMM) are exported under ``py*`` names in the same style.
 from __future__ import annotations
 
 import ctypes as C
+from typing import Optional
 
 import torch
 
@@ -55,8 +56,11 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
     """
     _lib.need_cuda(inputA, inputB, outputD)
     a = inputA.t() if transa else inputA
-    b = inputB.t() if transb else inputB
     stream = torch.cuda.current_stream()
+    if transb and not transa:
+        b = wgrad_lhs(inputB, inputA.shape[1])
+    else:
+        b = inputB.t() if transb else inputB
 
     def run():
         if grad_accumulate:
@@ -65,6 +69,38 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
             torch.matmul(b, a, out=outputD)
 
     return _timed(profiling, stream, run)
+
+
+def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row-major [rows, cols] -> row-major [cols, rows] (16-bit elements) on the current stream."""
+    _lib.need_cuda(src)
+    if not (src.dim() == 2 and src.stride(1) == 1):
+        raise RuntimeError("transpose_2d: src must be 2-D with unit inner stride")
+    rows, cols = src.shape
+    if out is None:
+        out = torch.empty((cols, rows), dtype=src.dtype, device=src.device)
+    elif not (out.shape == (cols, rows) and out.stride(1) == 1 and out.dtype == src.dtype):
+        raise RuntimeError("transpose_2d: out must be [cols, rows] of src's dtype with unit inner stride")
+    _lib.check(_lib.load().dh_transpose_2d(src.data_ptr(), out.data_ptr(), rows, cols, src.stride(0), out.stride(0),
+                                           _lib.dt(src), torch.cuda.current_stream().cuda_stream))
+    return out
+
+
+# The weight-gradient product dW[N, K] = dY[T, N]^T X[T, K] runs ~20 % faster in the GEMM library when dY^T is
+# row-major (measured at T = 4096: N, K = 7168, 8192: 482 -> 408 us; 8192, 3584: 257 -> 198 us), and the
+# transpose costs T N / (1 element per ps): it pays from K of about 2000.
+WGRAD_TRANSPOSE_MIN_K = 2048
+WGRAD_TRANSPOSE_MIN_ELEMS = 1 << 20
+
+
+def wgrad_lhs(grad: torch.Tensor, k: int) -> torch.Tensor:
+    """Left operand dY^T of the weight-gradient product for ``grad`` = dY [T, N] and an X of ``k`` columns:
+    a materialised row-major transpose where that makes the product faster, else the strided view."""
+    t, n = grad.shape
+    if (grad.dtype in (torch.bfloat16, torch.float16) and grad.is_contiguous() and k >= WGRAD_TRANSPOSE_MIN_K
+            and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and t % 8 == 0 and n % 8 == 0 and grad.data_ptr() % 16 == 0):
+        return transpose_2d(grad)
+    return grad.t()
 
 
 def pygelu(input, output, profiling):

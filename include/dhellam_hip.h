@@ -238,6 +238,13 @@ int dh_grouped_gemm_tn(const void *a, const void *b, void *c,
  * dhellam/core/dstb.py) when one GPU holds the whole sequence. */
 int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
 
+/* out[c * ld_out + r] = in[r * ld_in + c] for a [rows, cols] matrix of 16-bit elements
+ * (bf16 / fp16; rows, cols and both leading dimensions multiples of 8).  Feeds the
+ * weight-gradient product of the reference's GEMM operator (csrc/operators/gemm.cu:3-170 called
+ * with transb: D = B^T A) with a row-major B^T, the layout the GEMM library runs fastest. */
+int dh_transpose_2d(const void *in, void *out, int64_t rows, int64_t cols, int64_t ld_in,
+                    int64_t ld_out, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -142,3 +142,46 @@ def test_legacy_kernels():
     assert_close(o, O.bias_mask_add(x, b, r), torch.float16)
     s = _Clib.add_tensors(x.cuda(), b.cuda())
     assert torch.equal(s.cpu(), x + b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(8, 8), (64, 256), (72, 264), (4096, 1280), (1000, 24), (16, 4104)])
+def test_transpose_2d(dtype, rows, cols):
+    from dhellam_amd import _Clib
+    x = randn((rows, cols), dtype, rows + cols).cuda()
+    assert torch.equal(_Clib.transpose_2d(x), x.t().contiguous())
+    # strided source and destination: a column block of a wider matrix into a row block of a wider one
+    wide = randn((rows, cols + 16), dtype, 3).cuda()
+    out = torch.full((cols, rows + 8), 7.0, dtype=dtype, device="cuda")
+    _Clib.transpose_2d(wide[:, 8:8 + cols], out[:, :rows])
+    assert torch.equal(out[:, :rows], wide[:, 8:8 + cols].t())
+    assert bool((out[:, rows:] == 7.0).all())
+
+
+def test_transpose_2d_rejects():
+    from dhellam_amd import _Clib
+    with pytest.raises(RuntimeError):
+        _Clib.transpose_2d(torch.zeros(12, 16, dtype=torch.bfloat16, device="cuda"))     # rows not a multiple of 8
+    with pytest.raises(RuntimeError):
+        _Clib.transpose_2d(torch.zeros(16, 16, dtype=torch.float32, device="cuda"))      # 32-bit elements
+    assert _Clib.transpose_2d(torch.zeros(0, 16, dtype=torch.bfloat16, device="cuda")).shape == (16, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,N,K", [(1024, 1024, 2048), (512, 96, 4096), (1024, 1032, 1024)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_wgrad_product(dtype, T, N, K, accumulate):
+    """dW = dY^T X through both operator entry points, with and without the materialised dY^T."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.layernorm_column import wgrad_bwd
+    dy, x = randn((T, N), dtype, 11, std=0.5), randn((T, K), dtype, 12, std=0.5)
+    w0 = randn((N, K), dtype, 13)
+    ref = dy.double().t() @ x.double() + (w0.double() if accumulate else 0)
+    took_copy = _Clib.wgrad_lhs(dy.cuda(), K).is_contiguous()
+    assert took_copy == (dtype != torch.float32 and K >= 2048 and T * N >= 1 << 20)
+    d = w0.clone().cuda()
+    _Clib.pygemm(x.cuda(), dy.cuda(), d, None, 0, False, True, accumulate, 0, False)
+    assert_close(d, ref, dtype, "pygemm wgrad")
+    d2 = w0.clone().cuda() if accumulate else None
+    d2, _ = wgrad_bwd(None, dy.cuda(), x.cuda(), d2, accumulate, "NT", False, 0, True, None)
+    assert_close(d2, ref, dtype, "wgrad_bwd")

@@ -55,11 +55,11 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
     ``input_workspace`` / ``workspaceSize`` / ``math_sm_count`` are accepted and unused.
     """
     _lib.need_cuda(inputA, inputB, outputD)
-    a = inputA.t() if transa else inputA
     stream = torch.cuda.current_stream()
     if transb and not transa:
-        b = wgrad_lhs(inputB, inputA.shape[1])
+        b, a = wgrad_operands(inputB, inputA)
     else:
+        a = inputA.t() if transa else inputA
         b = inputB.t() if transb else inputB
 
     def run():
@@ -86,21 +86,32 @@ def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
-# The weight-gradient product dW[N, K] = dY[T, N]^T X[T, K] runs ~20 % faster in the GEMM library when dY^T is
-# row-major (measured at T = 4096: N, K = 7168, 8192: 482 -> 408 us; 8192, 3584: 257 -> 198 us), and the
-# transpose costs T N / (1 element per ps): it pays from K of about 2000.
-WGRAD_TRANSPOSE_MIN_K = 2048
+# The weight-gradient product dW[N, K] = dY[T, N]^T X[T, K] reads both operands along their strided dimension, the
+# GEMM library's slowest layout here.  Measured at T = 4096, bf16, accumulating (us; N, K = 7168, 8192 / 8192, 3584 /
+# 1280, 8192 / 8192, 1024):   as given 484 / 233-257 / 95 / 76;   dY^T row-major 409 / 203 / 82 / 67;
+# dY^T and X^T both row-major 364 / 178 / 70 / 60.  dh_transpose_2d moves 5.5-6 TB/s (a [4096, 8192] matrix in
+# 24 us), so materialising dY^T pays from K of about 3000 and X^T as well from N of about 4000.
+WGRAD_TRANSPOSE_GRAD_MIN_K = 3072
+WGRAD_TRANSPOSE_DATA_MIN_N = 4096
 WGRAD_TRANSPOSE_MIN_ELEMS = 1 << 20
 
 
-def wgrad_lhs(grad: torch.Tensor, k: int) -> torch.Tensor:
-    """Left operand dY^T of the weight-gradient product for ``grad`` = dY [T, N] and an X of ``k`` columns:
-    a materialised row-major transpose where that makes the product faster, else the strided view."""
-    t, n = grad.shape
-    if (grad.dtype in (torch.bfloat16, torch.float16) and grad.is_contiguous() and k >= WGRAD_TRANSPOSE_MIN_K
-            and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and t % 8 == 0 and n % 8 == 0 and grad.data_ptr() % 16 == 0):
-        return transpose_2d(grad)
-    return grad.t()
+def _can_transpose(t: torch.Tensor) -> bool:
+    return (t.dtype in (torch.bfloat16, torch.float16) and t.dim() == 2 and t.is_contiguous()
+            and t.shape[0] % 8 == 0 and t.shape[1] % 8 == 0 and t.data_ptr() % 16 == 0)
+
+
+def wgrad_operands(grad: torch.Tensor, data: torch.Tensor):
+    """(lhs, rhs) with lhs @ rhs = grad^T @ data for grad = dY [T, N], data = X [T, K]: the strided views, or
+    materialised row-major transposes of dY (and X) where that makes the product faster by more than they cost."""
+    (t, n), k = grad.shape, data.shape[1]
+    if (k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad)
+            and grad.dtype == data.dtype):
+        lhs = transpose_2d(grad)
+        if n >= WGRAD_TRANSPOSE_DATA_MIN_N and _can_transpose(data):
+            return lhs, transpose_2d(data).t()
+        return lhs, data
+    return grad.t(), data
 
 
 def pygelu(input, output, profiling):

@@ -17,7 +17,7 @@ from typing import Optional
 import torch
 
 from .._Clib import pygemm as gemm
-from .._Clib import wgrad_lhs
+from .._Clib import wgrad_operands
 from ._util import on_stream
 
 
@@ -71,8 +71,11 @@ def wgrad_bwd(args, input_grad: torch.Tensor, input_data: torch.Tensor, wgrad_ou
     el: list = []
     with on_stream(stream, profiling, el):
         if is_matmul:
-            d = input_data.t() if transa else input_data
-            g = (wgrad_lhs(input_grad, d.shape[1]) if not transa else input_grad.t()) if transb else input_grad
+            if transb and not transa:
+                g, d = wgrad_operands(input_grad, input_data)
+            else:
+                d = input_data.t() if transa else input_data
+                g = input_grad.t() if transb else input_grad
             if wgrad_output is None:
                 wgrad_output = torch.matmul(g, d)
             elif wgrad_output.dtype == g.dtype:

@@ -168,17 +168,19 @@ def test_transpose_2d_rejects():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("T,N,K", [(1024, 1024, 2048), (512, 96, 4096), (1024, 1032, 1024)])
+@pytest.mark.parametrize("T,N,K", [(1024, 1024, 3072), (512, 4096, 3080), (512, 96, 4096), (1024, 1032, 1024)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_wgrad_product(dtype, T, N, K, accumulate):
-    """dW = dY^T X through both operator entry points, with and without the materialised dY^T."""
+    """dW = dY^T X through both operator entry points, with and without materialised transposes."""
     from dhellam_amd import _Clib
     from dhellam_amd.operators.layernorm_column import wgrad_bwd
     dy, x = randn((T, N), dtype, 11, std=0.5), randn((T, K), dtype, 12, std=0.5)
     w0 = randn((N, K), dtype, 13)
     ref = dy.double().t() @ x.double() + (w0.double() if accumulate else 0)
-    took_copy = _Clib.wgrad_lhs(dy.cuda(), K).is_contiguous()
-    assert took_copy == (dtype != torch.float32 and K >= 2048 and T * N >= 1 << 20)
+    lhs, rhs = _Clib.wgrad_operands(dy.cuda(), x.cuda())
+    assert lhs.is_contiguous() == (dtype != torch.float32 and K >= 3072 and T * N >= 1 << 20)
+    assert (not rhs.is_contiguous()) == (lhs.is_contiguous() and N >= 4096)
+    assert torch.equal(lhs, dy.cuda().t()) and torch.equal(rhs, x.cuda())
     d = w0.clone().cuda()
     _Clib.pygemm(x.cuda(), dy.cuda(), d, None, 0, False, True, accumulate, 0, False)
     assert_close(d, ref, dtype, "pygemm wgrad")

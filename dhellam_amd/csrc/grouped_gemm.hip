@@ -285,6 +285,8 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 // BKS: the B operand is k-strided ([k][n] row-major, the NN product).  Its tile is then [64 k][256 n] with
 // 512-byte rows, copied two k rows per block with the transpose-read swizzle (chunk ^= 4 * (k % 4) +
 // (k / 4) % 4 inside each 256-byte half row), and its fragments come from LDS transpose reads.
+template <bool B> struct BoolC { static constexpr bool value = B; };
+
 template <typename T, int WVN, int BKT, int NST, bool BKS>
 __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGParams p) {
   using M = Mma<T>;
@@ -312,7 +314,9 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
 
   // A contiguous run of tiles per XCD, m fastest (tiles that share a weight panel run together).
   // Cutting the grid into 4 x 8 super-tiles per XCD instead lowers the L2 miss traffic by a third
-  // (measured) but is slower: the bound is not the fabric.
+  // (measured) but is slower: the bound is not the fabric.  Running every full tile first and the groups'
+  // cheap last tiles afterwards (long jobs first) is slower too, by 10 %: a last tile then re-reads from HBM
+  // the weight panel that its group's full tiles shared through L2 long before.
   const int ntiles = p.tiles_m * p.tiles_n;
   int pid = blockIdx.x;
   if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
@@ -430,17 +434,27 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
 
   Frag fa[2][WM], fb[2][WN];
   // fragments of k step ks of the stage whose row-fragment bases are fa_/fb_ (byte offset stage_ for the BKS form)
-  auto load_frags = [&](int buf, uint32_t fa_, uint32_t fb_, uint32_t stage_, int ks) {
+  // nvi: how many of this wavefront's WM 32-row blocks hold rows of the group (WM except in a group's last tile)
+  auto load_frags = [&](int buf, uint32_t fa_, uint32_t fb_, uint32_t stage_, int ks, int nvi) {
 #pragma unroll
-    for (int i = 0; i < WM; ++i) fa[buf][i] = *(lds_frag)((fa_ ^ (uint32_t)(ks << 5)) + i * 32 * ROWB);
+    for (int i = 0; i < WM; ++i)
+      if (i < nvi) fa[buf][i] = *(lds_frag)((fa_ ^ (uint32_t)(ks << 5)) + i * 32 * ROWB);
+    if (nvi > 0) {
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      if constexpr (BKS) fb[buf][j] = ld_b_tr(stage_, ks, j);
-      else fb[buf][j] = *(lds_frag)((fb_ ^ (uint32_t)(ks << 5)) + j * 32 * ROWB);
+      for (int j = 0; j < WN; ++j) {
+        if constexpr (BKS) fb[buf][j] = ld_b_tr(stage_, ks, j);
+        else fb[buf][j] = *(lds_frag)((fb_ ^ (uint32_t)(ks << 5)) + j * 32 * ROWB);
+      }
     }
   };
+  // A group's last tile usually holds fewer than 256 rows.  Its wavefronts skip the 32-row blocks past the end
+  // (fragment reads and MFMAs; the copies and barriers stay), so such a tile costs what its copies cost,
+  // about a quarter of a full one, instead of a full tile's time.  The full tile keeps a branch-free loop.
+  auto slices = [&](auto partial) {
+  constexpr bool PARTIAL = decltype(partial)::value;
+  const int nvi = PARTIAL ? min(WM, max(0, (a_rext - wm * 32 * WM + 31) >> 5)) : WM;
   if constexpr (CROSS) {
-    if (nslices > 0) load_frags(0, lds0 + fa_lane, lds0 + fb_lane, lds0, 0);
+    if (nslices > 0) load_frags(0, lds0 + fa_lane, lds0 + fb_lane, lds0, 0, nvi);
   }
   int st_cur = 0, st_nxt = DIST % NST;                  // stage of slice s, stage of slice s + DIST
 #pragma unroll 1
@@ -456,17 +470,17 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
     uint32_t fa1 = lds0 + nst1 + fa_lane, fb1 = lds0 + nst1 + fb_lane;
     uint32_t sg0 = lds0 + cur, sg1 = lds0 + nst1;
     asm volatile("" : "+v"(fa0), "+v"(fb0), "+v"(fa1), "+v"(fb1), "+v"(sg0), "+v"(sg1));   // derive the other addresses here, not ahead of the loop
-    if constexpr (!CROSS) load_frags(0, fa0, fb0, sg0, 0);
+    if constexpr (!CROSS) load_frags(0, fa0, fb0, sg0, 0, nvi);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int cu = ks & 1, nx = cu ^ 1;
-      if (ks + 1 < KS) load_frags(nx, fa0, fb0, sg0, ks + 1);
-      else if (CROSS && s + 1 < nslices) load_frags(nx, fa1, fb1, sg1, 0);   // first fragments of the next slice (already published)
+      if (ks + 1 < KS) load_frags(nx, fa0, fb0, sg0, ks + 1, nvi);
+      else if (CROSS && s + 1 < nslices) load_frags(nx, fa1, fb1, sg1, 0, nvi);   // first fragments of the next slice (already published)
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
 #pragma unroll
         for (int j = 0; j < WN; ++j) {  // C^T block: rows n, cols m
-          acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
+          if (!PARTIAL || i < nvi) acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
           // one 1 KB copy block after every DH_GG_CPI MFMAs until the slice's CPB blocks are out
           const int mi = (ks * WM + i) * WN + j;
           if (mi % DH_GG_CPI == DH_GG_CPI - 1 && mi / DH_GG_CPI < CPB && fcopy) {
@@ -492,29 +506,58 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
     // wavefront's fragment reads of slice s have returned before its last MFMAs of slice s were issued.
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
+  };
+  if (a_rext >= BM) slices(BoolC<false>{});
+  else slices(BoolC<true>{});
 
-  // Epilogue: lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad.
-  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0;
+  // Epilogue.  A lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad;
+  // stored straight from there, an instruction would touch 32 rows with two 8-byte pieces each, and such
+  // scattered partial-line stores run at a fraction of the memory system's rate (the stores were 5 % of the
+  // kernel).  Each wavefront instead passes its 128x64 block through a private LDS region, 64 rows at a time,
+  // and stores whole 128-byte lines: 8 adjacent lanes cover one row, 8 rows per instruction.  The stage
+  // buffers are free: the barrier that ended the last slice came after every wavefront's last fragment read.
+  // Rows of 136 bytes: the 8-byte writes of 32 lanes (32 rows, one column) fall on 64 different banks.
+  constexpr int EP = 136;
+  static_assert(NW * 64 * EP <= NST * STAGEB, "epilogue staging fits in the stage buffers");
+  unsigned char *ep = smem + w * (64 * EP);
+  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 32 * WN;
+  struct alignas(8) Q4 { T v[4]; };
+  struct alignas(8) Q8 { Q4 lo, hi; };
+  const int er = lane >> 3, ec = lane & 7;              // row inside a step of 8 rows, 16-byte chunk of the row
 #pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    const int m = wm * 32 * WM + 32 * i + c;
+  for (int h = 0; h < WM / 2; ++h) {
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const floatx16 av = acc[i][j];
-      if (m < a_rext) {
+    for (int i2 = 0; i2 < 2; ++i2) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        const floatx16 av = acc[2 * h + i2][j];
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {
-          const int n = wn * 32 * WN + 32 * j + 8 * vb + 4 * hh;
-          if (n < b_rext) {
-            struct alignas(8) Q4 { T v[4]; };
-            Q4 o;
+          Q4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
-            *reinterpret_cast<Q4 *>(cg + (int64_t)m * p.ldc + n) = o;
-          }
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
+          *reinterpret_cast<Q4 *>(ep + (32 * i2 + c) * EP + (32 * j + 8 * vb + 4 * hh) * (int)sizeof(T)) = o;
         }
       }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const int mh = wm * 32 * WM + 64 * h;               // first row of this half in the tile
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int r = 8 * it + er;
+      const unsigned char *src = ep + r * EP + ec * 16;
+      Q8 o;
+      o.lo = *reinterpret_cast<const Q4 *>(src);
+      o.hi = *reinterpret_cast<const Q4 *>(src + 8);
+      const int n = wn * 32 * WN + 8 * ec;
+      if (mh + r < a_rext && n < b_rext) {
+        T *dst = cg + (int64_t)(mh + r) * p.ldc + 8 * ec;
+        *reinterpret_cast<dh_u32x4 *>(dst) = __builtin_bit_cast(dh_u32x4, o);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
   }
 }
 

@@ -24,6 +24,14 @@ SIGNATURES = {
     "dh_last_error": (C.c_char_p, []),
     "dh_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
     "dh_transpose_2d": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp]),
+    "dh_cross_entropy_fwd": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _f32, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _vp,
+                                    _vp, _vp]),
+    "dh_cross_entropy_bwd": (_i32, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _i32, _vp, _i64,
+                                    _vp]),
+    "dh_embedding_fwd": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp]),
+    "dh_embedding_bwd": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i32, _vp]),
+    "dh_masked_mean_fwd": (_i32, [_vp, _vp, _i64, _f32, _vp, _vp]),
+    "dh_masked_mean_bwd": (_i32, [_vp, _vp, _i64, _f32, _vp, _vp]),
     "dh_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _vp]),
     "dh_norm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "dh_norm_bwd": (_i32, [_vp] * 10 + [_i64, _i64, _i32, _i32, _i32, _vp]),

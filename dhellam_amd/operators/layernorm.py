@@ -65,6 +65,8 @@ def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_ce
     with on_stream(stream, profiling, el) as st:
         dinp = torch.empty_like(inputmat)
         accumulate = dgamma_out is not None
+        assert not accumulate or dgamma_out.dtype == ln_weight.dtype, "dgamma_out must have the weight's dtype"
+        assert dbeta_out is None or dbeta_out.dtype == ln_weight.dtype, "dbeta_out must have the weight's dtype"
         dgamma = dgamma_out if accumulate else torch.empty_like(ln_weight)
         if mu is not None:
             dbeta = dbeta_out if dbeta_out is not None else torch.empty_like(ln_weight)

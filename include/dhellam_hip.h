@@ -245,6 +245,55 @@ int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
 int dh_transpose_2d(const void *in, void *out, int64_t rows, int64_t cols, int64_t ld_in,
                     int64_t ld_out, int dtype, void *stream);
 
+/* ---- head block: word embedding, cross entropy, masked mean loss ------------------------
+ * The per-rank arithmetic of the reference's vocab-parallel head; the all-reduces that join
+ * the ranks (dhellam/operators/loss.py:22-24,52-56,61-66) are outside this library.
+ * vocab_start = tp_rank * (rows of this rank's vocabulary slice). */
+
+/* Cross entropy of `rows` rows of `cols` logits (pitch ld, any dtype; fp32 arithmetic):
+ * dhellam/operators/loss.py:15-97.  Per row: row_max = max(x), sum_exp = sum exp(x - row_max),
+ * predicted = x[target - vocab_start] - row_max (0 when the target is outside this slice),
+ * loss = log(sum_exp) - predicted, with label smoothing
+ * loss = (1 - s) loss - s mean(log softmax), s = label_smoothing cols / (cols - 1).
+ * Optional outputs (NULL to skip): predicted, softmax (dtype of the logits, pitch ld_softmax),
+ * target_mask (1 = target outside the slice), masked_target (local index, 0 where masked). */
+int dh_cross_entropy_fwd(const void *logits, const int64_t *target, int64_t rows, int64_t cols,
+                         int64_t ld, int64_t vocab_start, float label_smoothing, int dtype,
+                         float *loss, float *row_max, float *sum_exp, float *predicted,
+                         void *softmax, int64_t ld_softmax, uint8_t *target_mask,
+                         int64_t *masked_target, void *stream);
+
+/* grad = (softmax - onehot(target) (1 - s) [target inside] - s / cols) * dout[row]:
+ * dhellam/operators/loss.py:99-127.  from_logits = 0: src is the softmax of the forward;
+ * from_logits = 1: src is the logits and the softmax is recomputed from row_max / sum_exp
+ * (nothing of size rows x cols is kept between forward and backward).  grad may be src. */
+int dh_cross_entropy_bwd(const void *src, int64_t ld_src, int from_logits, const float *row_max,
+                         const float *sum_exp, const int64_t *target, const float *dout,
+                         int64_t rows, int64_t cols, int64_t vocab_start, float label_smoothing,
+                         int dtype, void *grad, int64_t ld_grad, void *stream);
+
+/* out[i, :] = vocab[ids[i] - vocab_start, :], zero rows for ids outside
+ * [vocab_start, vocab_start + vocab_rows): dhellam/operators/embedding.py:16-39. */
+int dh_embedding_fwd(const void *vocab, const int64_t *ids, int64_t n, int64_t hidden,
+                     int64_t vocab_rows, int64_t vocab_start, int dtype, void *out, void *stream);
+
+/* dvocab[v, :] += sum of dout[i, :] over the positions i with ids[i] = vocab_start + v, in
+ * position order (deterministic): the gradient autograd forms in
+ * dhellam/operators/embedding.py:42-49.  dvocab is fp32 or of dout's type. */
+int dh_embedding_bwd(const void *dout, const int64_t *ids, int64_t n, int64_t hidden,
+                     int64_t vocab_rows, int64_t vocab_start, int dtype, void *dvocab,
+                     int dvocab_dtype, void *stream);
+
+/* out[0] = scale * sum(x mask) / sum(mask), out[1] = sum(mask):
+ * dhellam/operators/loss.py:131-153 with scale = loss_scale / num_microbatch. */
+int dh_masked_mean_fwd(const float *x, const float *mask, int64_t n, float scale, float *out,
+                       void *stream);
+
+/* grad[i] = scale * mask[i] / mask_sum[0] (dhellam/operators/loss.py:155-164: the reference
+ * backpropagates a gradient of one). */
+int dh_masked_mean_bwd(const float *mask, const float *mask_sum, int64_t n, float scale,
+                       float *grad, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

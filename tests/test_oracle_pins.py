@@ -290,3 +290,87 @@ def test_grouped_ffn_matches_per_expert_loop():
     r0 = F.silu(x[:4] @ w1[0, :Fh].T) * (x[:4] @ w1[0, Fh:].T) @ w2[0].T
     r1 = F.silu(x[4:] @ w1[1, :Fh].T) * (x[4:] @ w1[1, Fh:].T) @ w2[1].T
     assert torch.allclose(y, torch.cat((r0, r1)), atol=1e-12)
+
+
+# ---- head block: embedding, vocab-parallel cross entropy, masked mean ----------------------------
+from oracle import head as OH  # noqa: E402
+
+
+@pytest.mark.parametrize("ls", [0.0, 0.1])
+def test_cross_entropy_one_rank_is_the_library_cross_entropy(ls):
+    x, t = rnd(3, 5, 11), torch.randint(0, 11, (3, 5))
+    out = OH.cross_entropy_fwd([x], t, ls)[0]
+    # the reference's smoothing is the library's with eps' = eps K / (K - 1)
+    eps = ls * 11 / 10
+    xr = x.clone().requires_grad_(True)
+    ref = F.cross_entropy(xr.view(-1, 11), t.view(-1), reduction="none", label_smoothing=eps).view(3, 5)
+    assert torch.allclose(out["loss"], ref, atol=1e-12)
+    assert torch.allclose(out["softmax"], F.softmax(x, -1), atol=1e-14)
+    dout = rnd(3, 5)
+    (ref * dout).sum().backward()
+    assert torch.allclose(OH.cross_entropy_bwd(out, dout), xr.grad, atol=1e-12)
+    # a wrong sign on the one-hot term or a missing dout would not survive this
+    assert not torch.allclose(OH.cross_entropy_bwd(out, torch.ones(3, 5)), xr.grad, atol=1e-3)
+
+
+def test_cross_entropy_sharded_with_collectives_equals_unsharded():
+    world, part = 4, 6
+    x, t = rnd(7, world * part), torch.randint(0, world * part, (7,))
+    t[0], t[1] = 0, world * part - 1                       # first id of the first rank, last id of the last
+    outs = OH.cross_entropy_fwd(list(x.split(part, -1)), t)
+    ref = F.cross_entropy(x, t, reduction="none")
+    for r, o in enumerate(outs):
+        assert torch.allclose(o["loss"], ref, atol=1e-12)
+        inside = (t >= r * part) & (t < (r + 1) * part)
+        assert torch.equal(o["target_mask"], ~inside)
+        assert torch.equal(o["masked_target_1d"], torch.where(inside, t - r * part, torch.zeros_like(t)))
+    assert torch.allclose(torch.cat([o["softmax"] for o in outs], -1), F.softmax(x, -1), atol=1e-14)
+    xr = x.clone().requires_grad_(True)
+    dout = rnd(7)
+    (F.cross_entropy(xr, t, reduction="none") * dout).sum().backward()
+    got = torch.cat([OH.cross_entropy_bwd(o, dout) for o in outs], -1)
+    assert torch.allclose(got, xr.grad, atol=1e-12)
+
+
+def test_cross_entropy_single_rank_share_closed_form():
+    """Without the collectives a rank sees only its slice: loss = logsumexp(slice) - x[target] if the target is
+    inside; otherwise the predicted logit is 0 in the max-shifted frame (loss.py:27,50), which leaves
+    logsumexp(slice) - max(slice).  Smoothing averages log softmax over the SLICE (loss.py:72,86-90)."""
+    part, rank = 5, 2
+    x, t = rnd(6, part), torch.tensor([10, 14, 3, 12, 15, 9])      # slice of rank 2 is [10, 15)
+    o = OH.cross_entropy_fwd([x], t, 0.2, collectives=False, ranks=[rank])[0]
+    lse = torch.logsumexp(x, -1)
+    inside = (t >= 10) & (t < 15)
+    nll = lse - torch.where(inside, x[torch.arange(6), (t - 10).clamp(0, part - 1)], x.max(-1)[0])
+    s = 0.2 * part / (part - 1)
+    ref = (1 - s) * nll - s * (x - lse[:, None]).mean(-1)
+    assert torch.allclose(o["loss"], ref, atol=1e-12)
+    assert torch.equal(o["target_mask"], ~inside)
+    g = OH.cross_entropy_bwd(o, torch.ones(6))
+    onehot = torch.zeros(6, part, dtype=D)
+    onehot[torch.arange(6)[inside], (t - 10)[inside]] = 1.0
+    assert torch.allclose(g, F.softmax(x, -1) - (1 - s) * onehot - s / part, atol=1e-12)
+
+
+def test_word_embedding_shards_sum_to_the_library_embedding():
+    world, part, h = 3, 4, 5
+    table, ids = rnd(world * part, h), torch.randint(0, world * part, (2, 9))
+    ids[0, 0], ids[0, 1] = 0, world * part - 1
+    outs = [OH.word_embedding_fwd(table[r * part:(r + 1) * part], ids, r, world) for r in range(world)]
+    assert torch.allclose(sum(outs), F.embedding(ids, table), atol=0)
+    assert torch.equal(OH.word_embedding_fwd(table, ids), F.embedding(ids, table))
+    tr = table.clone().requires_grad_(True)
+    dout = rnd(2, 9, h)
+    (F.embedding(ids, tr) * dout).sum().backward()
+    got = torch.cat([OH.word_embedding_bwd(dout, ids, part, r, world) for r in range(world)], 0)
+    assert torch.allclose(got, tr.grad, atol=1e-13)
+    assert torch.allclose(OH.word_embedding_bwd(dout, ids, world * part), tr.grad, atol=1e-13)
+
+
+def test_masked_mean_loss_and_its_gradient():
+    losses, mask = rnd(2, 6), torch.tensor([[1, 0, 1, 1, 0, 0], [0, 0, 1, 0, 1, 1]])
+    ref = losses[mask.bool()].mean() / 4 * 8.0
+    assert torch.allclose(OH.mask_scale_loss_fwd(losses, mask, 4, 8.0), ref, atol=1e-14)
+    lr = losses.clone().requires_grad_(True)
+    (lr[mask.bool()].mean() / 4 * 8.0).backward()
+    assert torch.allclose(OH.mask_scale_loss_bwd(losses, mask, 4, 8.0), lr.grad, atol=1e-14)

@@ -27,62 +27,61 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 // A row of `cols` elements as seen by one thread of a BT-wide block: up to NV 16-byte vectors kept in
 // registers (vector i of the thread is vector i * BT + tid of the row), the rest of the row (long rows,
-// and the cols % N tail, and rows whose pitch breaks 16-byte alignment) visited element by element from
-// memory each time.
+// the cols % N tail, and rows whose pitch breaks 16-byte alignment) visited from memory each time.
+// Column arithmetic is 32-bit and nothing per element depends on the column: with a 64-bit column
+// compare per element the backward kernel was bound by the vector ALU, not by memory (2.8 TB/s).
 template <typename T, int BT, int NV> struct RowView {
   static constexpr int N = Vec<T>::N;
   const T *row;
-  int64_t cols, nvec;       // nvec: whole aligned vectors in the row (0 when the row is not 16-byte aligned)
+  int cols, nvec;           // nvec: whole aligned vectors in the row (0 when the row is not 16-byte aligned)
   Vec<T> held[NV];
 
-  __device__ __forceinline__ void load(const T *r, int64_t c, bool vec_ok) {
+  __device__ __forceinline__ void load(const T *r, int c, bool vec_ok) {
     row = r; cols = c; nvec = vec_ok ? c / N : 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int64_t v = (int64_t)i * BT + threadIdx.x;
-      if (v < nvec) held[i] = ldg(row + v * N);
+      const int v = i * BT + (int)threadIdx.x;
+      if (v < nvec) held[i] = ldg(row + (int64_t)v * N);
     }
   }
-  // f(column, value) over this thread's share of the row
+  // f(value) over this thread's share of the row
   template <typename F> __device__ __forceinline__ void for_each(F f) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int64_t v = (int64_t)i * BT + threadIdx.x;
+      const int v = i * BT + (int)threadIdx.x;
       if (v < nvec) {
 #pragma unroll
-        for (int e = 0; e < N; ++e) f(v * N + e, to_f(held[i].v[e]));
+        for (int e = 0; e < N; ++e) f(to_f(held[i].v[e]));
       }
     }
-    for (int64_t v = (int64_t)NV * BT + threadIdx.x; v < nvec; v += BT) {
-      const Vec<T> x = ldg(row + v * N);
+    for (int v = NV * BT + (int)threadIdx.x; v < nvec; v += BT) {
+      const Vec<T> x = ldg(row + (int64_t)v * N);
 #pragma unroll
-      for (int e = 0; e < N; ++e) f(v * N + e, to_f(x.v[e]));
+      for (int e = 0; e < N; ++e) f(to_f(x.v[e]));
     }
-    for (int64_t c = nvec * N + threadIdx.x; c < cols; c += BT) f(c, to_f(row[c]));
+    for (int c = nvec * N + (int)threadIdx.x; c < cols; c += BT) f(to_f(row[c]));
   }
-  // out[column] = g(column, value), same traversal, vector stores where the loads were vectors
-  template <typename TO, typename G> __device__ __forceinline__ void map_to(TO *out, bool out_vec_ok, G g) const {
-    static_assert(sizeof(TO) == sizeof(T), "map_to keeps the element size");
-    auto emit = [&](int64_t v, const Vec<T> &x) {
-      Vec<TO> o;
+  // out[c] = g(value) for every column; same traversal, vector stores where the loads were vectors
+  // (the caller enables vectors only when `out` is as aligned as the row: a run-time choice between a vector
+  // store and element stores of the same values gets merged by the compiler into the element stores)
+  template <typename G> __device__ __forceinline__ void map_to(T *out, G g) const {
+    auto emit = [&](int v, const Vec<T> &x) {
+      Vec<T> o;
 #pragma unroll
-      for (int e = 0; e < N; ++e) o.v[e] = from_f<TO>(g(v * N + e, to_f(x.v[e])));
-      if (out_vec_ok) {
-        stg(out + v * N, o);
-      } else {
-#pragma unroll
-        for (int e = 0; e < N; ++e) out[v * N + e] = o.v[e];
-      }
+      for (int e = 0; e < N; ++e) o.v[e] = from_f<T>(g(to_f(x.v[e])));
+      stg(out + (int64_t)v * N, o);
     };
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int64_t v = (int64_t)i * BT + threadIdx.x;
+      const int v = i * BT + (int)threadIdx.x;
       if (v < nvec) emit(v, held[i]);
     }
-    for (int64_t v = (int64_t)NV * BT + threadIdx.x; v < nvec; v += BT) emit(v, ldg(row + v * N));
-    for (int64_t c = nvec * N + threadIdx.x; c < cols; c += BT) out[c] = from_f<TO>(g(c, to_f(row[c])));
+    for (int v = NV * BT + (int)threadIdx.x; v < nvec; v += BT) emit(v, ldg(row + (int64_t)v * N));
+    for (int c = nvec * N + (int)threadIdx.x; c < cols; c += BT) out[c] = from_f<T>(g(to_f(row[c])));
   }
 };
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // x <= 0 here
 
 }  // namespace
 
@@ -97,18 +96,18 @@ __global__ void __launch_bounds__(BT) ce_fwd_kernel(const T *__restrict__ logits
                                                     float *__restrict__ loss, float *__restrict__ row_max,
                                                     float *__restrict__ sum_exp, float *__restrict__ predicted,
                                                     T *__restrict__ softmax, int64_t ld_sm, uint8_t *__restrict__ tmask,
-                                                    int64_t *__restrict__ mtarget, bool vec_in, bool vec_out) {
+                                                    int64_t *__restrict__ mtarget, bool vec) {
   __shared__ float red[BT / 64];
   const int64_t r = blockIdx.x;
   RowView<T, BT, NV> rv;
-  rv.load(logits + r * ld, cols, vec_in);
+  rv.load(logits + r * ld, (int)cols, vec);
   float m = -INFINITY, sx = 0.f;
-  rv.for_each([&](int64_t, float x) { m = fmaxf(m, x); sx += x; });
+  rv.for_each([&](float x) { m = fmaxf(m, x); sx += x; });
   m = block_max<BT>(m, red);
   // (x - m) first: the difference of two close numbers is exact, the product with log2(e) then errs by
   // one rounding of a small number (x * log2(e) - m * log2(e) would lose |x| * 2^-24 of the exponent).
   float s = 0.f;
-  rv.for_each([&](int64_t, float x) { s += exp2f((x - m) * LOG2E); });
+  rv.for_each([&](float x) { s += exp2_fast((x - m) * LOG2E); });
   s = block_sum<BT>(s, red);
   if (smoothing > 0.f) sx = block_sum<BT>(sx, red);
   const int64_t t = target[r] - vocab_start;
@@ -129,7 +128,7 @@ __global__ void __launch_bounds__(BT) ce_fwd_kernel(const T *__restrict__ logits
   }
   if (softmax) {
     const float inv = 1.f / s;
-    rv.map_to(softmax + r * ld_sm, vec_out, [&](int64_t, float x) { return exp2f((x - m) * LOG2E) * inv; });
+    rv.map_to(softmax + r * ld_sm, [&](float x) { return exp2_fast((x - m) * LOG2E) * inv; });
   }
 }
 
@@ -143,22 +142,31 @@ __global__ void __launch_bounds__(BT) ce_bwd_kernel(const T *src, int64_t ld_src
                                                     const float *__restrict__ sum_exp,
                                                     const int64_t *__restrict__ target, const float *__restrict__ dout,
                                                     int64_t cols, int64_t vocab_start, float smoothing, T *grad,
-                                                    int64_t ld_grad, bool vec_in, bool vec_out) {
+                                                    int64_t ld_grad, bool vec) {
   const int64_t r = blockIdx.x;
   RowView<T, BT, NV> rv;
-  rv.load(src + r * ld_src, cols, vec_in);
+  rv.load(src + r * ld_src, (int)cols, vec);
   const int64_t t = target[r] - vocab_start;
   const bool outside = t < 0 || t >= cols;
   const int64_t mt = outside ? 0 : t;
-  const float hit = outside ? 0.f : 1.f - smoothing;
   const float all = smoothing > 0.f ? smoothing / (float)cols : 0.f;
   const float d = dout[r];
   float m = 0.f, inv = 1.f;
   if (FROM_LOGITS) { m = row_max[r]; inv = 1.f / sum_exp[r]; }
-  rv.map_to(grad + r * ld_grad, vec_out, [&](int64_t c, float x) {
-    const float p = FROM_LOGITS ? exp2f((x - m) * LOG2E) * inv : x;
-    return (p - (c == mt ? hit : 0.f) - all) * d;
-  });
+  const float k = inv * d, c0 = all * d;
+  // Nothing per element depends on the column: the target's element is computed once, by thread 0, from the
+  // source value read BEFORE the row is overwritten (grad may be src), and stored after the row.
+  float at_target = 0.f;
+  if (threadIdx.x == 0 && !outside) {
+    const float x = to_f(rv.row[mt]);
+    const float p = FROM_LOGITS ? exp2_fast((x - m) * LOG2E) * inv : x;
+    at_target = (p - (1.f - smoothing) - all) * d;
+  }
+  T *out = grad + r * ld_grad;
+  if (FROM_LOGITS) rv.map_to(out, [&](float x) { return fmaf(exp2_fast((x - m) * LOG2E), k, -c0); });
+  else rv.map_to(out, [&](float x) { return fmaf(x, d, -c0); });
+  __syncthreads();                           // the row's stores are complete before the target element is replaced
+  if (threadIdx.x == 0 && !outside) out[mt] = from_f<T>(at_target);
 }
 
 // ---- word embedding ------------------------------------------------------------------------------------
@@ -307,14 +315,17 @@ extern "C" int dh_cross_entropy_fwd(const void *logits, const int64_t *target, i
   if (rows == 0) return DH_OK;
   DH_CHECK(logits && target && loss && row_max && sum_exp, "null pointer");
   DH_CHECK(!softmax || ld_softmax >= cols, "ld_softmax=%lld < cols", (long long)ld_softmax);
-  DH_CHECK(rows < (1ll << 31), "too many rows");
+  DH_CHECK(rows < (1ll << 31) && cols < (1ll << 31), "too many rows or columns");
   const float smoothing = label_smoothing > 0.f ? label_smoothing * (float)cols / (float)(cols - 1) : 0.f;
-  const bool vin = row_vec_ok(logits, ld, dtype), vout = softmax && row_vec_ok(softmax, ld_softmax, dtype);
+  // vector accesses only when the logits and (if asked for) the softmax rows are all 16-byte aligned
+  const bool vec = row_vec_ok(logits, ld, dtype) && (!softmax || row_vec_ok(softmax, ld_softmax, dtype));
   DH_DISPATCH_DTYPE(dtype, {
-    constexpr int BT = 1024, NV = 4;
+    // 256 threads x 128 bytes held per thread: rows up to 32 KB (16384 16-bit logits) stay in registers, and a
+    // CU keeps 5-8 rows in flight (with 1024 threads and 2 rows per CU the same kernel ran at half the rate).
+    constexpr int BT = 256, NV = 8;
     hipLaunchKernelGGL((ce_fwd_kernel<T, BT, NV>), dim3((unsigned)rows), dim3(BT), 0, (hipStream_t)stream,
                        (const T *)logits, target, cols, ld, vocab_start, smoothing, loss, row_max, sum_exp, predicted,
-                       (T *)softmax, ld_softmax, target_mask, masked_target, vin, vout);
+                       (T *)softmax, ld_softmax, target_mask, masked_target, vec);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;
@@ -332,19 +343,21 @@ extern "C" int dh_cross_entropy_bwd(const void *src, int64_t ld_src, int from_lo
   DH_CHECK(src && target && dout && grad, "null pointer");
   DH_CHECK(!from_logits || (row_max && sum_exp), "recomputing the softmax needs row_max and sum_exp");
   DH_CHECK(grad == src ? ld_grad == ld_src : true, "in-place gradient needs equal pitches");
-  DH_CHECK(rows < (1ll << 31), "too many rows");
+  DH_CHECK(rows < (1ll << 31) && cols < (1ll << 31), "too many rows or columns");
   const float smoothing = label_smoothing > 0.f ? label_smoothing * (float)cols / (float)(cols - 1) : 0.f;
-  const bool vin = row_vec_ok(src, ld_src, dtype), vout = row_vec_ok(grad, ld_grad, dtype);
+  const bool vec = row_vec_ok(src, ld_src, dtype) && row_vec_ok(grad, ld_grad, dtype);
   DH_DISPATCH_DTYPE(dtype, {
-    constexpr int BT = 1024, NV = 4;
+    // 256 threads x 128 bytes held per thread: rows up to 32 KB (16384 16-bit logits) stay in registers, and a
+    // CU keeps 5-8 rows in flight (with 1024 threads and 2 rows per CU the same kernel ran at half the rate).
+    constexpr int BT = 256, NV = 8;
     if (from_logits)
       hipLaunchKernelGGL((ce_bwd_kernel<T, BT, NV, true>), dim3((unsigned)rows), dim3(BT), 0, (hipStream_t)stream,
                          (const T *)src, ld_src, row_max, sum_exp, target, dout, cols, vocab_start, smoothing, (T *)grad,
-                         ld_grad, vin, vout);
+                         ld_grad, vec);
     else
       hipLaunchKernelGGL((ce_bwd_kernel<T, BT, NV, false>), dim3((unsigned)rows), dim3(BT), 0, (hipStream_t)stream,
                          (const T *)src, ld_src, row_max, sum_exp, target, dout, cols, vocab_start, smoothing, (T *)grad,
-                         ld_grad, vin, vout);
+                         ld_grad, vec);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;

@@ -159,13 +159,24 @@ moe_gather_kernel(const T *__restrict__ x, const int32_t *__restrict__ sorted_id
     const T *src = x + t * hidden;
     T *dst = permuted + r * hidden;
     if (vec_ok) {
-      for (int64_t c = threadIdx.x; c < hidden / N; c += 256) {
-        Vec<T> v = ldg(src + c * N);
-        if (row_scale) {
+      // four vectors in flight per lane: a row is only hidden / N / 256 (2 at hidden 4096) steps long, and one
+      // load per step left the copy latency-bound
+      const int64_t nv = hidden / N;
+      for (int64_t c0 = threadIdx.x; c0 < nv; c0 += 4 * 256) {
+        Vec<T> v[4];
 #pragma unroll
-          for (int j = 0; j < N; ++j) v.v[j] = from_f<T>(to_f(v.v[j]) * sc);
+        for (int u = 0; u < 4; ++u)
+          if (c0 + u * 256 < nv) v[u] = ldg(src + (c0 + u * 256) * N);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (c0 + u * 256 < nv) {
+            if (row_scale) {
+#pragma unroll
+              for (int j = 0; j < N; ++j) v[u].v[j] = from_f<T>(to_f(v[u].v[j]) * sc);
+            }
+            stg(dst + (c0 + u * 256) * N, v[u]);
+          }
         }
-        stg(dst + c * N, v);
       }
     } else {
       for (int64_t c = threadIdx.x; c < hidden; c += 256) dst[c] = row_scale ? from_f<T>(to_f(src[c]) * sc) : src[c];

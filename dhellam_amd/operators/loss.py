@@ -8,8 +8,16 @@ exponential sum) and the backward recomputes the softmax from the logits, which 
 between.  ``output_dict["softmax"]`` is then None.
 
 The all-reduces over the tensor-parallel group (loss.py:22-24,52-56,61-66) are the caller's:
-with a world size above one the outputs are this rank's share (row_max, sum_exp and predicted
-are what it would contribute).
+with a world size above one the outputs are this rank's share.  The ranks join their row
+statistics as
+
+    M = max_r row_max_r,   S = sum_r sum_exp_r * exp(row_max_r - M),
+    P = sum over the rank that holds the target of (predicted_r + row_max_r - M),
+    loss = log S - P,
+
+(two all-reduces of [rows] floats instead of the reference's three) and each rank's share of
+the gradient comes from ``cross_entropy_bwd`` with ``row_max`` / ``sum_exp`` in its context
+replaced by M / S (``keep_softmax=False``; a kept softmax is normalised by the rank's own sum).
 """
 from __future__ import annotations
 

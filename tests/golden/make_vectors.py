@@ -136,6 +136,21 @@ def route_topk(logits, k):
     return idx, gate
 
 
+def cross_entropy(x, target, label_smoothing):
+    """Per row: loss = log sum exp(x) - x[target]; with label smoothing eps over K classes
+    loss = (1 - a) loss - a mean(log softmax), a = eps K / (K - 1)."""
+    rows, k = x.shape
+    loss = np.zeros(rows)
+    for r in range(rows):
+        m = max(x[r])
+        lse = m + math.log(sum(math.exp(t - m) for t in x[r]))
+        loss[r] = lse - x[r, target[r]]
+        if label_smoothing > 0:
+            a = label_smoothing * k / (k - 1)
+            loss[r] = (1 - a) * loss[r] - a * sum(t - lse for t in x[r]) / k
+    return loss
+
+
 def main():
     rng = np.random.default_rng(20240521)
     v = {}
@@ -194,6 +209,30 @@ def main():
     lg[7, :] = 0.5
     idx, gate = route_topk(lg.astype(np.float64), 2)
     v.update(route_logits=lg, route_idx=idx, route_gate=gate)
+
+    # cross entropy over 40 classes (the tests cut the logits into 4 tensor-parallel slices of 10 and join the
+    # ranks' statistics) and over 10 classes with label smoothing; gradients by finite differences of
+    # sum(loss * dout).  Embedding of the slice [20, 30): a gather, and its gradient a scatter-add.
+    # (drawn from their own generator so that the vectors above keep their values)
+    rng2 = np.random.default_rng(977)
+    cx, cd = rnd(rng2, 6, 40, std=2.0), rnd(rng2, 6)
+    ct = np.array([20, 29, 5, 0, 39, 27], np.int64)
+    xd, dd = cx.astype(np.float64), cd.astype(np.float64)
+    v.update(ce_x=cx, ce_target=ct, ce_dout=cd, ce_loss=cross_entropy(xd, ct, 0.0),
+             ce_grad=fd_grad(lambda t: float((cross_entropy(t, ct, 0.0) * dd).sum()), xd.copy()))
+    sx, st = rnd(rng2, 6, 10, std=2.0), np.array([0, 9, 5, 3, 3, 7], np.int64)
+    sd = sx.astype(np.float64)
+    v.update(ce_ls_x=sx, ce_ls_target=st, ce_ls_loss=cross_entropy(sd, st, 0.1),
+             ce_ls_grad=fd_grad(lambda t: float((cross_entropy(t, st, 0.1) * dd).sum()), sd.copy()))
+    etab, eids, edo = rnd(rng2, 10, 16), np.array([[20, 3, 29, 20], [31, 25, 20, 29]], np.int64), rnd(rng2, 2, 4, 16)
+    eout, egrad = np.zeros((2, 4, 16)), np.zeros((10, 16))
+    for i in range(2):
+        for j in range(4):
+            t = eids[i, j] - 20
+            if 0 <= t < 10:
+                eout[i, j] = etab[t]
+                egrad[t] += edo[i, j].astype(np.float64)
+    v.update(emb_table=etab, emb_ids=eids, emb_dout=edo, emb_out=eout, emb_grad=egrad)
 
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.npz")
     np.savez_compressed(path, **v)

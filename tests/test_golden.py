@@ -15,6 +15,7 @@ import pytest
 import torch
 
 from oracle import attention as OA
+from oracle import head as OH
 from oracle import moe as OM
 from oracle import ops as O
 from tests.util import assert_close, rel_err
@@ -82,9 +83,70 @@ def test_oracle_merge_and_route():
     assert np.abs(gate - V["route_gate"]).max() < 1e-12
 
 
+def test_oracle_cross_entropy_and_embedding():
+    # 40 classes in 4 tensor-parallel slices, joined by the oracle's explicit collectives
+    outs = OH.cross_entropy_fwd(list(t("ce_x").split(10, -1)), t("ce_target"))
+    for o in outs:
+        close64(o["loss"], "ce_loss", 1e-12)
+    close64(torch.cat([OH.cross_entropy_bwd(o, t("ce_dout")) for o in outs], -1), "ce_grad")
+    # one rank, label smoothing
+    o = OH.cross_entropy_fwd([t("ce_ls_x")], t("ce_ls_target"), 0.1)[0]
+    close64(o["loss"], "ce_ls_loss", 1e-12)
+    close64(OH.cross_entropy_bwd(o, t("ce_dout")), "ce_ls_grad")
+    close64(OH.word_embedding_fwd(t("emb_table"), t("emb_ids"), 2, 4), "emb_out", 0)
+    close64(OH.word_embedding_bwd(t("emb_dout"), t("emb_ids"), 10, 2, 4), "emb_grad", 1e-14)
+
+
 # ------------------------------------------------------------------------------------------
 # GPU: the HIP path reproduces the vectors
 # ------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_hip_cross_entropy_and_embedding(dtype):
+    """The 40-class vector through FOUR ranks' kernels: each rank's statistics of its 10-column slice, joined the way
+    the all-reduces of the reference join them (max of maxima, rescaled sums, summed target logits), then each
+    rank's share of the gradient from the joined statistics."""
+    from dhellam_amd.common import parallel_state as ps
+    from dhellam_amd.operators.embedding import word_embedding_bwd, word_embedding_fwd
+    from dhellam_amd.operators.loss import cross_entropy_bwd, cross_entropy_fwd
+    try:
+        x, tgt, dout = t("ce_x", dtype).cuda(), t("ce_target").cuda(), t("ce_dout", torch.float32).cuda()
+        ctxs = []
+        for r in range(4):
+            ps.set_tensor_model_parallel(r, 4)
+            inputs = {"vocab_parallel_logits": x[:, 10 * r:10 * r + 10].contiguous(), "target": tgt}
+            ctxs.append([inputs, cross_entropy_fwd(inputs, 0.0, keep_softmax=False)])
+        m = torch.stack([c[1]["row_max"] for c in ctxs])
+        big = m.amax(0)
+        ssum = sum(c[1]["sum_exp"] * torch.exp(c[1]["row_max"] - big) for c in ctxs)
+        pred = sum(torch.where(c[1]["target_mask"], torch.zeros_like(big), c[1]["predicted"] + c[1]["row_max"] - big)
+                   for c in ctxs)
+        assert_close(torch.log(ssum) - pred, t("ce_loss"), torch.float32, "loss", scale=4)
+        grads = []
+        for r, c in enumerate(ctxs):
+            ps.set_tensor_model_parallel(r, 4)
+            c[1]["row_max"], c[1]["sum_exp"] = big, ssum
+            grads.append(cross_entropy_bwd(c, dout))
+        assert_close(torch.cat(grads, -1), t("ce_grad"), dtype, "grad")
+        # one rank, label smoothing, softmax kept and recomputed
+        ps.set_tensor_model_parallel(0, 1)
+        for keep in (True, False):
+            inputs = {"vocab_parallel_logits": t("ce_ls_x", dtype).cuda(), "target": t("ce_ls_target").cuda()}
+            out = cross_entropy_fwd(inputs, 0.1, keep_softmax=keep)
+            assert_close(out["loss"], t("ce_ls_loss"), torch.float32, "smoothed loss", scale=4)
+            assert_close(cross_entropy_bwd([inputs, out], dout), t("ce_ls_grad"), dtype, "smoothed grad")
+        ps.set_tensor_model_parallel(2, 4)
+        table = t("emb_table", dtype).cuda()
+        inputs = {"vocab": table, "token_ids": t("emb_ids").cuda()}
+        out = word_embedding_fwd(inputs)
+        assert torch.equal(out["word_embeddings"].double().cpu(), t("emb_out"))
+        table.main_grad = torch.zeros(10, 16, dtype=torch.float32, device="cuda")
+        word_embedding_bwd([inputs, out], t("emb_dout", dtype).cuda())
+        assert_close(table.main_grad, t("emb_grad"), torch.float32, "embedding grad")
+    finally:
+        ps.set_tensor_model_parallel(0, 1)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["rms", "ln"])

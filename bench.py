@@ -171,37 +171,6 @@ def kernel_rooflines(cfg):
     ms = time_gpu_graph(lambda: _Clib.pyattn_merge(outs, lses, [0] * 4, [S1] * 4, om, lm))
     add("attn_merge[4 steps x 4096x32x128]", "hbm", 5 * S1 * hq1 * d * e + 5 * 4 * S1 * hq1, ms, "(n+1)THde+(n+1)4TH bytes")
     del q1, k1, v1, do1, outs, lses, om, dq1, dk1, dv1, o1
-    # --- head block: Llama-3.1 vocabulary 128256 over TP = 8 (16032 columns), one micro-batch of 4096 tokens ----
-    from dhellam_amd.common import parallel_state
-    from dhellam_amd.operators.embedding import word_embedding_bwd, word_embedding_fwd
-    from dhellam_amd.operators.loss import cross_entropy_bwd, cross_entropy_fwd
-    from dhellam_amd import _lib as L
-    Vp = 128256 // 8
-    parallel_state.set_tensor_model_parallel(0, 8)
-    logits = (rn(T, Vp).float() * 3).to(dt)
-    tgt = torch.randint(0, 128256, (T,), generator=g, device=dev)
-    ce_in = {"vocab_parallel_logits": logits, "target": tgt}
-    ms = time_gpu_graph(lambda: cross_entropy_fwd(ce_in, 0.0, keep_softmax=False))
-    add(f"cross_entropy_fwd[{T}x{Vp}]", "hbm", T * Vp * e + 20 * T, ms, "TVe+20T bytes (loss and row statistics only)")
-    ce_out = cross_entropy_fwd(ce_in, 0.0, keep_softmax=False)
-    dl, gbuf = torch.randn(T, generator=g, device=dev), torch.empty_like(logits)
-    ms = time_gpu_graph(lambda: cross_entropy_bwd([ce_in, ce_out], dl, grad_out=gbuf))
-    add(f"cross_entropy_bwd[{T}x{Vp}]", "hbm", 2 * T * Vp * e + 20 * T, ms, "2TVe+20T bytes (softmax recomputed from the logits)")
-    del logits, gbuf, ce_out
-    table = rn(Vp, H)
-    ids = torch.randint(0, 128256, (1, T), generator=g, device=dev)
-    ids[0, : T // 2] = torch.randint(0, Vp, (T // 2,), generator=g, device=dev)   # every rank sees ~1/8 in real runs; here 9/16
-    inside = int(((ids >= 0) & (ids < Vp)).sum().item())
-    em_in = {"vocab": table, "token_ids": ids}
-    ms = time_gpu_graph(lambda: word_embedding_fwd(em_in))
-    add(f"embedding_fwd[{T}x{H}, {inside} ids inside]", "hbm", (inside + T) * H * e + 8 * T, ms, "(Tin+T)He+8T bytes")
-    table.main_grad = torch.zeros(Vp, H, device=dev, dtype=torch.float32)
-    dh_ = rn(1, T, H)
-    em_out = word_embedding_fwd(em_in)
-    ms = time_gpu_graph(lambda: word_embedding_bwd([em_in, em_out], dh_))
-    add(f"embedding_bwd[{T}x{H}, {inside} ids inside]", "hbm", inside * H * (e + 8) + 8 * T, ms, "Tin*H(e+8)+8T bytes (fp32 main_grad read+write)")
-    parallel_state.set_tensor_model_parallel(0, 1)
-    del table, dh_, em_out
     # --- MoE: 8192 tokens, 8 experts top-2, hidden 4096, expert FFN 14336, this rank holds experts 0,1 ----
     Tm, Hm, E, K, Fm = 8192, 4096, 8, 2, 14336
     logits = torch.randn(Tm, E, generator=g, device=dev)
@@ -223,6 +192,52 @@ def kernel_rooflines(cfg):
     dyp = rn(Rm, Hm)
     ms = time_gpu(lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved), iters=5, warmup=2)
     add(f"moe_expert_ffn_bwd[R={Rm} H={Hm} F={Fm}]", "mfma", 12.0 * Rm * Hm * Fm, ms, "12RHF flop")
+    # --- head block: Llama-3.1 vocabulary 128256 over TP = 8 (16032 columns), one micro-batch of 4096 tokens ----
+    from dhellam_amd.common import parallel_state
+    from dhellam_amd.operators.embedding import word_embedding_bwd, word_embedding_fwd
+    from dhellam_amd.operators.loss import cross_entropy_bwd, cross_entropy_fwd
+    from dhellam_amd import _lib as L
+    Vp = 128256 // 8
+    g2 = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s: torch.randn(s, generator=g2, device=dev, dtype=torch.float32).to(dt)
+    parallel_state.set_tensor_model_parallel(0, 8)
+    logits = (rn(T, Vp).float() * 3).to(dt)
+    tgt = torch.randint(0, 128256, (T,), generator=g2, device=dev)
+    ce_in = {"vocab_parallel_logits": logits, "target": tgt}
+    ms = time_gpu_graph(lambda: cross_entropy_fwd(ce_in, 0.0, keep_softmax=False))
+    add(f"cross_entropy_fwd[{T}x{Vp}]", "hbm", T * Vp * e + 20 * T, ms, "TVe+20T bytes (loss and row statistics only)")
+    ce_out = cross_entropy_fwd(ce_in, 0.0, keep_softmax=False)
+    dl, gbuf = torch.randn(T, generator=g2, device=dev), torch.empty_like(logits)
+    ms = time_gpu_graph(lambda: cross_entropy_bwd([ce_in, ce_out], dl, grad_out=gbuf))
+    add(f"cross_entropy_bwd[{T}x{Vp}]", "hbm", 2 * T * Vp * e + 20 * T, ms, "2TVe+20T bytes (softmax recomputed from the logits)")
+    del logits, gbuf, ce_out
+    table = rn(Vp, H)
+    ids = torch.randint(0, 128256, (1, T), generator=g2, device=dev)
+    ids[0, : T // 2] = torch.randint(0, Vp, (T // 2,), generator=g2, device=dev)   # every rank sees ~1/8 in real runs; here 9/16
+    inside = int(((ids >= 0) & (ids < Vp)).sum().item())
+    em_in = {"vocab": table, "token_ids": ids}
+    ms = time_gpu_graph(lambda: word_embedding_fwd(em_in))
+    add(f"embedding_fwd[{T}x{H}, {inside} ids inside]", "hbm", (inside + T) * H * e + 8 * T, ms, "(Tin+T)He+8T bytes")
+    table.main_grad = torch.zeros(Vp, H, device=dev, dtype=torch.float32)
+    dh_ = rn(1, T, H)
+    em_out = word_embedding_fwd(em_in)
+    ms = time_gpu_graph(lambda: word_embedding_bwd([em_in, em_out], dh_))
+    add(f"embedding_bwd[{T}x{H}, {inside} ids inside]", "hbm", inside * H * (e + 8) + 8 * T, ms, "Tin*H(e+8)+8T bytes (fp32 main_grad read+write)")
+    # the whole head: final norm -> logits GEMM -> cross entropy -> masked mean, and back (GEMM-dominated)
+    from dhellam_amd.core import dshb
+    hid = rn(T, 1, H)
+    gam = torch.ones(H, device=dev, dtype=dt)
+    labels = torch.randint(0, 128256, (1, T), generator=g2, device=dev)
+    lmask = torch.ones(1, T, device=dev, dtype=torch.int64)
+    gam.main_grad = torch.zeros_like(gam)
+
+    def head_step():
+        _, hctx = dshb.post_process(hid, gam, None, labels, lmask, table, 4, 1.0)
+        dshb.post_process_bwd(hctx)
+    ms = time_gpu(head_step, iters=5, warmup=2)
+    add(f"head_block_fwd_bwd[{T}x{H} -> {Vp}]", "mfma", 6.0 * T * H * Vp, ms, "6THV flop (logits GEMM fwd, dgrad, wgrad; norm, cross entropy, loss around them)")
+    parallel_state.set_tensor_model_parallel(0, 1)
+    del table, dh_, em_out, hid
     return res
 
 

@@ -210,7 +210,8 @@ def zigzag_dense(q, chunks, rank, scale, dtype=F64):
         src = (rank - i) % cp
         ks.append(k.reshape(b, 2 * c, -1, d)); vs.append(v.reshape(b, 2 * c, -1, d))
         pos_k.append(zigzag_positions(src, cp, c))
-    K = torch.cat(ks, 1).to(dtype); V = torch.cat(vs, 1).to(dtype); pk = torch.cat(pos_k)
+    K = torch.cat(ks, 1).to(dtype); V = torch.cat(vs, 1).to(dtype); pk = torch.cat(pos_k).to(q.device)
+    pos_q = pos_q.to(q.device)
     Kx = K.repeat_interleave(hq // K.shape[2], dim=2).permute(0, 2, 1, 3)     # [b, hq, S, d]
     Vx = V.repeat_interleave(hq // V.shape[2], dim=2).permute(0, 2, 1, 3)
     Q = q.reshape(b, 2 * c, hq, d).to(dtype).permute(0, 2, 1, 3)

@@ -82,9 +82,9 @@ def grouped_ffn(xp, w1, w2, group_offs, dtype=torch.float64, round_to=None):
     base = int(group_offs[0])
     R = int(group_offs[-1]) - base
     F = w2.shape[2]
-    h = torch.zeros((R, 2 * F), dtype=dtype)
-    a = torch.zeros((R, F), dtype=dtype)
-    y = torch.zeros((R, w2.shape[1]), dtype=dtype)
+    h = torch.zeros((R, 2 * F), dtype=dtype, device=xp.device)
+    a = torch.zeros((R, F), dtype=dtype, device=xp.device)
+    y = torch.zeros((R, w2.shape[1]), dtype=dtype, device=xp.device)
     rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
     for g in range(w1.shape[0]):
         r0, r1 = int(group_offs[g]) - base, int(group_offs[g + 1]) - base

@@ -201,3 +201,24 @@ def test_ring_step_matches_oracle_and_dense(dtype, b, c, hq, hk, d, rank):
     for s in range(cp):
         assert_close(dkv[s][0], dkvo[s][0], dtype, f"ring dk[{s}]")
         assert_close(dkv[s][1], dkvo[s][1], dtype, f"ring dv[{s}]")
+
+
+def test_ring_step_full_size():
+    """The ring configuration at its full shape (q [1, 2, 2048, 32, 128], four visiting KV chunks of 8 kv heads,
+    rank 1): forward and backward against ONE dense attention over the zig-zag positions, evaluated by the
+    oracle in fp32 with its matmuls on the GPU (the [32, 4096, 16384] score tensor is 8.6 GB), gradients by
+    autograd.  16-bit tolerance."""
+    dtype, b, c, hq, hk, d, cp, rank = torch.bfloat16, 1, 2048, 32, 8, 128, 4, 1
+    q, chunks, dout = _ring_inputs(dtype, b, c, hq, hk, d, cp, seed=3)
+    scale = 1.0 / math.sqrt(d)
+    out, lse, dq, dkv = _ring_gpu(q, chunks, dout, rank, cp)
+    qr = q.cuda().float().requires_grad_()
+    cr = [(k.cuda().float().requires_grad_(), v.cuda().float().requires_grad_()) for k, v in chunks]
+    do_, lo_ = OA.zigzag_dense(qr, cr, rank, scale, dtype=torch.float32)
+    assert_close(out.view(b, 2 * c, hq, d), do_, dtype, "ring out vs dense")
+    assert_close(lse, lo_, torch.float32, "ring lse", scale=1e3)
+    (do_ * dout.cuda().float().view(b, 2 * c, hq, d)).sum().backward()
+    assert_close(dq.view(q.shape), qr.grad, dtype, "ring dq")
+    for s in range(cp):
+        assert_close(dkv[s][0], cr[s][0].grad, dtype, f"ring dk[{s}]")
+        assert_close(dkv[s][1], cr[s][1].grad, dtype, f"ring dv[{s}]")

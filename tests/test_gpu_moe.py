@@ -159,3 +159,36 @@ def test_expert_ffn_fwd_bwd():
     assert_close(dxp, xr.grad, dtype, "dxp", scale=2)
     assert_close(dw1, w1r.grad, dtype, "dw1", scale=2)
     assert_close(dw2, w2r.grad, dtype, "dw2", scale=2)
+
+
+def test_expert_ffn_full_size():
+    """The MoE rank share at its full shape (8192 tokens, top-2 of 8 experts, hidden 4096, expert FFN 14336, two
+    local experts): forward against the oracle evaluated in fp32 with the 16-bit roundings of h and a, backward
+    against fp32 autograd of the oracle (no intermediate rounding there: tolerance 2x).  The oracle's matmuls
+    run on the GPU through the library here, a few seconds instead of minutes."""
+    from dhellam_amd.operators import moe
+    dtype = torch.bfloat16
+    T, H, F, E, k = 8192, 4096, 14336, 8, 2
+    idx, gates, _ = moe.route_topk(_logits(T, E, 21).cuda(), k)
+    plan, _ = moe.sort_assignments(idx, E)
+    offs_cpu = plan.expert_offsets.cpu().numpy()
+    R = int(offs_cpu[2] - offs_cpu[0])
+    assert 3500 < R < 4700
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rn = lambda *s_, std=1.0: (torch.randn(s_, generator=g, device="cuda") * std).to(dtype)
+    x, w1, w2, dy = rn(T, H), rn(2, 2 * F, H, std=0.02), rn(2, H, F, std=0.02), rn(R, H)
+    xp, _ = moe.permute_fwd(x, plan, 0, 2, R)
+    offs = plan.expert_offsets[0:3]
+    y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
+    yo, ho, _ = OM.grouped_ffn(xp, w1, w2, offs_cpu[0:3], dtype=torch.float32, round_to=dtype)
+    assert_close(saved[0], ho, dtype, "h")
+    assert_close(y, yo, dtype, "ffn out")
+    del yo, ho
+    xr = xp.float().requires_grad_()
+    w1r, w2r = w1.float().requires_grad_(), w2.float().requires_grad_()
+    yr, _, _ = OM.grouped_ffn(xr, w1r, w2r, offs_cpu[0:3], dtype=torch.float32)
+    (yr * dy.float()).sum().backward()
+    dxp, dw1, dw2, _ = moe.expert_ffn_bwd(dy, xp, w1, w2, offs, saved)
+    assert_close(dxp, xr.grad, dtype, "dxp", scale=2)
+    assert_close(dw1, w1r.grad, dtype, "dw1", scale=2)
+    assert_close(dw2, w2r.grad, dtype, "dw2", scale=2)

@@ -311,6 +311,19 @@ def profile_op(name: str, iters: int = 5):
             y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
             dyp = rn(Rm, Hm)
             fn = lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved)
+    elif name in ("gg_nt", "gemm_nt"):
+        # one [4096, 8192] x [7168, 8192]^T product: the grouped GEMM kernel (two groups of 2048 rows, full tiles
+        # only) and the library GEMM of the same shape, for side-by-side counter runs
+        from dhellam_amd.operators import moe
+        R, N, K = 4096, 7168, 8192
+        a, c = rn(R, K), torch.empty(R, N, device=dev, dtype=dt)
+        if name == "gg_nt":
+            b = (torch.randn(2, N, K, generator=g, device=dev) * 0.02).to(dt)
+            offs = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+            fn = lambda: moe.grouped_gemm_nt(a, b, offs, out=c)
+        else:
+            b = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(dt)
+            fn = lambda: torch.matmul(a, b.t(), out=c)
     elif name == "layer":
         # the serial schedule alone: four micro-batches of the 70B-shard layer, forward + backward
         from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights

@@ -162,6 +162,7 @@ __global__ void __launch_bounds__(BT) ce_bwd_kernel(const T *src, int64_t ld_src
     const float p = FROM_LOGITS ? exp2_fast((x - m) * LOG2E) * inv : x;
     at_target = (p - (1.f - smoothing) - all) * d;
   }
+  __syncthreads();                           // ... and before any other wavefront's stores can reach that element
   T *out = grad + r * ld_grad;
   if (FROM_LOGITS) rv.map_to(out, [&](float x) { return fmaf(exp2_fast((x - m) * LOG2E), k, -c0); });
   else rv.map_to(out, [&](float x) { return fmaf(x, d, -c0); });

@@ -56,24 +56,13 @@ def _rms(x, gamma, eps):
     return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * gamma
 
 
-def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=None):
-    """cfg: hidden, heads (q heads on this rank), groups (kv heads on this rank), head_dim,
-    ffn (per rank), seq, batch, tp, tp_rank, eps, theta.  w: column_attn_weight,
-    linear_attn_weight, column_mlp_weight, linear_mlp_weight, ln_attn_weight,
-    ln_mlp_weight.  mb: x, dy [b, seq/tp, hidden] (+ sp_peer_* [b*seq, hidden] when tp > 1).
-    ``round_to``: dtype every op's output is rounded to (models a 16-bit pipeline).
-    Returns (out, grads) with grads = {x, ln_attn_weight, ln_mlp_weight, column_attn_weight,
-    linear_attn_weight, column_mlp_weight, linear_mlp_weight}."""
-    rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
+def layer_forward(cfg: dict, P: dict, x, mb: dict, dtype=torch.float64, rnd=lambda t: t):
+    """Forward of the layer on x [rows, hidden] (autograd-capable).  cfg / P / mb as in ``layer_fwd_bwd``."""
     hq, hk, d, F = cfg["heads"], cfg["groups"], cfg["head_dim"], cfg["ffn"]
     b, s, tp, rk = cfg["batch"], cfg["seq"], cfg["tp"], cfg["tp_rank"]
-    H = cfg["hidden"]
     T = b * s
     rows = T // tp
     r0, r1 = rk * rows, (rk + 1) * rows
-    P = {k: v.to(dtype).requires_grad_() for k, v in w.items()}
-    x = mb["x"].to(dtype).reshape(rows, H).requires_grad_()
-    dy = mb["dy"].to(dtype).reshape(rows, H)
 
     def gather(h, key):
         return _Gather.apply(h, mb[key].to(dtype), r0, r1) if tp > 1 else h
@@ -106,8 +95,55 @@ def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=No
     u = rnd(X2 @ P["column_mlp_weight"].T)
     m = rnd(u[:, :F] * torch.sigmoid(u[:, :F]) * u[:, F:])
     y = rnd(m @ P["linear_mlp_weight"].T)
-    out = rnd(x2 + scatter(y, "sp_peer_mlp_bwd"))
+    return rnd(x2 + scatter(y, "sp_peer_mlp_bwd"))
+
+
+def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=None):
+    """cfg: hidden, heads (q heads on this rank), groups (kv heads on this rank), head_dim,
+    ffn (per rank), seq, batch, tp, tp_rank, eps, theta.  w: column_attn_weight,
+    linear_attn_weight, column_mlp_weight, linear_mlp_weight, ln_attn_weight,
+    ln_mlp_weight.  mb: x, dy [b, seq/tp, hidden] (+ sp_peer_* [b*seq, hidden] when tp > 1).
+    ``round_to``: dtype every op's output is rounded to (models a 16-bit pipeline).
+    Returns (out, grads) with grads = {x, ln_attn_weight, ln_mlp_weight, column_attn_weight,
+    linear_attn_weight, column_mlp_weight, linear_mlp_weight}."""
+    rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
+    b, s, tp, H = cfg["batch"], cfg["seq"], cfg["tp"], cfg["hidden"]
+    rows = b * s // tp
+    P = {k: v.to(dtype).requires_grad_() for k, v in w.items()}
+    x = mb["x"].to(dtype).reshape(rows, H).requires_grad_()
+    dy = mb["dy"].to(dtype).reshape(rows, H)
+    out = layer_forward(cfg, P, x, mb, dtype, rnd)
     (out * dy).sum().backward()
     grads = {k: v.grad for k, v in P.items()}
     grads["x"] = x.grad.view(b, rows // b, H)
     return out.detach().view(b, rows // b, H), grads
+
+
+def model_fwd_bwd(cfg: dict, layers: list, word_embeddings, final_ln_weight, batches: list, loss_scale=1.0,
+                  dtype=torch.float64):
+    """A complete one-rank model (tp = 1): embedding -> the layers -> final RMSNorm -> logits against the
+    embedding table -> cross entropy -> masked mean / number of micro-batches * loss_scale, for every
+    micro-batch {"token_ids", "labels", "loss_mask"} ([b, s] each); gradients summed over the micro-batches
+    (dhellam/core/dsllm.py:43-106 with dhellam/core/dshb.py:98-112).  Returns (losses, grads) with grads keyed
+    word_embeddings, final_ln_weight, layers.<l>.<name>."""
+    from . import head as OH
+    assert cfg["tp"] == 1
+    leaf = lambda t: t.detach().to(dtype).clone().requires_grad_()        # never the caller's own tensor
+    table, gamma = leaf(word_embeddings), leaf(final_ln_weight)
+    Ps = [{k: leaf(v) for k, v in w.items()} for w in layers]
+    losses = []
+    for mb in batches:
+        b, s = mb["token_ids"].shape
+        x = OH.word_embedding_fwd(table, mb["token_ids"]).reshape(b * s, -1)
+        for P in Ps:
+            x = layer_forward(cfg, P, x, {}, dtype)
+        logits = _rms(x, gamma, cfg["eps"]) @ table.T
+        tok = OH.cross_entropy_fwd([logits.view(b, s, -1)], mb["labels"])[0]["loss"]
+        loss = OH.mask_scale_loss_fwd(tok, mb["loss_mask"], len(batches), loss_scale)
+        loss.backward()
+        losses.append(loss.detach())
+    grads = {"word_embeddings": table.grad, "final_ln_weight": gamma.grad}
+    for l, P in enumerate(Ps):
+        for k, v in P.items():
+            grads[f"layers.{l}.{k}"] = v.grad
+    return losses, grads

@@ -86,6 +86,24 @@ def test_cross_entropy_strided_rows_and_in_place_over_logits(tp):
     assert_close(xc, OH.cross_entropy_bwd(ref, dout), torch.bfloat16, "grad over logits")
 
 
+def test_cross_entropy_in_place_equals_out_of_place():
+    """Short rows, many of them: the gradient written over the logits must be bit-identical to the one written
+    to a new tensor (the target's element is read before any wavefront of the row stores)."""
+    from dhellam_amd.operators.loss import cross_entropy_bwd, cross_entropy_fwd
+    for dtype, cols in ((torch.float32, 512), (torch.bfloat16, 1536), (torch.bfloat16, 40)):
+        x = randn((8192, cols), dtype, 11, std=2.0).cuda()
+        t = _targets((8192,), 0, cols, 12).cuda()
+        dout = randn((8192,), torch.float32, 13).cuda()
+        inputs = {"vocab_parallel_logits": x, "target": t}
+        out = cross_entropy_fwd(inputs, 0.0, keep_softmax=False)
+        g1 = cross_entropy_bwd([inputs, out], dout)
+        for _ in range(3):
+            xc = x.clone()
+            inputs2 = {"vocab_parallel_logits": xc, "target": t}
+            g2 = cross_entropy_bwd([inputs2, out], dout, grad_out=xc)
+            assert torch.equal(g1, g2)
+
+
 def test_cross_entropy_extreme_logits():
     """Large offsets and a dominant class: the max shift keeps everything finite."""
     from dhellam_amd.operators.loss import cross_entropy_fwd

@@ -1,0 +1,104 @@
+"""The model shell (embedding -> layers -> head, micro-batches paired across the whole model) against the
+oracle's complete model in fp64 with autograd, and a short training run that has to make the loss fall."""
+import pytest
+import torch
+
+from oracle import layer as OL
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(dtype, hidden=256, heads=4, groups=2, ffn=512, seq=128, batch=2):
+    from dhellam_amd.core.dstb import LayerConfig
+    return LayerConfig(hidden_size=hidden, num_attention_heads=heads, num_query_groups=groups, ffn_hidden_size=ffn,
+                       seq_length=seq, micro_batch_size=batch, tensor_model_parallel_size=1, tp_rank=0,
+                       rope_theta=10000.0, params_dtype=dtype)
+
+
+def _oracle_cfg(cfg):
+    return dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
+                ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size, tp=1, tp_rank=0,
+                eps=cfg.layernorm_epsilon, theta=cfg.rope_theta)
+
+
+def _batches(cfg, vocab, n, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(n):
+        ids = torch.randint(0, vocab, (cfg.micro_batch_size, cfg.seq_length), generator=g)
+        labels = torch.randint(0, vocab, (cfg.micro_batch_size, cfg.seq_length), generator=g)
+        mask = (torch.rand(cfg.micro_batch_size, cfg.seq_length, generator=g) > 0.3).long()
+        out.append({"token_ids": ids, "labels": labels, "loss_mask": mask})
+    return out
+
+
+def _cuda(batches):
+    return [{k: v.cuda() for k, v in mb.items()} for mb in batches]
+
+
+def _floats(w):
+    return {k: v.detach().cpu() for k, v in w.items() if v.is_floating_point()}
+
+
+def test_model_step_matches_oracle_and_schedules_agree():
+    from dhellam_amd.core.dsllm import DSLLM
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        cfg, vocab, L, n = _cfg(torch.float32), 512, 2, 3
+        batches = _batches(cfg, vocab, n)
+        model = DSLLM(cfg, L, vocab, seed=3)
+        losses_o, grads_o = OL.model_fwd_bwd(_oracle_cfg(cfg), [_floats(w) for w in model.layers],
+                                             model.word_embeddings.cpu(), model.final_ln_weight.cpu(), batches, 8.0)
+        losses = model.step(_cuda(batches), double_strand=True, loss_scale=8.0)
+        torch.cuda.synchronize()
+        for i in range(n):
+            assert_close(losses[i], losses_o[i], torch.float32, f"loss[{i}]", scale=4)
+        for name, p in model.named_parameters():
+            assert_close(p.main_grad, grads_o[name], torch.float32, name, scale=10)
+        # the serial schedule (one stream, forward then backward per micro-batch) gives the same bits
+        serial = DSLLM(cfg, L, vocab, seed=3)
+        losses_s = serial.step(_cuda(batches), double_strand=False, loss_scale=8.0)
+        torch.cuda.synchronize()
+        for a, b in zip(losses, losses_s):
+            assert torch.equal(a, b)
+        for (name, p), (_, q) in zip(model.named_parameters(), serial.named_parameters()):
+            assert torch.equal(p.main_grad, q.main_grad), name
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+
+
+def test_model_trains_in_bf16():
+    """Predict the token two positions back (needs attention): bf16 parameters and gradients, fp32 master weights
+    with Adam on the host side of the loop.  The loss has to fall well below its starting value ln(vocab)."""
+    from dhellam_amd.core.dsllm import DSLLM
+    cfg, vocab, L, n = _cfg(torch.bfloat16, hidden=256, heads=4, groups=2, ffn=512, seq=128, batch=4), 256, 2, 2
+    model = DSLLM(cfg, L, vocab, seed=1)
+    params = [p for _, p in model.named_parameters()]
+    master = [p.detach().float().clone().requires_grad_() for p in params]
+    opt = torch.optim.Adam(master, lr=2e-3)
+    g = torch.Generator().manual_seed(0)
+    first = last = None
+    for step in range(60):
+        batches = []
+        for _ in range(n):
+            ids = torch.randint(0, vocab, (cfg.micro_batch_size, cfg.seq_length), generator=g)
+            labels = torch.roll(ids, 2, dims=1)
+            mask = torch.ones_like(ids)
+            mask[:, :2] = 0
+            batches.append({"token_ids": ids.cuda(), "labels": labels.cuda(), "loss_mask": mask.cuda()})
+        model.zero_grads()
+        losses = model.step(batches, double_strand=True)
+        loss = float(sum(l.float() for l in losses))
+        assert loss == loss, "NaN loss"
+        for m, p in zip(master, params):
+            m.grad = p.main_grad.float()
+        opt.step()
+        with torch.no_grad():
+            for m, p in zip(master, params):
+                p.copy_(m)
+        first = loss if first is None else first
+        last = loss
+    assert first > 5.0, first                  # ln(256) = 5.55
+    assert last < 0.5 * first, (first, last)

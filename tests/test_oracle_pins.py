@@ -374,3 +374,25 @@ def test_masked_mean_loss_and_its_gradient():
     lr = losses.clone().requires_grad_(True)
     (lr[mask.bool()].mean() / 4 * 8.0).backward()
     assert torch.allclose(OH.mask_scale_loss_bwd(losses, mask, 4, 8.0), lr.grad, atol=1e-14)
+
+
+def test_model_oracle_without_layers_is_tied_embedding_cross_entropy():
+    """The composition around the layers: embedding -> RMSNorm -> logits against the same table -> masked mean
+    cross entropy, gradients summed over micro-batches, checked against the library routines."""
+    from oracle import layer as OL
+    vocab, h, b, s = 11, 8, 2, 5
+    table, gamma = rnd(vocab, h), 1 + 0.1 * rnd(h)
+    batches = [{"token_ids": torch.randint(0, vocab, (b, s)), "labels": torch.randint(0, vocab, (b, s)),
+                "loss_mask": torch.tensor([[1, 1, 0, 1, 1], [0, 1, 1, 1, 0]])} for _ in range(2)]
+    cfg = dict(tp=1, eps=1e-5)
+    losses, grads = OL.model_fwd_bwd(cfg, [], table, gamma, batches, loss_scale=4.0)
+    tr, gr = table.clone().requires_grad_(True), gamma.clone().requires_grad_(True)
+    for i, mb in enumerate(batches):
+        x = F.embedding(mb["token_ids"], tr)
+        logits = F.rms_norm(x, (h,), gr, 1e-5) @ tr.T
+        tok = F.cross_entropy(logits.view(-1, vocab), mb["labels"].view(-1), reduction="none")
+        loss = tok[mb["loss_mask"].view(-1).bool()].mean() / 2 * 4.0
+        assert torch.allclose(losses[i], loss.detach(), atol=1e-12)
+        loss.backward()
+    assert torch.allclose(grads["word_embeddings"], tr.grad, atol=1e-12)
+    assert torch.allclose(grads["final_ln_weight"], gr.grad, atol=1e-12)

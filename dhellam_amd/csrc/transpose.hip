@@ -61,6 +61,11 @@ extern "C" int dh_transpose_2d(const void *in, void *out, int64_t rows, int64_t 
            "rows=%lld cols=%lld ld_in=%lld ld_out=%lld: sizes and leading dimensions must be multiples of 8",
            (long long)rows, (long long)cols, (long long)ld_in, (long long)ld_out);
   DH_CHECK(aligned16(in) && aligned16(out), "in/out must be 16-byte aligned");
+  {
+    const char *a = (const char *)in, *b = (const char *)out;
+    const int64_t na = (rows - 1) * ld_in * 2 + cols * 2, nb = (cols - 1) * ld_out * 2 + rows * 2;
+    DH_CHECK(a + na <= b || b + nb <= a, "in and out overlap: the transpose is not in place");
+  }
   const dim3 grid((unsigned)cdiv(cols, 256), (unsigned)cdiv(rows, 64));
   DH_CHECK(grid.y < 65536, "too many rows for one launch");
   // Plain (cached) accesses at every size: non-temporal ones measured 5-25 % slower here.

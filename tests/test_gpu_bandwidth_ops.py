@@ -164,6 +164,9 @@ def test_transpose_2d_rejects():
         _Clib.transpose_2d(torch.zeros(12, 16, dtype=torch.bfloat16, device="cuda"))     # rows not a multiple of 8
     with pytest.raises(RuntimeError):
         _Clib.transpose_2d(torch.zeros(16, 16, dtype=torch.float32, device="cuda"))      # 32-bit elements
+    sq = torch.zeros(16, 16, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError):
+        _Clib.transpose_2d(sq, sq)                                                        # not in place
     assert _Clib.transpose_2d(torch.zeros(0, 16, dtype=torch.bfloat16, device="cuda")).shape == (16, 0)
 
 

@@ -190,3 +190,17 @@ def test_wgrad_product(dtype, T, N, K, accumulate):
     d2 = w0.clone().cuda() if accumulate else None
     d2, _ = wgrad_bwd(None, dy.cuda(), x.cuda(), d2, accumulate, "NT", False, 0, True, None)
     assert_close(d2, ref, dtype, "wgrad_bwd")
+
+
+def test_bandwidth_ops_are_deterministic():
+    """Norm backward (staged column sums), SwiGLU, RoPE: two runs, same bits."""
+    from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
+    from dhellam_amd.operators.swiglu import swiglu_back
+    dt = torch.bfloat16
+    x, g, dy = randn((4096, 8192), dt, 1).cuda(), randn((8192,), dt, 2).cuda(), randn((4096, 8192), dt, 3).cuda()
+    _, _, rs, _ = pylayernorm_fwd(x, g, None, 1e-5, 0, False, None)
+    a = pylayernorm_bwd(dy, x, None, rs, g, 0, False, None)
+    b = pylayernorm_bwd(dy, x, None, rs, g, 0, False, None)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    y, gg = randn((4096, 7168), dt, 4).cuda(), randn((4096, 3584), dt, 5).cuda()
+    assert torch.equal(swiglu_back(gg, y)[0], swiglu_back(gg, y)[0])

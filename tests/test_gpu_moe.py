@@ -192,3 +192,25 @@ def test_expert_ffn_full_size():
     assert_close(dxp, xr.grad, dtype, "dxp", scale=2)
     assert_close(dw1, w1r.grad, dtype, "dw1", scale=2)
     assert_close(dw2, w2r.grad, dtype, "dw2", scale=2)
+
+
+def test_expert_ffn_is_deterministic():
+    """Two runs on the same inputs give the same bits (no atomics, fixed reduction orders), forward and backward."""
+    from dhellam_amd.operators import moe
+    dtype = torch.bfloat16
+    T, H, F, E, k = 4096, 1024, 1536, 8, 2
+    idx, gates, _ = moe.route_topk(_logits(T, E, 31).cuda(), k)
+    plan, _ = moe.sort_assignments(idx, E)
+    R = int((plan.expert_offsets[3] - plan.expert_offsets[0]).item())
+    x, dy = randn((T, H), dtype, 1).cuda(), randn((R, H), dtype, 2).cuda()
+    w1, w2 = randn((3, 2 * F, H), dtype, 3, std=0.02).cuda(), randn((3, H, F), dtype, 4, std=0.02).cuda()
+    offs = plan.expert_offsets[0:4]
+    runs = []
+    for _ in range(2):
+        xp, _ = moe.permute_fwd(x, plan, 0, 3, R)
+        y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
+        dxp, dw1, dw2, _ = moe.expert_ffn_bwd(dy, xp, w1, w2, offs, saved)
+        out, _ = moe.unpermute_fwd(y, plan, gates, 0, 3)
+        runs.append((y, dxp, dw1, dw2, out))
+    for a, b in zip(*runs):
+        assert torch.equal(a, b)

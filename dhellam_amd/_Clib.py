@@ -16,7 +16,11 @@ import torch
 
 from . import _lib
 
-__all__ = ["add_tensors", "pygemm", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge"]
+__all__ = ["add_tensors", "pygemm", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
+           "pyrmsnorm_fwd", "pyrmsnorm_bwd", "pyrope_fwd", "pyrope_bwd", "pyswiglu_fwd", "pyswiglu_bwd",
+           "pymoe_route_topk", "pymoe_sort", "pymoe_permute", "pymoe_unpermute", "pygrouped_gemm_nt",
+           "pygrouped_gemm_nn", "pygrouped_gemm_tn", "pycross_entropy_fwd", "pycross_entropy_bwd",
+           "pyembedding_fwd", "pyembedding_bwd"]
 
 
 def _timed(profiling: bool, stream, fn):
@@ -271,3 +275,118 @@ def pyattn_merge(outs, lses, row_begin, rows, out, lse):
     _lib.check(lib.dh_attn_merge(C.cast(po, C.c_void_p), C.cast(pl, C.c_void_p), C.cast(rb, C.c_void_p),
                                  C.cast(rr, C.c_void_p), n, out.data_ptr(), lse.data_ptr(), b, sq, hq, d,
                                  _lib.dt(out), torch.cuda.current_stream().cuda_stream))
+
+
+# ---------------------------------------------------------------------------------------
+# Binding-level names for the operators the reference does not have (RMSNorm, RoPE, SwiGLU as a
+# kernel, MoE, grouped GEMM, the head block).  Same conventions as the six names above: positional
+# arguments, work on the current stream, a trailing ``profiling`` flag; results come back as a list
+# with the elapsed milliseconds appended when profiling.  They forward to ``dhellam_amd.operators``
+# (imported lazily: that package imports this module).
+# ---------------------------------------------------------------------------------------
+def _ret(values, ms, profiling):
+    values = list(values)
+    return values + [ms] if profiling else values
+
+
+def pyrmsnorm_fwd(inp, weight, eps, profiling=False):
+    """-> [out, rsigma]"""
+    from .operators.layernorm import pylayernorm_fwd
+    out, _, rsigma, ms = pylayernorm_fwd(inp, weight, None, eps, 0, False, None, profiling)
+    return _ret((out, rsigma), ms, profiling)
+
+
+def pyrmsnorm_bwd(dout, inp, rsigma, weight, profiling=False):
+    """-> [dinp, dweight]"""
+    from .operators.layernorm import pylayernorm_bwd
+    dinp, dweight, _, ms = pylayernorm_bwd(dout, inp, None, rsigma, weight, 0, False, None, profiling)
+    return _ret((dinp, dweight), ms, profiling)
+
+
+def pyrope_fwd(q, k, positions, theta, profiling=False):
+    """-> [q_rot, k_rot]; positions None = 0..T-1"""
+    from .operators.rope import rope_fwd
+    qr, kr, ms = rope_fwd(q, k, positions, theta, None, None, profiling)
+    return _ret((qr, kr), ms, profiling)
+
+
+def pyrope_bwd(dq, dk, positions, theta, profiling=False):
+    from .operators.rope import rope_bwd
+    a, b, ms = rope_bwd(dq, dk, positions, theta, None, None, profiling)
+    return _ret((a, b), ms, profiling)
+
+
+def pyswiglu_fwd(y, profiling=False):
+    from .operators.swiglu import swiglu
+    out, ms = swiglu(y, None, profiling)
+    return _ret((out,), ms, profiling)
+
+
+def pyswiglu_bwd(g, y, profiling=False):
+    from .operators.swiglu import swiglu_back
+    dy, ms = swiglu_back(g, y, None, None, profiling)
+    return _ret((dy,), ms, profiling)
+
+
+def pymoe_route_topk(logits, k, profiling=False):
+    """-> [topk_idx int32 [T, k], gates fp32 [T, k]]"""
+    from .operators.moe import route_topk
+    idx, gates, ms = route_topk(logits, k, None, profiling)
+    return _ret((idx, gates), ms, profiling)
+
+
+def pymoe_sort(topk_idx, num_experts, profiling=False):
+    """-> [plan] (sorted assignment order, destination rows, tokens per expert, expert offsets)"""
+    from .operators.moe import sort_assignments
+    plan, ms = sort_assignments(topk_idx, num_experts, None, profiling)
+    return _ret((plan,), ms, profiling)
+
+
+def pymoe_permute(x, plan, e_lo, e_hi, max_rows, profiling=False):
+    from .operators.moe import permute_fwd
+    xp, ms = permute_fwd(x, plan, e_lo, e_hi, max_rows, None, profiling)
+    return _ret((xp,), ms, profiling)
+
+
+def pymoe_unpermute(y, plan, gates, e_lo, e_hi, profiling=False):
+    from .operators.moe import unpermute_fwd
+    out, ms = unpermute_fwd(y, plan, gates, e_lo, e_hi, None, profiling)
+    return _ret((out,), ms, profiling)
+
+
+def pygrouped_gemm_nt(a, b, offs, out=None):
+    from .operators.moe import grouped_gemm_nt
+    return grouped_gemm_nt(a, b, offs, None, out)
+
+
+def pygrouped_gemm_nn(a, b, offs, out=None):
+    from .operators.moe import grouped_gemm_nn
+    return grouped_gemm_nn(a, b, offs, None, out)
+
+
+def pygrouped_gemm_tn(a, b, offs, out=None, accumulate=False):
+    from .operators.moe import grouped_gemm_tn
+    return grouped_gemm_tn(a, b, offs, out, accumulate)
+
+
+def pycross_entropy_fwd(vocab_parallel_logits, target, label_smoothing=0.0, keep_softmax=True):
+    """-> the reference's output dict (dhellam/operators/loss.py:91-97)"""
+    from .operators.loss import cross_entropy_fwd
+    return cross_entropy_fwd({"vocab_parallel_logits": vocab_parallel_logits, "target": target}, label_smoothing,
+                             keep_softmax)
+
+
+def pycross_entropy_bwd(vocab_parallel_logits, target, fwd_out, dout, grad_out=None):
+    from .operators.loss import cross_entropy_bwd
+    return cross_entropy_bwd([{"vocab_parallel_logits": vocab_parallel_logits, "target": target}, fwd_out], dout,
+                             grad_out)
+
+
+def pyembedding_fwd(vocab, token_ids):
+    from .operators.embedding import word_embedding_fwd
+    return word_embedding_fwd({"vocab": vocab, "token_ids": token_ids})["word_embeddings"]
+
+
+def pyembedding_bwd(vocab, token_ids, dout):
+    from .operators.embedding import word_embedding_bwd
+    return word_embedding_bwd([{"vocab": vocab, "token_ids": token_ids}, None], dout)

@@ -204,3 +204,45 @@ def test_bandwidth_ops_are_deterministic():
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
     y, gg = randn((4096, 7168), dt, 4).cuda(), randn((4096, 3584), dt, 5).cuda()
     assert torch.equal(swiglu_back(gg, y)[0], swiglu_back(gg, y)[0])
+
+
+def test_binding_level_names_for_the_added_operators():
+    """The `_Clib` names of the operators the reference lacks forward to the operator layer: same results, lists
+    with the elapsed time appended only when profiling."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators import moe
+    from dhellam_amd.operators.layernorm import pylayernorm_fwd
+    from dhellam_amd.operators.swiglu import swiglu
+    dt = torch.bfloat16
+    x, g = randn((64, 256), dt, 1).cuda(), randn((256,), dt, 2).cuda()
+    out, rs = _Clib.pyrmsnorm_fwd(x, g, 1e-5, False)
+    ref = pylayernorm_fwd(x, g, None, 1e-5, 0, False, None)
+    assert torch.equal(out, ref[0]) and torch.equal(rs, ref[2])
+    res = _Clib.pyrmsnorm_bwd(out, x, rs, g, True)
+    assert len(res) == 3 and res[2] >= 0 and res[0].shape == x.shape and res[1].shape == g.shape
+    q, k = randn((32, 4, 64), dt, 3).cuda(), randn((32, 2, 64), dt, 4).cuda()
+    qr, kr = _Clib.pyrope_fwd(q, k, None, 1e4, False)
+    q2, k2 = _Clib.pyrope_bwd(qr, kr, None, 1e4, False)
+    assert_close(q2, q.cpu(), dt, "rope inverse") and assert_close(k2, k.cpu(), dt, "rope inverse")
+    y = randn((64, 512), dt, 5).cuda()
+    (a,) = _Clib.pyswiglu_fwd(y, False)
+    assert torch.equal(a, swiglu(y)[0])
+    (dy,) = _Clib.pyswiglu_bwd(a, y, False)
+    assert dy.shape == y.shape
+    logits = randn((128, 8), torch.float32, 6).cuda()
+    idx, gates = _Clib.pymoe_route_topk(logits, 2, False)
+    (plan,) = _Clib.pymoe_sort(idx, 8, False)
+    rows = int(plan.expert_offsets[8].item())
+    h = randn((128, 64), dt, 7).cuda()
+    (xp,) = _Clib.pymoe_permute(h, plan, 0, 8, rows, False)
+    (back,) = _Clib.pymoe_unpermute(xp, plan, gates, 0, 8, False)
+    assert_close(back, h.cpu(), dt, "permute -> unpermute with gates summing to one")
+    w = randn((8, 32, 64), dt, 8).cuda()
+    c = _Clib.pygrouped_gemm_nt(xp, w, plan.expert_offsets)
+    assert torch.equal(c, moe.grouped_gemm_nt(xp, w, plan.expert_offsets))
+    lg, tg = randn((16, 100), dt, 9).cuda(), torch.arange(16, device="cuda") % 100
+    ce = _Clib.pycross_entropy_fwd(lg, tg, 0.0, False)
+    gr = _Clib.pycross_entropy_bwd(lg, tg, ce, torch.ones(16, device="cuda"))
+    assert ce["loss"].shape == (16,) and gr.shape == lg.shape
+    table = randn((100, 64), dt, 10).cuda()
+    assert torch.equal(_Clib.pyembedding_fwd(table, tg), table[tg])

@@ -338,6 +338,14 @@ def profile_op(name: str, iters: int = 5):
     torch.cuda.synchronize()
 
 
+def _device_info():
+    """Name, architecture, CU count and HBM size as the runtime reports them."""
+    p = torch.cuda.get_device_properties(0)
+    info = {"name": p.name, "arch": getattr(p, "gcnArchName", ""), "compute_units": p.multi_processor_count,
+            "hbm_gib": round(p.total_memory / 2**30, 1)}
+    return info
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -414,6 +422,7 @@ def main():
         "layer_mfma_frac": round(layer_flop / (best_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "device": _device_info(),
         "kernels": kernels,
     }
     print(json.dumps(line))

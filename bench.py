@@ -311,6 +311,27 @@ def profile_op(name: str, iters: int = 5):
             y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
             dyp = rn(Rm, Hm)
             fn = lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved)
+    elif name in ("norm", "swiglu", "cross_entropy", "transpose"):
+        # bandwidth kernels at sizes beyond the 256 MB last-level cache (norm, SwiGLU) / at the head-block and
+        # weight-gradient shapes (cross entropy, transpose); forward then backward in each iteration
+        from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
+        from dhellam_amd.operators.loss import cross_entropy_bwd, cross_entropy_fwd
+        from dhellam_amd.operators.swiglu import swiglu, swiglu_back
+        if name == "norm":
+            x, gm, dy = rn(32768, 8192), torch.ones(8192, device=dev, dtype=dt), rn(32768, 8192)
+            _, _, rs, _ = pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None)
+            fn = lambda: (pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None), pylayernorm_bwd(dy, x, None, rs, gm, 0, False, None))
+        elif name == "swiglu":
+            yy, gg = rn(16384, 7168), rn(16384, 3584)
+            fn = lambda: (swiglu(yy), swiglu_back(gg, yy))
+        elif name == "cross_entropy":
+            lg = rn(4096, 16032)
+            ce_in = {"vocab_parallel_logits": lg, "target": torch.randint(0, 16032, (4096,), generator=g, device=dev)}
+            dl, gbuf = torch.ones(4096, device=dev), torch.empty_like(lg)
+            fn = lambda: cross_entropy_bwd([ce_in, cross_entropy_fwd(ce_in, 0.0, keep_softmax=False)], dl, grad_out=gbuf)
+        else:
+            src, dst = rn(4096, 8192), torch.empty(8192, 4096, device=dev, dtype=dt)
+            fn = lambda: _Clib.transpose_2d(src, dst)
     elif name in ("gg_nt", "gemm_nt"):
         # one [4096, 8192] x [7168, 8192]^T product: the grouped GEMM kernel (two groups of 2048 rows, full tiles
         # only) and the library GEMM of the same shape, for side-by-side counter runs
@@ -356,7 +377,7 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
-                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, gg_nt, gemm_nt, layer, copy) and exit")
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "

@@ -102,3 +102,19 @@ def test_model_trains_in_bf16():
         last = loss
     assert first > 5.0, first                  # ln(256) = 5.55
     assert last < 0.5 * first, (first, last)
+
+
+@pytest.mark.parametrize("layers,n_mb", [(1, 1), (1, 2), (3, 1)])
+def test_model_edge_shapes(layers, n_mb):
+    """One layer and / or one micro-batch: the paired schedule degenerates to forward-only + backward-only phases."""
+    from dhellam_amd.core.dsllm import DSLLM
+    cfg, vocab = _cfg(torch.bfloat16, hidden=128, heads=2, groups=1, ffn=256, seq=64, batch=1), 128
+    batches = _cuda(_batches(cfg, vocab, n_mb, seed=5))
+    a, b = DSLLM(cfg, layers, vocab, seed=2), DSLLM(cfg, layers, vocab, seed=2)
+    la, lb = a.step(batches, double_strand=True), b.step(batches, double_strand=False)
+    torch.cuda.synchronize()
+    for x, y in zip(la, lb):
+        assert torch.isfinite(x) and torch.equal(x, y)
+    for (name, p), (_, q) in zip(a.named_parameters(), b.named_parameters()):
+        assert torch.equal(p.main_grad, q.main_grad), name
+        assert float(p.main_grad.float().abs().max()) > 0, name

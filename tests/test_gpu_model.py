@@ -71,7 +71,7 @@ def test_model_step_matches_oracle_and_schedules_agree():
 
 def test_model_trains_in_bf16():
     """Predict the token two positions back (needs attention): bf16 parameters and gradients, fp32 master weights
-    with Adam on the host side of the loop.  The loss has to fall well below its starting value ln(vocab)."""
+    with Adam on the host side of the loop.  The loss has to fall to a quarter of its starting value ln(vocab)."""
     from dhellam_amd.core.dsllm import DSLLM
     cfg, vocab, L, n = _cfg(torch.bfloat16, hidden=256, heads=4, groups=2, ffn=512, seq=128, batch=4), 256, 2, 2
     model = DSLLM(cfg, L, vocab, seed=1)
@@ -101,7 +101,7 @@ def test_model_trains_in_bf16():
         first = loss if first is None else first
         last = loss
     assert first > 5.0, first                  # ln(256) = 5.55
-    assert last < 0.5 * first, (first, last)
+    assert last < 0.25 * first, (first, last)       # observed: 5.6 -> 0.07
 
 
 @pytest.mark.parametrize("layers,n_mb", [(1, 1), (1, 2), (3, 1)])

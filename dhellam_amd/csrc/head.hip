@@ -206,19 +206,14 @@ __global__ void __launch_bounds__(256) embedding_bwd_kernel(const T *__restrict_
   constexpr int N = Vec<T>::N, CV = 4;
   __shared__ int64_t dup[256];
   __shared__ int wcount[4];
-  __shared__ int earlier_s;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int64_t i = blockIdx.x;
   const int64_t id = ids[i];
   const int64_t v = id - vocab_start;
   if (v < 0 || v >= vocab_rows) return;
-  if (tid == 0) earlier_s = 0;
-  __syncthreads();
-  bool earlier = false;
+  int earlier = 0;
   for (int64_t j = tid; j < i; j += 256) earlier |= ids[j] == id;
-  if (earlier) earlier_s = 1;                // every writer stores the same value
-  __syncthreads();
-  if (earlier_s) return;
+  if (__syncthreads_or(earlier)) return;     // an earlier position owns this id
 
   const int64_t c0 = (int64_t)blockIdx.y * (256 * N * CV) + (int64_t)tid * N;
   float acc[CV][N];

@@ -316,9 +316,10 @@ extern "C" int dh_cross_entropy_fwd(const void *logits, const int64_t *target, i
   // vector accesses only when the logits and (if asked for) the softmax rows are all 16-byte aligned
   const bool vec = row_vec_ok(logits, ld, dtype) && (!softmax || row_vec_ok(softmax, ld_softmax, dtype));
   DH_DISPATCH_DTYPE(dtype, {
-    // 256 threads x 128 bytes held per thread: rows up to 32 KB (16384 16-bit logits) stay in registers, and a
-    // CU keeps 5-8 rows in flight (with 1024 threads and 2 rows per CU the same kernel ran at half the rate).
-    constexpr int BT = 256, NV = 8;
+    // 256 threads per row holding 16384 logits in registers (128 bytes per thread for 16-bit types, 256 for fp32;
+    // an fp32 row half held and half re-read ran at 4.5 instead of 6.4 TB/s).  With 1024 threads and 2 rows per
+    // CU the kernel ran at half the rate; 128 threads per 16-bit row were slower as well (4.0 against 4.8 TB/s).
+    constexpr int BT = 256, NV = sizeof(T) == 4 ? 16 : 8;
     hipLaunchKernelGGL((ce_fwd_kernel<T, BT, NV>), dim3((unsigned)rows), dim3(BT), 0, (hipStream_t)stream,
                        (const T *)logits, target, cols, ld, vocab_start, smoothing, loss, row_max, sum_exp, predicted,
                        (T *)softmax, ld_softmax, target_mask, masked_target, vec);
@@ -343,9 +344,10 @@ extern "C" int dh_cross_entropy_bwd(const void *src, int64_t ld_src, int from_lo
   const float smoothing = label_smoothing > 0.f ? label_smoothing * (float)cols / (float)(cols - 1) : 0.f;
   const bool vec = row_vec_ok(src, ld_src, dtype) && row_vec_ok(grad, ld_grad, dtype);
   DH_DISPATCH_DTYPE(dtype, {
-    // 256 threads x 128 bytes held per thread: rows up to 32 KB (16384 16-bit logits) stay in registers, and a
-    // CU keeps 5-8 rows in flight (with 1024 threads and 2 rows per CU the same kernel ran at half the rate).
-    constexpr int BT = 256, NV = 8;
+    // 256 threads per row holding 16384 logits in registers (128 bytes per thread for 16-bit types, 256 for fp32;
+    // an fp32 row half held and half re-read ran at 4.5 instead of 6.4 TB/s).  With 1024 threads and 2 rows per
+    // CU the kernel ran at half the rate; 128 threads per 16-bit row were slower as well (4.0 against 4.8 TB/s).
+    constexpr int BT = 256, NV = sizeof(T) == 4 ? 16 : 8;
     if (from_logits)
       hipLaunchKernelGGL((ce_bwd_kernel<T, BT, NV, true>), dim3((unsigned)rows), dim3(BT), 0, (hipStream_t)stream,
                          (const T *)src, ld_src, row_max, sum_exp, target, dout, cols, vocab_start, smoothing, (T *)grad,

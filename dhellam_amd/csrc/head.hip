@@ -102,7 +102,8 @@ __global__ void __launch_bounds__(BT) ce_fwd_kernel(const T *__restrict__ logits
   RowView<T, BT, NV> rv;
   rv.load(logits + r * ld, (int)cols, vec);
   float m = -INFINITY, sx = 0.f;
-  rv.for_each([&](float x) { m = fmaxf(m, x); sx += x; });
+  if (smoothing > 0.f) rv.for_each([&](float x) { m = fmaxf(m, x); sx += x; });   // sum of x only feeds the smoothing term
+  else rv.for_each([&](float x) { m = fmaxf(m, x); });
   m = block_max<BT>(m, red);
   // (x - m) first: the difference of two close numbers is exact, the product with log2(e) then errs by
   // one rounding of a small number (x * log2(e) - m * log2(e) would lose |x| * 2^-24 of the exponent).

@@ -375,6 +375,8 @@ def main():
     ap.add_argument("--micro-batches", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
+    ap.add_argument("--emulate-comm-us", type=float, default=55.0,
+                    help="also time both schedules with each sequence-parallel stand-in taking this long (0: skip)")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
                     help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
@@ -413,6 +415,21 @@ def main():
     ms_serial = timed(runner.run_serial)
     ms_double = timed(runner.run_double_strand)
     best_ms, schedule = (ms_double, "double-strand") if ms_double <= ms_serial else (ms_serial, "serial")
+    # The same two schedules with every sequence-parallel stand-in ALSO occupying its stream for the time the
+    # collective it replaces would take (a one-wavefront delay kernel, no data moved): what the double strand is
+    # for.  Reported beside the real numbers, never part of `value`.
+    emulated = None
+    if args.emulate_comm_us > 0:
+        import dataclasses
+        runner_c = LayerRunner(dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us), w, plan=plan)
+        ser_c, dbl_c = timed(runner_c.run_serial), timed(runner_c.run_double_strand)
+        runner_l = LayerRunner(dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us, lockstep_blocks=True), w,
+                               plan=plan)
+        dbl_l = timed(runner_l.run_double_strand)
+        emulated = {"standin_us_per_collective": args.emulate_comm_us, "collectives_per_microbatch": 8,
+                    "serial_ms": round(ser_c, 4), "double_strand_ms": round(dbl_c, 4),
+                    "double_strand_lockstep_ms": round(dbl_l, 4),
+                    "double_strand_speedup": round(ser_c / min(dbl_c, dbl_l), 4)}
     layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
 
     kernels = [] if args.no_kernels else kernel_rooflines(cfg)
@@ -440,6 +457,7 @@ def main():
                    "tokens_per_step": tokens_per_step},
         "schedules": {"serial_ms": round(ms_serial, 4), "double_strand_ms": round(ms_double, 4),
                       "double_strand_speedup": round(ms_serial / ms_double, 4)},
+        "schedules_with_emulated_collectives": emulated,
         "layer_mfma_frac": round(layer_flop / (best_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,
         "cpu_baseline": cpu,

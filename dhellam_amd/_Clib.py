@@ -94,9 +94,11 @@ def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
 # GEMM library's slowest layout here.  Measured at T = 4096, bf16, accumulating (us; N, K = 7168, 8192 / 8192, 3584 /
 # 1280, 8192 / 8192, 1024):   as given 484 / 233-257 / 95 / 76;   dY^T row-major 409 / 203 / 82 / 67;
 # dY^T and X^T both row-major 364 / 178 / 70 / 60.  dh_transpose_2d moves 5.5-6 TB/s (a [4096, 8192] matrix in
-# 24 us), so materialising dY^T pays from K of about 3000 and X^T as well from N of about 4000.
+# 24 us), so materialising dY^T pays from K of about 3000.  X^T as well would pay from N of about 4000, but for
+# that layout the library picks a stream-K kernel whose accumulation into dW is not reproducible when another
+# kernel shares the GPU (1 run in 100 of the double-strand schedule differed from the serial one in the last
+# bits of one weight gradient), and the two schedules are required to give identical bits: not used.
 WGRAD_TRANSPOSE_GRAD_MIN_K = 3072
-WGRAD_TRANSPOSE_DATA_MIN_N = 4096
 WGRAD_TRANSPOSE_MIN_ELEMS = 1 << 20
 
 
@@ -106,15 +108,12 @@ def _can_transpose(t: torch.Tensor) -> bool:
 
 
 def wgrad_operands(grad: torch.Tensor, data: torch.Tensor):
-    """(lhs, rhs) with lhs @ rhs = grad^T @ data for grad = dY [T, N], data = X [T, K]: the strided views, or
-    materialised row-major transposes of dY (and X) where that makes the product faster by more than they cost."""
+    """(lhs, rhs) with lhs @ rhs = grad^T @ data for grad = dY [T, N], data = X [T, K]: the strided view of dY,
+    or its materialised row-major transpose where that makes the product faster by more than it costs."""
     (t, n), k = grad.shape, data.shape[1]
     if (k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad)
             and grad.dtype == data.dtype):
-        lhs = transpose_2d(grad)
-        if n >= WGRAD_TRANSPOSE_DATA_MIN_N and _can_transpose(data):
-            return lhs, transpose_2d(data).t()
-        return lhs, data
+        return transpose_2d(grad), data
     return grad.t(), data
 
 

@@ -23,6 +23,7 @@ SIGNATURES = {
     "dh_version": (_i32, []),
     "dh_last_error": (C.c_char_p, []),
     "dh_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
+    "dh_delay": (_i32, [_i64, _vp]),
     "dh_transpose_2d": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp]),
     "dh_cross_entropy_fwd": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _f32, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _vp,
                                     _vp, _vp]),

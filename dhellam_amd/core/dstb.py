@@ -105,6 +105,8 @@ class LayerConfig:
     rope_theta: Optional[float] = 10000.0
     params_dtype: torch.dtype = torch.bfloat16
     layernorm_bias: bool = False      # False: RMSNorm (Llama); True: LayerNorm with bias (the reference's TE call)
+    comm_standin_us: float = 0.0      # > 0: every sequence-parallel stand-in also occupies its stream this long
+    lockstep_blocks: bool = False     # the two strands enter every plan block together (events between the streams)
 
     @property
     def head_dim(self) -> int:
@@ -325,12 +327,22 @@ class DCFunc:
 
     # ---- sequence-parallel stand-ins (one GPU: no collective is issued) ---------------
     @staticmethod
+    def _comm_delay(config, stream):
+        """With ``comm_standin_us`` set, a stand-in also keeps its stream busy for that long (a one-wavefront
+        kernel that touches no memory): the duration of the collective it replaces, for schedule experiments."""
+        us = getattr(config, "comm_standin_us", 0.0)
+        if us > 0:
+            st = stream if stream is not None else torch.cuda.current_stream()
+            _lib.check(_lib.load().dh_delay(int(us * 1000), st.cuda_stream))
+
+    @staticmethod
     def allgather(config, data, stream):
         """(out, handle).  ``peer`` holds the other ranks' rows for this micro-batch."""
         input, peer = data
         tp = config.tensor_model_parallel_size
         if tp == 1:
             return input.view(-1, input.shape[-1]), None
+        DCFunc._comm_delay(config, stream)
         if peer is None:
             raise RuntimeError("sequence-parallel gather stand-in needs the micro-batch's peer buffer")
         rows = input.numel() // input.shape[-1]
@@ -348,6 +360,7 @@ class DCFunc:
         tp = config.tensor_model_parallel_size
         if tp == 1:
             return input, None
+        DCFunc._comm_delay(config, stream)
         rows = input.shape[0] // tp
         return input[config.tp_rank * rows:(config.tp_rank + 1) * rows], None
 
@@ -703,7 +716,18 @@ def exec(config, dcoperation, fwd_weight, bwd_weight, input, grad_output, dcbloc
     def stream_of(op):
         return stream1 if getattr(op, "strand", 1) == 1 else stream2
 
+    lockstep = (getattr(config, "lockstep_blocks", False) and stream1 is not None and stream2 is not None
+                and stream1 != stream2)
     for now_block in dcblocks:
+        if lockstep:
+            # both strands enter a block together (device-side events, no host wait): keeps the block's pairing,
+            # which matters when the stand-in collectives have a duration to hide; without it the forward strand
+            # simply runs ahead
+            e1, e2 = torch.cuda.Event(), torch.cuda.Event()
+            e1.record(stream1)
+            e2.record(stream2)
+            stream1.wait_event(e2)
+            stream2.wait_event(e1)
         fwd_comm_first = False
         if now_block.stream3_op is not None:
             for now_op in now_block.stream3_op:

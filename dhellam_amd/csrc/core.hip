@@ -45,6 +45,27 @@ __global__ void __launch_bounds__(256) copy_kernel(const uint4 *__restrict__ src
   if (blockIdx.x == 0 && (int)threadIdx.x < ntail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
+// One wavefront that does nothing for `ticks` ticks of the constant 100 MHz clock.  Bounded twice: by the
+// clock and by an iteration count, so it always ends.
+__global__ void __launch_bounds__(64) delay_kernel(unsigned long long ticks, unsigned long long max_iters) {
+  const unsigned long long t0 = wall_clock64();
+  for (unsigned long long i = 0; i < max_iters; ++i) {
+    if (wall_clock64() - t0 >= ticks) break;
+    __builtin_amdgcn_s_sleep(32);
+  }
+}
+
+extern "C" int dh_delay(int64_t nanoseconds, void *stream) {
+  DH_CHECK(nanoseconds >= 0 && nanoseconds <= 1000000000ll, "delay of %lld ns outside [0, 1 s]", (long long)nanoseconds);
+  if (nanoseconds == 0) return DH_OK;
+  const unsigned long long ticks = (unsigned long long)(nanoseconds / 10);             // 100 MHz
+  // one iteration sleeps 32 x 64 cycles, at least 0.8 us at any engine clock: 4 x the iterations that fill the time
+  const unsigned long long max_iters = (unsigned long long)(nanoseconds / 200) + 1024;
+  hipLaunchKernelGGL(delay_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, ticks, max_iters);
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
 extern "C" int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream) {
   DH_CHECK(nbytes >= 0, "nbytes must be >= 0");
   if (nbytes == 0) return DH_OK;

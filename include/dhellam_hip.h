@@ -238,6 +238,11 @@ int dh_grouped_gemm_tn(const void *a, const void *b, void *c,
  * dhellam/core/dstb.py) when one GPU holds the whole sequence. */
 int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
 
+/* Keeps `stream` busy with a one-wavefront kernel for about `nanoseconds` (at most 1 s) without using the
+ * memory system.  No counterpart in the reference: on one GPU it stands in for the DURATION of a collective
+ * (dhellam/common/comm.py) in scheduler experiments, so that the double-strand runtime has something to hide. */
+int dh_delay(int64_t nanoseconds, void *stream);
+
 /* out[c * ld_out + r] = in[r * ld_in + c] for a [rows, cols] matrix of 16-bit elements
  * (bf16 / fp16; rows, cols and both leading dimensions multiples of 8).  Feeds the
  * weight-gradient product of the reference's GEMM operator (csrc/operators/gemm.cu:3-170 called

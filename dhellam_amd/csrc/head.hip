@@ -312,6 +312,12 @@ extern "C" int dh_cross_entropy_fwd(const void *logits, const int64_t *target, i
   if (rows == 0) return DH_OK;
   DH_CHECK(logits && target && loss && row_max && sum_exp, "null pointer");
   DH_CHECK(!softmax || ld_softmax >= cols, "ld_softmax=%lld < cols", (long long)ld_softmax);
+  {
+    const char *a = (const char *)logits, *b = (const char *)softmax;
+    const int64_t e = (int64_t)dtype_size(dtype);
+    DH_CHECK(!softmax || a + ((rows - 1) * ld + cols) * e <= b || b + ((rows - 1) * ld_softmax + cols) * e <= a,
+             "softmax must not overlap the logits");
+  }
   DH_CHECK(rows < (1ll << 31) && cols < (1ll << 31), "too many rows or columns");
   const float smoothing = label_smoothing > 0.f ? label_smoothing * (float)cols / (float)(cols - 1) : 0.f;
   // vector accesses only when the logits and (if asked for) the softmax rows are all 16-byte aligned
@@ -340,7 +346,13 @@ extern "C" int dh_cross_entropy_bwd(const void *src, int64_t ld_src, int from_lo
   if (rows == 0) return DH_OK;
   DH_CHECK(src && target && dout && grad, "null pointer");
   DH_CHECK(!from_logits || (row_max && sum_exp), "recomputing the softmax needs row_max and sum_exp");
-  DH_CHECK(grad == src ? ld_grad == ld_src : true, "in-place gradient needs equal pitches");
+  {
+    const char *a = (const char *)src, *b = (const char *)grad;
+    const int64_t e = (int64_t)dtype_size(dtype);
+    DH_CHECK((a == b && ld_grad == ld_src) || a + ((rows - 1) * ld_src + cols) * e <= b ||
+                 b + ((rows - 1) * ld_grad + cols) * e <= a,
+             "grad is either src itself (same pitch) or does not overlap it");
+  }
   DH_CHECK(rows < (1ll << 31) && cols < (1ll << 31), "too many rows or columns");
   const float smoothing = label_smoothing > 0.f ? label_smoothing * (float)cols / (float)(cols - 1) : 0.f;
   const bool vec = row_vec_ok(src, ld_src, dtype) && row_vec_ok(grad, ld_grad, dtype);

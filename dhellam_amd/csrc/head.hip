@@ -44,8 +44,8 @@ template <typename T, int BT, int NV> struct RowView {
       if (v < nvec) held[i] = ldg(row + (int64_t)v * N);
     }
   }
-  // f(value) over this thread's share of the row
-  template <typename F> __device__ __forceinline__ void for_each(F f) const {
+  // f(value) over the part of this thread's share that sits in registers
+  template <typename F> __device__ __forceinline__ void for_each_held(F f) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = i * BT + (int)threadIdx.x;
@@ -54,12 +54,30 @@ template <typename T, int BT, int NV> struct RowView {
         for (int e = 0; e < N; ++e) f(to_f(held[i].v[e]));
       }
     }
-    for (int v = NV * BT + (int)threadIdx.x; v < nvec; v += BT) {
+  }
+  // ... and over the part that is read from memory on every visit
+  template <typename F> __device__ __forceinline__ void for_each_streamed(F f) const {
+    constexpr int U = 4;                     // vectors in flight per thread
+    int v = NV * BT + (int)threadIdx.x;
+    for (; v + (U - 1) * BT < nvec; v += U * BT) {
+      Vec<T> x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = ldg(row + (int64_t)(v + u * BT) * N);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int e = 0; e < N; ++e) f(to_f(x[u].v[e]));
+    }
+    for (; v < nvec; v += BT) {
       const Vec<T> x = ldg(row + (int64_t)v * N);
 #pragma unroll
       for (int e = 0; e < N; ++e) f(to_f(x.v[e]));
     }
     for (int c = nvec * N + (int)threadIdx.x; c < cols; c += BT) f(to_f(row[c]));
+  }
+  template <typename F> __device__ __forceinline__ void for_each(F f) const {
+    for_each_held(f);
+    for_each_streamed(f);
   }
   // out[c] = g(value) for every column; same traversal, vector stores where the loads were vectors
   // (the caller enables vectors only when `out` is as aligned as the row: a run-time choice between a vector
@@ -76,7 +94,16 @@ template <typename T, int BT, int NV> struct RowView {
       const int v = i * BT + (int)threadIdx.x;
       if (v < nvec) emit(v, held[i]);
     }
-    for (int v = NV * BT + (int)threadIdx.x; v < nvec; v += BT) emit(v, ldg(row + (int64_t)v * N));
+    constexpr int U = 4;
+    int v = NV * BT + (int)threadIdx.x;
+    for (; v + (U - 1) * BT < nvec; v += U * BT) {
+      Vec<T> x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = ldg(row + (int64_t)(v + u * BT) * N);
+#pragma unroll
+      for (int u = 0; u < U; ++u) emit(v + u * BT, x[u]);
+    }
+    for (; v < nvec; v += BT) emit(v, ldg(row + (int64_t)v * N));
     for (int c = nvec * N + (int)threadIdx.x; c < cols; c += BT) out[c] = from_f<T>(g(to_f(row[c])));
   }
 };
@@ -101,14 +128,24 @@ __global__ void __launch_bounds__(BT) ce_fwd_kernel(const T *__restrict__ logits
   const int64_t r = blockIdx.x;
   RowView<T, BT, NV> rv;
   rv.load(logits + r * ld, (int)cols, vec);
-  float m = -INFINITY, sx = 0.f;
-  if (smoothing > 0.f) rv.for_each([&](float x) { m = fmaxf(m, x); sx += x; });   // sum of x only feeds the smoothing term
-  else rv.for_each([&](float x) { m = fmaxf(m, x); });
-  m = block_max<BT>(m, red);
-  // (x - m) first: the difference of two close numbers is exact, the product with log2(e) then errs by
-  // one rounding of a small number (x * log2(e) - m * log2(e) would lose |x| * 2^-24 of the exponent).
-  float s = 0.f;
-  rv.for_each([&](float x) { s += exp2_fast((x - m) * LOG2E); });
+  // The registers are visited twice (maximum, then the exponentials against the block's maximum).  What does not
+  // fit in them (rows beyond 16384 logits) is read ONCE, with a running maximum ms and a sum ss of exp(x - ms)
+  // that is rescaled whenever ms moves, and joined afterwards: sum += ss * exp(ms - m).
+  float m = -INFINITY, sx = 0.f, ms = -INFINITY, ss = 0.f;
+  if (smoothing > 0.f) rv.for_each_held([&](float x) { m = fmaxf(m, x); sx += x; });   // sum of x only feeds the smoothing term
+  else rv.for_each_held([&](float x) { m = fmaxf(m, x); });
+  rv.for_each_streamed([&](float x) {
+    // (x - m) first: the difference of two close numbers is exact, the product with log2(e) then errs by
+    // one rounding of a small number (x * log2(e) - m * log2(e) would lose |x| * 2^-24 of the exponent).
+    const float mn = fmaxf(ms, x);
+    if (mn > -INFINITY)                      // (a -inf logit before any finite one contributes nothing)
+      ss = ss * exp2_fast((ms - mn) * LOG2E) + exp2_fast((x - mn) * LOG2E);   // ms = -inf at first: 0 * exp2(-inf) = 0
+    ms = mn;
+    sx += x;
+  });
+  m = block_max<BT>(fmaxf(m, ms), red);
+  float s = ms > -INFINITY ? ss * exp2_fast((ms - m) * LOG2E) : 0.f;
+  rv.for_each_held([&](float x) { s += exp2_fast((x - m) * LOG2E); });
   s = block_sum<BT>(s, red);
   if (smoothing > 0.f) sx = block_sum<BT>(sx, red);
   const int64_t t = target[r] - vocab_start;

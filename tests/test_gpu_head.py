@@ -29,7 +29,8 @@ def _targets(shape, lo, hi, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape,rank,world", [((64, 16032), 0, 1), ((4, 9, 1000), 0, 1), ((33, 16032), 3, 8),
-                                              ((5, 70000), 1, 2), ((7, 37), 0, 1), ((3, 1), 0, 1), ((0, 64), 0, 1)])
+                                              ((5, 70000), 1, 2), ((3, 131080), 0, 1), ((2, 140003), 0, 1), ((7, 37), 0, 1), ((3, 1), 0, 1),
+                                              ((0, 64), 0, 1)])
 @pytest.mark.parametrize("ls", [0.0, 0.1])
 @pytest.mark.parametrize("keep", [True, False])
 def test_cross_entropy(tp, dtype, shape, rank, world, ls, keep):

@@ -603,6 +603,26 @@ static int dispatch_gg(const GGParams &p, int64_t m_extent, int dtype, hipStream
              : launch_gg<f16_t, TA, TB, 2, 2, 2, GROUPED_OUT>(p, m_extent, st);
 }
 
+// Rows of c past the last group (up to max_rows) are zeroed, so that callers can hand over uninitialised
+// memory whatever the row count turns out to be on the device: usually no row at all (a full fill of the
+// output cost 45 us in front of the first expert GEMM).
+__global__ void __launch_bounds__(256) gg_zero_tail_kernel(uint16_t *c, const int32_t *__restrict__ offs, int groups,
+                                                           int64_t max_rows, int64_t n) {
+  const int64_t first = offs[groups] - offs[0];
+  const int64_t nv = n / 8;                                // n is a multiple of 8 (checked by the callers)
+  for (int64_t r = first + blockIdx.x; r < max_rows; r += gridDim.x)
+    for (int64_t v = threadIdx.x; v < nv; v += 256) {
+      Vec<uint16_t> z;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z.v[e] = 0;
+      stg(c + r * n + v * 8, z);
+    }
+}
+
+static void gg_zero_tail(void *c, const int32_t *offs, int groups, int64_t max_rows, int64_t n, hipStream_t st) {
+  hipLaunchKernelGGL(gg_zero_tail_kernel, dim3(64), dim3(256), 0, st, (uint16_t *)c, offs, groups, max_rows, n);
+}
+
 static int gg_common_checks(const void *a, const void *b, void *c, const int32_t *offs, int groups, int dtype) {
   DH_CHECK(groups >= 1 && groups <= GG_MAX_GROUPS, "groups=%d must be in [1, %d]", groups, GG_MAX_GROUPS);
   DH_CHECK(dtype == DH_BF16 || dtype == DH_F16, "grouped GEMM supports bf16/fp16 (dtype %d)", dtype);
@@ -625,6 +645,7 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0;
+  gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && k < (1ll << 30))
     rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream)
@@ -648,6 +669,7 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = n; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0;
+  gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
     rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream)

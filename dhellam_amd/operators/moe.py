@@ -129,7 +129,10 @@ def grouped_gemm_nt(a, b, offs, max_rows=None, out=None, stream=None):
     assert a.is_contiguous() and b.is_contiguous() and a.shape[1] == k and offs.numel() == g + 1
     st = stream or torch.cuda.current_stream()
     with torch.cuda.stream(st):
-        c = out if out is not None else torch.zeros((a.shape[0], n), dtype=a.dtype, device=a.device)
+        # rows past the last group are zeroed by the library; everything else is written
+        c = out if out is not None else torch.empty((a.shape[0], n), dtype=a.dtype, device=a.device)
+        if out is None and max_rows is not None and max_rows < a.shape[0]:
+            c[max_rows:].zero_()
         _lib.check(lib.dh_grouped_gemm_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g,
                                           a.shape[0] if max_rows is None else max_rows, n, k, _lib.dt(a),
                                           st.cuda_stream))
@@ -143,7 +146,10 @@ def grouped_gemm_nn(a, b, offs, max_rows=None, out=None, stream=None):
     assert a.is_contiguous() and b.is_contiguous() and a.shape[1] == k and offs.numel() == g + 1
     st = stream or torch.cuda.current_stream()
     with torch.cuda.stream(st):
-        c = out if out is not None else torch.zeros((a.shape[0], n), dtype=a.dtype, device=a.device)
+        # rows past the last group are zeroed by the library; everything else is written
+        c = out if out is not None else torch.empty((a.shape[0], n), dtype=a.dtype, device=a.device)
+        if out is None and max_rows is not None and max_rows < a.shape[0]:
+            c[max_rows:].zero_()
         _lib.check(lib.dh_grouped_gemm_nn(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g,
                                           a.shape[0] if max_rows is None else max_rows, n, k, _lib.dt(a),
                                           st.cuda_stream))

@@ -218,7 +218,8 @@ int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *dest_row,
  *   NT: c[rows_g, n] = a[rows_g, k] * b[g][n, k]^T          (forward)
  *   NN: c[rows_g, n] = a[rows_g, k] * b[g][k, n]            (dgrad)
  *   TN: c[g][m, n] (+)= a[rows_g, m]^T * b[rows_g, n]       (wgrad)
- * max_rows bounds the launch grid.
+ * max_rows bounds the launch grid; NT / NN zero the rows of c from the last group's end up to
+ * max_rows, so c may be uninitialised on entry.
  * ---------------------------------------------------------------------- */
 int dh_grouped_gemm_nt(const void *a, const void *b, void *c,
                        const int32_t *offs, int groups, int64_t max_rows,

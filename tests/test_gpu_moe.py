@@ -124,6 +124,13 @@ def test_grouped_gemm_variants(dtype, rows, N, K):
     wref = torch.stack([d[sum(rows[:g]):sum(rows[:g + 1])].double().T @ a[sum(rows[:g]):sum(rows[:g + 1])].double()
                         for g in range(G)])
     assert_close(w, wref, dtype, "TN")
+    # rows of a past the last group: the corresponding rows of c come back as zeros (c starts uninitialised)
+    a_pad = torch.cat([a, randn((9, K), dtype, 5)]).cuda()
+    for fn, bb in ((moe.grouped_gemm_nt, b.cuda()), (moe.grouped_gemm_nn, bt.cuda())):
+        torch.empty((R + 9, N), dtype=dtype, device="cuda").fill_(7.0)   # dirty the allocator's next block
+        cp = fn(a_pad, bb, offs.cuda())
+        assert_close(cp[:R], ref, dtype, "padded")
+        assert bool((cp[R:] == 0).all())
     acc0 = randn((G, N, K), dtype, 4)
     acc = acc0.clone().cuda()
     moe.grouped_gemm_tn(d.cuda(), a.cuda(), offs.cuda(), out=acc, accumulate=True)

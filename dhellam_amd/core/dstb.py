@@ -107,6 +107,9 @@ class LayerConfig:
     layernorm_bias: bool = False      # False: RMSNorm (Llama); True: LayerNorm with bias (the reference's TE call)
     comm_standin_us: float = 0.0      # > 0: every sequence-parallel stand-in also occupies its stream this long
     lockstep_blocks: bool = False     # the two strands enter every plan block together (events between the streams)
+    # (forward strand's, backward strand's) communication streams: the stand-ins' delays run there, with events
+    # to and from the strand's own stream, instead of on the strand's stream itself
+    comm_streams: Optional[tuple] = None
 
     @property
     def head_dim(self) -> int:
@@ -327,22 +330,32 @@ class DCFunc:
 
     # ---- sequence-parallel stand-ins (one GPU: no collective is issued) ---------------
     @staticmethod
-    def _comm_delay(config, stream):
+    def _comm_delay(config, stream, bwd_strand=False):
         """With ``comm_standin_us`` set, a stand-in also keeps its stream busy for that long (a one-wavefront
         kernel that touches no memory): the duration of the collective it replaces, for schedule experiments."""
         us = getattr(config, "comm_standin_us", 0.0)
         if us > 0:
             st = stream if stream is not None else torch.cuda.current_stream()
-            _lib.check(_lib.load().dh_delay(int(us * 1000), st.cuda_stream))
+            comm = getattr(config, "comm_streams", None)
+            if comm is None:
+                _lib.check(_lib.load().dh_delay(int(us * 1000), st.cuda_stream))
+                return
+            cs = comm[1] if bwd_strand else comm[0]
+            posted, done = torch.cuda.Event(), torch.cuda.Event()
+            posted.record(st)
+            cs.wait_event(posted)
+            _lib.check(_lib.load().dh_delay(int(us * 1000), cs.cuda_stream))
+            done.record(cs)
+            st.wait_event(done)
 
     @staticmethod
-    def allgather(config, data, stream):
+    def allgather(config, data, stream, bwd_strand=False):
         """(out, handle).  ``peer`` holds the other ranks' rows for this micro-batch."""
         input, peer = data
         tp = config.tensor_model_parallel_size
         if tp == 1:
             return input.view(-1, input.shape[-1]), None
-        DCFunc._comm_delay(config, stream)
+        DCFunc._comm_delay(config, stream, bwd_strand)
         if peer is None:
             raise RuntimeError("sequence-parallel gather stand-in needs the micro-batch's peer buffer")
         rows = input.numel() // input.shape[-1]
@@ -355,12 +368,12 @@ class DCFunc:
         return peer, None
 
     @staticmethod
-    def reduce_scatter(config, data, stream):
+    def reduce_scatter(config, data, stream, bwd_strand=False):
         (input,) = data
         tp = config.tensor_model_parallel_size
         if tp == 1:
             return input, None
-        DCFunc._comm_delay(config, stream)
+        DCFunc._comm_delay(config, stream, bwd_strand)
         rows = input.shape[0] // tp
         return input[config.tp_rank * rows:(config.tp_rank + 1) * rows], None
 
@@ -425,10 +438,11 @@ class DCoperation:
         elif op == 9:
             output, act["attn_mask"] = dcfunc.bda_attn(config, (x, g("ln_attn_residual")), stream)
         elif op == 10:
-            output = dcfunc.reduce_scatter(config, (x,), stream)
+            output = dcfunc.reduce_scatter(config, (x,), stream, bwd_strand=bool(name) and name.endswith("_bwd"))
         elif op == 11:
             peer = act.get(_PEER_KEY.get(name, ""))
-            output = dcfunc.allgather(config, (x, _use(peer, stream)), stream)
+            output = dcfunc.allgather(config, (x, _use(peer, stream)), stream,
+                                      bwd_strand=bool(name) and name.endswith("_bwd"))
         elif op == 12:
             output = dcfunc.swiglu(config, (x,), stream)
             act["swiglu_input"] = x

@@ -66,6 +66,29 @@ extern "C" int dh_delay(int64_t nanoseconds, void *stream) {
   return DH_OK;
 }
 
+// A stream whose kernels run only on the compute units whose bit is set in `mask` (bit i of word i / 32;
+// on a device with several XCDs bit i is compute unit i / n_xcd of XCD i % n_xcd).
+extern "C" int dh_stream_create_cu_mask(const uint32_t *mask, int words, void **stream_out) {
+  DH_CHECK(mask && stream_out, "null pointer");
+  int dev = 0, cus = 0;
+  DH_HIP(hipGetDevice(&dev));
+  DH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  DH_CHECK(words >= 1 && words * 32 >= cus && words <= 64, "mask of %d words does not cover the device's %d compute units", words, cus);
+  int set = 0;
+  for (int i = 0; i < cus; ++i) set += (mask[i / 32] >> (i % 32)) & 1;
+  DH_CHECK(set > 0, "the mask enables no compute unit");
+  hipStream_t st = nullptr;
+  DH_HIP(hipExtStreamCreateWithCUMask(&st, (uint32_t)words, mask));
+  *stream_out = (void *)st;
+  return DH_OK;
+}
+
+extern "C" int dh_stream_destroy(void *stream) {
+  DH_CHECK(stream, "null stream");
+  DH_HIP(hipStreamDestroy((hipStream_t)stream));
+  return DH_OK;
+}
+
 extern "C" int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream) {
   DH_CHECK(nbytes >= 0, "nbytes must be >= 0");
   if (nbytes == 0) return DH_OK;

@@ -244,6 +244,16 @@ int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
  * (dhellam/common/comm.py) in scheduler experiments, so that the double-strand runtime has something to hide. */
 int dh_delay(int64_t nanoseconds, void *stream);
 
+/* A stream whose kernels run only on the compute units named in `mask` (bit i of word i / 32; `words` x 32
+ * bits must cover the device; with several XCDs bit i is compute unit i / n_xcd of XCD i % n_xcd).  The
+ * MI355X form of the reference's libsmctrl partitioning (csrc/operators/smctrl.cpp:135-160, the `math_sm_count`
+ * argument of pygemm, csrc/operators/ops.h:30): a kernel that fills every register file (the library GEMMs do)
+ * keeps a later kernel of another stream from starting anywhere until its own last workgroup is placed, so a
+ * small kernel that must start on time -- a collective -- gets compute units the compute streams never use.
+ * `dh_stream_destroy` ends a stream created here (after its work has finished). */
+int dh_stream_create_cu_mask(const uint32_t *mask, int words, void **stream_out);
+int dh_stream_destroy(void *stream);
+
 /* out[c * ld_out + r] = in[r * ld_in + c] for a [rows, cols] matrix of 16-bit elements
  * (bf16 / fp16; rows, cols and both leading dimensions multiples of 8).  Feeds the
  * weight-gradient product of the reference's GEMM operator (csrc/operators/gemm.cu:3-170 called

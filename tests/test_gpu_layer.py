@@ -151,3 +151,69 @@ def test_delay_and_emulated_collectives():
         res.append((outs, dxs, [w[k].main_grad.clone() for k in GRAD_KEYS]))
     for x, y in zip(res[0][0] + res[0][1] + res[0][2], res[1][0] + res[1][1] + res[1][2]):
         assert torch.equal(x, y)
+
+
+def test_cu_partitioned_streams():
+    """Streams bound to a subset of the compute units (the MI355X form of the reference's libsmctrl masks,
+    csrc/operators/smctrl.cpp:135-160): the layer on masked compute streams, its stand-in collectives on
+    streams that own the reserved compute units, gives the same bits as on ordinary streams; bad masks are
+    refused."""
+    import ctypes
+    import dataclasses
+    from dhellam_amd import _lib
+    from dhellam_amd.common.streams import cu_mask_words, destroy_stream, partitioned_streams, stream_with_cu_mask
+    from dhellam_amd.core.dstb import LayerConfig
+    from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
+    n_cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert cu_mask_words(64, 60, 4) == [0, 0xF0000000]
+    with pytest.raises(ValueError):
+        cu_mask_words(64, 60, 8)
+    lib = _lib.load()
+    out = ctypes.c_void_p()
+    zero = (ctypes.c_uint32 * ((n_cus + 31) // 32))()
+    with pytest.raises(RuntimeError):                                    # enables nothing
+        _lib.check(lib.dh_stream_create_cu_mask(ctypes.cast(zero, ctypes.c_void_p), len(zero), ctypes.byref(out)))
+    one = (ctypes.c_uint32 * 1)(1)
+    if n_cus > 32:
+        with pytest.raises(RuntimeError):                                # does not cover the device
+            _lib.check(lib.dh_stream_create_cu_mask(ctypes.cast(one, ctypes.c_void_p), 1, ctypes.byref(out)))
+    # a kernel on a stream of 8 compute units does the same work, later
+    st = stream_with_cu_mask(cu_mask_words(n_cus, 0, 8))
+    x = torch.randn(1 << 22, device="cuda")
+    st.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(st):
+        y = x * 2.0
+    st.synchronize()
+    assert torch.equal(y, x * 2.0)
+    destroy_stream(st)
+
+    cfg = LayerConfig(hidden_size=512, num_attention_heads=8, num_query_groups=4, ffn_hidden_size=1024, seq_length=256,
+                      micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
+                      params_dtype=torch.bfloat16, comm_standin_us=30.0)
+    (c1, c2), comm = partitioned_streams(reserved_per_xcd=1)
+    res = []
+    for part in (False, True):
+        c = dataclasses.replace(cfg, comm_streams=tuple(comm)) if part else cfg
+        w = make_weights(c, 0)
+        mbs = [make_microbatch(c, i) for i in range(3)]
+        r = LayerRunner(c, w, stream1=c1, stream2=c2) if part else LayerRunner(c, w)
+        outs, dxs = r.run_double_strand(mbs)
+        torch.cuda.synchronize()
+        res.append(outs + dxs + [w[k].main_grad.clone() for k in GRAD_KEYS])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    # a stand-in on the reserved compute units starts when it is posted, whatever the compute streams run
+    a_ = torch.randn(4096, 8192, device="cuda", dtype=torch.bfloat16)
+    b_ = torch.randn(8192, 7168, device="cuda", dtype=torch.bfloat16)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    worst = 0.0
+    for _ in range(3):
+        with torch.cuda.stream(c1):
+            for _ in range(6):
+                a_ @ b_
+        e0.record(comm[0])
+        _lib.check(lib.dh_delay(50_000, comm[0].cuda_stream))
+        e1.record(comm[0])
+        torch.cuda.synchronize()
+        worst = max(worst, e0.elapsed_time(e1) * 1e3)
+    assert 45.0 <= worst <= 150.0, worst

@@ -68,3 +68,19 @@ def test_layer_config_derived_sizes():
     s = small_fp32_layer()
     assert (s.head_dim, s.heads_per_rank, s.groups_per_rank, s.ffn_per_rank, s.qkv_per_rank, s.sp_rows) == \
         (64, 16, 16, 2816, 3072, 1024)
+
+
+def test_cu_mask_words():
+    """Mask words for streams bound to a set of compute units: bit i of word i // 32."""
+    from dhellam_amd.common.streams import cu_mask_words
+    assert cu_mask_words(256, 0, 248) == [0xFFFFFFFF] * 7 + [0x00FFFFFF]
+    assert cu_mask_words(256, 248, 8) == [0] * 7 + [0xFF000000]
+    assert cu_mask_words(40, 30, 4) == [0xC0000000, 0x3]
+    a, b = cu_mask_words(256, 0, 248), cu_mask_words(256, 248, 8)
+    assert all(x & y == 0 and x | y == 0xFFFFFFFF for x, y in zip(a, b))     # a partition of the device
+    for bad in ((256, 250, 8), (256, -1, 4), (256, 0, 0)):
+        try:
+            cu_mask_words(*bad)
+        except ValueError:
+            continue
+        raise AssertionError(bad)

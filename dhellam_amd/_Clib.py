@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["add_tensors", "pygemm", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
+__all__ = ["add_tensors", "pygemm", "dense_gemm", "dense_ok", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
            "pyrmsnorm_fwd", "pyrmsnorm_bwd", "pyrope_fwd", "pyrope_bwd", "pyswiglu_fwd", "pyswiglu_bwd",
            "pymoe_route_topk", "pymoe_sort", "pymoe_permute", "pymoe_unpermute", "pygrouped_gemm_nt",
            "pygrouped_gemm_nn", "pygrouped_gemm_tn", "pycross_entropy_fwd", "pycross_entropy_bwd",
@@ -44,6 +44,51 @@ def add_tensors(a, b):
     return a + b
 
 
+GEMM_WORKSPACE_BYTES = 32 << 20
+_gemm_ws: dict = {}
+
+
+def _gemm_workspace(device, stream_ptr: int) -> torch.Tensor:
+    """One workspace per (device, stream): kernels that split a product over workgroups keep partial tiles
+    there, so two streams must not share one."""
+    key = (str(device), stream_ptr)
+    ws = _gemm_ws.get(key)
+    if ws is None:
+        ws = torch.empty(GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _gemm_ws[key] = ws
+    return ws
+
+
+def dense_ok(*tensors) -> bool:
+    """True when ``dh_gemm`` takes these operands as they are: 2-D, contiguous, on the GPU."""
+    return all(t.is_cuda and t.dim() == 2 and t.is_contiguous() for t in tensors)
+
+
+def dense_gemm(A, B, D, transa: bool, transb: bool, accumulate: bool, workspace=None, workspace_bytes: int = 0) -> None:
+    """``dh_gemm`` on the current stream, in the reference's operand convention (see ``pygemm``)."""
+    if not dense_ok(A, B, D):
+        raise RuntimeError("dense_gemm: operands must be contiguous 2-D GPU tensors")
+    if A.dtype != B.dtype or D.dtype not in (A.dtype, torch.float32):
+        raise RuntimeError(f"dense_gemm: operand types {A.dtype}, {B.dtype} -> {D.dtype} not supported")
+    m = A.shape[0] if transa else A.shape[1]
+    n = B.shape[1] if transb else B.shape[0]
+    if tuple(D.shape) != (n, m):
+        raise RuntimeError(f"dense_gemm: output is {tuple(D.shape)}, the product is {(n, m)}")
+    stream = torch.cuda.current_stream()
+    if workspace is None or not getattr(workspace, "is_cuda", False) or workspace_bytes <= 0:
+        workspace = _gemm_workspace(A.device, stream.cuda_stream)
+        workspace_bytes = workspace.numel()
+    elif workspace.numel() * workspace.element_size() < workspace_bytes:
+        raise RuntimeError("dense_gemm: workspace tensor smaller than workspaceSize")
+    if (transa and A.shape[1] == 0) or (not transa and A.shape[0] == 0):
+        if not accumulate:
+            D.zero_()
+        return
+    _lib.check(_lib.load().dh_gemm(A.data_ptr(), B.data_ptr(), D.data_ptr(), A.shape[0], A.shape[1], B.shape[0],
+                                   B.shape[1], int(transa), int(transb), int(accumulate), _lib.dt(A), _lib.dt(D),
+                                   workspace.data_ptr(), workspace_bytes, stream.cuda_stream))
+
+
 def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, transb, grad_accumulate, math_sm_count,
            profiling):
     """csrc/operators/gemm.cu:3-170.  Column-major cuBLASLt convention of the reference:
@@ -55,22 +100,22 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
         False   False    B   @ A       ("NN": dgrad)
         False   True     B.T @ A       ("NT": wgrad)
 
-    Dense GEMM is a library call on this path (hipBLASLt through torch.matmul);
-    ``input_workspace`` / ``workspaceSize`` / ``math_sm_count`` are accepted and unused.
+    The product is ``dh_gemm`` (hipBLASLt behind the C ABI).  ``input_workspace`` / ``workspaceSize`` are
+    used when given (a GPU tensor of at least that many bytes), otherwise a per-stream 32 MiB buffer;
+    ``math_sm_count`` is accepted and unused.  For the weight gradient, B^T is materialised first where that
+    makes the product faster by more than it costs (``wgrad_operands``).
     """
     _lib.need_cuda(inputA, inputB, outputD)
     stream = torch.cuda.current_stream()
-    if transb and not transa:
-        b, a = wgrad_operands(inputB, inputA)
-    else:
-        a = inputA.t() if transa else inputA
-        b = inputB.t() if transb else inputB
+    ws_bytes = int(workspaceSize or 0)
 
     def run():
-        if grad_accumulate:
-            outputD.addmm_(b, a)
-        else:
-            torch.matmul(b, a, out=outputD)
+        if transb and not transa:
+            bt, a = wgrad_operands(inputB, inputA)
+            if bt.is_contiguous():                      # the materialised transpose: now the "NN" form
+                dense_gemm(a, bt, outputD, False, False, grad_accumulate, input_workspace, ws_bytes)
+                return
+        dense_gemm(inputA, inputB, outputD, transa, transb, grad_accumulate, input_workspace, ws_bytes)
 
     return _timed(profiling, stream, run)
 

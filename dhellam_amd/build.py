@@ -72,7 +72,7 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
         objs = list(ex.map(lambda s: _compile(s, verbose), srcs))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc",
-           *map(str, objs), "-o", str(tmp)]
+           *map(str, objs), "-lhipblaslt", "-o", str(tmp)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -3,10 +3,12 @@
 Mirrors dhellam/operators/layernorm_column.py:7-62 (``gemm_fwd``), :209-263
 (``dgrad_bwd``) and :265-323 (``wgrad_bwd``).  Weights are stored [out, in];
 the layout letters are the reference's: "TN" computes input @ weight.T, "NN"
-grad @ weight, "NT" grad.T @ input.  Dense GEMM is a library call on this path
-(hipBLASLt through ``torch.matmul``), exactly what every scheduler call site of
-the reference selects with ``is_matmul=True`` (dhellam/core/dstb.py:84-106,
-300-340); with ``is_matmul=False`` the same product goes through ``_Clib.pygemm``.
+grad @ weight, "NT" grad.T @ input.  Dense GEMM is a library call on this path:
+``dh_gemm`` of the C ABI (hipBLASLt) whichever way it is asked for.  ``is_matmul=True``
+(what every scheduler call site of the reference selects, dhellam/core/dstb.py:84-106,
+300-340) takes inputs with leading dimensions, as ``torch.matmul`` does there, and falls back
+to ``torch.matmul`` only for operands ``dh_gemm`` does not take (strided views, mixed types);
+``is_matmul=False`` is ``_Clib.pygemm`` with its contiguous 2-D operands.
 Output dtype follows the inputs (the reference hard-codes fp16).  Elapsed time
 is in milliseconds, measured with events on the op's stream.
 """
@@ -16,6 +18,7 @@ from typing import Optional
 
 import torch
 
+from .._Clib import dense_gemm, dense_ok
 from .._Clib import pygemm as gemm
 from .._Clib import wgrad_operands
 from ._util import on_stream
@@ -29,9 +32,16 @@ def gemm_fwd(args, input: torch.Tensor, weight: torch.Tensor, output: Optional[t
     el: list = []
     with on_stream(stream, profiling, el):
         if is_matmul:
-            w = weight.t() if transa else weight
-            x = input.t() if transb else input
-            output = torch.matmul(x, w) if output is None else torch.matmul(x, w, out=output)
+            x2 = input.reshape(-1, input.shape[-1]) if input.is_contiguous() else input
+            if (transa and not transb and dense_ok(weight, x2) and weight.dtype == input.dtype
+                    and (output is None or (output.is_contiguous() and output.dtype == input.dtype))):
+                if output is None:
+                    output = torch.empty(*input.shape[:-1], weight.shape[0], dtype=input.dtype, device=input.device)
+                dense_gemm(weight, x2, output.view(-1, weight.shape[0]), True, False, False)
+            else:
+                w = weight.t() if transa else weight
+                x = input.t() if transb else input
+                output = torch.matmul(x, w) if output is None else torch.matmul(x, w, out=output)
         else:
             if output is None:
                 output = torch.empty(input.shape[1] if transb else input.shape[0],
@@ -53,9 +63,13 @@ def dgrad_bwd(args, input_grad: torch.Tensor, weight: torch.Tensor, dgrad_output
                                        weight.shape[0] if transa else weight.shape[1], dtype=input_grad.dtype,
                                        device=input_grad.device)
         if is_matmul:
-            w = weight.t() if transa else weight
-            g = input_grad.t() if transb else input_grad
-            torch.matmul(g, w, out=dgrad_output)
+            if (not transa and not transb and dense_ok(weight, input_grad, dgrad_output)
+                    and weight.dtype == input_grad.dtype == dgrad_output.dtype):
+                dense_gemm(weight, input_grad, dgrad_output, False, False, False)
+            else:
+                w = weight.t() if transa else weight
+                g = input_grad.t() if transb else input_grad
+                torch.matmul(g, w, out=dgrad_output)
         else:
             gemm(weight, input_grad, dgrad_output, None, 0, transa, transb, False, math_sm_count, False)
     return dgrad_output, el[0]
@@ -76,7 +90,16 @@ def wgrad_bwd(args, input_grad: torch.Tensor, input_data: torch.Tensor, wgrad_ou
             else:
                 d = input_data.t() if transa else input_data
                 g = input_grad.t() if transb else input_grad
-            if wgrad_output is None:
+            fresh = wgrad_output is None
+            if (transb and not transa and dense_ok(input_grad, input_data) and input_grad.dtype == input_data.dtype
+                    and (fresh or (dense_ok(wgrad_output) and wgrad_output.dtype in (g.dtype, torch.float32)))):
+                if fresh:
+                    wgrad_output = torch.empty(input_grad.shape[1], input_data.shape[1], dtype=g.dtype, device=g.device)
+                if g.is_contiguous():                   # dY^T was materialised: the "NN" form
+                    dense_gemm(d, g, wgrad_output, False, False, not fresh)
+                else:
+                    dense_gemm(input_data, input_grad, wgrad_output, False, True, not fresh)
+            elif fresh:
                 wgrad_output = torch.matmul(g, d)
             elif wgrad_output.dtype == g.dtype:
                 wgrad_output.addmm_(g, d)

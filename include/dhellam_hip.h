@@ -244,6 +244,21 @@ int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
  * (dhellam/common/comm.py) in scheduler experiments, so that the double-strand runtime has something to hide. */
 int dh_delay(int64_t nanoseconds, void *stream);
 
+/* Dense GEMM through hipBLASLt: cublas_gemm / pygemm, csrc/operators/gemm.cu:3-170 (csrc/operators/ops.h:54-65).
+ * The reference's convention is kept: A [a_rows, a_cols], B [b_rows, b_cols] and D are contiguous row-major
+ * arrays given to a column-major library, so with m = transa ? a_rows : a_cols, k = transa ? a_cols : a_rows,
+ * n = transb ? b_cols : b_rows the result is the row-major D [n, m] =
+ *   transa=1, transb=0: B @ A^T (forward: activations x weight^T)     transa=0, transb=0: B @ A (data gradient)
+ *   transa=0, transb=1: B^T @ A (weight gradient)                      transa=1, transb=1: refused, as there.
+ * `accumulate` (the reference's grad_accumulate) adds to D instead of overwriting it.  Operands are bf16 / fp16
+ * / fp32 (`dtype`), D is of the same type or fp32 (`out_dtype`); products are accumulated in fp32.
+ * `workspace` (device, 256-byte aligned) and its size are what the library may use, as in the reference;
+ * the kernel is chosen once per (shape, layout, types, workspace size, device) by the library's heuristic and
+ * cached.  `math_sm_count` has no counterpart (see dh_stream_create_cu_mask). */
+int dh_gemm(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+            int transa, int transb, int accumulate, int dtype, int out_dtype, void *workspace,
+            size_t workspace_bytes, void *stream);
+
 /* A stream whose kernels run only on the compute units named in `mask` (bit i of word i / 32; `words` x 32
  * bits must cover the device; with several XCDs bit i is compute unit i / n_xcd of XCD i % n_xcd).  The
  * MI355X form of the reference's libsmctrl partitioning (csrc/operators/smctrl.cpp:135-160, the `math_sm_count`

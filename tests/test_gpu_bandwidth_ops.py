@@ -246,3 +246,76 @@ def test_binding_level_names_for_the_added_operators():
     assert ce["loss"].shape == (16,) and gr.shape == lg.shape
     table = randn((100, 64), dt, 10).cuda()
     assert torch.equal(_Clib.pyembedding_fwd(table, tg), table[tg])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,n,k", [(256, 384, 512), (100, 72, 40), (1, 8, 8), (4096, 1280, 1024)])
+def test_dense_gemm_layouts(dtype, t, n, k):
+    """pygemm (csrc/operators/gemm.cu:3-170) in its three layouts and the wrappers of
+    dhellam/operators/layernorm_column.py on the same products, against fp64 matmul."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
+    x, w, dy = randn((t, k), dtype, 0), randn((n, k), dtype, 1, std=0.1), randn((t, n), dtype, 2)
+    acc0 = randn((n, k), dtype, 3)
+    xg, wg, dyg = x.cuda(), w.cuda(), dy.cuda()
+    ref_y, ref_dx = x.double() @ w.double().t(), dy.double() @ w.double()
+    ref_dw = dy.double().t() @ x.double()
+    y = torch.empty(t, n, dtype=dtype, device="cuda")
+    assert _Clib.pygemm(wg, xg, y, None, 0, True, False, False, 0, False) == 0.0
+    assert_close(y, ref_y, dtype, "TN")
+    dx = torch.empty(t, k, dtype=dtype, device="cuda")
+    ms = _Clib.pygemm(wg, dyg, dx, None, 0, False, False, False, 0, True)
+    assert ms > 0.0
+    assert_close(dx, ref_dx, dtype, "NN")
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")        # the caller's workspace
+    for accumulate in (False, True):
+        dw = acc0.clone().cuda()
+        _Clib.pygemm(xg, dyg, dw, ws, ws.numel(), False, True, accumulate, 0, False)
+        assert_close(dw, ref_dw + (acc0.double() if accumulate else 0), dtype, "NT")
+    # the wrappers: leading dimensions, a given output, accumulation into an fp32 gradient
+    y3, _ = gemm_fwd(None, xg.view(1, t, k), wg, None, "TN", False, 0, True, None)
+    assert y3.shape == (1, t, n) and torch.equal(y3.view(t, n), y)
+    y4, _ = gemm_fwd(None, xg, wg, None, "TN", False, 0, False, None)
+    assert torch.equal(y4, y)
+    dx2, _ = dgrad_bwd(None, dyg, wg, None, "NN", False, 0, True, None)
+    assert torch.equal(dx2, dx)
+    g32 = acc0.float().cuda()
+    out, _ = wgrad_bwd(None, dyg, xg, g32, True, "NT", False, 0, True, None)
+    assert out is g32
+    assert_close(g32, ref_dw + acc0.double(), torch.float32 if dtype == torch.float32 else dtype, "fp32 dW", scale=0.1 if dtype != torch.float32 else 1)
+    fresh, _ = wgrad_bwd(None, dyg, xg, None, False, "NT", False, 0, True, None)
+    assert_close(fresh, ref_dw, dtype, "fresh dW")
+    # operands the C entry point does not take still work through the wrapper (strided view of the weight)
+    wide = torch.cat([wg, wg], 1)[:, :k]
+    assert not wide.is_contiguous() or k == wide.stride(0)
+    y5, _ = gemm_fwd(None, xg, wide, None, "TN", False, 0, True, None)
+    assert_close(y5, ref_y, dtype, "strided weight")
+
+
+def test_dense_gemm_argument_errors():
+    import ctypes
+    from dhellam_amd import _Clib, _lib
+    lib = _lib.load()
+    a = torch.zeros(16, 32, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(8, 32, dtype=torch.bfloat16, device="cuda")
+    d = torch.zeros(8, 16, dtype=torch.bfloat16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call(ar, ac, br, bc, ta, tb, dt=1, odt=1, ws=None, wsb=0, acc=0):
+        return lib.dh_gemm(a.data_ptr(), b.data_ptr(), d.data_ptr(), ar, ac, br, bc, ta, tb, acc, dt, odt, ws, wsb, st)
+
+    assert call(16, 32, 8, 32, 1, 0) == 0                                  # TN, no workspace
+    for bad in (call(16, 32, 8, 32, 1, 1),                                # TT
+                call(16, 32, 8, 24, 1, 0),                                # inner sizes differ
+                call(16, 32, 8, 32, 1, 0, dt=7, odt=7),                   # unknown type
+                call(16, 32, 8, 32, 1, 0, dt=1, odt=2),                   # bf16 operands, fp16 result
+                call(16, 32, 8, 32, 1, 0, ws=None, wsb=1024),             # a size without a buffer
+                call(16, 0, 8, 0, 1, 0)):                                 # empty sum, not accumulating
+        assert bad < 0
+        assert len(_lib.load().dh_last_error()) > 0
+    assert call(16, 0, 8, 0, 1, 0, acc=1) == 0                            # empty sum, accumulating: nothing to do
+    assert call(0, 32, 8, 32, 1, 0) == 0                                  # empty result
+    with pytest.raises(RuntimeError):
+        _Clib.dense_gemm(a, b, torch.zeros(16, 8, dtype=torch.bfloat16, device="cuda"), True, False, False)   # D is [n, m]
+    with pytest.raises(RuntimeError):
+        _Clib.dense_gemm(a, b.float(), d, True, False, False)

@@ -238,6 +238,18 @@ def kernel_rooflines(cfg):
     add(f"head_block_fwd_bwd[{T}x{H} -> {Vp}]", "mfma", 6.0 * T * H * Vp, ms, "6THV flop (logits GEMM fwd, dgrad, wgrad; norm, cross entropy, loss around them)")
     parallel_state.set_tensor_model_parallel(0, 1)
     del table, dh_, em_out, hid
+    # --- the layer's twelve dense products (library kernels through dh_gemm), as the layer calls them -------
+    from dhellam_amd.operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
+    for name, n_out, k_in in (("qkv", cfg.qkv_per_rank, H), ("attn_out", H, hq * d), ("fc1", 2 * F, H), ("fc2", H, F)):
+        x, w, dy = rn(T, k_in), rn(n_out, k_in), rn(T, n_out)
+        dw = torch.zeros(n_out, k_in, device=dev, dtype=dt)
+        flop = 2.0 * T * n_out * k_in
+        for what, fn in (("fwd", lambda: gemm_fwd(None, x, w, None, "TN", False, 0, True, None)),
+                         ("dgrad", lambda: dgrad_bwd(None, dy, w, None, "NN", False, 0, True, None)),
+                         ("wgrad", lambda: wgrad_bwd(None, dy, x, dw, True, "NT", False, 0, True, None))):
+            add(f"dense_gemm[{name} {what} T={T} N={n_out} K={k_in}]", "mfma", flop, time_gpu(fn, iters=10, warmup=3),
+                "2TNK flop (hipBLASLt through dh_gemm; wgrad includes the transpose of dY where it is used)")
+        del x, w, dy, dw
     return res
 
 

@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["add_tensors", "pygemm", "dense_gemm", "dense_ok", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
+__all__ = ["add_tensors", "pygemm", "dense_gemm", "dense_ok", "wgrad_gemm", "wgrad_layout", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
            "pyrmsnorm_fwd", "pyrmsnorm_bwd", "pyrope_fwd", "pyrope_bwd", "pyswiglu_fwd", "pyswiglu_bwd",
            "pymoe_route_topk", "pymoe_sort", "pymoe_permute", "pymoe_unpermute", "pygrouped_gemm_nt",
            "pygrouped_gemm_nn", "pygrouped_gemm_tn", "pycross_entropy_fwd", "pycross_entropy_bwd",
@@ -102,8 +102,8 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
 
     The product is ``dh_gemm`` (hipBLASLt behind the C ABI).  ``input_workspace`` / ``workspaceSize`` are
     used when given (a GPU tensor of at least that many bytes), otherwise a per-stream 32 MiB buffer;
-    ``math_sm_count`` is accepted and unused.  For the weight gradient, B^T is materialised first where that
-    makes the product faster by more than it costs (``wgrad_operands``).
+    ``math_sm_count`` is accepted and unused.  For the weight gradient, B^T is materialised first
+    where that makes the product faster by more than it costs (``wgrad_layout``).
     """
     _lib.need_cuda(inputA, inputB, outputD)
     stream = torch.cuda.current_stream()
@@ -111,11 +111,9 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
 
     def run():
         if transb and not transa:
-            bt, a = wgrad_operands(inputB, inputA)
-            if bt.is_contiguous():                      # the materialised transpose: now the "NN" form
-                dense_gemm(a, bt, outputD, False, False, grad_accumulate, input_workspace, ws_bytes)
-                return
-        dense_gemm(inputA, inputB, outputD, transa, transb, grad_accumulate, input_workspace, ws_bytes)
+            wgrad_gemm(inputB, inputA, outputD, grad_accumulate, input_workspace, ws_bytes)
+        else:
+            dense_gemm(inputA, inputB, outputD, transa, transb, grad_accumulate, input_workspace, ws_bytes)
 
     return _timed(profiling, stream, run)
 
@@ -138,11 +136,13 @@ def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
 # The weight-gradient product dW[N, K] = dY[T, N]^T X[T, K] reads both operands along their strided dimension, the
 # GEMM library's slowest layout here.  Measured at T = 4096, bf16, accumulating (us; N, K = 7168, 8192 / 8192, 3584 /
 # 1280, 8192 / 8192, 1024):   as given 484 / 233-257 / 95 / 76;   dY^T row-major 409 / 203 / 82 / 67;
-# dY^T and X^T both row-major 364 / 178 / 70 / 60.  dh_transpose_2d moves 5.5-6 TB/s (a [4096, 8192] matrix in
-# 24 us), so materialising dY^T pays from K of about 3000.  X^T as well would pay from N of about 4000, but for
-# that layout the library picks a stream-K kernel whose accumulation into dW is not reproducible when another
-# kernel shares the GPU (1 run in 100 of the double-strand schedule differed from the serial one in the last
-# bits of one weight gradient), and the two schedules are required to give identical bits: not used.
+# dY^T and X^T both row-major (the forward's layout) 343 / 171 / 73 / 61.  dh_transpose_2d moves 5.5-6 TB/s (a
+# [4096, 8192] matrix in 24 us), so materialising dY^T pays from K of about 3000.  X^T as well would pay from N of
+# about 4000, but for that layout the library picks a kernel that splits tiles over workgroups, and its
+# accumulation into dW does not always give the same bits when another kernel shares the GPU (1 step in 40-100
+# of the double-strand schedule differed from the serial one in the last bits of one weight gradient; giving each
+# stream its own workspace does not change that), while the two schedules are required to agree bit for bit: not
+# used.
 WGRAD_TRANSPOSE_GRAD_MIN_K = 3072
 WGRAD_TRANSPOSE_MIN_ELEMS = 1 << 20
 
@@ -160,6 +160,24 @@ def wgrad_operands(grad: torch.Tensor, data: torch.Tensor):
             and grad.dtype == data.dtype):
         return transpose_2d(grad), data
     return grad.t(), data
+
+
+def wgrad_layout(grad: torch.Tensor, data: torch.Tensor) -> str:
+    """Which operand of dW = dY^T X is materialised transposed before the library call: "NT" (none) or "NN" (dY^T)."""
+    (t, n), k = grad.shape, data.shape[1]
+    if (k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad)
+            and grad.dtype == data.dtype):
+        return "NN"
+    return "NT"
+
+
+def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumulate: bool, workspace=None,
+               workspace_bytes: int = 0) -> None:
+    """out [N, K] (+)= grad [T, N]^T @ data [T, K] through ``dh_gemm``, in the layout ``wgrad_layout`` picks."""
+    if wgrad_layout(grad, data) == "NN":
+        dense_gemm(data, transpose_2d(grad), out, False, False, accumulate, workspace, workspace_bytes)
+    else:
+        dense_gemm(data, grad, out, False, True, accumulate, workspace, workspace_bytes)
 
 
 def pygelu(input, output, profiling):

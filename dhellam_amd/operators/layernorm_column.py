@@ -20,7 +20,7 @@ import torch
 
 from .._Clib import dense_gemm, dense_ok
 from .._Clib import pygemm as gemm
-from .._Clib import wgrad_operands
+from .._Clib import wgrad_gemm
 from ._util import on_stream
 
 
@@ -85,26 +85,22 @@ def wgrad_bwd(args, input_grad: torch.Tensor, input_data: torch.Tensor, wgrad_ou
     el: list = []
     with on_stream(stream, profiling, el):
         if is_matmul:
-            if transb and not transa:
-                g, d = wgrad_operands(input_grad, input_data)
+            fresh = wgrad_output is None
+            dt = input_grad.dtype
+            if (transb and not transa and dense_ok(input_grad, input_data) and dt == input_data.dtype
+                    and (fresh or (dense_ok(wgrad_output) and wgrad_output.dtype in (dt, torch.float32)))):
+                if fresh:
+                    wgrad_output = torch.empty(input_grad.shape[1], input_data.shape[1], dtype=dt, device=input_grad.device)
+                wgrad_gemm(input_grad, input_data, wgrad_output, not fresh)
             else:
                 d = input_data.t() if transa else input_data
                 g = input_grad.t() if transb else input_grad
-            fresh = wgrad_output is None
-            if (transb and not transa and dense_ok(input_grad, input_data) and input_grad.dtype == input_data.dtype
-                    and (fresh or (dense_ok(wgrad_output) and wgrad_output.dtype in (g.dtype, torch.float32)))):
                 if fresh:
-                    wgrad_output = torch.empty(input_grad.shape[1], input_data.shape[1], dtype=g.dtype, device=g.device)
-                if g.is_contiguous():                   # dY^T was materialised: the "NN" form
-                    dense_gemm(d, g, wgrad_output, False, False, not fresh)
-                else:
-                    dense_gemm(input_data, input_grad, wgrad_output, False, True, not fresh)
-            elif fresh:
-                wgrad_output = torch.matmul(g, d)
-            elif wgrad_output.dtype == g.dtype:
-                wgrad_output.addmm_(g, d)
-            else:  # fp32 main_grad with 16-bit operands
-                wgrad_output.add_(torch.matmul(g, d))
+                    wgrad_output = torch.matmul(g, d)
+                elif wgrad_output.dtype == g.dtype:
+                    wgrad_output.addmm_(g, d)
+                else:  # fp32 main_grad with 16-bit operands
+                    wgrad_output.add_(torch.matmul(g, d))
         else:
             if wgrad_output is None:
                 wgrad_output = torch.empty(input_grad.shape[1] if transb else input_grad.shape[0],

@@ -184,6 +184,7 @@ def test_wgrad_product(dtype, T, N, K, accumulate):
     assert lhs.is_contiguous() == (dtype != torch.float32 and K >= 3072 and T * N >= 1 << 20)
     assert rhs.is_contiguous()
     assert torch.equal(lhs, dy.cuda().t()) and torch.equal(rhs, x.cuda())
+    assert _Clib.wgrad_layout(dy.cuda(), x.cuda()) == ("NN" if lhs.is_contiguous() else "NT")
     d = w0.clone().cuda()
     _Clib.pygemm(x.cuda(), dy.cuda(), d, None, 0, False, True, accumulate, 0, False)
     assert_close(d, ref, dtype, "pygemm wgrad")

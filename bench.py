@@ -356,7 +356,8 @@ def profile_op(name: str, iters: int = 5):
             fn = lambda: moe.grouped_gemm_nt(a, b, offs, out=c)
         else:
             b = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(dt)
-            fn = lambda: torch.matmul(a, b.t(), out=c)
+            from dhellam_amd._Clib import dense_gemm
+            fn = lambda: dense_gemm(b, a, c, True, False, False)     # the library kernel through dh_gemm
     elif name == "layer":
         # the serial schedule alone: four micro-batches of the 70B-shard layer, forward + backward
         from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights

@@ -320,3 +320,28 @@ def test_dense_gemm_argument_errors():
         _Clib.dense_gemm(a, b, torch.zeros(16, 8, dtype=torch.bfloat16, device="cuda"), True, False, False)   # D is [n, m]
     with pytest.raises(RuntimeError):
         _Clib.dense_gemm(a, b.float(), d, True, False, False)
+
+
+def test_dense_gemm_on_two_streams():
+    """Products issued on two streams at once (each stream has its own library workspace) give the bits of the
+    same products issued alone."""
+    from dhellam_amd import _Clib
+    dtype = torch.bfloat16
+    x, w = randn((2048, 4096), dtype, 0).cuda(), randn((1280, 4096), dtype, 1, std=0.1).cuda()      # under-filled grid
+    x2, w2 = randn((2048, 1024), dtype, 2).cuda(), randn((4096, 1024), dtype, 3, std=0.1).cuda()
+    y_ref, y2_ref = torch.empty(2048, 1280, dtype=dtype, device="cuda"), torch.empty(2048, 4096, dtype=dtype, device="cuda")
+    _Clib.dense_gemm(w, x, y_ref, True, False, False)
+    _Clib.dense_gemm(w2, x2, y2_ref, True, False, False)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    y, y2 = torch.empty_like(y_ref), torch.empty_like(y2_ref)
+    for _ in range(50):
+        y.zero_(), y2.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s1):
+            _Clib.dense_gemm(w, x, y, True, False, False)
+        with torch.cuda.stream(s2):
+            _Clib.dense_gemm(w2, x2, y2, True, False, False)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_ref) and torch.equal(y2, y2_ref)
+    assert len({k for k in _Clib._gemm_ws if k[1] in (s1.cuda_stream, s2.cuda_stream)}) == 2

@@ -18,6 +18,7 @@
 // ends up with runs of 4 consecutive output columns of one row: 8-byte stores.
 // Group row ranges are read on the device from the offsets table.
 #include "mma.h"
+#include <atomic>
 #ifndef DH_GG_WVN
 #define DH_GG_WVN 4
 #endif
@@ -48,7 +49,12 @@ struct GGParams {
   int64_t b_group_stride, c_group_stride;
   int tiles_m, tiles_n;  // grid extents (tiles_m is an upper bound for NT/NN)
   int accumulate;
+  int max_rows;          // rows the stacked operands hold: group ranges read from offs are cut off there
 };
+
+// A group's row range as the kernels use it: relative to the first group and never past the rows the caller's
+// buffers hold, whatever the offsets say (they live on the device, so the host cannot check them).
+__device__ __forceinline__ int gg_clamp_row(int r, int max_rows) { return r < 0 ? 0 : (r > max_rows ? max_rows : r); }
 
 // Load one 64-deep k slice of an operand into registers.
 //   KC (k-contiguous): tile [R rows][64 k]; element (row, k) at src[row * ld + k]
@@ -126,12 +132,12 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
   if (GROUPED_OUT) {
     // wgrad: one full [m_dim, n_dim] output per group; blockIdx.y = group
     g = blockIdx.y;
-    row_begin = p.offs[g] - base;
-    row_end = p.offs[g + 1] - base;
+    row_begin = gg_clamp_row(p.offs[g] - base, p.max_rows);
+    row_end = gg_clamp_row(p.offs[g + 1] - base, p.max_rows);
   } else {
     bool found = false;
     for (int gi = 0; gi < p.groups; ++gi) {
-      const int rb = p.offs[gi] - base, re = p.offs[gi + 1] - base;
+      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
       const int t = (re - rb + BM - 1) / BM;
       if (!found && tm < t) {
         g = gi; row_begin = rb; row_end = re; found = true;
@@ -327,7 +333,7 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
   {
     bool found = false;
     for (int gi = 0; gi < p.groups; ++gi) {
-      const int rb = p.offs[gi] - base, re = p.offs[gi + 1] - base;
+      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
       const int t = (re - rb + BM - 1) / BM;
       if (!found && tm < t) {
         g = gi; row_begin = rb; row_end = re; found = true;
@@ -577,11 +583,15 @@ static int launch_gg(GGParams p, int64_t m_extent, hipStream_t st) {
   using LB = TileLoader<T, BN, TB, NT>;
   constexpr size_t smem = 2 * (LA::ELEMS + LB::ELEMS) * sizeof(T);
   static_assert(smem <= 160 * 1024, "LDS budget");
-  static bool attr_set = false;
-  if (!attr_set) {
+  // the attribute belongs to the (kernel, device) pair: one bit per device, set by whichever thread gets there first
+  static std::atomic<uint64_t> attr_set{0};
+  int dev = 0;
+  DH_HIP(hipGetDevice(&dev));
+  const uint64_t bit = 1ull << (dev & 63);
+  if (!(attr_set.load(std::memory_order_acquire) & bit)) {
     DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&grouped_gemm_kernel<T, TA, TB, WM, WN, WVN, GROUPED_OUT>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
+    attr_set.fetch_or(bit, std::memory_order_release);
   }
   p.tiles_n = (int)cdiv(p.n_dim, BN);
   p.tiles_m = GROUPED_OUT ? (int)cdiv(m_extent, BM) : (int)(cdiv(m_extent, BM) + p.groups);
@@ -608,7 +618,8 @@ static int dispatch_gg(const GGParams &p, int64_t m_extent, int dtype, hipStream
 // output cost 45 us in front of the first expert GEMM).
 __global__ void __launch_bounds__(256) gg_zero_tail_kernel(uint16_t *c, const int32_t *__restrict__ offs, int groups,
                                                            int64_t max_rows, int64_t n) {
-  const int64_t first = offs[groups] - offs[0];
+  int64_t first = (int64_t)offs[groups] - offs[0];
+  if (first < 0) first = 0;
   const int64_t nv = n / 8;                                // n is a multiple of 8 (checked by the callers)
   for (int64_t r = first + blockIdx.x; r < max_rows; r += gridDim.x)
     for (int64_t v = threadIdx.x; v < nv; v += 256) {
@@ -636,7 +647,7 @@ static int gg_common_checks(const void *a, const void *b, void *c, const int32_t
 extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const int32_t *offs, int groups,
                                   int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
   using namespace dh;
-  DH_CHECK(max_rows >= 0 && n >= 0 && k >= 0, "negative size");
+  DH_CHECK(max_rows >= 0 && max_rows < (1ll << 31) && n >= 0 && k >= 0, "size out of range");
   if (max_rows == 0 || n == 0) return DH_OK;
   int rc = gg_common_checks(a, b, c, offs, groups, dtype);
   if (rc) return rc;
@@ -644,7 +655,7 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   GGParams p{};
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
-  p.b_group_stride = n * k; p.accumulate = 0;
+  p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && k < (1ll << 30))
@@ -660,7 +671,7 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
 extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const int32_t *offs, int groups,
                                   int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
   using namespace dh;
-  DH_CHECK(max_rows >= 0 && n >= 0 && k >= 0, "negative size");
+  DH_CHECK(max_rows >= 0 && max_rows < (1ll << 31) && n >= 0 && k >= 0, "size out of range");
   if (max_rows == 0 || n == 0) return DH_OK;
   int rc = gg_common_checks(a, b, c, offs, groups, dtype);
   if (rc) return rc;
@@ -668,7 +679,7 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   GGParams p{};
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = n; p.ldc = n;
-  p.b_group_stride = n * k; p.accumulate = 0;
+  p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
@@ -684,7 +695,7 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
 extern "C" int dh_grouped_gemm_tn(const void *a, const void *b, void *c, const int32_t *offs, int groups,
                                   int64_t max_rows, int64_t m, int64_t n, int accumulate, int dtype, void *stream) {
   using namespace dh;
-  DH_CHECK(max_rows >= 0 && n >= 0 && m >= 0, "negative size");
+  DH_CHECK(max_rows >= 0 && max_rows < (1ll << 31) && n >= 0 && m >= 0, "size out of range");
   if (m == 0 || n == 0) return DH_OK;
   int rc = gg_common_checks(a, b, c, offs, groups, dtype);
   if (rc) return rc;
@@ -692,7 +703,7 @@ extern "C" int dh_grouped_gemm_tn(const void *a, const void *b, void *c, const i
   GGParams p{};
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.m_dim = m; p.n_dim = n; p.lda = m; p.ldb = n; p.ldc = n;
-  p.c_group_stride = m * n; p.accumulate = accumulate;
+  p.c_group_stride = m * n; p.accumulate = accumulate; p.max_rows = (int)max_rows;
   rc = dispatch_gg<true, true, true>(p, m, dtype, (hipStream_t)stream);
   if (rc) return rc;
   DH_LAUNCH_CHECK();

@@ -73,7 +73,10 @@ moe_hist_kernel(const int32_t *__restrict__ expert_of, int32_t *__restrict__ his
 #pragma unroll
   for (int r = 0; r < SORT_ITEMS / 256; ++r) {
     const int64_t i = base + r * 256 + threadIdx.x;
-    if (i < n) atomicAdd(&cnt[expert_of[i]], 1);
+    if (i < n) {
+      const int e = expert_of[i];
+      if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);  // ids outside [0, E) are left out of the sort
+    }
   }
   __syncthreads();
   if ((int)threadIdx.x < E) hist[(int64_t)blockIdx.x * E + threadIdx.x] = cnt[threadIdx.x];
@@ -125,7 +128,8 @@ moe_rank_scatter_kernel(const int32_t *__restrict__ expert_of, const int32_t *__
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   for (int r = 0; r < SORT_ITEMS / 256; ++r) {
     const int64_t i = base + r * 256 + threadIdx.x;
-    const int my = i < n ? expert_of[i] : -1;
+    int my = i < n ? expert_of[i] : -1;
+    if (my >= E) my = -1;  // an id outside [0, E) gets no place (its dest_row is -1)
     int rank_in_wave = 0;
     for (int e = 0; e < E; ++e) {
       const uint64_t m = __ballot(my == e);
@@ -138,6 +142,8 @@ moe_rank_scatter_kernel(const int32_t *__restrict__ expert_of, const int32_t *__
       for (int ww = 0; ww < w; ++ww) pos += wcnt[ww][my];
       dest_row[i] = pos;
       sorted_idx[pos] = (int32_t)i;
+    } else if (i < n) {
+      dest_row[i] = -1;
     }
     __syncthreads();
     if ((int)threadIdx.x < E) running[threadIdx.x] += wcnt[0][threadIdx.x] + wcnt[1][threadIdx.x] + wcnt[2][threadIdx.x] + wcnt[3][threadIdx.x];
@@ -145,93 +151,147 @@ moe_rank_scatter_kernel(const int32_t *__restrict__ expert_of, const int32_t *__
   }
 }
 
-template <typename T>
+// A workgroup moves RPB rows per trip and issues every load of the trip before its first store: a row is only
+// hidden / N / 256 (2 at hidden 4096) vectors per lane, and one row per workgroup left the copy latency-bound.
+// Rows past max_rows are never written, whatever expert_offsets says (the caller sized `permuted` by it).
+template <typename T, int RPB>
 __global__ void __launch_bounds__(256)
 moe_gather_kernel(const T *__restrict__ x, const int32_t *__restrict__ sorted_idx, const float *__restrict__ row_scale,
-                  T *__restrict__ permuted, const int32_t *__restrict__ offs, int e_lo, int e_hi, int K, int64_t hidden,
-                  int vec_ok) {
+                  T *__restrict__ permuted, const int32_t *__restrict__ offs, int e_lo, int e_hi, int64_t max_rows,
+                  int K, int64_t hidden, int vec_ok) {
   constexpr int N = Vec<T>::N;
-  const int first = offs[e_lo], n_rows = offs[e_hi] - first;
-  for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
-    const int a = sorted_idx[first + r];
-    const int64_t t = a / K;
-    const float sc = row_scale ? row_scale[a] : 1.0f;
-    const T *src = x + t * hidden;
+  constexpr int U = 2;
+  const int first = offs[e_lo];
+  int64_t n_rows = (int64_t)offs[e_hi] - first;
+  if (n_rows > max_rows) n_rows = max_rows;
+  if (n_rows < 0) n_rows = 0;
+  // rows between the real count and max_rows are zeroed, so the caller may hand over uninitialised memory
+  for (int64_t r = n_rows + blockIdx.x; r < max_rows; r += gridDim.x) {
     T *dst = permuted + r * hidden;
     if (vec_ok) {
-      // four vectors in flight per lane: a row is only hidden / N / 256 (2 at hidden 4096) steps long, and one
-      // load per step left the copy latency-bound
+      Vec<T> z;
+#pragma unroll
+      for (int j = 0; j < N; ++j) z.v[j] = from_f<T>(0.f);
+      for (int64_t c = threadIdx.x; c < hidden / N; c += 256) stg(dst + c * N, z);
+    } else {
+      for (int64_t c = threadIdx.x; c < hidden; c += 256) dst[c] = from_f<T>(0.f);
+    }
+  }
+  for (int64_t r0 = (int64_t)blockIdx.x * RPB; r0 < n_rows; r0 += (int64_t)gridDim.x * RPB) {
+    const T *src[RPB];
+    float sc[RPB];
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) {
+      const int64_t r = r0 + i < n_rows ? r0 + i : n_rows - 1;
+      const int a = sorted_idx[first + r];
+      src[i] = x + (int64_t)(a / K) * hidden;
+      sc[i] = row_scale ? row_scale[a] : 1.0f;
+    }
+    if (vec_ok) {
       const int64_t nv = hidden / N;
-      for (int64_t c0 = threadIdx.x; c0 < nv; c0 += 4 * 256) {
-        Vec<T> v[4];
+      for (int64_t c0 = threadIdx.x; c0 < nv; c0 += U * 256) {
+        Vec<T> v[RPB][U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (c0 + u * 256 < nv) v[u] = ldg(src + (c0 + u * 256) * N);
+        for (int i = 0; i < RPB; ++i)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          if (c0 + u * 256 < nv) {
-            if (row_scale) {
+          for (int u = 0; u < U; ++u)
+            if (c0 + u * 256 < nv) v[i][u] = ldg(src[i] + (c0 + u * 256) * N);
 #pragma unroll
-              for (int j = 0; j < N; ++j) v[u].v[j] = from_f<T>(to_f(v[u].v[j]) * sc);
+        for (int i = 0; i < RPB; ++i) {
+          if (r0 + i < n_rows) {
+            T *dst = permuted + (r0 + i) * hidden;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+              if (c0 + u * 256 < nv) {
+                if (row_scale) {
+#pragma unroll
+                  for (int j = 0; j < N; ++j) v[i][u].v[j] = from_f<T>(to_f(v[i][u].v[j]) * sc[i]);
+                }
+                stg(dst + (c0 + u * 256) * N, v[i][u]);
+              }
             }
-            stg(dst + (c0 + u * 256) * N, v[u]);
           }
         }
       }
     } else {
-      for (int64_t c = threadIdx.x; c < hidden; c += 256) dst[c] = row_scale ? from_f<T>(to_f(src[c]) * sc) : src[c];
+#pragma unroll
+      for (int i = 0; i < RPB; ++i) {
+        if (r0 + i < n_rows) {
+          T *dst = permuted + (r0 + i) * hidden;
+          for (int64_t c = threadIdx.x; c < hidden; c += 256)
+            dst[c] = row_scale ? from_f<T>(to_f(src[i][c]) * sc[i]) : src[i][c];
+        }
+      }
     }
   }
 }
 
-template <typename T>
+// A workgroup combines TPB tokens per trip; all row loads of the trip are issued before the first store.
+// KT: compile-time bound of the slots per token (K <= KT), so the slot loops unroll to what is needed.
+template <typename T, int TPB, int KT>
 __global__ void __launch_bounds__(256)
 moe_scatter_kernel(const T *__restrict__ y, const int32_t *__restrict__ dest_row, const float *__restrict__ gates,
                    T *__restrict__ out, const int32_t *__restrict__ offs, int e_lo, int e_hi, int64_t tokens, int K,
                    int64_t hidden, int vec_ok) {
   constexpr int N = Vec<T>::N;
-  const int first = offs[e_lo], n_rows = offs[e_hi] - first;
-  for (int64_t t = blockIdx.x; t < tokens; t += gridDim.x) {
-    int rows[MOE_MAX_K];
-    float wts[MOE_MAX_K];
+  const int first = offs[e_lo];
+  const int64_t n_rows = (int64_t)offs[e_hi] - first;
+  for (int64_t t0 = (int64_t)blockIdx.x * TPB; t0 < tokens; t0 += (int64_t)gridDim.x * TPB) {
+    int rows[TPB][KT];
+    float wts[TPB][KT];
 #pragma unroll
-    for (int j = 0; j < MOE_MAX_K; ++j) {
-      rows[j] = -1;
-      wts[j] = 0.f;
-      if (j < K) {
-        const int rr = dest_row[t * K + j] - first;
-        if (rr >= 0 && rr < n_rows) {
-          rows[j] = rr;
-          wts[j] = gates ? gates[t * K + j] : 1.0f;
-        }
-      }
-    }
-    T *dst = out + t * hidden;
-    if (vec_ok) {
-      for (int64_t c = threadIdx.x; c < hidden / N; c += 256) {
-        float acc[N];
+    for (int i = 0; i < TPB; ++i)
 #pragma unroll
-        for (int e = 0; e < N; ++e) acc[e] = 0.f;
-#pragma unroll
-        for (int j = 0; j < MOE_MAX_K; ++j) {
-          if (j < K && rows[j] >= 0) {
-            const Vec<T> v = ldg(y + (int64_t)rows[j] * hidden + c * N);
-#pragma unroll
-            for (int e = 0; e < N; ++e) acc[e] += wts[j] * to_f(v.v[e]);
+      for (int j = 0; j < KT; ++j) {
+        rows[i][j] = -1;
+        wts[i][j] = 0.f;
+        if (j < K && t0 + i < tokens) {
+          const int64_t rr = (int64_t)dest_row[(t0 + i) * K + j] - first;
+          if (rr >= 0 && rr < n_rows) {
+            rows[i][j] = (int)rr;
+            wts[i][j] = gates ? gates[(t0 + i) * K + j] : 1.0f;
           }
         }
-        Vec<T> o;
+      }
+    if (vec_ok) {
+      for (int64_t c = threadIdx.x; c < hidden / N; c += 256) {
+        Vec<T> v[TPB][KT];
 #pragma unroll
-        for (int e = 0; e < N; ++e) o.v[e] = from_f<T>(acc[e]);
-        stg(dst + c * N, o);
+        for (int i = 0; i < TPB; ++i)
+#pragma unroll
+          for (int j = 0; j < KT; ++j)
+            if (rows[i][j] >= 0) v[i][j] = ldg(y + (int64_t)rows[i][j] * hidden + c * N);
+#pragma unroll
+        for (int i = 0; i < TPB; ++i) {
+          if (t0 + i < tokens) {
+            float acc[N];
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[e] = 0.f;
+#pragma unroll
+            for (int j = 0; j < KT; ++j)
+              if (rows[i][j] >= 0) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[e] += wts[i][j] * to_f(v[i][j].v[e]);
+              }
+            Vec<T> o;
+#pragma unroll
+            for (int e = 0; e < N; ++e) o.v[e] = from_f<T>(acc[e]);
+            stg(out + (t0 + i) * hidden + c * N, o);
+          }
+        }
       }
     } else {
-      for (int64_t c = threadIdx.x; c < hidden; c += 256) {
-        float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < MOE_MAX_K; ++j)
-          if (j < K && rows[j] >= 0) acc += wts[j] * to_f(y[(int64_t)rows[j] * hidden + c]);
-        dst[c] = from_f<T>(acc);
+      for (int i = 0; i < TPB; ++i) {
+        if (t0 + i < tokens) {
+          for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < KT; ++j)
+              if (rows[i][j] >= 0) acc += wts[i][j] * to_f(y[(int64_t)rows[i][j] * hidden + c]);
+            out[(t0 + i) * hidden + c] = from_f<T>(acc);
+          }
+        }
       }
     }
   }
@@ -242,7 +302,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_gate_grad_kernel(const T *__restrict__ dout, const T *__restrict__ y, const int32_t *__restrict__ dest_row,
                      float *__restrict__ dgates, const int32_t *__restrict__ offs, int e_lo, int e_hi, int64_t tokens,
-                     int K, int64_t hidden) {
+                     int K, int64_t hidden, int vec_ok) {
   __shared__ float red[4];
   const int first = offs[e_lo], n_rows = offs[e_hi] - first;
   for (int64_t a = blockIdx.x; a < tokens * K; a += gridDim.x) {
@@ -251,7 +311,16 @@ moe_gate_grad_kernel(const T *__restrict__ dout, const T *__restrict__ y, const 
     if (rr >= 0 && rr < n_rows) {  // uniform over the block
       const T *p = dout + (a / K) * hidden;
       const T *q = y + (int64_t)rr * hidden;
-      for (int64_t c = threadIdx.x; c < hidden; c += 256) s += to_f(p[c]) * to_f(q[c]);
+      if (vec_ok) {
+        constexpr int N = Vec<T>::N;
+        for (int64_t c = threadIdx.x; c < hidden / N; c += 256) {
+          const Vec<T> pv = ldg(p + c * N), qv = ldg(q + c * N);
+#pragma unroll
+          for (int e = 0; e < N; ++e) s += to_f(pv.v[e]) * to_f(qv.v[e]);
+        }
+      } else {
+        for (int64_t c = threadIdx.x; c < hidden; c += 256) s += to_f(p[c]) * to_f(q[c]);
+      }
     }
     s = block256_sum(s, red);
     if (threadIdx.x == 0) dgates[a] = s;
@@ -281,15 +350,10 @@ extern "C" size_t dh_moe_sort_workspace_bytes(int64_t n_assign, int experts) {
   return (size_t)(nb * (experts > 0 ? experts : 1) * sizeof(int32_t)) + 16;
 }
 
-extern "C" int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert, int32_t *expert_offsets,
-                           int32_t *sorted_idx, int32_t *dest_row, void *workspace, int64_t n_assign, int experts,
-                           void *stream) {
+static int moe_sort_launch(const int32_t *topk_idx, int32_t *tokens_per_expert, int32_t *expert_offsets,
+                           int32_t *sorted_idx, int32_t *dest_row, int32_t *hist, int64_t n_assign, int experts,
+                           hipStream_t st) {
   using namespace dh;
-  DH_CHECK(n_assign >= 0 && n_assign < (1ll << 31), "n_assign out of range");
-  DH_CHECK(experts >= 1 && experts <= MOE_MAX_E, "experts=%d must be in [1, %d]", experts, MOE_MAX_E);
-  DH_CHECK(tokens_per_expert && expert_offsets && workspace, "null pointer");
-  hipStream_t st = (hipStream_t)stream;
-  int32_t *hist = (int32_t *)workspace;
   const int nb = (int)cdiv(n_assign, SORT_ITEMS);
   if (nb > 0) {
     DH_CHECK(topk_idx && sorted_idx && dest_row, "null pointer");
@@ -303,6 +367,17 @@ extern "C" int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert, 
   return DH_OK;
 }
 
+extern "C" int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert, int32_t *expert_offsets,
+                           int32_t *sorted_idx, int32_t *dest_row, void *workspace, int64_t n_assign, int experts,
+                           void *stream) {
+  using namespace dh;
+  DH_CHECK(n_assign >= 0 && n_assign < (1ll << 31), "n_assign out of range");
+  DH_CHECK(experts >= 1 && experts <= MOE_MAX_E, "experts=%d must be in [1, %d]", experts, MOE_MAX_E);
+  DH_CHECK(tokens_per_expert && expert_offsets && workspace, "null pointer");
+  return moe_sort_launch(topk_idx, tokens_per_expert, expert_offsets, sorted_idx, dest_row, (int32_t *)workspace,
+                         n_assign, experts, (hipStream_t)stream);
+}
+
 static int moe_range_check(int e_lo, int e_hi) { return e_lo >= 0 && e_hi >= e_lo && e_hi <= dh::MOE_MAX_E; }
 
 extern "C" int dh_moe_gather_rows(const void *x, const int32_t *sorted_idx, const float *row_scale, void *permuted,
@@ -313,16 +388,22 @@ extern "C" int dh_moe_gather_rows(const void *x, const int32_t *sorted_idx, cons
   DH_CHECK(moe_range_check(e_lo, e_hi), "bad expert range [%d, %d)", e_lo, e_hi);
   if (max_rows == 0 || hidden == 0) return DH_OK;
   DH_CHECK(x && sorted_idx && permuted && expert_offsets, "null pointer");
-  int64_t blocks = max_rows < 65536 ? max_rows : 65536;
+  constexpr int RPB = 4;
+  int64_t blocks = cdiv(max_rows, RPB);
+  if (blocks > 65536) blocks = 65536;
   DH_DISPATCH_DTYPE(dtype, {
     const int vec_ok = hidden % Vec<T>::N == 0 && aligned16(x) && aligned16(permuted);
-    hipLaunchKernelGGL((moe_gather_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const T *)x, sorted_idx, row_scale, (T *)permuted, expert_offsets, e_lo, e_hi, k, hidden,
-                       vec_ok);
+    hipLaunchKernelGGL((moe_gather_kernel<T, RPB>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const T *)x, sorted_idx, row_scale, (T *)permuted, expert_offsets, e_lo, e_hi, max_rows, k,
+                       hidden, vec_ok);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;
 }
+
+#define DH_SCATTER(KT)                                                                                             \
+  hipLaunchKernelGGL((moe_scatter_kernel<T, TPB, KT>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, \
+                     (const T *)y, dest_row, gates, (T *)out, expert_offsets, e_lo, e_hi, tokens, k, hidden, vec_ok)
 
 extern "C" int dh_moe_scatter_rows(const void *y, const int32_t *dest_row, const float *gates, void *out,
                                    const int32_t *expert_offsets, int e_lo, int e_hi, int64_t tokens, int k,
@@ -333,11 +414,15 @@ extern "C" int dh_moe_scatter_rows(const void *y, const int32_t *dest_row, const
   DH_CHECK(moe_range_check(e_lo, e_hi), "bad expert range [%d, %d)", e_lo, e_hi);
   if (tokens == 0 || hidden == 0) return DH_OK;
   DH_CHECK(dest_row && out && expert_offsets, "null pointer");
-  int64_t blocks = tokens < 65536 ? tokens : 65536;
+  constexpr int TPB = 2;
+  int64_t blocks = cdiv(tokens, TPB);
+  if (blocks > 65536) blocks = 65536;
   DH_DISPATCH_DTYPE(dtype, {
     const int vec_ok = hidden % Vec<T>::N == 0 && aligned16(y) && aligned16(out);
-    hipLaunchKernelGGL((moe_scatter_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const T *)y, dest_row, gates, (T *)out, expert_offsets, e_lo, e_hi, tokens, k, hidden, vec_ok);
+    if (k <= 1) DH_SCATTER(1);
+    else if (k <= 2) DH_SCATTER(2);
+    else if (k <= 4) DH_SCATTER(4);
+    else DH_SCATTER(8);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;
@@ -353,8 +438,10 @@ extern "C" int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *
   DH_CHECK(dout && dest_row && dgates && expert_offsets, "null pointer");
   int64_t blocks = tokens * k < 65536 ? tokens * k : 65536;
   DH_DISPATCH_DTYPE(dtype, {
+    const int vec_ok = hidden % Vec<T>::N == 0 && aligned16(dout) && aligned16(y);
     hipLaunchKernelGGL((moe_gate_grad_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const T *)dout, (const T *)y, dest_row, dgates, expert_offsets, e_lo, e_hi, tokens, k, hidden);
+                       (const T *)dout, (const T *)y, dest_row, dgates, expert_offsets, e_lo, e_hi, tokens, k, hidden,
+                       vec_ok);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;

@@ -593,6 +593,12 @@ extern "C" size_t dh_norm_bwd_workspace_bytes(int64_t rows, int64_t cols) {
   return (size_t)(2 * (a > b ? a : b) * cols * (int64_t)sizeof(float));
 }
 
+namespace dh {
+__global__ void __launch_bounds__(256) zero_bytes_kernel(uint8_t *p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0;
+}
+}  // namespace dh
+
 extern "C" int dh_norm_bwd(const void *dy, const void *x, const float *mu, const float *rsigma, const void *gamma,
                            const void *add_to_dx, void *dx, void *dgamma, void *dbeta, void *workspace,
                            int64_t rows, int64_t cols, int zero_centered_gamma, int accumulate_wgrad, int dtype,
@@ -606,9 +612,13 @@ extern "C" int dh_norm_bwd(const void *dy, const void *x, const float *mu, const
   hipStream_t st = (hipStream_t)stream;
   if (rows == 0) {
     // no rows: the weight gradients are zero (or unchanged when accumulating)
+    // (a fill kernel, not a memset: memset nodes are unreliable inside a captured graph)
     if (!accumulate_wgrad) {
-      DH_HIP(hipMemsetAsync(dgamma, 0, cols * dtype_size(dtype), st));
-      if (mu && dbeta) DH_HIP(hipMemsetAsync(dbeta, 0, cols * dtype_size(dtype), st));
+      const int64_t nbytes = cols * (int64_t)dtype_size(dtype);
+      const unsigned blocks = (unsigned)(cdiv(nbytes, 256) < 1024 ? cdiv(nbytes, 256) : 1024);
+      hipLaunchKernelGGL(zero_bytes_kernel, dim3(blocks), dim3(256), 0, st, (uint8_t *)dgamma, nbytes);
+      if (mu && dbeta) hipLaunchKernelGGL(zero_bytes_kernel, dim3(blocks), dim3(256), 0, st, (uint8_t *)dbeta, nbytes);
+      DH_LAUNCH_CHECK();
     }
     return DH_OK;
   }

@@ -67,7 +67,7 @@ def _gather(x, plan, e_lo, e_hi, max_rows, row_scale, stream, profiling):
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2
     el: list = []
     with on_stream(stream, profiling, el) as st:
-        out = torch.zeros((max_rows, x.shape[1]), dtype=x.dtype, device=x.device)
+        out = torch.empty((max_rows, x.shape[1]), dtype=x.dtype, device=x.device)   # the kernel zeroes the unused rows
         _lib.check(lib.dh_moe_gather_rows(x.data_ptr(), plan.sorted_idx.data_ptr(), _lib.ptr(row_scale),
                                           out.data_ptr(), plan.expert_offsets.data_ptr(), e_lo, e_hi, max_rows,
                                           plan.k, x.shape[1], _lib.dt(x), st.cuda_stream))

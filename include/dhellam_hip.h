@@ -185,7 +185,9 @@ int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert,
 /* The rows of local experts [e_lo, e_hi) are the sorted positions
  * [first, first + n_rows) with first = expert_offsets[e_lo] and n_rows =
  * expert_offsets[e_hi] - first, both read ON DEVICE (no host sync); launches
- * cover max_rows / tokens.
+ * cover max_rows / tokens.  `permuted` holds max_rows rows: rows past that are
+ * never written, whatever the offsets say, and rows [n_rows, max_rows) are
+ * zeroed (so `permuted` may be uninitialised on entry).
  *
  * gather: permuted[r] = scale * x[sorted_idx[first + r] / k] for r < n_rows,
  * scale = row_scale[sorted_idx[first + r]] if row_scale != NULL else 1. */
@@ -218,8 +220,9 @@ int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *dest_row,
  *   NT: c[rows_g, n] = a[rows_g, k] * b[g][n, k]^T          (forward)
  *   NN: c[rows_g, n] = a[rows_g, k] * b[g][k, n]            (dgrad)
  *   TN: c[g][m, n] (+)= a[rows_g, m]^T * b[rows_g, n]       (wgrad)
- * max_rows bounds the launch grid; NT / NN zero the rows of c from the last group's end up to
- * max_rows, so c may be uninitialised on entry.
+ * max_rows is the number of rows the stacked operands hold: it bounds the launch grid, group ranges read
+ * from offs are cut off there (no row past it is read or written), and NT / NN zero the rows of c from the
+ * last group's end up to max_rows, so c may be uninitialised on entry.
  * ---------------------------------------------------------------------- */
 int dh_grouped_gemm_nt(const void *a, const void *b, void *c,
                        const int32_t *offs, int groups, int64_t max_rows,

@@ -103,14 +103,16 @@ def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=No
     ffn (per rank), seq, batch, tp, tp_rank, eps, theta.  w: column_attn_weight,
     linear_attn_weight, column_mlp_weight, linear_mlp_weight, ln_attn_weight,
     ln_mlp_weight.  mb: x, dy [b, seq/tp, hidden] (+ sp_peer_* [b*seq, hidden] when tp > 1).
-    ``round_to``: dtype every op's output is rounded to (models a 16-bit pipeline).
+    ``round_to``: dtype every op's output is rounded to, and with it the gradient that comes back
+    through that output (a 16-bit pipeline stores both in that type).
     Returns (out, grads) with grads = {x, ln_attn_weight, ln_mlp_weight, column_attn_weight,
     linear_attn_weight, column_mlp_weight, linear_mlp_weight}."""
-    rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
+    rnd = O.pipeline_round(round_to)
     b, s, tp, H = cfg["batch"], cfg["seq"], cfg["tp"], cfg["hidden"]
     rows = b * s // tp
-    P = {k: v.to(dtype).requires_grad_() for k, v in w.items()}
-    x = mb["x"].to(dtype).reshape(rows, H).requires_grad_()
+    leaf = lambda t: t.detach().to(dtype).clone().requires_grad_()         # never the caller's own tensor
+    P = {k: leaf(v) for k, v in w.items()}
+    x = leaf(mb["x"].reshape(rows, H))
     dy = mb["dy"].to(dtype).reshape(rows, H)
     out = layer_forward(cfg, P, x, mb, dtype, rnd)
     (out * dy).sum().backward()

@@ -78,14 +78,16 @@ def grouped_ffn(xp, w1, w2, group_offs, dtype=torch.float64, round_to=None):
     dhellam/operators/swiglu.py:15), w2 [G, H, F]; group g owns rows
     [group_offs[g]-group_offs[0], group_offs[g+1]-group_offs[0]).
     ``round_to``: dtype the intermediate h and a are rounded to (what a 16-bit pipeline
-    stores between its GEMMs).  Returns (y, h, a)."""
+    stores between its GEMMs; the gradients that come back through h and a are rounded to it as
+    well).  Returns (y, h, a)."""
     base = int(group_offs[0])
     R = int(group_offs[-1]) - base
     F = w2.shape[2]
     h = torch.zeros((R, 2 * F), dtype=dtype, device=xp.device)
     a = torch.zeros((R, F), dtype=dtype, device=xp.device)
     y = torch.zeros((R, w2.shape[1]), dtype=dtype, device=xp.device)
-    rnd = (lambda t: t.to(round_to).to(dtype)) if round_to is not None else (lambda t: t)
+    from .ops import pipeline_round
+    rnd = pipeline_round(round_to)
     for g in range(w1.shape[0]):
         r0, r1 = int(group_offs[g]) - base, int(group_offs[g + 1]) - base
         hg = rnd(xp[r0:r1].to(dtype) @ w1[g].to(dtype).T)

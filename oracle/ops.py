@@ -11,6 +11,28 @@ import torch
 F64 = torch.float64
 
 
+class _PipelineRound(torch.autograd.Function):
+    """What a 16-bit pipeline does to a tensor it hands from one operator to the next: the value is
+    rounded to the storage type on the way forward, and the gradient that comes back through the same
+    hand-over (the output of the next operator's backward) is rounded to it too."""
+
+    @staticmethod
+    def forward(ctx, t, store):
+        ctx.store = store
+        return t.to(store).to(t.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.to(ctx.store).to(g.dtype), None
+
+
+def pipeline_round(store):
+    """t -> t stored as ``store`` (forward value and backward gradient both); the identity for ``store`` None."""
+    if store is None:
+        return lambda t: t
+    return lambda t: _PipelineRound.apply(t, store)
+
+
 # --------------------------------------------------------------------------------------
 # RMSNorm / LayerNorm.  API slot: dhellam/operators/layernorm.py:6-45 (fwd), :47-91 (bwd).
 # The arithmetic is TransformerEngine's (un-vendored); this is the textbook definition.

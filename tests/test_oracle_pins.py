@@ -396,3 +396,175 @@ def test_model_oracle_without_layers_is_tied_embedding_cross_entropy():
         loss.backward()
     assert torch.allclose(grads["word_embeddings"], tr.grad, atol=1e-12)
     assert torch.allclose(grads["final_ln_weight"], gr.grad, atol=1e-12)
+
+
+# ---- decoder layer ---------------------------------------------------------------------------
+def _angles(s, d, theta):
+    """Rotation angles as the path defines them: position times theta^(-2j/d), both factors and their product in
+    fp32 (one rounding each), [s, d/2]."""
+    inv = torch.tensor([theta ** (-2.0 * j / d) for j in range(d // 2)], dtype=D).float()
+    return (torch.arange(s, dtype=torch.float32)[:, None] * inv[None, :]).to(D)
+
+
+def _independent_layer(cfg, W, x):
+    """The layer of ``oracle.layer.layer_forward`` at tp = 1, written again from library routines only
+    (F.rms_norm, F.linear, F.scaled_dot_product_attention, F.silu) with its own QKV unpacking (a Python loop
+    over kv groups) and its own RoPE (complex multiplication of the (j, j + d/2) pairs)."""
+    hq, hk, d, F_ = cfg["heads"], cfg["groups"], cfg["head_dim"], cfg["ffn"]
+    b, s, H = cfg["batch"], cfg["seq"], cfg["hidden"]
+    r = hq // hk
+    h1 = F.rms_norm(x, (H,), W["ln_attn_weight"], cfg["eps"])
+    qkv = F.linear(h1, W["column_attn_weight"]).view(b, s, (hq + 2 * hk) * d)
+    qs, ks, vs = [], [], []
+    width = (r + 2) * d
+    for g in range(hk):                                    # group g: [its r q heads | k_g | v_g]
+        blk = qkv[..., g * width:(g + 1) * width]
+        for j in range(r):
+            qs.append(blk[..., j * d:(j + 1) * d])
+        ks.append(blk[..., r * d:(r + 1) * d])
+        vs.append(blk[..., (r + 1) * d:(r + 2) * d])
+    q, k, v = torch.stack(qs, 1), torch.stack(ks, 1), torch.stack(vs, 1)           # [b, heads, s, d]
+
+    def rotate(t):
+        ang = _angles(s, d, cfg["theta"])
+        z = torch.complex(t[..., : d // 2], t[..., d // 2:]) * torch.polar(torch.ones_like(ang), ang)
+        return torch.cat((z.real, z.imag), -1)
+
+    q, k = rotate(q), rotate(k)
+    o = F.scaled_dot_product_attention(q, k.repeat_interleave(r, 1), v.repeat_interleave(r, 1), is_causal=True)
+    o = o.transpose(1, 2).reshape(b * s, hq * d)
+    x2 = x + F.linear(o, W["linear_attn_weight"])
+    u = F.linear(F.rms_norm(x2, (H,), W["ln_mlp_weight"], cfg["eps"]), W["column_mlp_weight"])
+    return x2 + F.linear(F.silu(u[:, :F_]) * u[:, F_:], W["linear_mlp_weight"])
+
+
+def _layer_case(tp=1, tp_rank=0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    r_ = lambda *s_, std=1.0: torch.randn(*s_, generator=g, dtype=D) * std
+    cfg = dict(hidden=24, heads=4, groups=2, head_dim=6, ffn=10, seq=8, batch=2, tp=tp, tp_rank=tp_rank, eps=1e-5,
+               theta=10000.0)
+    H, T = cfg["hidden"], cfg["batch"] * cfg["seq"]
+    W = {"column_attn_weight": r_((4 + 4) * 6, H, std=0.3), "linear_attn_weight": r_(H, 24, std=0.3),
+         "column_mlp_weight": r_(20, H, std=0.3), "linear_mlp_weight": r_(H, 10, std=0.3),
+         "ln_attn_weight": 1 + 0.2 * r_(H), "ln_mlp_weight": 1 + 0.2 * r_(H)}
+    rows = T // tp
+    mb = {"x": r_(cfg["batch"], rows // cfg["batch"], H) if rows % cfg["batch"] == 0 else r_(1, rows, H),
+          "dy": r_(cfg["batch"], rows // cfg["batch"], H) if rows % cfg["batch"] == 0 else r_(1, rows, H)}
+    if tp > 1:
+        for key in ("sp_peer_attn", "sp_peer_attn_bwd", "sp_peer_mlp", "sp_peer_mlp_bwd"):
+            mb[key] = r_(T, H)
+    return cfg, W, mb
+
+
+def test_layer_oracle_matches_an_independently_written_layer():
+    """Output and every gradient of ``layer_fwd_bwd`` (tp = 1, GQA 4 q / 2 kv heads, batch 2, so the packing per
+    kv group, the per-sequence RoPE positions and the causal mask per sequence all matter) against fp64 autograd
+    of ``_independent_layer``.  A swapped q/k/v block, head-major instead of group-major packing, positions that
+    run over the batch, or up/gate exchanged each fail it."""
+    from oracle import layer as OL
+    cfg, W, mb = _layer_case()
+    out, grads = OL.layer_fwd_bwd(cfg, W, mb)
+    Wr = {k_: v_.clone().requires_grad_() for k_, v_ in W.items()}
+    xr = mb["x"].reshape(-1, cfg["hidden"]).clone().requires_grad_()
+    ref = _independent_layer(cfg, Wr, xr)
+    (ref * mb["dy"].reshape(ref.shape)).sum().backward()
+    assert torch.allclose(out.reshape(ref.shape), ref.detach(), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(grads["x"].reshape(xr.shape), xr.grad, rtol=1e-11, atol=1e-12)
+    for k_ in W:
+        assert torch.allclose(grads[k_], Wr[k_].grad, rtol=1e-11, atol=1e-12), k_
+    # the pin must be able to fail: head-major packing ([all q | all k | all v]) is a different layer
+    Wswap = dict(W)
+    d, r = cfg["head_dim"], cfg["heads"] // cfg["groups"]
+    idx = torch.arange((cfg["heads"] + 2 * cfg["groups"]) * d).view(cfg["groups"], (r + 2) * d)
+    head_major = torch.cat((idx[:, : r * d].reshape(-1), idx[:, r * d:(r + 1) * d].reshape(-1), idx[:, (r + 1) * d:].reshape(-1)))
+    Wswap["column_attn_weight"] = W["column_attn_weight"][head_major]
+    out_swapped, _ = OL.layer_fwd_bwd(cfg, Wswap, mb)
+    assert not torch.allclose(out_swapped, out, atol=1e-3)
+
+
+@pytest.mark.parametrize("tp_rank", [0, 2, 3])
+def test_layer_oracle_sequence_parallel_stand_ins(tp_rank):
+    """tp = 4: the gather stand-in puts the rank's rows into the peer tensor (all other rows stay the peer's),
+    its backward hands back the rank's row slice; the scatter stand-in takes the rank's row slice, its backward
+    puts the slice's gradient into the peer gradient.  Checked on the layer as a whole against explicit slicing
+    in ``_sp_reference`` (every op from the library), output and all gradients."""
+    from oracle import layer as OL
+    cfg, W, mb = _layer_case(tp=4, tp_rank=tp_rank, seed=1)
+    H, T, b, s = cfg["hidden"], cfg["batch"] * cfg["seq"], cfg["batch"], cfg["seq"]
+    rows = T // 4
+    r0, r1 = tp_rank * rows, (tp_rank + 1) * rows
+    out, grads = OL.layer_fwd_bwd(cfg, W, mb)
+
+    Wr = {k_: v_.clone().requires_grad_() for k_, v_ in W.items()}
+    xr = mb["x"].reshape(rows, H).clone().requires_grad_()
+    hq, hk, d, F_ = cfg["heads"], cfg["groups"], cfg["head_dim"], cfg["ffn"]
+
+    def put(peer, mine):                       # the peer tensor with this rank's rows replaced
+        return torch.cat((peer[:r0], mine, peer[r1:]), 0)
+
+    def take_with_peer_grad(a, peer_grad):
+        # (this rank's rows of a, a scalar whose gradient is the peer gradient on all OTHER rows of a): adding
+        # the scalar to the loss gives ``a`` the gradient the scatter stand-in hands back
+        mask = torch.ones(T, 1, dtype=D)
+        mask[r0:r1] = 0
+        return a[r0:r1], (a * mask * peer_grad).sum()
+
+    # attention half on the gathered rows, with the library pieces of _independent_layer
+    h1 = F.rms_norm(xr, (H,), Wr["ln_attn_weight"], cfg["eps"])
+    X = put(mb["sp_peer_attn"], h1)
+    qkv = F.linear(X, Wr["column_attn_weight"]).view(b, s, -1)
+    r = hq // hk
+    width = (r + 2) * d
+    q = torch.stack([qkv[..., g * width + j * d: g * width + (j + 1) * d] for g in range(hk) for j in range(r)], 1)
+    k = torch.stack([qkv[..., g * width + r * d: g * width + (r + 1) * d] for g in range(hk)], 1)
+    v = torch.stack([qkv[..., g * width + (r + 1) * d: (g + 1) * width] for g in range(hk)], 1)
+    ang = _angles(s, d, cfg["theta"])
+    rot = lambda t: torch.cat(((t[..., : d // 2] * ang.cos() - t[..., d // 2:] * ang.sin()),
+                               (t[..., d // 2:] * ang.cos() + t[..., : d // 2] * ang.sin())), -1)
+    o = F.scaled_dot_product_attention(rot(q), rot(k).repeat_interleave(r, 1), v.repeat_interleave(r, 1), is_causal=True)
+    a = F.linear(o.transpose(1, 2).reshape(T, hq * d), Wr["linear_attn_weight"])
+    a_sp, carry1 = take_with_peer_grad(a, mb["sp_peer_attn_bwd"])
+    x2 = xr + a_sp
+    X2 = put(mb["sp_peer_mlp"], F.rms_norm(x2, (H,), Wr["ln_mlp_weight"], cfg["eps"]))
+    u = F.linear(X2, Wr["column_mlp_weight"])
+    y = F.linear(F.silu(u[:, :F_]) * u[:, F_:], Wr["linear_mlp_weight"])
+    y_sp, carry2 = take_with_peer_grad(y, mb["sp_peer_mlp_bwd"])
+    ref = x2 + y_sp
+    # loss: <out, dy> plus the peer gradients flowing into the rows of a and y that belong to other ranks
+    ((ref * mb["dy"].reshape(rows, H)).sum() + carry1 + carry2).backward()
+    assert torch.allclose(out.reshape(rows, H), ref.detach(), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(grads["x"].reshape(rows, H), xr.grad, rtol=1e-11, atol=1e-12)
+    for k_ in W:
+        assert torch.allclose(grads[k_], Wr[k_].grad, rtol=1e-11, atol=1e-12), k_
+
+
+def test_layer_oracle_stand_in_nodes():
+    """The two autograd nodes on their own: rows outside [r0, r1) of the gathered tensor are the peer's, dx is the
+    row slice; the scattered tensor is the row slice and the gradient handed back is the peer gradient with the
+    slice replaced."""
+    from oracle.layer import _Gather, _Scatter
+    h, peer, pg = rnd(3, 5).requires_grad_(), rnd(12, 5), rnd(12, 5)
+    X = _Gather.apply(h, peer, 6, 9)
+    assert torch.equal(X[:6], peer[:6]) and torch.equal(X[9:], peer[9:]) and torch.equal(X[6:9], h.detach())
+    G = rnd(12, 5)
+    X.backward(G)
+    assert torch.equal(h.grad, G[6:9])
+    a = rnd(12, 5).requires_grad_()
+    sl = _Scatter.apply(a, pg, 6, 9)
+    assert torch.equal(sl, a.detach()[6:9])
+    g = rnd(3, 5)
+    sl.backward(g)
+    want = pg.clone()
+    want[6:9] = g
+    assert torch.equal(a.grad, want)
+
+
+def test_pipeline_round_rounds_value_and_gradient():
+    """round_to: the value handed on and the gradient handed back are both stored in the 16-bit type."""
+    x = (torch.arange(16, dtype=D) / 7 + 1).requires_grad_()
+    y = O.pipeline_round(torch.bfloat16)(x)
+    assert torch.equal(y.detach(), x.detach().to(torch.bfloat16).to(D))
+    g = torch.arange(16, dtype=D) / 11 + 1
+    y.backward(g)
+    assert torch.equal(x.grad, g.to(torch.bfloat16).to(D))
+    assert O.pipeline_round(None)(x) is x

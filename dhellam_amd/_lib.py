@@ -52,6 +52,8 @@ SIGNATURES = {
     "dh_moe_route_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "dh_moe_sort_workspace_bytes": (_sz, [_i64, _i32]),
     "dh_moe_sort": (_i32, [_vp] * 6 + [_i64, _i32, _vp]),
+    "dh_moe_sort_static_max_assign": (_i64, []),
+    "dh_moe_sort_static": (_i32, [_vp] * 5 + [_i64, _i32, _vp]),
     "dh_moe_gather_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
     "dh_moe_scatter_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
     "dh_moe_gate_grad": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),

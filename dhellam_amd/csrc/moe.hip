@@ -12,6 +12,7 @@
 //   scatter : out[t] = sum_j gate * y[row of (t, j)]   (fixed j order, fp32)
 // Row counts live on the device (expert_offsets), so nothing here syncs the host.
 #include "common.h"
+#include <mutex>
 
 namespace dh {
 
@@ -376,6 +377,51 @@ extern "C" int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert, 
   DH_CHECK(tokens_per_expert && expert_offsets && workspace, "null pointer");
   return moe_sort_launch(topk_idx, tokens_per_expert, expert_offsets, sorted_idx, dest_row, (int32_t *)workspace,
                          n_assign, experts, (hipStream_t)stream);
+}
+
+// ---- the sort for callers that cannot allocate ---------------------------------------------------------------
+// The per-block histogram / start-position table lives in a file-scope device array instead of a caller's
+// workspace.  The array's name is only a host-side handle: its device address is asked for once per device
+// (hipGetSymbolAddress, with that device current) and every launch gets that address.
+constexpr int64_t MOE_STATIC_MAX_ASSIGN = 1ll << 20;
+constexpr int MOE_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) int32_t scratch[(MOE_STATIC_MAX_ASSIGN / dh::SORT_ITEMS) * dh::MOE_MAX_E];
+static int32_t *g_scratch_ptr[MOE_STATIC_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int moe_static_scratch(int32_t **out) {
+  int dev = -1;
+  DH_HIP(hipGetDevice(&dev));
+  DH_CHECK(dev >= 0 && dev < MOE_STATIC_MAX_DEVICES, "device %d outside [0, %d)", dev, MOE_STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    DH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    DH_CHECK(p != nullptr, "no device address for the static sort table");
+    g_scratch_ptr[dev] = (int32_t *)p;
+  }
+  *out = g_scratch_ptr[dev];
+  return DH_OK;
+}
+
+extern "C" int64_t dh_moe_sort_static_max_assign(void) { return MOE_STATIC_MAX_ASSIGN; }
+
+extern "C" int dh_moe_sort_static(const int32_t *topk_idx, int32_t *tokens_per_expert, int32_t *expert_offsets,
+                                  int32_t *sorted_idx, int32_t *dest_row, int64_t n_assign, int experts,
+                                  void *stream) {
+  using namespace dh;
+  DH_CHECK(n_assign >= 0 && n_assign <= MOE_STATIC_MAX_ASSIGN,
+           "n_assign=%lld exceeds what the static table holds (%lld); use dh_moe_sort with a workspace",
+           (long long)n_assign, (long long)MOE_STATIC_MAX_ASSIGN);
+  DH_CHECK(experts >= 1 && experts <= MOE_MAX_E, "experts=%d must be in [1, %d]", experts, MOE_MAX_E);
+  DH_CHECK(tokens_per_expert && expert_offsets, "null pointer");
+  int32_t *hist = nullptr;
+  const int rc = moe_static_scratch(&hist);
+  if (rc != DH_OK) return rc;
+  // Nothing of the table has to start at zero: the histogram kernel writes every (block, expert) entry that the
+  // scan and the ranked scatter of this call read, so what an earlier call left behind is never seen.
+  return moe_sort_launch(topk_idx, tokens_per_expert, expert_offsets, sorted_idx, dest_row, hist, n_assign, experts,
+                         (hipStream_t)stream);
 }
 
 static int moe_range_check(int e_lo, int e_hi) { return e_lo >= 0 && e_hi >= e_lo && e_hi <= dh::MOE_MAX_E; }

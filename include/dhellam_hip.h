@@ -182,6 +182,18 @@ int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert,
                 int32_t *expert_offsets, int32_t *sorted_idx, int32_t *dest_row,
                 void *workspace, int64_t n_assign, int experts, void *stream);
 
+/* dh_moe_sort for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same results as
+ * dh_moe_sort; the per-block histogram table lives in a device array inside the library (256 KiB per GPU, held
+ * until the process ends), so n_assign is limited to dh_moe_sort_static_max_assign() (2^20) and a larger list
+ * is refused with DH_ERR_INVALID.  Calls no hipMalloc / hipFree.  Every call on a GPU uses that GPU's one
+ * table: calls that overlap on one GPU (two streams) race; calls in stream order do not. */
+int64_t dh_moe_sort_static_max_assign(void);
+int dh_moe_sort_static(const int32_t *topk_idx, int32_t *tokens_per_expert,
+                       int32_t *expert_offsets, int32_t *sorted_idx,
+                       int32_t *dest_row, int64_t n_assign, int experts,
+                       void *stream);
+
 /* The rows of local experts [e_lo, e_hi) are the sorted positions
  * [first, first + n_rows) with first = expert_offsets[e_lo] and n_rows =
  * expert_offsets[e_hi] - first, both read ON DEVICE (no host sync); launches

@@ -23,6 +23,11 @@ Re-designed for one MI355X:
   row slice.  With tensor_model_parallel_size == 1 they are the identity.
 * RoPE ops (``rope``, ``rope_bwd``) are added to the graph; plans that do not name them
   get them inserted next to ``fl_attn`` / ``attn_bwd``.
+* Context parallelism (``context_parallel_size`` = cp > 1): the graph holds the ring steps
+  ``cp_attn_block_fwd_1 .. _cp`` and ``cp_attn_block_bwd_1 .. _cp+1`` in place of ``fl_attn`` /
+  ``attn_bwd`` (the reference builds them for cp = 2 only, dstb.py:711-722,801-817); the KV
+  chunks that would arrive over the ring are the micro-batch's pre-generated
+  ``cp_kv_chunks``, nothing is exchanged, and ``seq_length`` is the rank's local length.
 * GQA: the fused QKV weight is packed per kv-group as [q heads of the group | k | v]
   (for MHA this is the reference's per-head q|k|v interleave, dstb.py:111-122); with one
   group per rank q, k, v are strided views of the projection output (no copies), and
@@ -45,6 +50,7 @@ from .._Clib import pymha_varlen_bwd, pymha_varlen_fwd, _attn_bwd_raw
 from ..operators.bda import bda_bwd, bda_fwd
 from ..operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
 from ..operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
+from ..operators.ring_attn import RingGroup, fa_cp_block_bwd, fa_cp_block_fwd
 from ..operators.rope import rope_bwd, rope_fwd
 from ..operators.swiglu import swiglu, swiglu_back
 
@@ -100,7 +106,8 @@ class LayerConfig:
     micro_batch_size: int = 1
     tensor_model_parallel_size: int = 1
     tp_rank: int = 0
-    context_parallel_size: int = 1
+    context_parallel_size: int = 1    # > 1: seq_length is this rank's LOCAL length (zig-zag chunks cp_rank, 2cp-1-cp_rank)
+    cp_rank: int = 0
     layernorm_epsilon: float = 1e-5
     rope_theta: Optional[float] = 10000.0
     params_dtype: torch.dtype = torch.bfloat16
@@ -227,6 +234,62 @@ class DCFunc:
                 config.softmax_scale, True, False, 0, False)
             output = out.view(config.tokens, -1)
         return output, q_p, k_p, v_p, out_p, rng_state, lse
+
+    @staticmethod
+    def ring_attn_fwd(config, data, stream):
+        """One ring step (dstb.py:146-197).  ``input`` is the projection output [T, qkv] on the first step,
+        afterwards the carry list of fa_cp_block_fwd.  ``visiting``: the KV chunks [2, b, 2, s/2, hk, d] that
+        arrive at steps 1 .. cp-1 (already rotated by the ranks they come from).  Returns the carry list, or on
+        the last step (out [T, hq d], q, kv buffers, softmax_lse, rng_states)."""
+        input, cu_seqlens_q, cu_seqlens_kv, positions, visiting = data
+        cp, s, b = config.context_parallel_size, config.seq_length, config.micro_batch_size
+        hq, hk, d = config.heads_per_rank, config.groups_per_rank, config.head_dim
+        with torch.cuda.stream(stream):
+            if isinstance(input, torch.Tensor):
+                if visiting is None or len(visiting) != cp - 1:
+                    raise RuntimeError(f"ring attention needs the micro-batch's {cp - 1} visiting KV chunks")
+                q, k, v = _split_qkv(config, input)
+                if config.rope_theta is not None:
+                    rope_fwd(q, k, positions, config.rope_theta, s, stream, False, inplace=True)
+                own = torch.stack((k.reshape(b, 2, s // 2, hk, d), v.reshape(b, 2, s // 2, hk, d)))
+                input = [q.view(b, 2, s // 2, hq, d), [own, *visiting], None, None, None, None, None, 0]
+            i = input[7]
+            r = fa_cp_block_fwd(input[0], cu_seqlens_q, cu_seqlens_kv, s, s, input[1], input[2], input[3], input[4],
+                                input[5], input[6], i, True, RingGroup(config.cp_rank, cp), list(range(cp)), stream,
+                                softmax_scale=config.softmax_scale)
+            if i == cp - 1:
+                out, q, _, softmax_lse, rng_states = r
+                return out.view(config.tokens, -1), q, input[1], softmax_lse, rng_states
+        return r[0]
+
+    @staticmethod
+    def ring_attn_bwd(config, data, stream):
+        """One backward ring call (dstb.py:199-263), cp + 1 of them.  ``input`` is the gradient of the attention
+        output on the first call, afterwards the state list of fa_cp_block_bwd.  The last call returns the packed
+        gradient [T, qkv] of the projection output: dq, and dk / dv of this rank's OWN chunk (what the other
+        ranks would add to it travels with the ring and is absent here)."""
+        input, out, q, kv, softmax_lse, rng_states, cu_seqlens_q, cu_seqlens_kv, positions = data
+        cp, s, b = config.context_parallel_size, config.seq_length, config.micro_batch_size
+        hq, hk, d = config.heads_per_rank, config.groups_per_rank, config.head_dim
+        T = config.tokens
+        with torch.cuda.stream(stream):
+            if isinstance(input, torch.Tensor):
+                input = [input, None, None, kv, 0]
+            i = input[4]
+            r = fa_cp_block_bwd(input[0], out, q, input[1], None, input[2], softmax_lse, rng_states, cu_seqlens_q,
+                                cu_seqlens_kv, s, s, input[3], i, True, RingGroup(config.cp_rank, cp),
+                                list(range(cp)), stream, softmax_scale=config.softmax_scale)
+            if i < cp:
+                return r[0]
+            dq, dkv = r
+            dq = dq.reshape(T, hq, d)
+            dk, dv = dkv[0][0].reshape(T, hk, d), dkv[0][1].reshape(T, hk, d)
+            if config.rope_theta is not None:
+                rope_bwd(dq, dk, positions, config.rope_theta, s, stream, False, inplace=True)
+            dqkv = torch.empty((T, config.qkv_per_rank), dtype=dq.dtype, device=dq.device)
+            rr = hq // hk
+            torch.cat((dq.view(T, hk, rr * d), dk, dv), dim=2, out=dqkv.view(T, hk, (rr + 2) * d))
+        return dqkv
 
     @staticmethod
     def bda_mlp(config, data, stream):
@@ -489,6 +552,28 @@ class DCoperation:
                                      apply_rope=config.groups_per_rank != 1)
         elif op == 32:
             output = dcfunc.rope_bwd(config, (x,), stream)
+        elif op == 29:
+            last = (0 if isinstance(x, torch.Tensor) else x[7]) == config.context_parallel_size - 1
+            visiting = act.get("cp_kv_chunks")
+            if visiting is not None:
+                for t in visiting:
+                    _use(t, stream)
+            output = dcfunc.ring_attn_fwd(config, (x, weight["cu_seqlens_q"], weight["cu_seqlens_kv"],
+                                                   weight.get("rope_positions"), visiting), stream)
+            if last:
+                output, act["q"], act["kv"], act["softmax_lse"], act["rng_states"] = output
+                act["out"] = output
+        elif op == 30:
+            last = (0 if isinstance(x, torch.Tensor) else x[4]) == config.context_parallel_size
+            for t in act["kv"]:
+                _use(t, stream)
+            output = dcfunc.ring_attn_bwd(config, (x, g("out"), g("q"), act["kv"], g("softmax_lse"), act.get("rng_states"),
+                                                   weight["cu_seqlens_q"], weight["cu_seqlens_kv"],
+                                                   weight.get("rope_positions")), stream)
+            if last:
+                for key in ("out", "q", "kv", "softmax_lse", "rng_states"):
+                    act.pop(key, None)
+                act["attn_dgrad"] = output
         elif op in (25, 26):
             p = "mlp" if op == 25 else "attn"
             lw, lb = weight[f"ln_{p}_weight"], weight.get(f"ln_{p}_bias")
@@ -499,6 +584,8 @@ class DCoperation:
         else:
             raise ValueError(f"operation {op} is not part of the single-GPU decoder-layer path")
 
+        if op == 18:
+            act.pop("attn_dgrad", None)          # kept by the last ring call for the qkv weight gradient
         for key in _FREE_AFTER.get(op, ()):
             act.pop(key, None)
         return output
@@ -622,6 +709,72 @@ def _names(entry):
     return [e for e in entry if e != "None"] or None
 
 
+def ring_op_names(cp: int):
+    """Plan names of the ring steps: cp forward steps, cp + 1 backward calls (the reference writes them out for
+    cp = 2: cp_attn_block_fwd_1/2, cp_attn_block_bwd_1/2/3, dstb.py:711-722,801-817)."""
+    return ([f"cp_attn_block_fwd_{i}" for i in range(1, cp + 1)],
+            [f"cp_attn_block_bwd_{i}" for i in range(1, cp + 2)])
+
+
+def _graph(cp: int):
+    """The op graph as (name, op id, strand, is_comm, predecessor) rows; with cp > 1 the ring steps stand where
+    rope + fl_attn and attn_bwd + rope_bwd stand otherwise (RoPE then runs inside the first / last ring call)."""
+    if cp <= 1:
+        return _GRAPH
+    fwd, bwd = ring_op_names(cp)
+    rows = []
+    for row in _GRAPH:
+        name, num, strand, is_comm, pre = row
+        if name in ("rope", "rope_bwd"):
+            continue
+        if name == "fl_attn":
+            prev = "gemm_attn_c"
+            for n in fwd:
+                rows.append((n, 29, 1, 0, prev))
+                prev = n
+            continue
+        if name == "attn_bwd":
+            prev = "gemm_dgrad_attn_l"
+            for n in bwd:
+                rows.append((n, 30, 2, 0, prev))
+                prev = n
+            continue
+        if pre == "fl_attn":
+            pre = fwd[-1]
+        elif pre == "rope_bwd":
+            pre = bwd[-1]
+        rows.append((name, num, strand, is_comm, pre))
+    return rows
+
+
+def _ring_names_for(blocks_json, cp):
+    """A plan written without context parallelism, used with cp > 1: fl_attn / attn_bwd become the ring steps
+    (in the same column), the RoPE ops disappear."""
+    fwd, bwd = ring_op_names(cp)
+    named = {n for blk in blocks_json for col in blk for n in (_names(col) or [])}
+    has_ring = any(n.startswith("cp_attn_block_") for n in named)
+    out = []
+    for blk in blocks_json:
+        cols = []
+        for col in blk:
+            names = _names(col)
+            if names is not None:
+                new = []
+                for n in names:
+                    if n in ("rope", "rope_bwd"):
+                        continue
+                    if n == "fl_attn" and not has_ring:
+                        new.extend(fwd)
+                    elif n == "attn_bwd" and not has_ring:
+                        new.extend(bwd)
+                    else:
+                        new.append(n)
+                names = new or None
+            cols.append(names)
+        out.append(cols)
+    return out
+
+
 def _insert_rope(blocks_json):
     """Plans written for the reference never name the RoPE ops: put ``rope`` right before
     ``fl_attn`` and ``rope_bwd`` right after ``attn_bwd``, in the same column."""
@@ -645,13 +798,16 @@ def _insert_rope(blocks_json):
     return out
 
 
-def init_DCBlocks(config=None, stream1=None, stream2=None) -> Plan:
+def init_DCBlocks(config=None, stream1=None, stream2=None, context_parallel_size: int = 1) -> Plan:
     """Build the op graph and map a plan onto it.  ``config``: path of a plan JSON, a dict in
     the same schema, or None for the built-in plans.  Schema (search/search.py:180-244):
     {"DCBlocks": [[stream1, stream2, stream3], ...], "fwd_only": [...], "bwd_only": [...]},
-    each column a list of op names, one name, or "None"; missing sections use the built-ins."""
+    each column a list of op names, one name, or "None"; missing sections use the built-ins.
+    ``context_parallel_size`` > 1 builds the graph with the ring steps (the reference reads it
+    from Megatron's global arguments, dstb.py:709)."""
     ops = {}
-    for name, num, strand, is_comm, pre in _GRAPH:
+    cp = int(context_parallel_size)
+    for name, num, strand, is_comm, pre in _graph(cp):
         node = DCOP(ops.get(pre), stream1 if strand == 1 else stream2, num, name == "ln_attn", is_comm, name)
         node.strand = strand
         if pre is not None:
@@ -668,7 +824,8 @@ def init_DCBlocks(config=None, stream1=None, stream2=None) -> Plan:
 
     def build(section):
         blocks = []
-        for blk in _insert_rope(data.get(section) or DEFAULT_PLAN[section]):
+        raw = data.get(section) or DEFAULT_PLAN[section]
+        for blk in (_insert_rope(raw) if cp <= 1 else _ring_names_for(raw, cp)):
             if len(blk) != 3:
                 raise ValueError(f"a plan block has 3 columns [stream1, stream2, stream3], got {blk!r}")
             cols = []

@@ -64,25 +64,35 @@ def make_weights(cfg: LayerConfig, seed: int = 0, device="cuda", gen_device="cpu
     cu = torch.arange(0, (cfg.micro_batch_size + 1) * s, s, dtype=torch.int32, device=device)
     w["cu_seqlens_q"] = cu
     w["cu_seqlens_kv"] = cu
+    if cfg.context_parallel_size > 1:
+        # global positions of the rank's local tokens: zig-zag chunks cp_rank and 2 cp - 1 - cp_rank of every sequence
+        c, cp, r = s // 2, cfg.context_parallel_size, cfg.cp_rank
+        a = torch.arange(c, dtype=torch.int32)
+        w["rope_positions"] = torch.cat((r * c + a, (2 * cp - 1 - r) * c + a)).repeat(cfg.micro_batch_size).to(device)
     return w
 
 
 def make_microbatch(cfg: LayerConfig, seed: int, device="cuda", gen_device="cpu") -> Dict[str, torch.Tensor]:
     """Activations and upstream gradient N(0,1), drawn in the order x, dy, then (sequence
     parallel only) the four peer tensors that stand for the other ranks' rows: P_attn,
-    G_attn, P_mlp, G_mlp, each [tokens, hidden]."""
+    G_attn, P_mlp, G_mlp, each [tokens, hidden], then (context parallel only) the visiting
+    KV chunks of the ring."""
     g = torch.Generator(device=gen_device).manual_seed(1000 + seed)
     b, rows, h, dt = cfg.micro_batch_size, cfg.seq_length // cfg.tensor_model_parallel_size, cfg.hidden_size, cfg.params_dtype
     mb = {"x": _randn((b, rows, h), g, device, dt), "dy": _randn((b, rows, h), g, device, dt)}
     if cfg.tensor_model_parallel_size > 1:
         for key in ("sp_peer_attn", "sp_peer_attn_bwd", "sp_peer_mlp", "sp_peer_mlp_bwd"):
             mb[key] = _randn((cfg.tokens, h), g, device, dt)
+    if cfg.context_parallel_size > 1:
+        # the KV chunks that visit at ring steps 1 .. cp-1, [2, b, 2, s/2, hk, d] each (as their owners rotated them)
+        shape = (2, b, 2, cfg.seq_length // 2, cfg.groups_per_rank, cfg.head_dim)
+        mb["cp_kv_chunks"] = [_randn(shape, g, device, dt) for _ in range(cfg.context_parallel_size - 1)]
     return mb
 
 
 def fresh_activation_dict(mb: Dict[str, torch.Tensor]) -> dict:
-    """Activation dict of a micro-batch about to start its forward: only the peer buffers."""
-    return {k: v for k, v in mb.items() if k.startswith("sp_peer")}
+    """Activation dict of a micro-batch about to start its forward: only the peer buffers and the visiting KV."""
+    return {k: v for k, v in mb.items() if k.startswith("sp_peer") or k == "cp_kv_chunks"}
 
 
 class LayerRunner:
@@ -94,7 +104,7 @@ class LayerRunner:
         self.weights = weights
         self.stream1 = stream1 or torch.cuda.Stream()
         self.stream2 = stream2 or torch.cuda.Stream()
-        self.plan: Plan = init_DCBlocks(plan, self.stream1, self.stream2)
+        self.plan: Plan = init_DCBlocks(plan, self.stream1, self.stream2, cfg.context_parallel_size)
 
     def _exec(self, blocks, x, dy, act_prev, act_new, s1, s2):
         return exec_blocks(self.cfg, DCoperation, self.weights if act_new is not None else None,

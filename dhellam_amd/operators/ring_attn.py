@@ -14,9 +14,12 @@ zig-zag cases, the same argument order and carry lists.  Differences, all forced
   (ring_attn.py:95).
 * softmax scale and dropout are parameters (``softmax_scale`` default 1/sqrt(d); dropout
   is not implemented) instead of the hard-coded 0.125 / 0.1 (ring_attn.py:100).
-* The log-sum-exp merge runs once, fused, in fp32 on the last step, instead of an fp64
-  exp/log update per step plus one pass over ``out`` per step (ring_attn.py:146-195);
-  the carried ``softmax_lse`` / ``softmax_lse_`` stay None until then.
+* The merge of the partial outputs runs once, fused, in fp32 on the last step, instead of one
+  pass over ``out`` per step (ring_attn.py:171-195).  The carried ``softmax_lse`` /
+  ``softmax_lse_`` are kept up to date as in the reference (step i folds step i - 1's
+  log-sum-exp into them, ring_attn.py:146-164), in fp32 instead of fp64, so a caller that
+  looks at the carry between steps sees the running value; the value returned after the
+  last step is the one the fused merge computes from all steps.
 * Backward keeps one dKV buffer per visiting chunk (``dkv_`` is a list) instead of adding
   into a buffer that travels round the ring (ring_attn.py:239-272).
 """
@@ -104,6 +107,18 @@ def fa_cp_block_fwd(q, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p
             cq, ck, mq, mk, cz = cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, False
         res = _Clib.pymha_varlen_fwd(q_in, k_in, v_in, cq, ck, mq, mk, 0.0, scale, cz, False, 0, False)
         out_per_step[i], softmax_lse_per_step[i], rng_states[i] = res[0], res[5], res[7]
+
+        # running log-sum-exp over the steps before this one (ring_attn.py:146-164): step i folds step i - 1
+        if i == 1:
+            softmax_lse = softmax_lse_per_step[0].clone()
+            if causal:
+                softmax_lse_ = softmax_lse.view(*softmax_lse.shape[:-1], 2, -1)
+        elif i > 1:
+            prev = softmax_lse_per_step[i - 1]
+            if causal and i - 1 > rank:            # a half-q step: only the second half of the rows
+                torch.logaddexp(softmax_lse_[..., 1, :], prev, out=softmax_lse_[..., 1, :])
+            else:
+                torch.logaddexp(softmax_lse, prev, out=softmax_lse)
 
         if i == cp_size - 1:
             sq = max_seqlen_q

@@ -4,7 +4,8 @@ Counterpart of search/op_table.py: ``OP_TABLE_IDX`` (:1-37, the ids stored in
 ``op_profile_num.txt``), ``operator_list_prune`` (:42-92) and
 ``get_candidate_operator_groups`` (:405-420).  On one GPU there is no communication to
 hide, so the communication ops are not search variables: the boundary groups are the
-reference's compute groups, with the two RoPE ops added next to the attention ops, and the
+reference's compute groups, with the two RoPE ops added next to the attention ops (or, with
+context parallelism, the ring steps in their place), and the
 sequence-parallel stand-in ops are attached to the block of their consumer when a plan is
 written (search.plan_to_json).
 """
@@ -22,7 +23,23 @@ OP_TABLE_IDX = {
     'cp_attn_block_bwd_3': 34,
     'rope': 35, 'rope_bwd': 36,                  # not in the reference
 }
+# Ring steps beyond the five names the reference's table holds (it is written for cp = 2): forward step k >= 3
+# gets id 100 + k, backward call k >= 4 gets id 200 + k.
+for _k in range(3, 17):
+    OP_TABLE_IDX[f'cp_attn_block_fwd_{_k}'] = 100 + _k
+for _k in range(4, 18):
+    OP_TABLE_IDX[f'cp_attn_block_bwd_{_k}'] = 200 + _k
+# Deferred weight-gradient placeholders (dhellam/core/dstb.py:45-48,551-598; plan names string_to_OP :886-889).
+# The reference's search never proposes them; here they are search variables (search.search_plan_with_parking),
+# with ids of their own.
+for _k, _n in enumerate(('gemm_wgrad_mlp_c_n', 'gemm_wgrad_mlp_l_n', 'gemm_wgrad_attn_c_n', 'gemm_wgrad_attn_l_n')):
+    OP_TABLE_IDX[_n] = 40 + _k
 ID_TO_NAME = {v: k for k, v in OP_TABLE_IDX.items()}
+# search id of a weight-gradient op -> search id of its placeholder
+PLACEHOLDER_OF = {OP_TABLE_IDX['gemm_wgrad_mlp_c_reduce_scatter_mlp_c_bwd']: OP_TABLE_IDX['gemm_wgrad_mlp_c_n'],
+                  OP_TABLE_IDX['gemm_wgrad_mlp_l']: OP_TABLE_IDX['gemm_wgrad_mlp_l_n'],
+                  OP_TABLE_IDX['gemm_wgrad_attn_c_reduce_scatter_attn_c_bwd']: OP_TABLE_IDX['gemm_wgrad_attn_c_n'],
+                  OP_TABLE_IDX['gemm_wgrad_attn_l']: OP_TABLE_IDX['gemm_wgrad_attn_l_n']}
 
 # Plan-file name of a search op: the reference fuses the column wgrads with the reduce-scatter
 # that follows them into one search op and splits the name again when it writes the plan
@@ -40,11 +57,22 @@ COMM_CONSUMER = {'allgather_attn': 'gemm_attn_c', 'reduce_scatter_attn': 'bda_at
 def operator_list_prune(context_parallel_size: int = 1):
     """Boundary groups (lists of op ids).  Returns ((min groups, max groups, fwd list),
     (min groups, max groups, bwd list)) like the reference."""
-    if context_parallel_size != 1:
-        raise ValueError("the single-GPU search covers context_parallel_size == 1")
+    cp = int(context_parallel_size)
+    if not 1 <= cp <= 16:
+        raise ValueError(f"context_parallel_size={cp} outside [1, 16]")
     n = OP_TABLE_IDX
+    if cp == 1:
+        attn_fwd = [[n['gemm_attn_c'], n['rope'], n['fl_attn'], n['gemm_attn_l']]]
+        attn_bwd = [[n['gemm_dgrad_attn_l'], n['gemm_wgrad_attn_l'], n['attn_bwd'], n['rope_bwd'], n['gemm_dgrad_attn_c']]]
+    else:
+        # every ring step but the last posts an exchange in the reference, which makes it a group of its own
+        # (op_table.py:68-89 for cp = 2); the last step joins the GEMM that follows it
+        f = [n[f'cp_attn_block_fwd_{i}'] for i in range(1, cp + 1)]
+        b = [n[f'cp_attn_block_bwd_{i}'] for i in range(1, cp + 2)]
+        attn_fwd = [[n['gemm_attn_c']]] + [[i] for i in f[:-1]] + [[f[-1], n['gemm_attn_l']]]
+        attn_bwd = [[n['gemm_dgrad_attn_l'], n['gemm_wgrad_attn_l']]] + [[i] for i in b[:-1]] + [[b[-1], n['gemm_dgrad_attn_c']]]
     fwd = [[n['ln_attn']],
-           [n['gemm_attn_c'], n['rope'], n['fl_attn'], n['gemm_attn_l']],
+           *attn_fwd,
            [n['bda_attn'], n['ln_mlp']],
            [n['gemm_mlp_c'], n['swiglu_mlp'], n['gemm_mlp_l']],
            [n['bda_mlp']]]
@@ -52,7 +80,7 @@ def operator_list_prune(context_parallel_size: int = 1):
            [n['gemm_dgrad_mlp_l'], n['gemm_wgrad_mlp_l'], n['swiglu_bwd'], n['gemm_dgrad_mlp_c']],
            [n['gemm_wgrad_mlp_c_reduce_scatter_mlp_c_bwd']],
            [n['ln_mlp_bwd'], n['bda_attn_bwd']],
-           [n['gemm_dgrad_attn_l'], n['gemm_wgrad_attn_l'], n['attn_bwd'], n['rope_bwd'], n['gemm_dgrad_attn_c']],
+           *attn_bwd,
            [n['gemm_wgrad_attn_c_reduce_scatter_attn_c_bwd']],
            [n['ln_attn_bwd']]]
     cnt = lambda l: sum(len(g) for g in l)

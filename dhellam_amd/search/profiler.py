@@ -80,7 +80,7 @@ def profile_pairs(runner: LayerRunner, mb: dict, out_path: Optional[str] = None,
     """Time every candidate pair; returns {(fwd ids, bwd ids): para_time ms} and, when
     ``out_path`` is given, appends the records to it in the op_profile_num.txt format."""
     records = record_layer(runner, mb)
-    fwd_c, bwd_c = get_candidate_operator_groups(1)
+    fwd_c, bwd_c = get_candidate_operator_groups(runner.cfg.context_parallel_size)
     s1, s2 = runner.stream1, runner.stream2
     prof = {}
     fp = open(out_path, "a") if out_path else None

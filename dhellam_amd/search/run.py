@@ -19,7 +19,7 @@ import torch
 from ..core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
 from .op_table import operator_list_prune
 from .profiler import profile_pairs
-from .search import dump_plan, parse_op_file, search_plan
+from .search import dump_plan, parse_op_file, search_plan_with_parking
 
 
 def validate(cfg, weights, mbs, plan_path, steps=10, warmup=3):
@@ -58,11 +58,13 @@ def main():
                   progress=lambda i, n: print(f"profiled forward group {i}/{n}", flush=True))
     print(f"profiling took {time.perf_counter() - t0:.1f} s", flush=True)
     prof = parse_op_file(prof_path)
-    (_, _, fwd), (_, _, bwd) = operator_list_prune(1)
-    cost, blocks = search_plan(prof, fwd, bwd)
+    (_, _, fwd), (_, _, bwd) = operator_list_prune(cfg.context_parallel_size)
+    cost, blocks, alias = search_plan_with_parking(prof, fwd, bwd)
     serial_cost = sum(prof[(tuple(g), ())] for g in fwd) + sum(prof[((), tuple(g))] for g in bwd)
     plan_path = os.path.join(args.out_dir, "best_result.json")
-    dump_plan(blocks, plan_path)
+    dump_plan(blocks, plan_path, alias=alias, bwd_order=[x for g in bwd for x in g])
+    if alias:
+        print("deferred weight gradients:", sorted(alias.values()), flush=True)
     print(f"predicted: paired {cost:.3f} ms vs unpaired groups {serial_cost:.3f} ms per micro-batch", flush=True)
     print(json.dumps(json.load(open(plan_path))["DCBlocks"]), flush=True)
     ser, dbl = validate(cfg, w, mbs, plan_path)

@@ -6,6 +6,10 @@ exactly m and n groups and runs a 2-D DP for each pair of refinements; the same 
 reached here by ONE DP over (forward ops consumed, backward ops consumed) whose moves are
 "take the next contiguous forward group", "take the next backward group" or "pair the two",
 a group never crossing a boundary.  Profile strings are parsed with ``ast.literal_eval``.
+Beyond the reference: ``search_plan_with_parking`` also decides which weight gradients to defer
+to a later block under their ``*_n`` placeholders (the runtime and the plan format support
+that, dhellam/core/dstb.py:543-598,931-939; the reference's search never proposes it), and the
+writer emits the ``fwd_only`` / ``bwd_only`` sections the loader reads.
 """
 from __future__ import annotations
 
@@ -14,7 +18,7 @@ import json
 import re
 from typing import Dict, List, Sequence, Tuple
 
-from .op_table import COMM_CONSUMER, ID_TO_NAME, PLAN_NAME
+from .op_table import COMM_CONSUMER, ID_TO_NAME, PLACEHOLDER_OF, PLAN_NAME
 
 Key = Tuple[Tuple[int, ...], Tuple[int, ...]]
 _LINE = re.compile(r'\[\s*(\[[\d,\s]*\])\s*,\s*(\[[\d,\s]*\])\s*\]\s*speedup:\s*([0-9.eE+-]+)\s*'
@@ -52,11 +56,12 @@ def _starts(groups: List[List[int]]):
 
 
 def search_plan(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_groups: List[List[int]],
-                illegal=None) -> Tuple[float, List[Tuple[List[int], List[int]]]]:
+                illegal=None, alias=None) -> Tuple[float, List[Tuple[List[int], List[int]]]]:
     """Best sequence of blocks [(fwd group, bwd group)], either possibly empty, that covers
     both op lists in order and minimises the sum of the blocks' measured times.  ``illegal(f, b)``
     forbids pairing two groups (the reference forbids pairs where both sides communicate,
-    search.py:13-21).  Raises KeyError if the profile lacks a needed record."""
+    search.py:13-21).  ``alias``: {op id: op id whose records time it} (a parked weight gradient
+    runs the kernel of the op it was parked from).  Raises KeyError if the profile lacks a needed record."""
     F, fs = _starts(fwd_groups)
     B, bs = _starts(bwd_groups)
     nf, nb = len(F), len(B)
@@ -64,7 +69,8 @@ def search_plan(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_grou
     cost = [[INF] * (nb + 1) for _ in range(nf + 1)]
     back = [[None] * (nb + 1) for _ in range(nf + 1)]
     cost[0][0] = 0.0
-    t = lambda f, b: profile[(tuple(f), tuple(b))]
+    al = alias or {}
+    t = lambda f, b: profile[(tuple(al.get(x, x) for x in f), tuple(al.get(x, x) for x in b))]
     for i in range(nf + 1):
         for j in range(nb + 1):
             if i == 0 and j == 0:
@@ -99,25 +105,110 @@ def search_plan(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_grou
     return cost[nf][nb], blocks
 
 
-def plan_to_json(blocks, with_comm_standins: bool = True) -> dict:
-    """{"DCBlocks": [[stream1, stream2, stream3], ...]} in the reference's schema
-    (search.py:180-244): op-name lists, or the string "None" for an empty column.  The
+def park_choices(bwd_groups: List[List[int]], movable: Sequence[int]):
+    """Every way of deferring weight gradients: each movable op either stays, or leaves its place and runs as a
+    group of its own right after a LATER boundary group (where its ``*_n`` placeholder then sits,
+    dhellam/core/dstb.py:543-598).  Yields (modified backward groups, {placeholder id: op id}); the group an op
+    leaves is cut in two at its place."""
+    where = {op: gi for gi, g in enumerate(bwd_groups) for op in g}
+    movable = [m for m in movable if m in where]
+    options = [[None] + list(range(where[m] + 1, len(bwd_groups))) for m in movable]
+
+    def rec(k, chosen):
+        if k == len(movable):
+            yield dict(chosen)
+            return
+        for o in options[k]:
+            chosen.append((movable[k], o))
+            yield from rec(k + 1, chosen)
+            chosen.pop()
+
+    for choice in rec(0, []):
+        groups, alias = [], {}
+        after = {}
+        for m, o in choice.items():
+            if o is not None:
+                after.setdefault(o, []).append(m)
+        for gi, g in enumerate(bwd_groups):
+            cur = []
+            for op in g:
+                if choice.get(op) is not None:
+                    if cur:
+                        groups.append(cur)
+                    cur = []
+                else:
+                    cur.append(op)
+            if cur:
+                groups.append(cur)
+            for m in after.get(gi, []):
+                groups.append([PLACEHOLDER_OF[m]])
+                alias[PLACEHOLDER_OF[m]] = m
+        yield groups, alias
+
+
+def search_plan_with_parking(profile: Dict[Key, float], fwd_groups, bwd_groups, movable=None, illegal=None):
+    """``search_plan`` over every choice of deferred weight gradients.  Returns (cost, blocks, alias): in the
+    blocks a deferred op appears as its placeholder id at the place where it runs; ``alias`` maps the
+    placeholders used to the ops they defer (``plan_to_json`` puts the op's own name back where it was parked)."""
+    movable = list(PLACEHOLDER_OF) if movable is None else list(movable)
+    best = (float("inf"), None, None)
+    for groups, alias in park_choices(bwd_groups, movable):
+        try:
+            cost, blocks = search_plan(profile, fwd_groups, groups, illegal, alias)
+        except KeyError:
+            continue                      # the profile has no record for a group this choice needs
+        if cost < best[0]:
+            best = (cost, blocks, alias)
+    if best[1] is None:
+        raise KeyError("the profile lacks the records of every candidate plan")
+    return best
+
+
+def plan_to_json(blocks, with_comm_standins: bool = True, alias=None, bwd_order: Sequence[int] = ()) -> dict:
+    """{"DCBlocks": [...], "fwd_only": [...], "bwd_only": [...]}, each a list of
+    [stream1, stream2, stream3] in the reference's schema (writer search.py:180-244, reader
+    dhellam/core/dstb.py:901-1041): op-name lists, or the string "None" for an empty column.  The
     sequence-parallel stand-in ops go into the third column of the block that holds their
-    consumer."""
+    consumer.  ``fwd_only`` / ``bwd_only`` (the schedules of the first forward and the last
+    backward) hold the same groups in the same order, one strand each.
+    ``alias`` ({placeholder id: deferred op id}, from ``search_plan_with_parking``) with ``bwd_order`` (the
+    backward ops in their original order): a deferred op is named again right after the op it followed, where
+    the runtime parks it, and its placeholder stays where the search put it."""
     comm_of = {}
     for comm, consumer in COMM_CONSUMER.items():
         comm_of.setdefault(consumer, []).append(comm)
-    out = []
-    for fg, bg in blocks:
-        names = lambda ids: [PLAN_NAME.get(ID_TO_NAME[i], ID_TO_NAME[i]) for i in ids]
-        first, second = names(fg), names(bg)
-        third = [c for op in first + second for c in comm_of.get(op, [])] if with_comm_standins else []
-        out.append([first or "None", second or "None", third or "None"])
-    return {"DCBlocks": out}
+    nm = lambda i: PLAN_NAME.get(ID_TO_NAME[i], ID_TO_NAME[i])
+    blocks = [(list(f), list(b)) for f, b in blocks]
+    for ph, op in (alias or {}).items():
+        order = list(bwd_order)
+        k = order.index(op)
+        placed = False
+        for prev in reversed(order[:k]):                  # nearest earlier op that is still at its place
+            for _, bg in blocks:
+                if prev in bg:
+                    bg.insert(bg.index(prev) + 1, op)
+                    placed = True
+                    break
+            if placed:
+                break
+        if not placed:                                    # nothing before it: park it in the first backward block
+            next(bg for _, bg in blocks if bg).insert(0, op)
+
+    def section(blks):
+        out = []
+        for fg, bg in blks:
+            first, second = [nm(i) for i in fg], [nm(i) for i in bg]
+            third = [c for op in first + second for c in comm_of.get(op, [])] if with_comm_standins else []
+            out.append([first or "None", second or "None", third or "None"])
+        return out
+
+    return {"DCBlocks": section(blocks),
+            "fwd_only": section([(f, []) for f, _ in blocks if f]),
+            "bwd_only": section([([], b) for _, b in blocks if b])}
 
 
-def dump_plan(blocks, path: str) -> dict:
-    data = plan_to_json(blocks)
+def dump_plan(blocks, path: str, alias=None, bwd_order: Sequence[int] = ()) -> dict:
+    data = plan_to_json(blocks, alias=alias, bwd_order=bwd_order)
     with open(path, "w") as f:
         json.dump(data, f, indent=4)
     return data

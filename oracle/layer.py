@@ -19,6 +19,7 @@ import math
 
 import torch
 
+from . import attention as OA
 from . import ops as O
 
 
@@ -78,16 +79,33 @@ def layer_forward(cfg: dict, P: dict, x, mb: dict, dtype=torch.float64, rnd=lamb
     q = g[:, :, : r * d].reshape(T, hq, d)
     k = g[:, :, r * d:(r + 1) * d]
     v = g[:, :, (r + 1) * d:]
-    pos = torch.arange(T) % s
+    cp, cr = cfg.get("cp", 1), cfg.get("cp_rank", 0)
+    pos = torch.arange(T) % s if cp == 1 else OA.zigzag_positions(cr, cp, s // 2).repeat(b)
     if cfg.get("theta") is not None:
         q = rnd(O.rope(q, pos, cfg["theta"], dtype=dtype))
         k = rnd(O.rope(k, pos, cfg["theta"], dtype=dtype))
+    if cp > 1:
+        # Context parallel: this rank's tokens are the zig-zag chunks cr and 2 cp - 1 - cr of a sequence of
+        # cp * s tokens; its q rows attend to its own K/V and to the cp - 1 visiting chunks (as their owners
+        # rotated them) under the causal mask of the GLOBAL positions -- what the ring steps and their merge
+        # amount to (dhellam/operators/ring_attn.py:90-201).  The visiting chunks get no gradient here.
+        c = s // 2
+        chunks = [(k.reshape(b, 2, c, hk, d), v.reshape(b, 2, c, hk, d))]
+        chunks += [(kv[0].to(dtype), kv[1].to(dtype)) for kv in mb["cp_kv_chunks"]]
+        o, _ = OA.zigzag_dense(q.reshape(b, 2, c, hq, d), chunks, cr, 1.0 / math.sqrt(d), dtype=dtype)
+        o = rnd(o.reshape(T, hq * d))
+        return _after_attention(cfg, P, x, o, rnd, scatter, gather, F)
     qh = q.view(b, s, hq, d).permute(0, 2, 1, 3)
     kh = k.reshape(b, s, hk, d).repeat_interleave(r, dim=2).permute(0, 2, 1, 3)
     vh = v.reshape(b, s, hk, d).repeat_interleave(r, dim=2).permute(0, 2, 1, 3)
     sc = torch.matmul(qh, kh.transpose(2, 3)) / math.sqrt(d)
     sc = sc.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
     o = rnd(torch.matmul(torch.softmax(sc, -1), vh).permute(0, 2, 1, 3).reshape(T, hq * d))
+    return _after_attention(cfg, P, x, o, rnd, scatter, gather, F)
+
+
+def _after_attention(cfg, P, x, o, rnd, scatter, gather, F):
+    """Output projection, residual, second norm and the SwiGLU FFN (steps 6-11 of the layer)."""
     a = rnd(o @ P["linear_attn_weight"].T)
     x2 = rnd(x + scatter(a, "sp_peer_attn_bwd"))
     h2 = rnd(_rms(x2, P["ln_mlp_weight"], cfg["eps"]))
@@ -100,7 +118,8 @@ def layer_forward(cfg: dict, P: dict, x, mb: dict, dtype=torch.float64, rnd=lamb
 
 def layer_fwd_bwd(cfg: dict, w: dict, mb: dict, dtype=torch.float64, round_to=None):
     """cfg: hidden, heads (q heads on this rank), groups (kv heads on this rank), head_dim,
-    ffn (per rank), seq, batch, tp, tp_rank, eps, theta.  w: column_attn_weight,
+    ffn (per rank), seq, batch, tp, tp_rank, eps, theta (+ cp, cp_rank: context parallelism, seq then being the
+    rank's local length and mb holding cp_kv_chunks, the cp - 1 visiting KV chunks [2, b, 2, seq/2, groups, head_dim]).  w: column_attn_weight,
     linear_attn_weight, column_mlp_weight, linear_mlp_weight, ln_attn_weight,
     ln_mlp_weight.  mb: x, dy [b, seq/tp, hidden] (+ sp_peer_* [b*seq, hidden] when tp > 1).
     ``round_to``: dtype every op's output is rounded to, and with it the gradient that comes back

@@ -203,12 +203,14 @@ def test_ring_step_matches_oracle_and_dense(dtype, b, c, hq, hk, d, rank):
         assert_close(dkv[s][1], dkvo[s][1], dtype, f"ring dv[{s}]")
 
 
-def test_ring_step_full_size():
-    """The ring configuration at its full shape (q [1, 2, 2048, 32, 128], four visiting KV chunks of 8 kv heads,
-    rank 1): forward and backward against ONE dense attention over the zig-zag positions, evaluated by the
+@pytest.mark.parametrize("rank", [0, 1, 3])
+def test_ring_step_full_size(rank):
+    """The ring configuration at its full shape (q [1, 2, 2048, 32, 128], four visiting KV chunks of 8 kv heads;
+    rank 0: a diagonal step and three half-q steps, rank 3: a diagonal step and three half-kv steps, rank 1:
+    both kinds): forward and backward against ONE dense attention over the zig-zag positions, evaluated by the
     oracle in fp32 with its matmuls on the GPU (the [32, 4096, 16384] score tensor is 8.6 GB), gradients by
     autograd.  16-bit tolerance."""
-    dtype, b, c, hq, hk, d, cp, rank = torch.bfloat16, 1, 2048, 32, 8, 128, 4, 1
+    dtype, b, c, hq, hk, d, cp = torch.bfloat16, 1, 2048, 32, 8, 128, 4
     q, chunks, dout = _ring_inputs(dtype, b, c, hq, hk, d, cp, seed=3)
     scale = 1.0 / math.sqrt(d)
     out, lse, dq, dkv = _ring_gpu(q, chunks, dout, rank, cp)

@@ -17,11 +17,13 @@ def _oracle_cfg(cfg):
     return dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
                 ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size,
                 tp=cfg.tensor_model_parallel_size, tp_rank=cfg.tp_rank, eps=cfg.layernorm_epsilon,
-                theta=cfg.rope_theta)
+                theta=cfg.rope_theta, cp=cfg.context_parallel_size, cp_rank=cfg.cp_rank)
 
 
 def _cpu(d):
-    return {k: v.detach().cpu() for k, v in d.items() if isinstance(v, torch.Tensor) and v.is_floating_point()}
+    out = {k: v.detach().cpu() for k, v in d.items() if isinstance(v, torch.Tensor) and v.is_floating_point()}
+    out.update({k: [t.detach().cpu() for t in v] for k, v in d.items() if isinstance(v, list)})
+    return out
 
 
 def _check_layer(cfg, oracle_dtype, round_to=None):
@@ -68,11 +70,54 @@ def test_layer_70b_shard_full_shape():
     _check_layer(llama70b_tp8_shard(), torch.float32, round_to=torch.bfloat16)
 
 
-def test_serial_and_double_strand_are_bit_identical():
+def _ring_layer_cfg(seq, cp_rank, hidden=4096, ffn=2048):
+    """A layer whose attention is the ring configuration: 32 q / 8 kv heads of 128, cp = 4, local sequence ``seq``
+    (the q chunk of the rank; four KV chunks of the same length visit)."""
+    from dhellam_amd.core.dstb import LayerConfig
+    return LayerConfig(hidden_size=hidden, num_attention_heads=hidden // 128, num_query_groups=hidden // 512,
+                       ffn_hidden_size=ffn, seq_length=seq, micro_batch_size=1, tensor_model_parallel_size=1,
+                       context_parallel_size=4, cp_rank=cp_rank, rope_theta=500000.0, params_dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("cp_rank", [0, 1, 3])
+def test_layer_with_ring_attention_through_the_runtime(cp_rank):
+    """The ring step inside the layer, driven by the runtime's cp_attn_block_fwd_1..4 / cp_attn_block_bwd_1..5 ops
+    (op ids 29 / 30), against the oracle layer whose attention is ONE dense causal attention over the zig-zag
+    positions of all four chunks.  Small hidden size so that the fp64 oracle runs in seconds."""
+    _check_layer(_ring_layer_cfg(512, cp_rank, hidden=1024, ffn=1024), torch.float64, round_to=torch.bfloat16)
+
+
+def test_ring_layer_full_shape_serial_and_double_strand_are_bit_identical():
+    """The ring configuration at its full shape (32 q / 8 kv heads x 128, local q 4096, four visiting KV chunks of
+    4096) inside a layer, rank 1: the double-strand schedule (ring steps of micro-batch i+1 beside the backward
+    ring calls of micro-batch i) gives the bits of the serial one."""
+    from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
+    cfg = _ring_layer_cfg(4096, 1)
+    w = make_weights(cfg, 0, gen_device="cuda")
+    mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(3)]
+    runner = LayerRunner(cfg, w)
+    names = [str(o) for blk in runner.plan.dcblocks for o in (blk.stream1_op or []) + (blk.stream2_op or [])]
+    assert "cp_attn_block_fwd_4" in names and "cp_attn_block_bwd_5" in names and "fl_attn" not in names
+    outs_s, dxs_s = runner.run_serial(mbs)
+    torch.cuda.synchronize()
+    g_s = {k: v.clone() for k, v in runner.grads().items()}
+    for _ in range(5):
+        runner.zero_grads()
+        outs_d, dxs_d = runner.run_double_strand(mbs)
+        torch.cuda.synchronize()
+        for a, b in zip(outs_s + dxs_s, outs_d + dxs_d):
+            assert torch.equal(a, b)
+        for k, v in runner.grads().items():
+            assert torch.equal(v, g_s[k]), k
+
+
+@pytest.mark.parametrize("seq", [1024, 4096])
+def test_serial_and_double_strand_are_bit_identical(seq):
     """Same kernels, different stream order: outputs, input grads and accumulated weight grads must be
-    identical bit for bit over 4 micro-batches."""
+    identical bit for bit over 4 micro-batches.  seq 4096 is the double-strand configuration at its own size
+    (four micro-batches of the full 70B shard layer)."""
     from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
-    cfg = llama70b_tp8_shard(seq_length=1024)
+    cfg = llama70b_tp8_shard(seq_length=seq)
     w = make_weights(cfg, 0, gen_device="cuda")
     mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(4)]
     runner = LayerRunner(cfg, w)

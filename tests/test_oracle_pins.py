@@ -399,14 +399,15 @@ def test_model_oracle_without_layers_is_tied_embedding_cross_entropy():
 
 
 # ---- decoder layer ---------------------------------------------------------------------------
-def _angles(s, d, theta):
+def _angles(s, d, theta, pos=None):
     """Rotation angles as the path defines them: position times theta^(-2j/d), both factors and their product in
     fp32 (one rounding each), [s, d/2]."""
     inv = torch.tensor([theta ** (-2.0 * j / d) for j in range(d // 2)], dtype=D).float()
-    return (torch.arange(s, dtype=torch.float32)[:, None] * inv[None, :]).to(D)
+    pos = torch.arange(s, dtype=torch.float32) if pos is None else pos.float()
+    return (pos[:, None] * inv[None, :]).to(D)
 
 
-def _independent_layer(cfg, W, x):
+def _independent_layer(cfg, W, x, pos=None, attention=None):
     """The layer of ``oracle.layer.layer_forward`` at tp = 1, written again from library routines only
     (F.rms_norm, F.linear, F.scaled_dot_product_attention, F.silu) with its own QKV unpacking (a Python loop
     over kv groups) and its own RoPE (complex multiplication of the (j, j + d/2) pairs)."""
@@ -426,12 +427,15 @@ def _independent_layer(cfg, W, x):
     q, k, v = torch.stack(qs, 1), torch.stack(ks, 1), torch.stack(vs, 1)           # [b, heads, s, d]
 
     def rotate(t):
-        ang = _angles(s, d, cfg["theta"])
+        ang = _angles(s, d, cfg["theta"], pos)
         z = torch.complex(t[..., : d // 2], t[..., d // 2:]) * torch.polar(torch.ones_like(ang), ang)
         return torch.cat((z.real, z.imag), -1)
 
     q, k = rotate(q), rotate(k)
-    o = F.scaled_dot_product_attention(q, k.repeat_interleave(r, 1), v.repeat_interleave(r, 1), is_causal=True)
+    if attention is None:
+        o = F.scaled_dot_product_attention(q, k.repeat_interleave(r, 1), v.repeat_interleave(r, 1), is_causal=True)
+    else:
+        o = attention(q, k.repeat_interleave(r, 1), v.repeat_interleave(r, 1))
     o = o.transpose(1, 2).reshape(b * s, hq * d)
     x2 = x + F.linear(o, W["linear_attn_weight"])
     u = F.linear(F.rms_norm(x2, (H,), W["ln_mlp_weight"], cfg["eps"]), W["column_mlp_weight"])
@@ -534,6 +538,51 @@ def test_layer_oracle_sequence_parallel_stand_ins(tp_rank):
     ((ref * mb["dy"].reshape(rows, H)).sum() + carry1 + carry2).backward()
     assert torch.allclose(out.reshape(rows, H), ref.detach(), rtol=1e-12, atol=1e-12)
     assert torch.allclose(grads["x"].reshape(rows, H), xr.grad, rtol=1e-11, atol=1e-12)
+    for k_ in W:
+        assert torch.allclose(grads[k_], Wr[k_].grad, rtol=1e-11, atol=1e-12), k_
+
+
+@pytest.mark.parametrize("cp,cp_rank", [(2, 0), (2, 1), (3, 1)])
+def test_layer_oracle_context_parallel(cp, cp_rank):
+    """cp > 1: the rank holds the zig-zag chunks cp_rank and 2 cp - 1 - cp_rank of a sequence cp times as long.
+    Checked by laying the WHOLE sequence out in its natural order -- own K/V and the visiting chunks at their global
+    places, the rank's q rows at theirs (zeros elsewhere) -- and calling the library's plain causal attention on
+    it; the rank's rows of that result, and autograd through it, must be what the oracle layer gives."""
+    from oracle import layer as OL
+    cfg, W, mb = _layer_case(seed=3)
+    cfg = dict(cfg, cp=cp, cp_rank=cp_rank)
+    b, s, hk, d, r = cfg["batch"], cfg["seq"], cfg["groups"], cfg["head_dim"], cfg["heads"] // cfg["groups"]
+    c = s // 2
+    g = torch.Generator().manual_seed(9)
+    mb["cp_kv_chunks"] = [torch.randn(2, b, 2, c, hk, d, generator=g, dtype=D) for _ in range(cp - 1)]
+    out, grads = OL.layer_fwd_bwd(cfg, W, mb)
+
+    chunk_of = lambda rank: (rank, 2 * cp - 1 - rank)           # global chunk numbers a rank owns
+    mine = chunk_of(cp_rank)
+    pos = torch.cat([torch.arange(c) + m * c for m in mine])
+
+    def attention(q, k, v):                                     # [b, heads, s, d], already rotated, kv heads repeated
+        S = 2 * cp * c
+        Q = torch.zeros(b, q.shape[1], S, d, dtype=D)
+        K, V = torch.zeros_like(Q), torch.zeros_like(Q)
+        idx = pos
+        Q = Q.index_copy(2, idx, q)
+        K = K.index_copy(2, idx, k)
+        V = V.index_copy(2, idx, v)
+        for i, kv in enumerate(mb["cp_kv_chunks"], start=1):     # step i brings the chunk of rank (cp_rank - i) % cp
+            src = chunk_of((cp_rank - i) % cp)
+            for half in (0, 1):
+                sl = slice(src[half] * c, (src[half] + 1) * c)
+                K[:, :, sl] = kv[0][:, half].permute(0, 2, 1, 3).repeat_interleave(r, 1)
+                V[:, :, sl] = kv[1][:, half].permute(0, 2, 1, 3).repeat_interleave(r, 1)
+        return F.scaled_dot_product_attention(Q, K, V, is_causal=True)[:, :, idx]
+
+    Wr = {k_: v_.clone().requires_grad_() for k_, v_ in W.items()}
+    xr = mb["x"].reshape(-1, cfg["hidden"]).clone().requires_grad_()
+    ref = _independent_layer(cfg, Wr, xr, pos=pos, attention=attention)
+    (ref * mb["dy"].reshape(ref.shape)).sum().backward()
+    assert torch.allclose(out.reshape(ref.shape), ref.detach(), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(grads["x"].reshape(xr.shape), xr.grad, rtol=1e-11, atol=1e-12)
     for k_ in W:
         assert torch.allclose(grads[k_], Wr[k_].grad, rtol=1e-11, atol=1e-12), k_
 

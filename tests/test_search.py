@@ -105,7 +105,7 @@ def test_plan_json_is_loadable_and_complete(tmp_path):
     # a plan that pairs group by group where possible
     blocks = [(fwd[i] if i < len(fwd) else [], bwd[i] if i < len(bwd) else []) for i in range(max(len(fwd), len(bwd)))]
     data = search.dump_plan(blocks, str(tmp_path / "best_result.json"))
-    assert set(data) == {"DCBlocks"} and all(len(b) == 3 for b in data["DCBlocks"])
+    assert set(data) == {"DCBlocks", "fwd_only", "bwd_only"} and all(len(b) == 3 for b in data["DCBlocks"])
     assert data["DCBlocks"][0] == [["ln_attn"], ["bda_mlp_bwd"], "None"]
     assert data["DCBlocks"][1][2] == ["allgather_attn", "allgather_mlp_bwd"]
     assert data["DCBlocks"][2][1] == ["gemm_wgrad_mlp_c"]                      # fused search op written under its plan name
@@ -117,3 +117,112 @@ def test_plan_json_is_loadable_and_complete(tmp_path):
     pos = {str(o): i for i, blk in enumerate(plan.dcblocks) for col in (blk.stream1_op, blk.stream2_op, blk.stream3_op) for o in (col or [])}
     for comm, consumer in op_table.COMM_CONSUMER.items():
         assert pos[comm] == pos[consumer] and pos[str(plan.ops[comm].pre)] < pos[comm]
+
+
+def _ops_of(blocks, col):
+    return [str(o) for blk in blocks for o in (getattr(blk, col) or [])]
+
+
+def test_plan_writer_emits_fwd_only_and_bwd_only_sections(tmp_path):
+    """The writer's three sections round-trip through the loader: fwd_only holds every forward op once, in order,
+    with nothing in the backward column; bwd_only the mirror image; stand-in collectives ride with their consumers."""
+    (_, _, fwd), (_, _, bwd) = op_table.operator_list_prune()
+    blocks = [(fwd[i] if i < len(fwd) else [], bwd[i] if i < len(bwd) else []) for i in range(max(len(fwd), len(bwd)))]
+    data = search.dump_plan(blocks, str(tmp_path / "p.json"))
+    assert all(b[1] == "None" for b in data["fwd_only"]) and all(b[0] == "None" for b in data["bwd_only"])
+    assert len(data["fwd_only"]) == len(fwd) and len(data["bwd_only"]) == len(bwd)
+    plan = dstb.init_DCBlocks(str(tmp_path / "p.json"))
+    name = lambda i: op_table.PLAN_NAME.get(op_table.ID_TO_NAME[i], op_table.ID_TO_NAME[i])
+    assert _ops_of(plan.fwd_only, "stream1_op") == [name(i) for g in fwd for i in g]
+    assert _ops_of(plan.bwd_only, "stream2_op") == [name(i) for g in bwd for i in g]
+    assert sorted(_ops_of(plan.fwd_only, "stream3_op")) == sorted(c for c in op_table.COMM_CONSUMER if not c.endswith("_bwd"))
+    assert sorted(_ops_of(plan.bwd_only, "stream3_op")) == sorted(c for c in op_table.COMM_CONSUMER if c.endswith("_bwd"))
+
+
+def _synthetic_profile(fwd_groups, bwd_groups, rng, cheap_pair=None):
+    solo, prof = {}, {}
+    for f in op_table.candidate_groups(fwd_groups):
+        for b in op_table.candidate_groups(bwd_groups):
+            if not f and not b:
+                continue
+            base = sum(solo.setdefault(x, rng.uniform(0.1, 1.0)) for x in f + b)
+            save = rng.uniform(0, 0.9) * min(sum(solo[x] for x in f), sum(solo[x] for x in b)) if f and b else 0.0
+            prof[(tuple(f), tuple(b))] = base - save
+    return prof, solo
+
+
+def test_parking_search_matches_brute_force_over_every_choice():
+    """The deferred-weight-gradient search against the reference-style enumeration run on every park choice."""
+    rng = random.Random(1)
+    W1, W2 = 12, 15
+    fwd_groups, bwd_groups = [[1], [2, 3], [4]], [[11, W1, 13], [14], [W2], [16]]
+    saved = dict(op_table.PLACEHOLDER_OF)
+    op_table.PLACEHOLDER_OF.clear()
+    op_table.PLACEHOLDER_OF.update({W1: 912, W2: 915})
+    search.PLACEHOLDER_OF = op_table.PLACEHOLDER_OF
+    try:
+        for trial in range(4):
+            prof, _ = _synthetic_profile(fwd_groups, bwd_groups, rng)
+            cost, blocks, alias = search.search_plan_with_parking(prof, fwd_groups, bwd_groups)
+            best = float("inf")
+            n_choices = 0
+            for groups, al in search.park_choices(bwd_groups, [W1, W2]):
+                n_choices += 1
+                p2 = dict(prof)
+                for (f, b), v in prof.items():            # the placeholder runs the kernel of the op it defers
+                    for ph, op in al.items():
+                        if b == (op,):
+                            p2[(f, (ph,))] = v
+                best = min(best, _brute(p2, fwd_groups, groups))
+            assert n_choices == 4 * 2                     # W1: stay or after group 1, 2, 3; W2: stay or after group 3
+            assert abs(cost - best) < 1e-9
+            no_parking, _ = search.search_plan(prof, fwd_groups, bwd_groups)
+            assert cost <= no_parking + 1e-12
+            ran = [alias.get(x, x) for _, b in blocks for x in b]
+            assert sorted(ran) == [11, 12, 13, 14, 15, 16]
+    finally:
+        op_table.PLACEHOLDER_OF.clear()
+        op_table.PLACEHOLDER_OF.update(saved)
+
+
+def test_parked_plan_names_the_op_where_it_is_parked_and_its_placeholder_where_it_runs(tmp_path):
+    (_, _, fwd), (_, _, bwd) = op_table.operator_list_prune()
+    n = op_table.OP_TABLE_IDX
+    w = n["gemm_wgrad_mlp_l"]
+    # hand-made result of the search: the mlp_l weight gradient leaves its group and runs after the 4th group
+    groups, alias = next((g, a) for g, a in search.park_choices(bwd, [w]) if a and g.index([n["gemm_wgrad_mlp_l_n"]]) == 5)
+    blocks = [(fwd[i] if i < len(fwd) else [], groups[i] if i < len(groups) else []) for i in range(max(len(fwd), len(groups)))]
+    order = [x for g in bwd for x in g]
+    data = search.dump_plan(blocks, str(tmp_path / "p.json"), alias=alias, bwd_order=order)
+    col2 = [b[1] for b in data["DCBlocks"]]
+    assert col2[1] == ["gemm_dgrad_mlp_l", "gemm_wgrad_mlp_l"]          # parked right after the op it followed
+    assert ["gemm_wgrad_mlp_l_n"] in col2
+    plan = dstb.init_DCBlocks(str(tmp_path / "p.json"))
+    assert plan.movable == {"gemm_wgrad_mlp_l_n"}
+    flat = _ops_of(plan.dcblocks, "stream2_op")
+    assert flat.index("gemm_wgrad_mlp_l") < flat.index("gemm_wgrad_mlp_l_n")
+    assert "gemm_wgrad_mlp_l_n" in _ops_of(plan.bwd_only, "stream2_op")
+
+
+def test_context_parallel_groups_and_graph():
+    """cp = 4: ring steps replace fl_attn / attn_bwd in the boundary groups, the graph and the built-in plans."""
+    (nf, _, fwd), (nb, _, bwd) = op_table.operator_list_prune(4)
+    n = op_table.OP_TABLE_IDX
+    assert n["cp_attn_block_fwd_1"] == 30 and n["cp_attn_block_bwd_3"] == 34                      # search/op_table.py:31-36
+    assert [n["cp_attn_block_fwd_1"]] in fwd and [n["cp_attn_block_fwd_4"], n["gemm_attn_l"]] in fwd
+    assert [n["cp_attn_block_bwd_5"], n["gemm_dgrad_attn_c"]] in bwd and [n["cp_attn_block_bwd_4"]] in bwd
+    assert all(n["fl_attn"] not in g and n["rope"] not in g for g in fwd)
+    (_, _, f2), (_, _, b2) = op_table.operator_list_prune(2)
+    assert [30] in f2 and [31, 17] in f2 and [32] in b2 and [33] in b2 and [34, 6] in b2           # op_table.py:68-89
+    plan = dstb.init_DCBlocks(None, context_parallel_size=4)
+    fl = _ops_of(plan.fwd_only, "stream1_op")
+    assert fl[fl.index("gemm_attn_c") + 1: fl.index("gemm_attn_l")] == [f"cp_attn_block_fwd_{i}" for i in range(1, 5)]
+    bl = _ops_of(plan.bwd_only, "stream2_op")
+    i0 = bl.index("cp_attn_block_bwd_1")
+    assert bl[i0:i0 + 5] == [f"cp_attn_block_bwd_{i}" for i in range(1, 6)] and "attn_bwd" not in bl and "rope_bwd" not in bl
+    assert plan.ops["gemm_attn_l"].pre is plan.ops["cp_attn_block_fwd_4"]
+    assert plan.ops["gemm_wgrad_attn_c"].pre is plan.ops["cp_attn_block_bwd_5"]
+    # a searched plan over these groups loads
+    blocks = [(fwd[i] if i < len(fwd) else [], bwd[i] if i < len(bwd) else []) for i in range(max(len(fwd), len(bwd)))]
+    loaded = dstb.init_DCBlocks(search.plan_to_json(blocks), context_parallel_size=4)
+    assert "cp_attn_block_bwd_5" in _ops_of(loaded.dcblocks, "stream2_op")

@@ -121,7 +121,7 @@ def test_hip_cross_entropy_and_embedding(dtype):
         ssum = sum(c[1]["sum_exp"] * torch.exp(c[1]["row_max"] - big) for c in ctxs)
         pred = sum(torch.where(c[1]["target_mask"], torch.zeros_like(big), c[1]["predicted"] + c[1]["row_max"] - big)
                    for c in ctxs)
-        assert_close(torch.log(ssum) - pred, t("ce_loss"), torch.float32, "loss", scale=4)
+        assert_close(torch.log(ssum) - pred, t("ce_loss"), torch.float32, "loss")
         grads = []
         for r, c in enumerate(ctxs):
             ps.set_tensor_model_parallel(r, 4)
@@ -133,7 +133,7 @@ def test_hip_cross_entropy_and_embedding(dtype):
         for keep in (True, False):
             inputs = {"vocab_parallel_logits": t("ce_ls_x", dtype).cuda(), "target": t("ce_ls_target").cuda()}
             out = cross_entropy_fwd(inputs, 0.1, keep_softmax=keep)
-            assert_close(out["loss"], t("ce_ls_loss"), torch.float32, "smoothed loss", scale=4)
+            assert_close(out["loss"], t("ce_ls_loss"), torch.float32, "smoothed loss")
             assert_close(cross_entropy_bwd([inputs, out], dout), t("ce_ls_grad"), dtype, "smoothed grad")
         ps.set_tensor_model_parallel(2, 4)
         table = t("emb_table", dtype).cuda()
@@ -157,7 +157,7 @@ def test_hip_norm(dtype, name):
     b = t("norm_beta", dtype).cuda() if ln else None
     y, mu, rs, _ = pylayernorm_fwd(x, g, b, 1e-5, 0, False, None)
     assert_close(y, t(f"{name}_y"), dtype, "y")
-    assert_close(rs, t(f"{name}_rsigma"), torch.float32, "rsigma", scale=4)
+    assert_close(rs, t(f"{name}_rsigma"), torch.float32, "rsigma")
     mu32 = t(f"{name}_mu", torch.float32).cuda() if ln else None
     rs32 = t(f"{name}_rsigma", torch.float32).cuda()
     dx, dg, db, _ = pylayernorm_bwd(dy, x, mu32, rs32, g, 0, False, None)
@@ -194,8 +194,7 @@ def test_hip_attention(dtype, name, causal):
     out, lse = res[0], res[5]
     assert_close(out, t(f"{name}_out"), dtype, "out")
     for i, n in enumerate(lq):
-        assert_close(lse[i, :, :n], t(f"{name}_lse")[i, :, :n], torch.float32, f"lse[{i}]",
-                     scale=1e3 if dtype != torch.float32 else 1)
+        assert_close(lse[i, :, :n], t(f"{name}_lse")[i, :, :n], torch.float32, f"lse[{i}]")
     # backward from the exact out / lse, so the gradients are compared with the vectors alone
     out_x = t(f"{name}_out", dtype).cuda()
     lse_x = t(f"{name}_lse", torch.float32).cuda()
@@ -217,7 +216,7 @@ def test_hip_merge_and_route():
                            [t("merge_l1", torch.float32).cuda(), t("merge_l2", torch.float32).cuda()],
                            [0, 0], [8, 8], out, lse)
         assert_close(out, t("merge_out"), dtype, "merged out")
-        assert_close(lse, t("merge_lse"), torch.float32, "merged lse", scale=2)
+        assert_close(lse, t("merge_lse"), torch.float32, "merged lse")
     idx, gate, _ = route_topk(t("route_logits").cuda(), 2)
     assert np.array_equal(idx.cpu().numpy(), V["route_idx"])
     assert_close(gate, t("route_gate"), torch.float32, "gates")

@@ -49,7 +49,7 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     assert_close(out, oo, dtype, "out")
     for i, n in enumerate(lens_q):
         if n:
-            assert_close(lse[i, :, :n], lo[i, :, :n], torch.float32, f"lse[{i}]", scale=1e3 if dtype != torch.float32 else 1)
+            assert_close(lse[i, :, :n], lo[i, :, :n], torch.float32, f"lse[{i}]")
     # backward consumes the forward's own (rounded) out and lse, like the layer does
     stream = torch.cuda.current_stream()
     r = _Clib.pymha_varlen_bwd(do.cuda(), qg, kg, vg, out, lse, cq.cuda(), ck.cuda(), mq, mk, 0.0, scale, causal,
@@ -63,7 +63,7 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     assert_close(dv, dvo, dtype, "dv")
     for i, n in enumerate(lens_q):
         if n:
-            assert_close(dl[i, :, :n], dlo[i, :, :n], torch.float32, f"delta[{i}]", scale=1e3 if dtype != torch.float32 else 10)
+            assert_close(dl[i, :, :n], dlo[i, :, :n], torch.float32, f"delta[{i}]")
     return out, lse, dq, dk, dv
 
 
@@ -141,7 +141,7 @@ def test_merge_kernel(dtype):
     _Clib.pyattn_merge([o.cuda() for o in outs], [l.cuda() for l in lses], row_begin, rows, out, lse)
     oo, lo = OA.merge(outs, lses, row_begin, rows, b, sq, hq, d)
     assert_close(out, oo, dtype, "merged out")
-    assert_close(lse, lo, torch.float32, "merged lse", scale=2)
+    assert_close(lse, lo, torch.float32, "merged lse")
 
 
 def _ring_inputs(dtype, b, c, hq, hk, d, cp, seed=0):
@@ -191,7 +191,7 @@ def test_ring_step_matches_oracle_and_dense(dtype, b, c, hq, hk, d, rank):
     out, lse, dq, dkv = _ring_gpu(q, chunks, dout, rank, cp)
     oo, lo, _ = OA.ring_fwd(q, chunks, rank, scale)
     assert_close(out, oo, dtype, "ring out")
-    assert_close(lse, lo, torch.float32, "ring lse", scale=1e3 if dtype != torch.float32 else 2)
+    assert_close(lse, lo, torch.float32, "ring lse")
     # the same thing as ONE dense causal attention over the zig-zag order
     do_, lo_ = OA.zigzag_dense(q, chunks, rank, scale)
     assert_close(out.view(b, 2 * c, hq, d), do_, dtype, "ring out vs dense")
@@ -218,7 +218,7 @@ def test_ring_step_full_size(rank):
     cr = [(k.cuda().float().requires_grad_(), v.cuda().float().requires_grad_()) for k, v in chunks]
     do_, lo_ = OA.zigzag_dense(qr, cr, rank, scale, dtype=torch.float32)
     assert_close(out.view(b, 2 * c, hq, d), do_, dtype, "ring out vs dense")
-    assert_close(lse, lo_, torch.float32, "ring lse", scale=1e3)
+    assert_close(lse, lo_, torch.float32, "ring lse")
     (do_ * dout.cuda().float().view(b, 2 * c, hq, d)).sum().backward()
     assert_close(dq.view(q.shape), qr.grad, dtype, "ring dq")
     for s in range(cp):

@@ -74,7 +74,7 @@ def test_norm_past_2_31_elements():
     xc = x[idx.cuda()].cpu()
     yo, _, rso = O.norm_fwd(xc, gamma, None, 1e-5)
     assert_close(y[idx.cuda()], yo, BF, "y")
-    assert_close(rs[idx.cuda()], rso, torch.float32, "rsigma", scale=4)
+    assert_close(rs[idx.cuda()], rso, torch.float32, "rsigma")
     del y
     dy = _randn((rows, cols), 5)
     dx, dg, _, _ = pylayernorm_bwd(dy, x, None, rs, gamma.cuda(), 0, False, None)
@@ -102,7 +102,7 @@ def test_cross_entropy_past_2_31_elements():
     idx = _rows_to_check(rows, cols)
     xc = logits[0, idx.cuda()].cpu()
     ref = H.cross_entropy_fwd([xc], target[0, idx])[0]
-    assert_close(out["loss"][0, idx.cuda()], ref["loss"], torch.float32, "loss", scale=10)
+    assert_close(out["loss"][0, idx.cuda()], ref["loss"], torch.float32, "loss")
     grad = cross_entropy_bwd([inputs, out], dout.cuda(), grad_out=logits)      # over the logits
     assert grad.data_ptr() == logits.data_ptr()
     assert_close(grad[0, idx.cuda()], H.cross_entropy_bwd(ref, dout[0, idx]), BF, "d logits")

@@ -54,9 +54,9 @@ def test_model_step_matches_oracle_and_schedules_agree():
         losses = model.step(_cuda(batches), double_strand=True, loss_scale=8.0)
         torch.cuda.synchronize()
         for i in range(n):
-            assert_close(losses[i], losses_o[i], torch.float32, f"loss[{i}]", scale=4)
+            assert_close(losses[i], losses_o[i], torch.float32, f"loss[{i}]")
         for name, p in model.named_parameters():
-            assert_close(p.main_grad, grads_o[name], torch.float32, name, scale=10)
+            assert_close(p.main_grad, grads_o[name], torch.float32, name)
         # the serial schedule (one stream, forward then backward per micro-batch) gives the same bits
         serial = DSLLM(cfg, L, vocab, seed=3)
         losses_s = serial.step(_cuda(batches), double_strand=False, loss_scale=8.0)

@@ -26,7 +26,7 @@ def test_route_topk_bit_exact(T, E, k, ties):
     idx, gates, ms = route_topk(lg.cuda(), k)
     io, go = OM.route_topk(lg.numpy(), k)
     assert np.array_equal(idx.cpu().numpy(), io), "top-k indices must be bit-exact"
-    assert_close(gates, torch.from_numpy(go), torch.float32, "gates", scale=2)
+    assert_close(gates, torch.from_numpy(go), torch.float32, "gates")
     assert torch.allclose(gates.sum(1).cpu(), torch.ones(T), atol=1e-6)
 
 
@@ -83,7 +83,7 @@ def test_permute_unpermute(dtype, T, H, E, k, e_lo, e_hi):
     dyo = OM.permute(dout, sidx, offs, e_lo, e_hi, k, row_scale=gates.cpu())
     assert_close(dy[:R], dyo, dtype, "unpermute_bwd dy")
     dgo = OM.gate_grad(dout, y[:R], dest, offs, e_lo, e_hi, T, k)
-    assert_close(dg, dgo, torch.float32, "dgates", scale=10 if dtype == torch.float32 else 1e3)
+    assert_close(dg, dgo, torch.float32, "dgates")
 
 
 def test_permute_roundtrip_identity():

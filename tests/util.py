@@ -1,4 +1,6 @@
 """Helpers shared by the parity tests."""
+import os
+
 import torch
 
 # Tolerances of the path: relative L2 error of outputs and gradients against the oracle.
@@ -58,6 +60,8 @@ def local_err(a: torch.Tensor, ref: torch.Tensor):
 def assert_close(a, ref, dtype, what="", scale=1.0, local=True):
     e = rel_err(a, ref)
     tol = TOL[dtype] * scale
+    if scale > 1.0 and os.environ.get("DH_REPORT_SCALED"):       # which widened bounds are really needed
+        print(f"[scaled] {what}: rel err {e:.3e}, base tol {TOL[dtype]:.0e}, scale {scale:g}")
     assert e <= tol, f"{what}: rel err {e:.3e} > {tol:.1e}"
     if local:
         l2, mx, where = local_err(a, ref)

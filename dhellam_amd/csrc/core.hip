@@ -2,7 +2,11 @@
 #include "common.h"
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
+#include <algorithm>
+#include <mutex>
+#include <vector>
 
 namespace dh {
 static thread_local char g_err[1024] = "";
@@ -66,6 +70,31 @@ extern "C" int dh_delay(int64_t nanoseconds, void *stream) {
   return DH_OK;
 }
 
+// Masked streams that are alive, and their owner of last resort.  A caller that wraps such a stream in an object
+// that only borrows the handle (torch's ExternalStream) and never calls dh_stream_destroy would leave it open
+// until the HIP runtime's own exit-time destructors run; with a profiler attached (rocprofv3), whose tool has
+// finalised by then, a process that had made four of them ended with SIGSEGV after printing its result.
+// The first creation therefore registers an exit handler.  Handlers run in reverse order of registration, so
+// this one runs before those of the runtime and of a preloaded tool (both registered at load time) and after
+// the host program's own shutdown (a Python interpreter has freed its tensors by then: a tensor freed AFTER a
+// stream it was used on is destroyed would make the caching allocator record an event on a dead stream).
+namespace dh {
+static std::mutex g_streams_mutex;
+static std::vector<hipStream_t> g_masked_streams;
+static bool g_exit_hook = false;
+
+static void destroy_masked_streams_at_exit() {
+  std::vector<hipStream_t> left;
+  {
+    std::lock_guard<std::mutex> lock(g_streams_mutex);
+    left.swap(g_masked_streams);
+  }
+  for (hipStream_t st : left) {
+    if (hipStreamSynchronize(st) == hipSuccess) (void)hipStreamDestroy(st);
+  }
+}
+}  // namespace dh
+
 // A stream whose kernels run only on the compute units whose bit is set in `mask` (bit i of word i / 32;
 // on a device with several XCDs bit i is compute unit i / n_xcd of XCD i % n_xcd).
 extern "C" int dh_stream_create_cu_mask(const uint32_t *mask, int words, void **stream_out) {
@@ -79,12 +108,27 @@ extern "C" int dh_stream_create_cu_mask(const uint32_t *mask, int words, void **
   DH_CHECK(set > 0, "the mask enables no compute unit");
   hipStream_t st = nullptr;
   DH_HIP(hipExtStreamCreateWithCUMask(&st, (uint32_t)words, mask));
+  {
+    std::lock_guard<std::mutex> lock(dh::g_streams_mutex);
+    dh::g_masked_streams.push_back(st);
+    if (!dh::g_exit_hook) {
+      dh::g_exit_hook = true;
+      atexit(dh::destroy_masked_streams_at_exit);
+    }
+  }
   *stream_out = (void *)st;
   return DH_OK;
 }
 
 extern "C" int dh_stream_destroy(void *stream) {
   DH_CHECK(stream, "null stream");
+  {
+    std::lock_guard<std::mutex> lock(dh::g_streams_mutex);
+    auto &v = dh::g_masked_streams;
+    auto it = std::find(v.begin(), v.end(), (hipStream_t)stream);
+    DH_CHECK(it != v.end(), "not a live stream of dh_stream_create_cu_mask (destroyed twice?)");
+    v.erase(it);
+  }
   DH_HIP(hipStreamDestroy((hipStream_t)stream));
   return DH_OK;
 }

@@ -228,7 +228,16 @@ def test_cu_partitioned_streams():
     cfg = LayerConfig(hidden_size=512, num_attention_heads=8, num_query_groups=4, ffn_hidden_size=1024, seq_length=256,
                       micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
                       params_dtype=torch.bfloat16, comm_standin_us=30.0)
-    (c1, c2), comm = partitioned_streams(reserved_per_xcd=1)
+    with partitioned_streams(reserved_per_xcd=1) as ((c1, c2), comm):
+        _partitioned_checks(cfg, c1, c2, comm, lib)
+    from dhellam_amd.common import streams as S
+    assert not S._LIVE, "the partition's streams are ended with the block"
+
+
+def _partitioned_checks(cfg, c1, c2, comm, lib):
+    import dataclasses
+    from dhellam_amd import _lib
+    from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
     res = []
     for part in (False, True):
         c = dataclasses.replace(cfg, comm_streams=tuple(comm)) if part else cfg
@@ -255,3 +264,26 @@ def test_cu_partitioned_streams():
         torch.cuda.synchronize()
         worst = max(worst, e0.elapsed_time(e1) * 1e3)
     assert 45.0 <= worst <= 150.0, worst
+
+
+def test_masked_streams_do_not_outlive_the_interpreter(tmp_path):
+    """A process that makes masked streams and never destroys them by hand ends normally (exit status 0): the
+    streams module ends them in an exit hook, before the runtime's own exit-time destructors run."""
+    import subprocess
+    import sys
+    code = (
+        "import torch\n"
+        "from dhellam_amd.common.streams import partitioned_streams\n"
+        "(c1, c2), comm = partitioned_streams()\n"
+        "x = torch.ones(1 << 20, device='cuda')\n"
+        "for st in (c1, c2, *comm):\n"
+        "    st.wait_stream(torch.cuda.current_stream())\n"
+        "    with torch.cuda.stream(st):\n"
+        "        y = x * 2\n"
+        "torch.cuda.synchronize()\n"
+        "print('done', float(y[0]))\n")
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=110)
+    assert "done 2.0" in res.stdout, res.stderr[-2000:]
+    assert res.returncode == 0, (res.returncode, res.stderr[-2000:])

@@ -101,21 +101,58 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
         False   True     B.T @ A       ("NT": wgrad)
 
     The product is ``dh_gemm`` (hipBLASLt behind the C ABI).  ``input_workspace`` / ``workspaceSize`` are
-    used when given (a GPU tensor of at least that many bytes), otherwise a per-stream 32 MiB buffer;
-    ``math_sm_count`` is accepted and unused.  For the weight gradient, B^T is materialised first
+    used when given (a GPU tensor of at least that many bytes), otherwise a per-stream 32 MiB buffer.
+    ``math_sm_count`` > 0 confines the product to that many compute units, as the reference's libsmctrl
+    mask does (csrc/operators/gemm.cu:66-70, smctrl.cpp:135-160): it runs on a stream created with that
+    compute-unit mask (cached per device and count), ordered after and before the current stream by events;
+    a count above the device's compute units is refused.  For the weight gradient, B^T is materialised first
     where that makes the product faster by more than it costs (``wgrad_layout``).
     """
     _lib.need_cuda(inputA, inputB, outputD)
     stream = torch.cuda.current_stream()
     ws_bytes = int(workspaceSize or 0)
 
-    def run():
+    def product():
         if transb and not transa:
             wgrad_gemm(inputB, inputA, outputD, grad_accumulate, input_workspace, ws_bytes)
         else:
             dense_gemm(inputA, inputB, outputD, transa, transb, grad_accumulate, input_workspace, ws_bytes)
 
-    return _timed(profiling, stream, run)
+    return _timed(profiling, stream, lambda: _confined(stream, math_sm_count, lambda st: product()))
+
+
+_masked_streams: dict = {}
+
+
+def _masked_stream(count: int) -> torch.cuda.Stream:
+    """The stream that owns ``|count|`` compute units of the current device: the first ones for a positive
+    count, the last ones for a negative count (the reference's ``reverse``, gemm.cu:20-21).  Mask bits are spread
+    over the XCDs round-robin, so the units are shared evenly between them."""
+    from .common.streams import cu_mask_words, stream_with_cu_mask
+    dev = torch.cuda.current_device()
+    n_cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    n = abs(count)
+    if not 0 < n <= n_cus:
+        raise RuntimeError(f"math_sm_count={count} outside the {n_cus} compute units of this device")
+    key = (dev, count)
+    if key not in _masked_streams:
+        _masked_streams[key] = stream_with_cu_mask(cu_mask_words(n_cus, 0 if count > 0 else n_cus - n, n))
+    return _masked_streams[key]
+
+
+def _confined(stream, math_sm_count, launch):
+    """``launch(stream_to_use)`` on ``stream``, or -- with a non-zero ``math_sm_count`` -- on the masked stream of
+    that many compute units, ordered after and before ``stream`` by events (the MI355X form of the reference's
+    per-launch libsmctrl mask, csrc/operators/smctrl.cpp:135-160)."""
+    math_sm_count = int(math_sm_count or 0)
+    if math_sm_count == 0:
+        return launch(stream)
+    masked = _masked_stream(math_sm_count)
+    masked.wait_stream(stream)
+    with torch.cuda.stream(masked):
+        res = launch(masked)
+    stream.wait_stream(masked)
+    return res
 
 
 def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -235,7 +272,8 @@ def _zero_rng_state(device) -> torch.Tensor:
 
 def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
                      is_causal, return_softmax, math_sm_count, profiling):
-    """ops.h:18-32 / flash_atten.cu:436-477.  Runs on the current stream.
+    """ops.h:18-32 / flash_atten.cu:436-477.  Runs on the current stream (``math_sm_count`` != 0: confined to
+    that many compute units, see ``_confined``).
 
     Returns [out, q, k, v, out, softmax_lse, p, rng_state] (+ a CPU fp32 [1] tensor of
     milliseconds when ``profiling``), positions as in flash_atten.cu:429-433.  The
@@ -255,9 +293,9 @@ def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     b = cu_seqlens_q.numel() - 1
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     lse = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
-    ms = _timed(profiling, stream, lambda: _attn_fwd_raw(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k,
-                                                        max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
-                                                        stream.cuda_stream))
+    ms = _timed(profiling, stream, lambda: _confined(stream, math_sm_count, lambda st: _attn_fwd_raw(
+        q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
+        st.cuda_stream)))
     p = torch.empty(0, dtype=q.dtype, device=q.device)
     res = [out, q, k, v, out, lse, p, _zero_rng_state(q.device)]
     if profiling:
@@ -309,9 +347,9 @@ def pymha_varlen_bwd(dout, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k
         dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
         dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
         softmax_d = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
-        ms = _timed(profiling, ext, lambda: _attn_bwd_raw(dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d,
-                                                          cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                                                          softmax_scale, is_causal, int(stream_ptr or 0)))
+        ms = _timed(profiling, ext, lambda: _confined(ext, math_sm_count, lambda st: _attn_bwd_raw(
+            dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
+            max_seqlen_k, softmax_scale, is_causal, int(st.cuda_stream))))
     res = [dq, dk, dv, softmax_d]
     if profiling:
         res.append(torch.tensor([ms], dtype=torch.float32))

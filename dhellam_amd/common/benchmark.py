@@ -22,6 +22,22 @@ def benchmark(repeat, fn, *args, **kwargs):
     return sum(times) / repeat
 
 
+def benchmark_ms(repeat, s1, s2, fn1, fn2, *args):
+    """Mean ms of ``repeat`` rounds of one prepared op on s1 and one on s2 (benchmark.py:17-29); a factory is
+    ``fn(*args) -> (call_args, callable)``."""
+    a1, k1 = fn1(*args)
+    a2, k2 = fn2(*args)
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for _ in range(repeat):
+        with torch.cuda.stream(s1):
+            k1(*a1)
+        with torch.cuda.stream(s2):
+            k2(*a2)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - start) / repeat * 1000
+
+
 def trimmed_mean(samples):
     """Mean after dropping the lowest and highest 20 %, only when more than 10 samples."""
     s = sorted(samples)

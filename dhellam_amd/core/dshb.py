@@ -97,3 +97,96 @@ def _main_grad(p: torch.Tensor) -> torch.Tensor:
         g = torch.zeros_like(p)
         p.main_grad = g
     return g
+
+
+class DSHB_(torch.autograd.Function):
+    """The head block of the folded model (dshb.py:114-237).  Forward traversal: backward of the PREVIOUS
+    micro-batch's loss (its gradient becomes the backward strand's input) and the embedding of the NEW one.
+    Autograd traversal: the new micro-batch's loss, and the previous micro-batch's embedding gradient."""
+
+    @staticmethod
+    def forward(ctx, placeholder, block):
+        from ..common.global_variables import GLOBAL_VARIABLES as G
+        ctx.block = block
+        bwd_input, fwd_input = G['inputs']
+        s_f, s_b = block.stream_fwd, block.stream_bwd
+        dgrad = fwd_result = None
+        with torch.no_grad():
+            if bwd_input is not None:
+                (head_ctx,) = G['bwd_activations'][0].pop()
+                if G['bwd_activations'][0].is_empty():
+                    G['bwd_activations'].pop(0)
+                s_b.wait_event(head_ctx["_ready"])
+                _record_stream(head_ctx, s_b)
+                with torch.cuda.stream(s_b):
+                    dgrad = post_process_bwd(head_ctx)
+            if fwd_input is not None:
+                token_ids, labels, loss_mask = fwd_input
+                ctx.labels, ctx.loss_mask = labels, loss_mask
+                with torch.cuda.stream(s_f):
+                    fwd_result, emb_ctx = pre_process(token_ids, block.word_embeddings, batch_first=True)
+                G['fwd_activations'][-1].push([emb_ctx])
+        G['inputs'] = [dgrad, fwd_result]
+        return placeholder.view_as(placeholder)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        from ..common.global_variables import GLOBAL_VARIABLES as G
+        block = ctx.block
+        bwd_input, fwd_input = G['inputs']
+        s_f, s_b = block.stream_fwd, block.stream_bwd
+        loss = None
+        with torch.no_grad():
+            if bwd_input is not None:
+                (emb_ctx,) = G['fwd_activations'][0].pop()
+                if G['fwd_activations'][0].is_empty():
+                    G['fwd_activations'].pop(0)
+                with torch.cuda.stream(s_b):
+                    pre_process_bwd(emb_ctx, bwd_input, batch_first=True)
+            if fwd_input is not None:
+                with torch.cuda.stream(s_f):
+                    loss, head_ctx = post_process(fwd_input, block.ln_weight, block.ln_bias, ctx.labels, ctx.loss_mask,
+                                                  block.word_embeddings, block.num_mb, block.loss_scale,
+                                                  block.config.layernorm_epsilon, batch_first=True)
+                    head_ctx["_ready"] = torch.cuda.Event()
+                    head_ctx["_ready"].record(s_f)
+                G['bwd_activations'][-1].push([head_ctx])
+                G['loss'].append({'lm loss': loss})
+        G['inputs'] = [None, loss]
+        return grads[0], None
+
+
+def _record_stream(obj, stream) -> None:
+    if isinstance(obj, torch.Tensor):
+        if obj.is_cuda:
+            obj.record_stream(stream)
+    elif isinstance(obj, dict):
+        for v in obj.values():
+            _record_stream(v, stream)
+    elif isinstance(obj, (list, tuple)):
+        for v in obj:
+            _record_stream(v, stream)
+
+
+class DSHB(torch.nn.Module):
+    """Embedding table (tied to the output layer), final norm and loss (dshb.py:239-275), without Megatron's
+    ``LanguageModelEmbedding`` / ``ColumnParallelLinear`` and without learned position embeddings (the layers
+    rotate q and k instead).  ``num_mb``: micro-batches per step; ``loss_scale``: the reference's
+    ``loss_scale_func`` as a factor."""
+
+    def __init__(self, config, vocab_size: int, stream1=None, stream2=None, num_mb: int = 1, loss_scale: float = 1.0,
+                 seed: int = 0, device="cuda"):
+        super().__init__()
+        self.config, self.stream_fwd, self.stream_bwd = config, stream1, stream2
+        self.num_mb, self.loss_scale = num_mb, loss_scale
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        dt = config.params_dtype
+        self.word_embeddings = torch.nn.Parameter((torch.randn(vocab_size, config.hidden_size, generator=g) * 0.02).to(dt).to(device))
+        self.ln_weight = torch.nn.Parameter(torch.ones(config.hidden_size, dtype=dt, device=device))
+        self.ln_bias = None
+        for p in (self.word_embeddings, self.ln_weight):
+            p.main_grad = torch.zeros_like(p)
+        self.logits_weight = self.word_embeddings
+
+    def forward(self, placeholder):
+        return DSHB_.apply(placeholder, self)

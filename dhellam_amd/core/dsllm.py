@@ -3,8 +3,11 @@ a step paired the reference's way (dhellam/core/dsllm.py:43-106, dhellam/core/ds
 the first micro-batch runs forward only, then forward of micro-batch i + 1 runs beside backward
 of micro-batch i through the whole model, and the last micro-batch runs backward only.
 
-The reference hides this inside Megatron modules and autograd hooks; here it is one explicit
-schedule over this package's operators.  In a paired phase the forward strand (stream 1) walks
+Two forms of the same schedule live here.  ``DSLLM`` is the reference's shell: a ``torch.nn.Module`` of
+head block + folded ``DSTB`` modules driven by ``model(x1, x2)`` followed by ``.backward()``
+on the placeholder it returns (autograd functions and a backward pre-hook move the micro-batches,
+``Stack``s hold their activations), without Megatron.  ``DSLLMStep`` is the same thing written as
+one explicit schedule over this package's operators.  In a paired phase the forward strand (stream 1) walks
 the layers upward while the backward strand (stream 2) walks them downward, so slot k pairs
 forward of layer k with backward of layer L - 1 - k under the plan's DCBlocks:
 
@@ -38,7 +41,7 @@ def _record(obj, stream) -> None:
             _record(v, stream)
 
 
-class DSLLM:
+class DSLLMStep:
     def __init__(self, cfg: LayerConfig, num_layers: int, vocab_size: int, seed: int = 0, plan=None,
                  stream1: Optional[torch.cuda.Stream] = None, stream2: Optional[torch.cuda.Stream] = None,
                  device="cuda"):
@@ -146,3 +149,126 @@ class DSLLM:
         cur.wait_stream(s1)
         cur.wait_stream(s2)
         return losses
+
+
+# ---- the reference's module shell (dsllm.py:10-115) -----------------------------------------------
+class Stack:
+    def __init__(self):
+        self.items = []
+
+    def __str__(self) -> str:
+        return f"dhellam.Stack object({len(self.items)} items)"
+
+    def is_empty(self):
+        return len(self.items) == 0
+
+    def push(self, item):
+        self.items.append(item)
+
+    def pop(self):
+        if not self.is_empty():
+            return self.items.pop()
+        raise IndexError("pop from empty stack")
+
+    def size(self):
+        return len(self.items)
+
+
+def pre_backward_hook(module, grad_output):
+    """dsllm.py:108-115: the autograd traversal of a call that took a new micro-batch forward collects that
+    micro-batch's second-half activations on a stack of its own."""
+    from ..common.global_variables import GLOBAL_VARIABLES
+    x1, x2 = GLOBAL_VARIABLES["inputs"]
+    if x2 is not None:
+        GLOBAL_VARIABLES['bwd_activations'].append(Stack())
+    return grad_output
+
+
+class DSLLM(torch.nn.Module):
+    """``num_layers`` decoder layers (even) folded into ``num_layers / 2`` DSTB modules behind a head block
+    (dsllm.py:43-106).  One call + backward moves the new micro-batch forward through ALL layers and the
+    previous one backward through all of them::
+
+        out = model(previous_loss_or_None, (token_ids, labels, loss_mask) or None); out.backward()
+
+    x1 (the reference passes the previous micro-batch's loss) only says whether a previous micro-batch
+    waits for its backward; x2 is the new micro-batch's data.  ``run_microbatches`` drives a whole step.
+    One rank (tensor_model_parallel_size == 1), no pipeline stages, no Megatron."""
+
+    def __init__(self, config: LayerConfig, vocab_size: int, num_layers: int, num_mb: int = 1, loss_scale: float = 1.0,
+                 seed: int = 0, plan=None, stream1: Optional[torch.cuda.Stream] = None,
+                 stream2: Optional[torch.cuda.Stream] = None, pre_process: bool = True, device="cuda"):
+        super().__init__()
+        from ..common.global_variables import GLOBAL_VARIABLES
+        from .dstb import DSTB
+        if config.tensor_model_parallel_size != 1:
+            raise ValueError("the model shell runs one complete rank: tensor_model_parallel_size must be 1")
+        assert num_layers % 2 == 0, "Only support the llm with even number of layers in each pipeline stage!"
+        self.config = config
+        self.stream1 = stream1 or torch.cuda.Stream()
+        self.stream2 = stream2 or torch.cuda.Stream()
+        n = num_layers // 2
+        # layer l of the network is first_l for l < n and second_{2n-1-l} otherwise; seeds follow the layer number
+        self.pre_process = pre_process
+        if pre_process:
+            self.dchb = dshb.DSHB(config, vocab_size, self.stream1, self.stream2, num_mb, loss_scale, seed, device)
+        mods = []
+        for k in range(n):
+            m = DSTB(config, self.stream1, self.stream2, plan, seed=0, device=device)
+            for tag, layer in (("first", k), ("second", 2 * n - 1 - k)):
+                w = make_weights(config, seed + 1 + layer, device)
+                wd = m.weight_first if tag == "first" else m.weight_second
+                with torch.no_grad():
+                    for key, p in wd.items():
+                        if isinstance(p, torch.nn.Parameter):
+                            p.copy_(w[key])
+            mods.append(m)
+        self.dctb = torch.nn.Sequential(*mods)
+        self.input_tensor = None
+        GLOBAL_VARIABLES['loss'] = []
+        GLOBAL_VARIABLES['fwd_activations'] = []
+        GLOBAL_VARIABLES['bwd_activations'] = []
+        self.register_full_backward_pre_hook(pre_backward_hook)
+
+    def set_input_tensor(self, input_tensor) -> None:
+        self.input_tensor = input_tensor if isinstance(input_tensor, list) else [input_tensor]
+
+    def layer_weights(self, l: int) -> Dict[str, torch.Tensor]:
+        """Weight dict of network layer ``l`` (see the folding rule above)."""
+        n = len(self.dctb)
+        return self.dctb[l].weight_first if l < n else self.dctb[2 * n - 1 - l].weight_second
+
+    def forward(self, x1, x2):
+        from ..common.global_variables import GLOBAL_VARIABLES
+        if not self.pre_process:
+            x1, x2 = self.input_tensor
+        backward_only, forward_only = x2 is None, x1 is None
+        assert not (forward_only and backward_only), "it's necessary to execute forward pass or backward pass"
+        if not backward_only:
+            GLOBAL_VARIABLES['fwd_activations'].append(Stack())
+        cur = torch.cuda.current_stream()
+        self.stream1.wait_stream(cur)
+        self.stream2.wait_stream(cur)
+        placeholder = torch.zeros(1, dtype=torch.float32, device="cuda", requires_grad=True)
+        GLOBAL_VARIABLES['inputs'] = [x1, x2]
+        if self.pre_process:
+            placeholder = self.dchb(placeholder)
+        return self.dctb(placeholder)
+
+
+def run_microbatches(model: DSLLM, batches: List[dict]) -> List[torch.Tensor]:
+    """A whole step through the module shell: forward of micro-batch 0, then forward(i + 1) beside backward(i),
+    then the last backward -- the order the reference's patched no-pipelining schedule produces.  Returns the
+    micro-batch losses; gradients are in the parameters' ``main_grad``."""
+    from ..common.global_variables import GLOBAL_VARIABLES
+    GLOBAL_VARIABLES['loss'] = []
+    prev = None
+    for mb in list(batches) + [None]:
+        x2 = None if mb is None else (mb["token_ids"], mb["labels"], mb["loss_mask"])
+        out = model(prev, x2)
+        out.backward()
+        prev = GLOBAL_VARIABLES['inputs'][1]           # the new micro-batch's loss (None after the last call)
+    cur = torch.cuda.current_stream()
+    cur.wait_stream(model.stream1)
+    cur.wait_stream(model.stream2)
+    return [d['lm loss'] for d in GLOBAL_VARIABLES['loss']]

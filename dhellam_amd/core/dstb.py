@@ -46,6 +46,7 @@ from typing import List, Optional
 import torch
 
 from .. import _lib
+from ..common.global_variables import GLOBAL_VARIABLES
 from .._Clib import pymha_varlen_bwd, pymha_varlen_fwd, _attn_bwd_raw
 from ..operators.bda import bda_bwd, bda_fwd
 from ..operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
@@ -460,134 +461,217 @@ _PEER_KEY = {"allgather_attn": "sp_peer_attn", "allgather_mlp": "sp_peer_mlp",
              "allgather_mlp_bwd": "sp_peer_mlp_bwd", "allgather_attn_bwd": "sp_peer_attn_bwd"}
 
 
+class _Ctx:
+    """What one dispatch hands to an op handler."""
+    __slots__ = ("dcfunc", "op", "config", "weight", "act", "x", "stream", "name", "movable")
+
+    def __init__(self, dcfunc, op, config, weight, act, x, stream, name, movable):
+        self.dcfunc, self.op, self.config, self.weight, self.act = dcfunc, op, config, weight, act
+        self.x, self.stream, self.name, self.movable = x, stream, name, movable
+
+    def g(self, key):
+        """A saved activation, registered with the stream that is about to read it."""
+        return _use(self.act[key], self.stream)
+
+
+def _h_norm(c):
+    p = "attn" if c.op == 1 else "mlp"
+    fn = c.dcfunc.ln_attn if c.op == 1 else c.dcfunc.ln_mlp
+    act = c.act
+    output, act[f"{p}_mu"], act[f"{p}_rsigma"], act[f"ln_{p}_input"], act[f"ln_{p}_residual"], _ = fn(
+        c.config, (c.x, c.weight[f"ln_{p}_weight"], c.weight.get(f"ln_{p}_bias")), c.stream)
+    return output
+
+
+def _h_gemm_attn_c(c):
+    c.act["gemm_attn_c_input"] = c.x
+    return c.dcfunc.gemm_attn_column(c.config, (c.x, c.weight["column_attn_weight"]), c.stream)
+
+
+def _h_rope(c):
+    return c.dcfunc.rope(c.config, (c.x,), c.stream)
+
+
+def _h_attn(c):
+    act = c.act
+    (output, act["q_padded"], act["k_padded"], act["v_padded"], act["out_padded"], act["rng_state"],
+     act["softmax_lse"]) = c.dcfunc.attn(c.config, (c.x, c.weight["cu_seqlens_q"], c.weight["cu_seqlens_kv"]), c.stream,
+                                         apply_rope=c.config.groups_per_rank != 1)
+    return output
+
+
+def _h_gemm_attn_l(c):
+    output, c.act["linear_attn_input"] = c.dcfunc.gemm_attn_linear(c.config, (c.x, c.weight["linear_attn_weight"]), c.stream)
+    return output
+
+
+def _h_gemm_mlp_c(c):
+    c.act["gemm_mlp_c_input"] = c.x
+    return c.dcfunc.gemm_mlp_column(c.config, (c.x, c.weight["column_mlp_weight"]), c.stream)
+
+
+def _h_gemm_mlp_l(c):
+    output, c.act["linear_mlp_input"] = c.dcfunc.gemm_mlp_linear(c.config, (c.x, c.weight["linear_mlp_weight"]), c.stream)
+    return output
+
+
+def _h_bda_mlp(c):
+    output, c.act["mlp_mask"] = c.dcfunc.bda_mlp(c.config, (c.x, c.g("ln_mlp_residual")), c.stream)
+    return output
+
+
+def _h_bda_attn(c):
+    output, c.act["attn_mask"] = c.dcfunc.bda_attn(c.config, (c.x, c.g("ln_attn_residual")), c.stream)
+    return output
+
+
+def _h_reduce_scatter(c):
+    return c.dcfunc.reduce_scatter(c.config, (c.x,), c.stream, bwd_strand=bool(c.name) and c.name.endswith("_bwd"))
+
+
+def _h_all_gather(c):
+    peer = c.act.get(_PEER_KEY.get(c.name, ""))
+    return c.dcfunc.allgather(c.config, (c.x, _use(peer, c.stream)), c.stream,
+                              bwd_strand=bool(c.name) and c.name.endswith("_bwd"))
+
+
+def _h_swiglu(c):
+    output = c.dcfunc.swiglu(c.config, (c.x,), c.stream)
+    c.act["swiglu_input"] = c.x
+    return output
+
+
+_DGRAD_WEIGHT = {13: "column_mlp_weight", 15: "linear_mlp_weight", 17: "column_attn_weight", 19: "linear_attn_weight"}
+
+
+def _h_dgrad(c):
+    return c.dcfunc._dgrad(c.config, (c.x, c.weight[_DGRAD_WEIGHT[c.op]]), c.stream)
+
+
+def _run_or_park(c, fn, args):
+    """A weight gradient runs now, or -- when the plan names its placeholder -- is parked until the placeholder
+    op (or the end of the block list) runs it (dstb.py:543-598)."""
+    if _WGRAD_PLACEHOLDER[c.op] in c.movable:
+        c.act.setdefault("_parked", {})[_WGRAD_PLACEHOLDER[c.op]] = (fn, (c.config, args, c.stream))
+    else:
+        fn(c.config, args, c.stream)
+    return None
+
+
+def _h_wgrad_column(c):
+    # (saved GEMM input, incoming gradient, main_grad)
+    if c.op == 14:
+        args = (c.g("gemm_mlp_c_input"), c.g("swiglu_dgrad"), c.weight["column_mlp_weight"].main_grad)
+        return _run_or_park(c, c.dcfunc.gemm_wgrad_mlp_c, args)
+    c.act.pop("attn_dgrad", None)          # kept by the last ring call for this weight gradient
+    args = (c.g("gemm_attn_c_input"), c.x, c.weight["column_attn_weight"].main_grad)
+    return _run_or_park(c, c.dcfunc.gemm_wgrad_attn_c, args)
+
+
+def _h_wgrad_linear(c):
+    key, wkey = ("linear_mlp_input", "linear_mlp_weight") if c.op == 16 else ("linear_attn_input", "linear_attn_weight")
+    args = (c.x, c.g(key), c.weight[wkey].main_grad)
+    return _run_or_park(c, c.dcfunc.gemm_wgrad_mlp_l if c.op == 16 else c.dcfunc.gemm_wgrad_attn_l, args)
+
+
+def _h_placeholder(c):
+    parked = c.act.get("_parked", {}).pop(_PLACEHOLDER_ID[c.op], None)
+    if parked is not None:
+        fn, (cfg, args, _) = parked
+        fn(cfg, args, c.stream)
+    return None
+
+
+def _h_swiglu_bwd(c):
+    output = c.dcfunc.swiglu_bwd(c.config, (c.g("swiglu_input"), c.x), c.stream)
+    c.act["swiglu_dgrad"] = output
+    return output
+
+
+def _h_bda_mlp_bwd(c):
+    output, c.act["mlp_residual_bwd"] = c.dcfunc.bda_mlp_bwd(c.config, (c.x, c.act.get("mlp_mask")), c.stream)
+    return output
+
+
+def _h_bda_attn_bwd(c):
+    output, c.act["attn_residual_bwd"] = c.dcfunc.bda_attn_bwd(c.config, (c.x, c.act.get("attn_mask")), c.stream)
+    return output
+
+
+def _h_attn_bwd(c):
+    return c.dcfunc.attn_bwd(c.config, (c.x, c.g("q_padded"), c.g("k_padded"), c.g("v_padded"), c.g("out_padded"),
+                                        c.g("softmax_lse"), c.weight["cu_seqlens_q"], c.weight["cu_seqlens_kv"],
+                                        c.act.get("rng_state")), c.stream, apply_rope=c.config.groups_per_rank != 1)
+
+
+def _h_rope_bwd(c):
+    return c.dcfunc.rope_bwd(c.config, (c.x,), c.stream)
+
+
+def _h_ring_fwd(c):
+    act, x = c.act, c.x
+    last = (0 if isinstance(x, torch.Tensor) else x[7]) == c.config.context_parallel_size - 1
+    visiting = act.get("cp_kv_chunks")
+    for t in visiting or ():
+        _use(t, c.stream)
+    output = c.dcfunc.ring_attn_fwd(c.config, (x, c.weight["cu_seqlens_q"], c.weight["cu_seqlens_kv"],
+                                               c.weight.get("rope_positions"), visiting), c.stream)
+    if last:       # dstb.py:471-481
+        output, act["q"], act["kv"], act["softmax_lse"], act["rng_states"] = output
+        act["out"] = output
+    return output
+
+
+def _h_ring_bwd(c):
+    act, x = c.act, c.x
+    last = (0 if isinstance(x, torch.Tensor) else x[4]) == c.config.context_parallel_size
+    for t in act["kv"]:
+        _use(t, c.stream)
+    output = c.dcfunc.ring_attn_bwd(c.config, (x, c.g("out"), c.g("q"), act["kv"], c.g("softmax_lse"), act.get("rng_states"),
+                                               c.weight["cu_seqlens_q"], c.weight["cu_seqlens_kv"],
+                                               c.weight.get("rope_positions")), c.stream)
+    if last:       # dstb.py:492-504
+        for key in ("out", "q", "kv", "softmax_lse", "rng_states"):
+            act.pop(key, None)
+        act["attn_dgrad"] = output
+    return output
+
+
+def _h_norm_bwd(c):
+    p = "mlp" if c.op == 25 else "attn"
+    lw, lb = c.weight[f"ln_{p}_weight"], c.weight.get(f"ln_{p}_bias")
+    mu = c.act.get(f"{p}_mu")
+    data = (c.x, c.g(f"ln_{p}_input"), _use(mu, c.stream), c.g(f"{p}_rsigma"), lw, lb, c.g(f"{p}_residual_bwd"),
+            lw.main_grad, lb.main_grad if lb is not None else None)
+    return (c.dcfunc.ln_mlp_bwd if c.op == 25 else c.dcfunc.ln_attn_bwd)(c.config, data, c.stream)
+
+
+# op id -> handler (the reference: one ``if operation == N`` after another, dstb.py:431-657)
+_HANDLERS = {
+    1: _h_norm, 2: _h_norm, 3: _h_gemm_attn_c, 4: _h_gemm_attn_l, 5: _h_gemm_mlp_c, 6: _h_gemm_mlp_l, 7: _h_attn,
+    8: _h_bda_mlp, 9: _h_bda_attn, 10: _h_reduce_scatter, 11: _h_all_gather, 12: _h_swiglu,
+    13: _h_dgrad, 15: _h_dgrad, 17: _h_dgrad, 19: _h_dgrad,
+    14: _h_wgrad_column, 18: _h_wgrad_column, 16: _h_wgrad_linear, 20: _h_wgrad_linear,
+    114: _h_placeholder, 116: _h_placeholder, 118: _h_placeholder, 120: _h_placeholder,
+    21: _h_swiglu_bwd, 22: _h_bda_mlp_bwd, 23: _h_bda_attn_bwd, 24: _h_attn_bwd, 25: _h_norm_bwd, 26: _h_norm_bwd,
+    29: _h_ring_fwd, 30: _h_ring_bwd, 31: _h_rope, 32: _h_rope_bwd,
+}
+
+
 class DCoperation:
     """Dispatch one op id: fetch its inputs (previous op's output, weights, saved
     activations), run the adapter, save / free activations (dstb.py:427-660)."""
 
     @staticmethod
     def perform_operation(dcfunc, operation, config, weight, activation_dict, **kwargs):
-        stream = kwargs["stream"]
-        x = kwargs.get("output")
-        name = kwargs.get("name")
-        movable = kwargs.get("movable", ())
-        act = activation_dict
         op = operation.value if isinstance(operation, FuncChoice) else int(operation)
-        g = lambda key: _use(act[key], stream)
-        output = None
-
-        if op in (1, 2):
-            p = "attn" if op == 1 else "mlp"
-            fn = dcfunc.ln_attn if op == 1 else dcfunc.ln_mlp
-            output, act[f"{p}_mu"], act[f"{p}_rsigma"], act[f"ln_{p}_input"], act[f"ln_{p}_residual"], _ = fn(
-                config, (x, weight[f"ln_{p}_weight"], weight.get(f"ln_{p}_bias")), stream)
-        elif op == 3:
-            act["gemm_attn_c_input"] = x
-            output = dcfunc.gemm_attn_column(config, (x, weight["column_attn_weight"]), stream)
-        elif op == 31:
-            output = dcfunc.rope(config, (x,), stream)
-        elif op == 7:
-            (output, act["q_padded"], act["k_padded"], act["v_padded"], act["out_padded"], act["rng_state"],
-             act["softmax_lse"]) = dcfunc.attn(config, (x, weight["cu_seqlens_q"], weight["cu_seqlens_kv"]), stream,
-                                               apply_rope=config.groups_per_rank != 1)
-        elif op == 4:
-            output, act["linear_attn_input"] = dcfunc.gemm_attn_linear(config, (x, weight["linear_attn_weight"]), stream)
-        elif op == 5:
-            act["gemm_mlp_c_input"] = x
-            output = dcfunc.gemm_mlp_column(config, (x, weight["column_mlp_weight"]), stream)
-        elif op == 6:
-            output, act["linear_mlp_input"] = dcfunc.gemm_mlp_linear(config, (x, weight["linear_mlp_weight"]), stream)
-        elif op == 8:
-            output, act["mlp_mask"] = dcfunc.bda_mlp(config, (x, g("ln_mlp_residual")), stream)
-        elif op == 9:
-            output, act["attn_mask"] = dcfunc.bda_attn(config, (x, g("ln_attn_residual")), stream)
-        elif op == 10:
-            output = dcfunc.reduce_scatter(config, (x,), stream, bwd_strand=bool(name) and name.endswith("_bwd"))
-        elif op == 11:
-            peer = act.get(_PEER_KEY.get(name, ""))
-            output = dcfunc.allgather(config, (x, _use(peer, stream)), stream,
-                                      bwd_strand=bool(name) and name.endswith("_bwd"))
-        elif op == 12:
-            output = dcfunc.swiglu(config, (x,), stream)
-            act["swiglu_input"] = x
-        elif op in (13, 15, 17, 19):
-            wkey = {13: "column_mlp_weight", 15: "linear_mlp_weight", 17: "column_attn_weight",
-                    19: "linear_attn_weight"}[op]
-            output = dcfunc._dgrad(config, (x, weight[wkey]), stream)
-        elif op in (14, 18):
-            # (saved GEMM input, incoming gradient, main_grad)
-            if op == 14:
-                args = (g("gemm_mlp_c_input"), g("swiglu_dgrad"), weight["column_mlp_weight"].main_grad)
-                fn = dcfunc.gemm_wgrad_mlp_c
-            else:
-                args = (g("gemm_attn_c_input"), x, weight["column_attn_weight"].main_grad)
-                fn = dcfunc.gemm_wgrad_attn_c
-            if _WGRAD_PLACEHOLDER[op] in movable:
-                act.setdefault("_parked", {})[_WGRAD_PLACEHOLDER[op]] = (fn, (config, args, stream))
-            else:
-                fn(config, args, stream)
-        elif op in (16, 20):
-            key, wkey = ("linear_mlp_input", "linear_mlp_weight") if op == 16 else ("linear_attn_input", "linear_attn_weight")
-            args = (x, g(key), weight[wkey].main_grad)
-            fn = dcfunc.gemm_wgrad_mlp_l if op == 16 else dcfunc.gemm_wgrad_attn_l
-            if _WGRAD_PLACEHOLDER[op] in movable:
-                act.setdefault("_parked", {})[_WGRAD_PLACEHOLDER[op]] = (fn, (config, args, stream))
-            else:
-                fn(config, args, stream)
-        elif op in _PLACEHOLDER_ID:
-            parked = act.get("_parked", {}).pop(_PLACEHOLDER_ID[op], None)
-            if parked is not None:
-                fn, (cfg, args, _) = parked
-                fn(cfg, args, stream)
-        elif op == 21:
-            output = dcfunc.swiglu_bwd(config, (g("swiglu_input"), x), stream)
-            act["swiglu_dgrad"] = output
-        elif op == 22:
-            output, act["mlp_residual_bwd"] = dcfunc.bda_mlp_bwd(config, (x, act.get("mlp_mask")), stream)
-        elif op == 23:
-            output, act["attn_residual_bwd"] = dcfunc.bda_attn_bwd(config, (x, act.get("attn_mask")), stream)
-        elif op == 24:
-            output = dcfunc.attn_bwd(config, (x, g("q_padded"), g("k_padded"), g("v_padded"), g("out_padded"),
-                                              g("softmax_lse"), weight["cu_seqlens_q"], weight["cu_seqlens_kv"],
-                                              act.get("rng_state")), stream,
-                                     apply_rope=config.groups_per_rank != 1)
-        elif op == 32:
-            output = dcfunc.rope_bwd(config, (x,), stream)
-        elif op == 29:
-            last = (0 if isinstance(x, torch.Tensor) else x[7]) == config.context_parallel_size - 1
-            visiting = act.get("cp_kv_chunks")
-            if visiting is not None:
-                for t in visiting:
-                    _use(t, stream)
-            output = dcfunc.ring_attn_fwd(config, (x, weight["cu_seqlens_q"], weight["cu_seqlens_kv"],
-                                                   weight.get("rope_positions"), visiting), stream)
-            if last:
-                output, act["q"], act["kv"], act["softmax_lse"], act["rng_states"] = output
-                act["out"] = output
-        elif op == 30:
-            last = (0 if isinstance(x, torch.Tensor) else x[4]) == config.context_parallel_size
-            for t in act["kv"]:
-                _use(t, stream)
-            output = dcfunc.ring_attn_bwd(config, (x, g("out"), g("q"), act["kv"], g("softmax_lse"), act.get("rng_states"),
-                                                   weight["cu_seqlens_q"], weight["cu_seqlens_kv"],
-                                                   weight.get("rope_positions")), stream)
-            if last:
-                for key in ("out", "q", "kv", "softmax_lse", "rng_states"):
-                    act.pop(key, None)
-                act["attn_dgrad"] = output
-        elif op in (25, 26):
-            p = "mlp" if op == 25 else "attn"
-            lw, lb = weight[f"ln_{p}_weight"], weight.get(f"ln_{p}_bias")
-            mu = act.get(f"{p}_mu")
-            data = (x, g(f"ln_{p}_input"), _use(mu, stream), g(f"{p}_rsigma"), lw, lb, g(f"{p}_residual_bwd"),
-                    lw.main_grad, lb.main_grad if lb is not None else None)
-            output = (dcfunc.ln_mlp_bwd if op == 25 else dcfunc.ln_attn_bwd)(config, data, stream)
-        else:
+        handler = _HANDLERS.get(op)
+        if handler is None:
             raise ValueError(f"operation {op} is not part of the single-GPU decoder-layer path")
-
-        if op == 18:
-            act.pop("attn_dgrad", None)          # kept by the last ring call for the qkv weight gradient
+        output = handler(_Ctx(dcfunc, op, config, weight, activation_dict, kwargs.get("output"), kwargs["stream"],
+                              kwargs.get("name"), kwargs.get("movable", ())))
         for key in _FREE_AFTER.get(op, ()):
-            act.pop(key, None)
+            activation_dict.pop(key, None)
         return output
 
 
@@ -933,3 +1017,85 @@ def exec(config, dcoperation, fwd_weight, bwd_weight, input, grad_output, dcbloc
 
 
 exec_plan = exec
+
+
+class DSTB_(torch.autograd.Function):
+    """One module of the folded model (dstb.py:1294-1366).  The model is walked twice per micro-batch: the
+    forward traversal calls ``forward`` (the module's FIRST layer takes the new micro-batch forward, its SECOND
+    layer takes the previous micro-batch backward), the autograd traversal that follows calls ``backward`` with
+    the two weight sets exchanged.  Inputs and results travel through ``GLOBAL_VARIABLES['inputs']`` =
+    [backward strand's gradient, forward strand's hidden states]; activation dicts are pushed on the stack of
+    the micro-batch that made them and popped by the traversal that differentiates them."""
+
+    @staticmethod
+    def _walk(config, fwd_weight, bwd_weight, plan, stream1, stream2, push_to, pop_from):
+        bwd_input, fwd_input = GLOBAL_VARIABLES['inputs']
+        new_act = {}
+        if bwd_input is None:                               # only the new micro-batch: forward
+            fwd_result, _ = exec(config, DCoperation, fwd_weight, None, fwd_input, None, plan.fwd_only, stream1,
+                                 stream2, None, new_act, movable=plan.movable)
+            GLOBAL_VARIABLES[push_to][-1].push(new_act)
+            GLOBAL_VARIABLES['inputs'] = [None, fwd_result]
+            return
+        act = GLOBAL_VARIABLES[pop_from][0].pop()           # activations of the previous micro-batch
+        if GLOBAL_VARIABLES[pop_from][0].is_empty():
+            GLOBAL_VARIABLES[pop_from].pop(0)
+        if fwd_input is None:                               # only the previous micro-batch: backward
+            _, bwd_result = exec(config, DCoperation, None, bwd_weight, None, bwd_input, plan.bwd_only, stream1,
+                                 stream2, act, None, movable=plan.movable)
+            GLOBAL_VARIABLES['inputs'] = [bwd_result, None]
+            return
+        fwd_result, bwd_result = exec(config, DCoperation, fwd_weight, bwd_weight, fwd_input, bwd_input,
+                                      plan.dcblocks, stream1, stream2, act, new_act, movable=plan.movable)
+        GLOBAL_VARIABLES[push_to][-1].push(new_act)
+        GLOBAL_VARIABLES['inputs'] = [bwd_result, fwd_result]
+
+    @staticmethod
+    def forward(ctx, placeholder, config, bwd_weight, fwd_weight, plan, stream1, stream2):
+        ctx.args = (config, fwd_weight, bwd_weight, plan, stream1, stream2)
+        with torch.no_grad():
+            DSTB_._walk(config, fwd_weight, bwd_weight, plan, stream1, stream2, 'fwd_activations', 'bwd_activations')
+        return placeholder.view_as(placeholder)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        config, fwd_weight, bwd_weight, plan, stream1, stream2 = ctx.args
+        with torch.no_grad():                               # the two weight sets change places (dstb.py:1333-1335)
+            DSTB_._walk(config, bwd_weight, fwd_weight, plan, stream1, stream2, 'bwd_activations', 'fwd_activations')
+        return grads[0], None, None, None, None, None, None
+
+
+_DSTB_WEIGHTS = ("ln_attn_weight", "column_attn_weight", "linear_attn_weight", "ln_mlp_weight", "column_mlp_weight",
+                 "linear_mlp_weight")
+
+
+class DSTB(torch.nn.Module):
+    """Two decoder layers in one module (dstb.py:1368-1468): ``*_first`` is the layer the forward traversal runs,
+    ``*_second`` the one the autograd traversal runs, so a model of n such modules is the 2n-layer network
+    first_0 .. first_{n-1}, second_{n-1} .. second_0.  Parameters are ``torch.nn.Parameter`` with a ``main_grad``
+    buffer each (Megatron's distributed optimizer provides it in the reference)."""
+
+    def __init__(self, config: LayerConfig, stream1, stream2, plan=None, seed: int = 0, device="cuda"):
+        super().__init__()
+        from .layer import make_weights
+        self.config, self.stream1, self.stream2 = config, stream1, stream2
+        self.weight_first, self.weight_second = {}, {}
+        for tag, wd, sd in (("first", self.weight_first, seed), ("second", self.weight_second, seed + 1)):
+            w = make_weights(config, sd, device)
+            names = _DSTB_WEIGHTS + (("ln_attn_bias", "ln_mlp_bias") if config.layernorm_bias else ())
+            for k in names:
+                p = torch.nn.Parameter(w[k])
+                p.main_grad = torch.zeros_like(w[k])
+                if k.startswith("ln_"):
+                    p.sequence_parallel = config.tensor_model_parallel_size > 1
+                setattr(self, f"{k}_{tag}", p)
+                wd[k] = p
+            for k in ("cu_seqlens_q", "cu_seqlens_kv", "rope_positions"):
+                if k in w:
+                    wd[k] = w[k]
+        self.plan = init_DCBlocks(plan, stream1, stream2, config.context_parallel_size)
+        self.dcblocks, self.fwd_only_dcblocks, self.bwd_only_dcblocks = self.plan
+
+    def forward(self, inputs):
+        return DSTB_.apply(inputs, self.config, self.weight_second, self.weight_first, self.plan, self.stream1,
+                           self.stream2)

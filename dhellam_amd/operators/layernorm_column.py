@@ -51,6 +51,13 @@ def gemm_fwd(args, input: torch.Tensor, weight: torch.Tensor, output: Optional[t
     return output, el[0]
 
 
+def gemm_fwd_event(args, input: torch.Tensor, weight: torch.Tensor, output: Optional[torch.Tensor] = None,
+                   layout: str = "TN", profiling: bool = False, math_sm_count: int = 0, is_matmul: bool = False):
+    """layernorm_column.py:64-119: ``gemm_fwd`` on the current stream (the reference's variant without a
+    ``stream`` argument, timed with events like every operator here)."""
+    return gemm_fwd(args, input, weight, output, layout, profiling, math_sm_count, is_matmul, None)
+
+
 def dgrad_bwd(args, input_grad: torch.Tensor, weight: torch.Tensor, dgrad_output: Optional[torch.Tensor],
               layout: str = "NN", profiling: bool = False, math_sm_count: int = 0, is_matmul: bool = False,
               stream=None):

@@ -59,7 +59,7 @@ def test_version_and_error_string_without_gpu():
 
 def test_product_does_not_import_the_oracle():
     """Nothing under dhellam_amd/ may import, read or run the oracle (it is the checker)."""
-    for dirpath, _, files in os.walk(os.path.join(ROOT, "dhellam_amd")):
+    for dirpath, _, files in list(os.walk(os.path.join(ROOT, "dhellam_amd"))) + list(os.walk(os.path.join(ROOT, "dhellam"))):
         for f in files:
             if f.endswith((".py", ".hip", ".h")):
                 src = open(os.path.join(dirpath, f)).read()

@@ -345,3 +345,38 @@ def test_dense_gemm_on_two_streams():
         torch.cuda.synchronize()
         assert torch.equal(y, y_ref) and torch.equal(y2, y2_ref)
     assert len({k for k in _Clib._gemm_ws if k[1] in (s1.cuda_stream, s2.cuda_stream)}) == 2
+
+
+def test_math_sm_count_confines_a_launch_to_that_many_compute_units():
+    """``math_sm_count`` of the reference's bindings (libsmctrl mask, csrc/operators/gemm.cu:20-21,66-70,108;
+    flash_atten.cu:248-249,407) maps to a stream with a compute-unit mask: same bits as the unconfined launch, a
+    longer run on a sixteenth of the GPU, negative counts take the units from the other end, counts beyond the
+    device are refused."""
+    from dhellam_amd import _Clib
+    n_cus = torch.cuda.get_device_properties(0).multi_processor_count
+    dt = torch.bfloat16
+    a, b = randn((2048, 4096), dt, 1, 0.1).cuda(), randn((4096, 4096), dt, 2, 0.1).cuda()     # weight [N, K], input [T, K]
+    outs, ms = [], []
+    for count in (0, n_cus // 16, -(n_cus // 16)):
+        d = torch.empty((4096, 2048), dtype=dt, device="cuda")
+        _Clib.pygemm(a, b, d, None, 0, True, False, False, count, False)                       # warm-up (stream creation)
+        t = [_Clib.pygemm(a, b, d, None, 0, True, False, False, count, True) for _ in range(5)]
+        outs.append(d)
+        ms.append(sorted(t)[2])
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert ms[1] > 3 * ms[0] and ms[2] > 3 * ms[0], ms
+    with pytest.raises(RuntimeError):
+        _Clib.pygemm(a, b, outs[0], None, 0, True, False, False, n_cus + 1, False)
+    # attention forward and backward on a quarter of the GPU: same bits
+    T, hq, hk, dd = 1024, 8, 2, 128
+    q, k, v, do = (randn((T, h, dd), dt, s).cuda() for h, s in ((hq, 3), (hk, 4), (hk, 5), (hq, 6)))
+    cu = torch.tensor([0, T], dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    res = []
+    for count in (0, n_cus // 4):
+        r = _Clib.pymha_varlen_fwd(q, k, v, cu, cu, T, T, 0.0, dd ** -0.5, True, False, count, False)
+        g = _Clib.pymha_varlen_bwd(do, q, k, v, r[0], r[5], cu, cu, T, T, 0.0, dd ** -0.5, True, None, False, count, False, st)
+        torch.cuda.synchronize()
+        res.append([r[0], r[5]] + g[:4])
+    for x, y in zip(*res):
+        assert torch.equal(x, y)

@@ -228,10 +228,12 @@ def test_cu_partitioned_streams():
     cfg = LayerConfig(hidden_size=512, num_attention_heads=8, num_query_groups=4, ffn_hidden_size=1024, seq_length=256,
                       micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
                       params_dtype=torch.bfloat16, comm_standin_us=30.0)
-    with partitioned_streams(reserved_per_xcd=1) as ((c1, c2), comm):
-        _partitioned_checks(cfg, c1, c2, comm, lib)
     from dhellam_amd.common import streams as S
-    assert not S._LIVE, "the partition's streams are ended with the block"
+    before = set(S._LIVE)              # masked streams other tests made and keep (math_sm_count caches them)
+    with partitioned_streams(reserved_per_xcd=1) as ((c1, c2), comm):
+        assert len(S._LIVE) == len(before) + 4
+        _partitioned_checks(cfg, c1, c2, comm, lib)
+    assert S._LIVE == before, "the partition's streams are ended with the block"
 
 
 def _partitioned_checks(cfg, c1, c2, comm, lib):

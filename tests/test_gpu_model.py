@@ -42,13 +42,13 @@ def _floats(w):
 
 
 def test_model_step_matches_oracle_and_schedules_agree():
-    from dhellam_amd.core.dsllm import DSLLM
+    from dhellam_amd.core.dsllm import DSLLMStep
     prev = torch.backends.cuda.matmul.allow_tf32
     torch.backends.cuda.matmul.allow_tf32 = False
     try:
         cfg, vocab, L, n = _cfg(torch.float32), 512, 2, 3
         batches = _batches(cfg, vocab, n)
-        model = DSLLM(cfg, L, vocab, seed=3)
+        model = DSLLMStep(cfg, L, vocab, seed=3)
         losses_o, grads_o = OL.model_fwd_bwd(_oracle_cfg(cfg), [_floats(w) for w in model.layers],
                                              model.word_embeddings.cpu(), model.final_ln_weight.cpu(), batches, 8.0)
         losses = model.step(_cuda(batches), double_strand=True, loss_scale=8.0)
@@ -58,7 +58,7 @@ def test_model_step_matches_oracle_and_schedules_agree():
         for name, p in model.named_parameters():
             assert_close(p.main_grad, grads_o[name], torch.float32, name)
         # the serial schedule (one stream, forward then backward per micro-batch) gives the same bits
-        serial = DSLLM(cfg, L, vocab, seed=3)
+        serial = DSLLMStep(cfg, L, vocab, seed=3)
         losses_s = serial.step(_cuda(batches), double_strand=False, loss_scale=8.0)
         torch.cuda.synchronize()
         for a, b in zip(losses, losses_s):
@@ -72,9 +72,9 @@ def test_model_step_matches_oracle_and_schedules_agree():
 def test_model_trains_in_bf16():
     """Predict the token two positions back (needs attention): bf16 parameters and gradients, fp32 master weights
     with Adam on the host side of the loop.  The loss has to fall to a quarter of its starting value ln(vocab)."""
-    from dhellam_amd.core.dsllm import DSLLM
+    from dhellam_amd.core.dsllm import DSLLMStep
     cfg, vocab, L, n = _cfg(torch.bfloat16, hidden=256, heads=4, groups=2, ffn=512, seq=128, batch=4), 256, 2, 2
-    model = DSLLM(cfg, L, vocab, seed=1)
+    model = DSLLMStep(cfg, L, vocab, seed=1)
     params = [p for _, p in model.named_parameters()]
     master = [p.detach().float().clone().requires_grad_() for p in params]
     opt = torch.optim.Adam(master, lr=2e-3)
@@ -107,10 +107,10 @@ def test_model_trains_in_bf16():
 @pytest.mark.parametrize("layers,n_mb", [(1, 1), (1, 2), (3, 1)])
 def test_model_edge_shapes(layers, n_mb):
     """One layer and / or one micro-batch: the paired schedule degenerates to forward-only + backward-only phases."""
-    from dhellam_amd.core.dsllm import DSLLM
+    from dhellam_amd.core.dsllm import DSLLMStep
     cfg, vocab = _cfg(torch.bfloat16, hidden=128, heads=2, groups=1, ffn=256, seq=64, batch=1), 128
     batches = _cuda(_batches(cfg, vocab, n_mb, seed=5))
-    a, b = DSLLM(cfg, layers, vocab, seed=2), DSLLM(cfg, layers, vocab, seed=2)
+    a, b = DSLLMStep(cfg, layers, vocab, seed=2), DSLLMStep(cfg, layers, vocab, seed=2)
     la, lb = a.step(batches, double_strand=True), b.step(batches, double_strand=False)
     torch.cuda.synchronize()
     for x, y in zip(la, lb):
@@ -118,3 +118,48 @@ def test_model_edge_shapes(layers, n_mb):
     for (name, p), (_, q) in zip(a.named_parameters(), b.named_parameters()):
         assert torch.equal(p.main_grad, q.main_grad), name
         assert float(p.main_grad.float().abs().max()) > 0, name
+
+
+@pytest.mark.parametrize("two_streams", [False, True])
+def test_module_shell_matches_the_explicit_schedule_and_the_oracle(two_streams):
+    """The reference's shell -- ``torch.nn.Module``s, autograd functions, a backward pre-hook and activation
+    stacks, driven by ``model(x1, x2)`` + ``.backward()`` per micro-batch -- moves the micro-batches exactly as
+    the explicit schedule does: same losses and parameter gradients, bit for bit, and both match the oracle."""
+    from dhellam_amd.common.global_variables import GLOBAL_VARIABLES
+    from dhellam_amd.core.dsllm import DSLLM, DSLLMStep, run_microbatches
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        cfg, vocab, L, n = _cfg(torch.float32), 512, 4, 3
+        batches = _batches(cfg, vocab, n, seed=5)
+        s1 = torch.cuda.Stream()
+        s2 = torch.cuda.Stream() if two_streams else s1
+        model = DSLLM(cfg, vocab, L, num_mb=n, loss_scale=8.0, seed=3, stream1=s1, stream2=s2)
+        assert isinstance(model, torch.nn.Module) and len(model.dctb) == L // 2
+        names = [k for k, _ in model.named_parameters()]
+        assert "dctb.0.column_attn_weight_first" in names and "dctb.1.linear_mlp_weight_second" in names
+        losses = run_microbatches(model, _cuda(batches))
+        torch.cuda.synchronize()
+        assert not GLOBAL_VARIABLES['fwd_activations'] and not GLOBAL_VARIABLES['bwd_activations']   # every stack consumed
+        step = DSLLMStep(cfg, L, vocab, seed=3)
+        losses_s = step.step(_cuda(batches), double_strand=two_streams, loss_scale=8.0)
+        torch.cuda.synchronize()
+        for a, b in zip(losses, losses_s):
+            assert torch.equal(a, b)
+        assert torch.equal(model.dchb.word_embeddings.main_grad, step.word_embeddings.main_grad)
+        assert torch.equal(model.dchb.ln_weight.main_grad, step.final_ln_weight.main_grad)
+        for l in range(L):
+            for k, p in model.layer_weights(l).items():
+                if hasattr(p, "main_grad"):
+                    assert torch.equal(p, step.layers[l][k]), (l, k)
+                    assert torch.equal(p.main_grad, step.layers[l][k].main_grad), (l, k)
+        losses_o, grads_o = OL.model_fwd_bwd(_oracle_cfg(cfg), [_floats(w) for w in step.layers],
+                                             step.word_embeddings.cpu(), step.final_ln_weight.cpu(), batches, 8.0)
+        for i in range(n):
+            assert_close(losses[i], losses_o[i], torch.float32, f"loss[{i}]")
+        for l in range(L):
+            for k, p in model.layer_weights(l).items():
+                if hasattr(p, "main_grad"):
+                    assert_close(p.main_grad, grads_o[f"layers.{l}.{k}"], torch.float32, f"layers.{l}.{k}")
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev

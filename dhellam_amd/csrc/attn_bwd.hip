@@ -631,8 +631,8 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
             }
             S = M::mma(__builtin_bit_cast(Frag, fk[a]), Qf[ks], S);
             dP = M::mma(__builtin_bit_cast(Frag, fv[a]), dOf[ks], dP);
-            if (CPW == 8 && (ks & 1)) DH_DQ_COPY(ks >> 1);           // copy blocks 0..3
-            if (CPW == 4 && (ks & 3) == 3) DH_DQ_COPY(ks >> 2);      // copy blocks 0..1
+            if (CPW == 8) DH_DQ_COPY(ks);                            // all copy blocks go out in this phase, so
+            if (CPW == 4 && (ks & 1)) DH_DQ_COPY(ks >> 1);           // that they have the rest of the iteration to land
           }
         }
         // dQ^T += K^T dS^T needs K^T fragments (transpose reads of the K tile): those of the first 16-key
@@ -676,13 +676,10 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
           }
           dQt[0] = M::mma(frag_join<T>(g[0], g[1]), dSb[s], dQt[0]);
           dQt[1] = M::mma(frag_join<T>(g[2], g[3]), dSb[s], dQt[1]);
-          if (CPW == 8) DH_DQ_COPY(4 + 2 * s);
           if (s + 1 < NS) lds_wait<8>(g[4], g[5], g[6], g[7]);
           else lds_wait<0>(g[4], g[5], g[6], g[7]);
           dQt[2] = M::mma(frag_join<T>(g[4], g[5]), dSb[s], dQt[2]);
           dQt[3] = M::mma(frag_join<T>(g[6], g[7]), dSb[s], dQt[3]);
-          if (CPW == 8) DH_DQ_COPY(5 + 2 * s);
-          else DH_DQ_COPY(2 + s);
         }
       } else {
 #pragma unroll
@@ -956,6 +953,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
             S = M::mma(fq[cb], fk[cb], S);
             dP = M::mma(fo[cb], fv[cb], dP);
             __builtin_amdgcn_sched_barrier(0);
+            DH_DKV_COPY(ks);                          // one copy block per step: all eight are out before the softmax
           }
         }
         if ((causal && i0 < jw0 + 31) || (i0 + BM > sq)) {
@@ -1008,7 +1006,6 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
             if (which == 0) dVt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), Pb[sx], dVt[t]);
             else dKt[t] = M::mma(frag_join<T>(x0[cb], x1[cb]), dSb[sx], dKt[t]);
             __builtin_amdgcn_sched_barrier(0);
-            if (u & 1) DH_DKV_COPY(u >> 1);
           }
         }
       } else {

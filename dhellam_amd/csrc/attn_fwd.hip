@@ -361,7 +361,8 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
       }                                                                                                 \
     } while (0)
 
-    // O^T += V^T P^T for the tile in V slot `vs`; copy blocks 4..7 go out between the MFMAs.
+    // O^T += V^T P^T for the tile in V slot `vs`; the wavefront's eight copy blocks go out between the MFMAs
+    // of this phase, the first of the iteration, so that they have the rest of it to land.
     auto pv = [&](int vs) {
       uint32_t va = ldsV + (uint32_t)(vs * SLOTB) + va_lane, vb = ldsV + (uint32_t)(vs * SLOTB) + vb_lane;
       asm volatile("" : "+v"(va), "+v"(vb));     // derive the other addresses here, not ahead of the loop
@@ -390,17 +391,18 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
         }
         O[0] = M::mma(frag_join<T>(g[0], g[1]), Pb[s], O[0]);
         O[1] = M::mma(frag_join<T>(g[2], g[3]), Pb[s], O[1]);
-        if (NS == 2) DH_FWD_COPY(4 + 2 * s);
+        if (NS == 2) { DH_FWD_COPY(4 * s); DH_FWD_COPY(4 * s + 1); }
+        else DH_FWD_COPY(2 * s);
         if (s + 1 < NS) lds_wait<8>(g[4], g[5], g[6], g[7]);
         else lds_wait<0>(g[4], g[5], g[6], g[7]);
         O[2] = M::mma(frag_join<T>(g[4], g[5]), Pb[s], O[2]);
         O[3] = M::mma(frag_join<T>(g[6], g[7]), Pb[s], O[3]);
-        if (NS == 2) DH_FWD_COPY(5 + 2 * s);
-        else DH_FWD_COPY(4 + s);
+        if (NS == 2) { DH_FWD_COPY(4 * s + 2); DH_FWD_COPY(4 * s + 3); }
+        else DH_FWD_COPY(2 * s + 1);
       }
     };
 
-    // S^T = K Q^T for this wavefront's tile of the current iteration; copy blocks 0..3 go out between the MFMAs.
+    // S^T = K Q^T for this wavefront's tile of the current iteration.
     floatx16 S[NB];
     auto qk = [&](uint32_t k_slot) {
       uint32_t kb = k_slot + kb_lane;
@@ -435,7 +437,6 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
         else lds_wait<6>(ka[a], ka[a + 1]);
         S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a]), Qf[ks], S[nb]);
         S[nb] = M::mma(__builtin_bit_cast(Frag, ka[a + 1]), Qf[ks + 1], S[nb]);
-        if (pr % NB == NB - 1) DH_FWD_COPY(pr / NB);      // copy blocks 0..3
       }
     };
 
@@ -509,9 +510,8 @@ __global__ void __launch_bounds__(512) attn_fwd_d128_kernel(const AttnFwdParams 
 
       if (lag && act_prev) softmax(n0_prev);
       if (act_prev) pv(v_prev);
-      else { DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
+      else { DH_FWD_COPY(0); DH_FWD_COPY(1); DH_FWD_COPY(2); DH_FWD_COPY(3); DH_FWD_COPY(4); DH_FWD_COPY(5); DH_FWD_COPY(6); DH_FWD_COPY(7); }
       if (act) qk(k_cur);
-      else { DH_FWD_COPY(0); DH_FWD_COPY(1); DH_FWD_COPY(2); DH_FWD_COPY(3); }
       if (!lag && act) softmax(n0);
 
       act_prev = act;

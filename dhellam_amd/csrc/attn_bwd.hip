@@ -2,7 +2,8 @@
 // floating-point atomics).
 //
 // Three kernels:
-//   delta   : delta_i = sum_d dO[i,d] * O[i,d]                      (streaming)
+//   delta   : delta_i = sum_d dO[i,d] * O[i,d]                      (streaming; head dim 64 only: the
+//             head dim 128 dQ kernel forms delta in its prologue and runs first)
 //   dK/dV   : a workgroup owns 64 key/value rows (K, V fragments stay in
 //             registers for head dim 64, in LDS for head dim 128), walks the
 //             query heads of its GQA group and the query tiles that attend to
@@ -25,8 +26,11 @@ namespace dh {
 
 struct AttnBwdParams {
   const void *dout, *q, *k, *v;
-  const float *lse, *delta;
-  const float *ld2;          // fp32 [2][plane]: lse * log2(e), then delta, each [batch][hq][ld2_pitch] (d = 128 kernels)
+  const void *out;           // forward output (d = 128: the dQ kernel forms delta from it)
+  int64_t o_stride;
+  const float *lse;
+  float *delta;              // fp32 [batch][hq][max_sq]: rowsum(dO * O); written by the delta kernel, or (d = 128) by the dQ kernel
+  float *ld2;                // fp32 [2][plane]: lse * log2(e), then delta, each [batch][hq][ld2_pitch] (d = 128 kernels)
   int64_t ld2_plane;         // elements between the two planes
   int ld2_pitch;             // max_sq rounded up to 32: every 32-row query tile of a head is one aligned 128-byte run
   void *dq, *dk, *dv;
@@ -482,6 +486,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
   constexpr int CPW = SPLIT * 2 * BPT / 8;        // copy blocks per wavefront and iteration (4 or 8)
   static_assert(CPW == 4 || CPW == 8, "copy blocks per wavefront");
   __shared__ __attribute__((aligned(1024))) T sAll[4 * SLOT];   // K slots 0..1, V slots 0..1
+  __shared__ float sDel[RG * 32];                               // delta of the workgroup's rows
 
   const int b = blockIdx.y;
   // the query heads of one kv head read the same K / V rows: keep a kv head on one XCD's L2
@@ -558,7 +563,33 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
       }
     }
     const float lse_c = row_ok ? p.lse[((int64_t)b * p.hq + h) * p.max_sq + row_q] * 1.4426950408889634f : INFINITY;
-    const float del_c = row_ok ? p.delta[((int64_t)b * p.hq + h) * p.max_sq + row_q] : 0.f;
+    // delta = rowsum(dO * O) of this lane's row, formed by the first key split of each row group: the lane holds
+    // one half of the row's dO (its k-step chunks), reads the same chunks of O, and the two halves meet through
+    // the partner lane.  The other splits get it through LDS after the barrier that publishes the first tiles.
+    // Split 0 also writes it out, together with the copy the dK/dV kernel streams (lse in exp2 units next to
+    // delta, zeros in the rows that pad the last 32-row tile), so that no separate pass over dO and O is
+    // needed.  The dK/dV kernel therefore runs after this one.
+    float del_c = 0.f;
+    if (sp == 0) {
+      const T *op = reinterpret_cast<const T *>(p.out) + (int64_t)(q0 + row_ld) * p.o_stride + (int64_t)h * D;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const Frag of = frag_ld<T>(op + ks * 16 + 8 * hh);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) del_c += to_f(dOf[ks][j]) * to_f(of[j]);
+      }
+      del_c += __shfl_xor(del_c, 32, 64);
+      if (!row_ok) del_c = 0.f;
+      if (hh == 0) {
+        sDel[rg * 32 + c] = del_c;
+        if (row_ok) p.delta[((int64_t)b * p.hq + h) * p.max_sq + row_q] = del_c;
+        if (row_q < p.ld2_pitch) {
+          const int64_t a2 = ((int64_t)b * p.hq + h) * p.ld2_pitch + row_q;
+          p.ld2[a2] = row_ok ? lse_c : 0.f;
+          p.ld2[p.ld2_plane + a2] = del_c;
+        }
+      }
+    }
     int nk_end = sk;
     if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
     const int ntiles = (nk_end + BN - 1) / BN;
@@ -575,6 +606,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
       dma_tile32_general<T, CPW>(sAll + (cp_v ? 2 * SLOT : 0) + cp_dst0, cp_gt, cp_stride, 1, cp_tile * BN + cp_r0, cp_r0, sk, cl0);
     dma_wait_all();
     __syncthreads();
+    del_c = sDel[rg * 32 + c];
 
     const char *cp_src = nullptr;
     uint32_t cp_dst = 0;
@@ -1218,7 +1250,9 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   DH_CHECK(d % n == 0 || dtype == DH_F32, "head dim %d must be a multiple of %d", d, n);
   DH_CHECK(do_stride % n == 0 && o_stride % n == 0 && aligned16(dout) && aligned16(out),
            "dout/out rows must be 16-byte aligned");
-  if (max_seqlen_q > 0) {
+  // head dim 128 in 16 bits: the dQ kernel forms delta itself (and runs first); everything else uses the delta kernel
+  const bool delta_in_dq = dtype != DH_F32 && d == 128;
+  if (max_seqlen_q > 0 && !delta_in_dq) {
     DH_DISPATCH_DTYPE(dtype, {
       launch_delta<T>(dout, out, delta, lse, ld2, (int64_t)(plane2 / sizeof(float)), ld2_pitch, cu_seqlens_q, batch, max_seqlen_q, hq, d,
                       do_stride, o_stride, st);
@@ -1238,6 +1272,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
            "pointers must be 16-byte aligned");
   AttnBwdParams p;
   p.dout = dout; p.q = q; p.k = k; p.v = v; p.lse = lse; p.delta = delta;
+  p.out = out; p.o_stride = o_stride;
   p.ld2 = ld2; p.ld2_plane = (int64_t)(plane2 / sizeof(float)); p.ld2_pitch = ld2_pitch;
   p.dq = dq; p.dk = dk; p.dv = dv;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
@@ -1263,7 +1298,9 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   int rc = DH_OK;
 #define DH_BWD(TT, DD)                                                                         \
   do {                                                                                         \
-    if (max_seqlen_k > 0)                                                                      \
+    if (DD == 128 && max_seqlen_q > 0)                                                         \
+      rc = big_q ? launch_dq_d128<TT, 4, 2, 32>(p, batch, st) : launch_dq_d128<TT, 2, 4, 32>(p, batch, st); \
+    if (rc == DH_OK && max_seqlen_k > 0)                                                       \
       rc = DD == 128 ? launch_dkv_d128<TT>(p, batch, max_seqlen_k, st) : launch_dkv<TT, DD, DKV_NW>(p, batch, max_seqlen_k, st); \
     if (rc == DH_OK && p.hsplit > 1 && total_k > 0) {                                          \
       int64_t blocks = cdiv(total_k * hk * (DD / 4), 256);                                     \
@@ -1271,10 +1308,8 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
       hipLaunchKernelGGL((attn_bwd_gqa_sum_kernel<TT>), dim3((unsigned)blocks), dim3(256), 0, st, p.dk_part, \
                          p.dv_part, (TT *)dk, (TT *)dv, total_k, hk, DD, p.hsplit, dk_stride, dv_stride);    \
     }                                                                                          \
-    if (rc == DH_OK && max_seqlen_q > 0) {                                                     \
-      if (DD == 128) rc = big_q ? launch_dq_d128<TT, 4, 2, 32>(p, batch, st) : launch_dq_d128<TT, 2, 4, 32>(p, batch, st); \
-      else rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st); \
-    }                                                                                          \
+    if (rc == DH_OK && max_seqlen_q > 0 && DD != 128)                                          \
+      rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st);  \
   } while (0)
   if (dtype == DH_BF16) {
     if (d == 128) DH_BWD(bf16_t, 128); else DH_BWD(bf16_t, 64);

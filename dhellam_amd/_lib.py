@@ -37,6 +37,7 @@ SIGNATURES = {
     "dh_masked_mean_fwd": (_i32, [_vp, _vp, _i64, _f32, _vp, _vp]),
     "dh_masked_mean_bwd": (_i32, [_vp, _vp, _i64, _f32, _vp, _vp]),
     "dh_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _vp]),
+    "dh_add_norm_fwd": (_i32, [_vp] * 8 + [_i64, _i64, _f32, _i32, _i32, _vp]),
     "dh_norm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "dh_norm_bwd": (_i32, [_vp] * 10 + [_i64, _i64, _i32, _i32, _i32, _vp]),
     "dh_swiglu_fwd": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp]),

@@ -118,6 +118,7 @@ class LayerConfig:
     # (forward strand's, backward strand's) communication streams: the stand-ins' delays run there, with events
     # to and from the strand's own stream, instead of on the strand's stream itself
     comm_streams: Optional[tuple] = None
+    fuse_adjacent: bool = True        # ops a plan lists next to each other run as one kernel where one exists (bda_attn + ln_mlp)
 
     @property
     def head_dim(self) -> int:
@@ -189,6 +190,18 @@ class DCFunc:
         return output, mu, rsigma, inputmat, input, output
 
     ln_mlp = ln_attn
+
+    @staticmethod
+    def bda_attn_ln_mlp(config, data, stream):
+        """``bda_attn`` and ``ln_mlp`` (dstb.py:273-277, 73-78), adjacent in the layer, in one kernel: the residual
+        sum is written once and normalised from registers.  Returns (ln output, mu, rsigma, norm input as a
+        matrix, the residual sum in the layer's [b, s/tp, h] shape)."""
+        input, residual, ln_weight, ln_bias = data
+        input = input.view(config.micro_batch_size, config.seq_length // config.tensor_model_parallel_size, -1)
+        output, mu, rsigma, _, x2 = pylayernorm_fwd(input, ln_weight, ln_bias, config.layernorm_epsilon, 0, False,
+                                                    stream, profiling=False, residual=residual)
+        x2 = x2.view(input.shape)
+        return output.view(-1, ln_weight.numel()), mu, rsigma, x2.view(-1, ln_weight.numel()), x2
 
     @staticmethod
     def gemm_attn_column(config, data, stream):
@@ -646,6 +659,20 @@ def _h_norm_bwd(c):
     return (c.dcfunc.ln_mlp_bwd if c.op == 25 else c.dcfunc.ln_attn_bwd)(c.config, data, c.stream)
 
 
+def _h_bda_attn_ln_mlp(c):
+    """bda_attn followed by ln_mlp in one column of a plan: what the two handlers would save, from one kernel."""
+    act = c.act
+    output, act["mlp_mu"], act["mlp_rsigma"], act["ln_mlp_input"], act["ln_mlp_residual"] = c.dcfunc.bda_attn_ln_mlp(
+        c.config, (c.x, c.g("ln_attn_residual"), c.weight["ln_mlp_weight"], c.weight.get("ln_mlp_bias")), c.stream)
+    act["attn_mask"] = None
+    act.pop("ln_attn_residual", None)
+    return output
+
+
+# (name, name of the op that follows it in the same column) -> handler that runs both
+_FUSED = {("bda_attn", "ln_mlp"): _h_bda_attn_ln_mlp}
+
+
 # op id -> handler (the reference: one ``if operation == N`` after another, dstb.py:431-657)
 _HANDLERS = {
     1: _h_norm, 2: _h_norm, 3: _h_gemm_attn_c, 4: _h_gemm_attn_l, 5: _h_gemm_mlp_c, 6: _h_gemm_mlp_l, 7: _h_attn,
@@ -661,6 +688,14 @@ _HANDLERS = {
 class DCoperation:
     """Dispatch one op id: fetch its inputs (previous op's output, weights, saved
     activations), run the adapter, save / free activations (dstb.py:427-660)."""
+
+    @staticmethod
+    def perform_fused(dcfunc, names, config, weight, activation_dict, **kwargs):
+        """Two ops that a plan lists next to each other in one column, run as one kernel (the plan keeps both
+        names; the result is what running them one after the other gives, bit for bit)."""
+        handler = _FUSED[tuple(names)]
+        return handler(_Ctx(dcfunc, None, config, weight, activation_dict, kwargs.get("output"), kwargs["stream"],
+                            names[0], kwargs.get("movable", ())))
 
     @staticmethod
     def perform_operation(dcfunc, operation, config, weight, activation_dict, **kwargs):
@@ -932,10 +967,31 @@ def init_DCBlocks(config=None, stream1=None, stream2=None, context_parallel_size
 
 
 def _run_column(col, dcoperation, config, weight, act, first_input, stream_of, result, movable):
-    for now_op in col:
+    skip = False
+    for idx, now_op in enumerate(col):
+        if skip:                    # ran together with the op before it
+            skip = False
+            continue
         src = now_op.get_output()
         inp = first_input if src is None else src
         st = stream_of(now_op)
+        nxt_in_col = col[idx + 1] if idx + 1 < len(col) else None
+        if (nxt_in_col is not None and (now_op.name, nxt_in_col.name) in _FUSED and getattr(config, "fuse_adjacent", True)
+                and hasattr(dcoperation, "perform_fused") and nxt_in_col in now_op.get_next_op()):
+            output = dcoperation.perform_fused(DCFunc, (now_op.name, nxt_in_col.name), config, weight, act, output=inp,
+                                               stream=st, movable=movable)
+            now_op.set_output(None)
+            now_op = nxt_in_col         # successors and result bookkeeping are those of the second op
+            skip = True
+            handle = None
+            now_op.set_output(None)
+            nxt = now_op.get_next_op()
+            if output is not None and len(nxt) == 0:
+                result[0] = output
+            for nop in nxt:
+                nop.set_output(output)
+                nop.set_handle(handle)
+            continue
         output = dcoperation.perform_operation(DCFunc, now_op.get_op_num(), config, weight, act, output=inp, stream=st,
                                                name=now_op.name, movable=movable)
         handle = None

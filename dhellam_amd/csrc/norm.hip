@@ -14,7 +14,8 @@ namespace dh {
 
 template <typename T, int BT, int TPR, int VPT, bool LN, bool NT>
 __global__ void __launch_bounds__(BT)
-norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *__restrict__ beta,
+norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ residual, T *__restrict__ sum_out,
+                const T *__restrict__ gamma, const T *__restrict__ beta,
                 T *__restrict__ y, float *__restrict__ mu_out, float *__restrict__ rs_out, int64_t rows,
                 int cols, float eps, float gamma_shift) {
   constexpr int N = Vec<T>::N;
@@ -46,6 +47,14 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
       const int v = lane + i * TPR;
       if (active && v < nvec) {
         xv[i] = ldg_s<NT>(xr + (int64_t)v * N);
+        if (residual) {
+          // the row that is normalised is x + residual, rounded to the storage type and written out: what a
+          // separate residual-add kernel in front of the norm would have stored and this one read back
+          const Vec<T> rv = ldg_s<NT>(residual + row * cols + (int64_t)v * N);
+#pragma unroll
+          for (int j = 0; j < N; ++j) xv[i].v[j] = from_f<T>(to_f(xv[i].v[j]) + to_f(rv.v[j]));
+          stg_s<NT>(sum_out + row * cols + (int64_t)v * N, xv[i]);
+        }
 #pragma unroll
         for (int j = 0; j < N; ++j) {
           const float f = to_f(xv[i].v[j]);
@@ -104,13 +113,19 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *_
 // Any cols / alignment: one block per row, scalar accesses, row re-read from cache.
 template <typename T, bool LN>
 __global__ void __launch_bounds__(256)
-norm_fwd_generic_kernel(const T *__restrict__ x, const T *__restrict__ gamma, const T *__restrict__ beta,
+norm_fwd_generic_kernel(const T *__restrict__ x, const T *__restrict__ residual, T *__restrict__ sum_out,
+                        const T *__restrict__ gamma, const T *__restrict__ beta,
                         T *__restrict__ y, float *__restrict__ mu_out, float *__restrict__ rs_out,
                         int64_t rows, int64_t cols, float eps, float gamma_shift) {
   __shared__ float red[4];
   const float inv_cols = 1.0f / (float)cols;
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const T *xr = x + row * cols;
+    if (residual) {     // x + residual first, stored; every thread re-reads only the columns it wrote itself
+      T *sr = sum_out + row * cols;
+      for (int64_t c = threadIdx.x; c < cols; c += 256) sr[c] = from_f<T>(to_f(xr[c]) + to_f(residual[row * cols + c]));
+      xr = sr;
+    }
     float mean = 0.f;
     if (LN) {
       float s = 0.f;
@@ -486,21 +501,21 @@ static int64_t bwd_blocks(int64_t rows, int64_t cols, int elt) {
 }
 
 template <typename T, bool LN>
-static int launch_fwd(const NormPlan &p, const T *x, const T *gamma, const T *beta, T *y, float *mu, float *rs,
-                      int64_t rows, int64_t cols, float eps, float shift, hipStream_t st) {
+static int launch_fwd(const NormPlan &p, const T *x, const T *residual, T *sum_out, const T *gamma, const T *beta, T *y,
+                      float *mu, float *rs, int64_t rows, int64_t cols, float eps, float shift, hipStream_t st) {
   if (!p.vec) {
     int64_t nb = rows < 4096 ? rows : 4096;
-    hipLaunchKernelGGL((norm_fwd_generic_kernel<T, LN>), dim3((unsigned)nb), dim3(256), 0, st, x, gamma, beta, y,
-                       mu, rs, rows, cols, eps, shift);
+    hipLaunchKernelGGL((norm_fwd_generic_kernel<T, LN>), dim3((unsigned)nb), dim3(256), 0, st, x, residual, sum_out,
+                       gamma, beta, y, mu, rs, rows, cols, eps, shift);
     return 0;
   }
   const int rpb = p.tpr == 64 ? 4 : 1;
   int64_t nb = cdiv(rows, rpb);
   if (nb > 256 * 16) nb = 256 * 16;
-  const bool nt = stream_hint(2 * rows * cols * (int64_t)sizeof(T));
+  const bool nt = stream_hint((residual ? 4 : 2) * rows * cols * (int64_t)sizeof(T));
 #define L2(BT, TPR, VPT, NT)                                                                                 \
-  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT), 0, st, x, gamma,  \
-                     beta, y, mu, rs, rows, (int)cols, eps, shift)
+  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT), 0, st, x, residual, \
+                     sum_out, gamma, beta, y, mu, rs, rows, (int)cols, eps, shift)
 #define L(BT, TPR, VPT)                                                                                      \
   do {                                                                                                       \
     if (nt) L2(BT, TPR, VPT, true); else L2(BT, TPR, VPT, false);                                             \
@@ -560,29 +575,47 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
 
 }  // namespace dh
 
-extern "C" int dh_norm_fwd(const void *x, const void *gamma, const void *beta, void *y, float *mu, float *rsigma,
-                           int64_t rows, int64_t cols, float eps, int zero_centered_gamma, int dtype,
-                           void *stream) {
+static int norm_fwd_entry(const void *x, const void *residual, void *sum_out, const void *gamma, const void *beta,
+                          void *y, float *mu, float *rsigma, int64_t rows, int64_t cols, float eps,
+                          int zero_centered_gamma, int dtype, void *stream) {
   using namespace dh;
   DH_CHECK(rows >= 0 && cols > 0, "bad shape rows=%lld cols=%lld", (long long)rows, (long long)cols);
   if (rows == 0) return DH_OK;
   DH_CHECK(x && gamma && y && rsigma, "null pointer");
+  DH_CHECK((residual == nullptr) == (sum_out == nullptr), "residual and sum_out go together");
   DH_CHECK(beta == nullptr || mu != nullptr, "LayerNorm (beta given) needs a mu output");
   DH_CHECK(cols < (1ll << 31), "cols too large");
-  const bool al = aligned16(x) && aligned16(y) && aligned16(gamma) && (beta == nullptr || aligned16(beta));
+  const bool al = aligned16(x) && aligned16(y) && aligned16(gamma) && (beta == nullptr || aligned16(beta)) &&
+                  (residual == nullptr || (aligned16(residual) && aligned16(sum_out)));
   const float shift = zero_centered_gamma ? 1.0f : 0.0f;
   hipStream_t st = (hipStream_t)stream;
   DH_DISPATCH_DTYPE(dtype, {
     const NormPlan p = norm_plan(cols, sizeof(T), al);
     if (beta)
-      launch_fwd<T, true>(p, (const T *)x, (const T *)gamma, (const T *)beta, (T *)y, mu, rsigma, rows, cols, eps,
-                          shift, st);
+      launch_fwd<T, true>(p, (const T *)x, (const T *)residual, (T *)sum_out, (const T *)gamma, (const T *)beta, (T *)y,
+                          mu, rsigma, rows, cols, eps, shift, st);
     else
-      launch_fwd<T, false>(p, (const T *)x, (const T *)gamma, nullptr, (T *)y, mu, rsigma, rows, cols, eps, shift,
-                           st);
+      launch_fwd<T, false>(p, (const T *)x, (const T *)residual, (T *)sum_out, (const T *)gamma, nullptr, (T *)y, mu,
+                           rsigma, rows, cols, eps, shift, st);
   });
   DH_LAUNCH_CHECK();
   return DH_OK;
+}
+
+extern "C" int dh_norm_fwd(const void *x, const void *gamma, const void *beta, void *y, float *mu, float *rsigma,
+                           int64_t rows, int64_t cols, float eps, int zero_centered_gamma, int dtype,
+                           void *stream) {
+  return norm_fwd_entry(x, nullptr, nullptr, gamma, beta, y, mu, rsigma, rows, cols, eps, zero_centered_gamma, dtype,
+                        stream);
+}
+
+extern "C" int dh_add_norm_fwd(const void *x, const void *residual, void *sum_out, const void *gamma, const void *beta,
+                               void *y, float *mu, float *rsigma, int64_t rows, int64_t cols, float eps,
+                               int zero_centered_gamma, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(rows <= 0 || (residual && sum_out), "null pointer");
+  return norm_fwd_entry(x, residual, sum_out, gamma, beta, y, mu, rsigma, rows, cols, eps, zero_centered_gamma, dtype,
+                        stream);
 }
 
 extern "C" size_t dh_norm_bwd_workspace_bytes(int64_t rows, int64_t cols) {

@@ -25,7 +25,11 @@ def _workspace(nbytes: int, device, stream) -> torch.Tensor:
     return ws
 
 
-def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_gamma, stream, profiling=False):
+def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_gamma, stream, profiling=False,
+                    residual=None, sum_out=None):
+    """Returns (ln_out, mu, rsigma, ms).  Extension over the reference signature: with ``residual`` the row that
+    is normalised is ``inp + residual``, which is also stored in ``sum_out`` (default: a new tensor, returned
+    as a fifth value) -- the reference's bda op and the norm after it (dstb.py:273-277, 73-78) in one pass."""
     in_features = ln_weight.numel()
     assert inp.is_cuda, "dhellam needs a GPU."
     assert inp.shape[-1] == in_features, "LayerNorm not possible"
@@ -38,9 +42,21 @@ def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_g
         ln_out = torch.empty_like(inputmat)
         rsigma = torch.empty(rows, dtype=torch.float32, device=inp.device)
         mu = torch.empty(rows, dtype=torch.float32, device=inp.device) if ln_bias is not None else None
-        _lib.check(lib.dh_norm_fwd(inputmat.data_ptr(), ln_weight.data_ptr(), _lib.ptr(ln_bias), ln_out.data_ptr(),
-                                   _lib.ptr(mu), rsigma.data_ptr(), rows, in_features, float(eps),
-                                   int(bool(zero_centered_gamma)), _lib.dt(inp), st.cuda_stream))
+        if residual is None:
+            _lib.check(lib.dh_norm_fwd(inputmat.data_ptr(), ln_weight.data_ptr(), _lib.ptr(ln_bias), ln_out.data_ptr(),
+                                       _lib.ptr(mu), rsigma.data_ptr(), rows, in_features, float(eps),
+                                       int(bool(zero_centered_gamma)), _lib.dt(inp), st.cuda_stream))
+        else:
+            assert residual.is_contiguous() and residual.numel() == inp.numel() and residual.dtype == inp.dtype
+            if sum_out is None:
+                sum_out = torch.empty_like(residual)
+            assert sum_out.is_contiguous() and sum_out.numel() == inp.numel() and sum_out.dtype == inp.dtype
+            _lib.check(lib.dh_add_norm_fwd(inputmat.data_ptr(), residual.data_ptr(), sum_out.data_ptr(),
+                                           ln_weight.data_ptr(), _lib.ptr(ln_bias), ln_out.data_ptr(), _lib.ptr(mu),
+                                           rsigma.data_ptr(), rows, in_features, float(eps),
+                                           int(bool(zero_centered_gamma)), _lib.dt(inp), st.cuda_stream))
+    if residual is not None:
+        return ln_out.view_as(inp), mu, rsigma, el[0], sum_out
     return ln_out.view_as(inp), mu, rsigma, el[0]
 
 

@@ -52,6 +52,16 @@ int dh_norm_fwd(const void *x, const void *gamma, const void *beta, void *y,
                 float *mu, float *rsigma, int64_t rows, int64_t cols,
                 float eps, int zero_centered_gamma, int dtype, void *stream);
 
+/* The residual add of the reference's bda operator (dhellam/operators/bda.py:3-7 with the dropout mask all ones,
+ * dhellam/core/dstb.py:273-277) and the norm that follows it (dstb.py:73-78) in one pass:
+ * sum_out = x + residual (rounded to `dtype`, exactly what dh_residual_add stores) and y = norm(sum_out).
+ * The two ops are adjacent in the layer (bda_attn, ln_mlp); fused, the sum is not read back from memory and
+ * one launch goes away.  sum_out may alias x or residual. */
+int dh_add_norm_fwd(const void *x, const void *residual, void *sum_out,
+                    const void *gamma, const void *beta, void *y, float *mu,
+                    float *rsigma, int64_t rows, int64_t cols, float eps,
+                    int zero_centered_gamma, int dtype, void *stream);
+
 /* Bytes of fp32 scratch dh_norm_bwd needs for its dgamma/dbeta partial sums. */
 size_t dh_norm_bwd_workspace_bytes(int64_t rows, int64_t cols);
 

@@ -380,3 +380,28 @@ def test_math_sm_count_confines_a_launch_to_that_many_compute_units():
         res.append([r[0], r[5]] + g[:4])
     for x, y in zip(*res):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols,ln", [(512, 8192, False), (37, 1000, True), (300, 4104, False), (64, 16384, True), (5, 99, False)])
+def test_residual_add_fused_into_norm_is_the_two_ops_bit_for_bit(dtype, rows, cols, ln):
+    """dh_add_norm_fwd = the bda residual add followed by the norm: same sum, same normalised rows, same statistics,
+    bit for bit (and therefore the oracle's, at the operators' tolerance)."""
+    from dhellam_amd.operators.bda import bda_fwd
+    from dhellam_amd.operators.layernorm import pylayernorm_fwd
+    x, r = randn((rows, cols), dtype, 1).cuda(), randn((rows, cols), dtype, 2).cuda()
+    g = (1 + 0.1 * randn((cols,), torch.float32, 3)).to(dtype).cuda()
+    b = (0.1 * randn((cols,), torch.float32, 4)).to(dtype).cuda() if ln else None
+    s_ref, _, _ = bda_fwd(x, r, out=torch.empty_like(x))
+    y_ref, mu_ref, rs_ref, _ = pylayernorm_fwd(s_ref, g, b, 1e-5, 0, False, None)
+    y, mu, rs, _, s = pylayernorm_fwd(x, g, b, 1e-5, 0, False, None, residual=r)
+    assert torch.equal(s, s_ref) and torch.equal(y, y_ref) and torch.equal(rs, rs_ref)
+    if ln:
+        assert torch.equal(mu, mu_ref)
+    yo, _, rso = O.norm_fwd(x.cpu().double() + r.cpu().double() if dtype == torch.float32 else s_ref.cpu(), g.cpu(),
+                            b.cpu() if ln else None, 1e-5)
+    assert_close(y, yo, dtype, "fused add + norm")
+    # in place on the input, as the reference's bda is
+    x2 = x.clone()
+    y2, _, _, _, s2 = pylayernorm_fwd(x2, g, b, 1e-5, 0, False, None, residual=r, sum_out=x2)
+    assert s2 is x2 and torch.equal(x2, s_ref) and torch.equal(y2, y_ref)

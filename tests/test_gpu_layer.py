@@ -289,3 +289,21 @@ def test_masked_streams_do_not_outlive_the_interpreter(tmp_path):
     res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=110)
     assert "done 2.0" in res.stdout, res.stderr[-2000:]
     assert res.returncode == 0, (res.returncode, res.stderr[-2000:])
+
+
+def test_fused_adjacent_ops_give_the_bits_of_the_separate_ops():
+    """bda_attn + ln_mlp run as one kernel when a plan lists them next to each other (all built-in plans do);
+    with ``fuse_adjacent`` off they run one after the other.  Same outputs and gradients, bit for bit."""
+    import dataclasses
+    from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
+    res = []
+    for fuse in (True, False):
+        cfg = dataclasses.replace(llama70b_tp8_shard(seq_length=1024), fuse_adjacent=fuse)
+        w = make_weights(cfg, 0, gen_device="cuda")
+        mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(2)]
+        r = LayerRunner(cfg, w)
+        outs, dxs = r.run_double_strand(mbs)
+        torch.cuda.synchronize()
+        res.append(outs + dxs + [w[k].main_grad.clone() for k in GRAD_KEYS])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)

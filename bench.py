@@ -372,6 +372,83 @@ def profile_op(name: str, iters: int = 5):
     torch.cuda.synchronize()
 
 
+def analyze_trace(path: str, cus: int = 256, lds_per_cu: int = 160 * 1024, regs_per_simd: int = 512,
+                  max_waves_per_simd: int = 8) -> str:
+    """Overlap headroom of the SERIAL schedule from a `rocprofv3 --kernel-trace --output-format csv` trace of
+    `bench.py --profile-op layer` (no GPU needed): how much compute-unit time one step leaves unused, i.e. the most
+    any co-schedule of a second strand could fill.  Per kernel: workgroups, how many fit the GPU at once (limited
+    by LDS, registers and wave slots), rounds, and the share of its CU-time that the last, partly filled round
+    leaves idle (compute units without any workgroup); plus the gaps between consecutive kernels on the stream.
+    All workgroups of a kernel are taken to run equally long.  Returns a markdown report."""
+    import csv
+    import re
+    rows = []
+    with open(path, newline="") as f:
+        for r in csv.DictReader(f):
+            rows.append(r)
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    first = next(i for i, r in enumerate(rows) if "norm_fwd_kernel" in r["Kernel_Name"])
+    layer = rows[first:]
+    per_iter = len(layer) // 5                   # --profile-op runs the step five times
+    win = layer[-per_iter:]
+    span = int(win[-1]["End_Timestamp"]) - int(win[0]["Start_Timestamp"])
+    busy = sum(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]) for r in win)
+
+    def short(name):
+        name = re.sub(r"\(.*", "", name)
+        name = re.sub(r"<.*", "", name)
+        name = name.replace("void ", "").replace("dh::", "")
+        m = re.match(r"_ZN2dh(\d+)(\w+)", name)
+        if m:
+            name = m.group(2)[: int(m.group(1))]
+        return name[:44]
+
+    agg = {}
+    idle_tail = 0.0
+    for r in win:
+        dur = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+        wg = int(r["Workgroup_Size_X"]) * int(r["Workgroup_Size_Y"]) * int(r["Workgroup_Size_Z"])
+        grid = int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
+        n_wg = max(1, grid // max(wg, 1))
+        waves = max(1, (wg + 63) // 64)
+        regs = max(8, int(r["VGPR_Count"]) + int(r["Accum_VGPR_Count"]))
+        per_simd = max(1, min(max_waves_per_simd, regs_per_simd // regs))
+        fit = max(1, (per_simd * 4) // waves)
+        lds = int(r["LDS_Block_Size"])
+        if lds > 0:
+            fit = max(1, min(fit, lds_per_cu // lds))
+        cap = fit * cus
+        rounds = -(-n_wg // cap)
+        # a compute unit counts as busy while it holds at least one workgroup (workgroups of the last round spread
+        # one per compute unit first): slots a resident workgroup leaves free on its own compute unit are not idle
+        # time a second strand could have, because the resident kernel already owns that unit's pipes
+        last = n_wg - (rounds - 1) * cap
+        fill = ((rounds - 1) + min(last, cus) / cus) / rounds
+        idle_tail += dur * (1.0 - fill)
+        a = agg.setdefault(short(r["Kernel_Name"]), dict(calls=0, ns=0, idle=0.0, wgs=set(), fit=set(), rounds=set()))
+        a["calls"] += 1
+        a["ns"] += dur
+        a["idle"] += dur * (1.0 - fill)
+        a["wgs"].add(n_wg)
+        a["fit"].add(fit)
+        a["rounds"].add(rounds)
+    gaps = span - busy
+    headroom = (gaps + idle_tail) / span
+    out = ["| kernel | calls | total us | share of step | workgroups | fit per CU | rounds | idle share of its CU-time |",
+           "|---|---|---|---|---|---|---|---|"]
+    fmt = lambda s_: "/".join(str(x) for x in sorted(s_)[:4]) + ("/.." if len(s_) > 4 else "")
+    for name, a in sorted(agg.items(), key=lambda kv: -kv[1]["ns"]):
+        out.append(f"| {name} | {a['calls']} | {a['ns'] / 1e3:.1f} | {a['ns'] / span:.3f} | {fmt(a['wgs'])} | {fmt(a['fit'])} | "
+                   f"{fmt(a['rounds'])} | {a['idle'] / max(a['ns'], 1):.3f} |")
+    out.append("")
+    out.append(f"step (4 micro-batches, serial): {span / 1e6:.3f} ms; kernels busy {busy / 1e6:.3f} ms; gaps between kernels "
+               f"{gaps / 1e6:.3f} ms ({gaps / span:.3f}); CU-time idle in partly filled rounds {idle_tail / 1e6:.3f} ms "
+               f"({idle_tail / span:.3f})")
+    out.append(f"idle CU-time / CU-time = {headroom:.3f}  ->  no co-schedule of the same kernels can be faster than "
+               f"{1.0 / (1.0 - headroom):.3f}x the serial schedule")
+    return "\n".join(out)
+
+
 def _device_info():
     """Name, architecture, CU count and HBM size as the runtime reports them."""
     p = torch.cuda.get_device_properties(0)
@@ -393,7 +470,13 @@ def main():
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
                     help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
+    ap.add_argument("--analyze-trace", default=None,
+                    help="kernel-trace CSV of `rocprofv3 --kernel-trace -- python bench.py --profile-op layer`: print the "
+                         "overlap headroom of the serial schedule and exit (no GPU needed)")
     args = ap.parse_args()
+    if args.analyze_trace:
+        print(analyze_trace(args.analyze_trace))
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures ONE GPU (one rank's share of the layer, no collectives); "
               "--gpus must be 1", file=sys.stderr)

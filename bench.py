@@ -31,7 +31,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
-ATTN_BWD_TRAFFIC_BYTES = 167.8e6   # measured; see profiles/attn_70b_shard_hbm_traffic.md
+def _measured():
+    """Counter- and trace-derived figures kept under profiles/ (hardware counters cannot be read from inside the
+    timed run): HBM bytes per launch of the attention backward, ceiling of any co-schedule of the layer's kernels."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "measured.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
 
 
 def _ensure_built():
@@ -135,6 +142,9 @@ def kernel_rooflines(cfg):
     o = torch.empty_like(a)
     ms = time_gpu_graph(lambda: bda_fwd(a, b, out=o))
     add(f"residual_add[{R}x{H}]", "hbm", 3 * R * H * e, ms, "3RHe bytes")
+    gm, so = torch.ones(H, device=dev, dtype=dt), torch.empty_like(a)
+    ms = time_gpu_graph(lambda: pylayernorm_fwd(a, gm, None, 1e-5, 0, False, None, residual=b, sum_out=so))
+    add(f"residual_add_rmsnorm_fwd[{R}x{H}]", "hbm", 4 * R * H * e + H * e + 4 * R, ms, "4RHe+He+4R bytes")
     del yy, gg
     # --- attention (70B shard: causal, S=4096, 8q/1kv, d=128) --------------------------------
     v = qkv[:, (hq + hk) * d:].view(T, hk, d)
@@ -149,7 +159,7 @@ def kernel_rooflines(cfg):
     dq, dk, dv = torch.empty_like(do), torch.empty(T, hk, d, device=dev, dtype=dt), torch.empty(T, hk, d, device=dev, dtype=dt)
     bw = lambda: _Clib._attn_bwd_raw(do, q, k, v, out_l[0], out_l[5], dq, dk, dv, None, cu, cu, T, T, sc, True, sp)
     ms_bwd = time_gpu(bw)
-    add(f"attn_bwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", 2.5 * fl_fwd, ms_bwd, "2.5 * fwd flop (delta+dkv+dq kernels)")
+    add(f"attn_bwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", 2.5 * fl_fwd, ms_bwd, "2.5 * fwd flop (dQ incl. delta, dK/dV and head-split sum kernels)")
     # --- ring step (32q/8kv, d=128, q 4096, kv chunk 4096): one causal and one full-block step -------
     hq1, hk1, S1 = 32, 8, 4096
     q1, k1, v1, do1 = rn(S1, hq1, d), rn(S1, hk1, d), rn(S1, hk1, d), rn(S1, hq1, d)
@@ -528,6 +538,7 @@ def main():
                     "double_strand_speedup": round(ser_c / min(dbl_c, dbl_l), 4)}
     layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
 
+    measured = _measured()
     kernels = [] if args.no_kernels else kernel_rooflines(cfg)
     dom = next((k for k in kernels if k["kernel"].startswith("attn_bwd")), None)
     roofline = None
@@ -535,8 +546,9 @@ def main():
         # HBM bytes per launch of the backward (its four kernels), from two rocprofv3 --pmc runs
         # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000: factors from the 1 GiB copy kernel) at this exact shape.
         roofline = {"kernel": dom["kernel"], "bound": "mfma", "achieved": dom["achieved"], "peak": dom["peak"],
-                    "unit": dom["unit"], "frac": dom["frac"], "traffic": ATTN_BWD_TRAFFIC_BYTES,
-                    "traffic_unit": "bytes/launch (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, calibrated)"}
+                    "unit": dom["unit"], "frac": dom["frac"],
+                    "traffic": measured.get("attn_bwd_70b_shard_hbm_traffic_bytes"),
+                    "traffic_unit": "bytes/launch (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, calibrated; profiles/measured.json)"}
     cpu = None if args.no_cpu_baseline else cpu_baseline(cfg)
 
     line = {
@@ -552,7 +564,9 @@ def main():
                                f"{len(mbs)} micro-batches per step", "schedule": schedule,
                    "tokens_per_step": tokens_per_step},
         "schedules": {"serial_ms": round(ms_serial, 4), "double_strand_ms": round(ms_double, 4),
-                      "double_strand_speedup": round(ms_serial / ms_double, 4)},
+                      "double_strand_speedup": round(ms_serial / ms_double, 4),
+                      # what ANY co-schedule of these kernels could reach: idle compute-unit time of the serial trace
+                      "double_strand_ceiling": measured.get("double_strand_ceiling")},
         "schedules_with_emulated_collectives": emulated,
         "layer_mfma_frac": round(layer_flop / (best_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,

@@ -12,7 +12,7 @@
 
 namespace dh {
 
-template <typename T, int BT, int TPR, int VPT, bool LN, bool NT>
+template <typename T, int BT, int TPR, int VPT, bool LN, bool NT, bool RES>
 __global__ void __launch_bounds__(BT)
 norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ residual, T *__restrict__ sum_out,
                 const T *__restrict__ gamma, const T *__restrict__ beta,
@@ -47,7 +47,7 @@ norm_fwd_kernel(const T *__restrict__ x, const T *__restrict__ residual, T *__re
       const int v = lane + i * TPR;
       if (active && v < nvec) {
         xv[i] = ldg_s<NT>(xr + (int64_t)v * N);
-        if (residual) {
+        if (RES) {
           // the row that is normalised is x + residual, rounded to the storage type and written out: what a
           // separate residual-add kernel in front of the norm would have stored and this one read back
           const Vec<T> rv = ldg_s<NT>(residual + row * cols + (int64_t)v * N);
@@ -152,7 +152,7 @@ norm_fwd_generic_kernel(const T *__restrict__ x, const T *__restrict__ residual,
 }
 
 // Backward main pass.  part: fp32 [2][gridDim.x][cols] (dgamma rows, then dbeta rows).
-template <typename T, int BT, int TPR, int VPT, bool LN, bool NT>
+template <typename T, int BT, int TPR, int VPT, bool LN, bool NT, bool ADD>
 __global__ void __launch_bounds__(BT)
 norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *__restrict__ mu,
                 const float *__restrict__ rsigma, const T *__restrict__ gamma, const T *__restrict__ add_to_dx,
@@ -203,6 +203,14 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
       dv[i] = dn[i];
     }
     fetch(row + (int64_t)gridDim.x * RPB);
+    Vec<T> rv[VPT];       // the gradient added to dx: requested ahead of the reduction
+    if (ADD) {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int v = lane + i * TPR;
+        if (active && v < nvec) rv[i] = ldg_s<NT>(add_to_dx + row * cols + (int64_t)v * N);
+      }
+    }
     float rs = 0.f, mean = 0.f;
     if (active) {
       rs = rsigma[row];
@@ -238,14 +246,13 @@ norm_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *
       for (int i = 0; i < VPT; ++i) {
         const int v = lane + i * TPR;
         if (v < nvec) {
-          Vec<T> o, r;
-          if (add_to_dx) r = ldg_s<NT>(add_to_dx + row * cols + (int64_t)v * N);
+          Vec<T> o;
 #pragma unroll
           for (int j = 0; j < N; ++j) {
             const float xh = (to_f(xv[i].v[j]) - mean) * rs;
             const float gg = to_f(dv[i].v[j]) * (to_f(g[i].v[j]) + gamma_shift);
             float f = rs * (gg - xh * c1 - c2);
-            if (add_to_dx) f += to_f(r.v[j]);
+            if (ADD) f += to_f(rv[i].v[j]);
             o.v[j] = from_f<T>(f);
           }
           stg_s<NT>(dx + row * cols + (int64_t)v * N, o);
@@ -513,9 +520,13 @@ static int launch_fwd(const NormPlan &p, const T *x, const T *residual, T *sum_o
   int64_t nb = cdiv(rows, rpb);
   if (nb > 256 * 16) nb = 256 * 16;
   const bool nt = stream_hint((residual ? 4 : 2) * rows * cols * (int64_t)sizeof(T));
+#define L3(BT, TPR, VPT, NT, RES)                                                                            \
+  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN, NT, RES>), dim3((unsigned)nb), dim3(BT), 0, st, x,     \
+                     residual, sum_out, gamma, beta, y, mu, rs, rows, (int)cols, eps, shift)
 #define L2(BT, TPR, VPT, NT)                                                                                 \
-  hipLaunchKernelGGL((norm_fwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT), 0, st, x, residual, \
-                     sum_out, gamma, beta, y, mu, rs, rows, (int)cols, eps, shift)
+  do {                                                                                                       \
+    if (residual) L3(BT, TPR, VPT, NT, true); else L3(BT, TPR, VPT, NT, false);                               \
+  } while (0)
 #define L(BT, TPR, VPT)                                                                                      \
   do {                                                                                                       \
     if (nt) L2(BT, TPR, VPT, true); else L2(BT, TPR, VPT, false);                                             \
@@ -529,6 +540,7 @@ static int launch_fwd(const NormPlan &p, const T *x, const T *residual, T *sum_o
   }
 #undef L
 #undef L2
+#undef L3
   return 0;
 }
 
@@ -546,10 +558,14 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
                        dim3(256), 0, st, dy, x, mu, rs, part, rows, cols, rpc);
   } else {
     const bool nt = stream_hint((add ? 4 : 3) * rows * cols * (int64_t)sizeof(T));
-#define L2(BT, TPR, VPT, NT)                                                                                 \
-  hipLaunchKernelGGL((norm_bwd_kernel<T, BT, TPR, VPT, LN, NT>), dim3((unsigned)nb), dim3(BT),                    \
+#define L3(BT, TPR, VPT, NT, ADD)                                                                            \
+  hipLaunchKernelGGL((norm_bwd_kernel<T, BT, TPR, VPT, LN, NT, ADD>), dim3((unsigned)nb), dim3(BT),               \
                      (TPR == 64 ? 4 * 64 * VPT * (16 / sizeof(T)) * sizeof(float) : 0), st, dy, x, mu, rs, gamma, \
                      add, dx, part, rows, (int)cols, shift)
+#define L2(BT, TPR, VPT, NT)                                                                                 \
+  do {                                                                                                       \
+    if (add) L3(BT, TPR, VPT, NT, true); else L3(BT, TPR, VPT, NT, false);                                    \
+  } while (0)
 #define L(BT, TPR, VPT)                                                                                      \
   do {                                                                                                       \
     if (nt) L2(BT, TPR, VPT, true); else L2(BT, TPR, VPT, false);                                             \
@@ -563,6 +579,7 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
     }
 #undef L
 #undef L2
+#undef L3
   }
   if (cols % 4 == 0)
     hipLaunchKernelGGL((norm_bwd_finalize_kernel<T, LN>), dim3((unsigned)cdiv(cols, 64)), dim3(256), 0, st, part,

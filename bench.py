@@ -241,6 +241,8 @@ def kernel_rooflines(cfg):
     lmask = torch.ones(1, T, device=dev, dtype=torch.int64)
     gam.main_grad = torch.zeros_like(gam)
 
+    from dhellam_amd._Clib import keep_transposed as _keep_t
+    _keep_t(table)                             # as DSHB / DSLLMStep hold it: the logits product's data gradient runs against W^T
     def head_step():
         _, hctx = dshb.post_process(hid, gam, None, labels, lmask, table, 4, 1.0)
         dshb.post_process_bwd(hctx)
@@ -249,16 +251,18 @@ def kernel_rooflines(cfg):
     parallel_state.set_tensor_model_parallel(0, 1)
     del table, dh_, em_out, hid
     # --- the layer's twelve dense products (library kernels through dh_gemm), as the layer calls them -------
+    from dhellam_amd._Clib import keep_transposed
     from dhellam_amd.operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
     for name, n_out, k_in in (("qkv", cfg.qkv_per_rank, H), ("attn_out", H, hq * d), ("fc1", 2 * F, H), ("fc2", H, F)):
         x, w, dy = rn(T, k_in), rn(n_out, k_in), rn(T, n_out)
+        keep_transposed(w)                      # as the layer holds its weights: dgrad runs against W^T
         dw = torch.zeros(n_out, k_in, device=dev, dtype=dt)
         flop = 2.0 * T * n_out * k_in
         for what, fn in (("fwd", lambda: gemm_fwd(None, x, w, None, "TN", False, 0, True, None)),
                          ("dgrad", lambda: dgrad_bwd(None, dy, w, None, "NN", False, 0, True, None)),
                          ("wgrad", lambda: wgrad_bwd(None, dy, x, dw, True, "NT", False, 0, True, None))):
             add(f"dense_gemm[{name} {what} T={T} N={n_out} K={k_in}]", "mfma", flop, time_gpu(fn, iters=10, warmup=3),
-                "2TNK flop (hipBLASLt through dh_gemm; wgrad includes the transpose of dY where it is used)")
+                "2TNK flop (hipBLASLt through dh_gemm; dgrad against the resident W^T; wgrad includes the transpose of dY where it is used)")
         del x, w, dy, dw
     return res
 
@@ -508,12 +512,16 @@ def main():
     runner = LayerRunner(cfg, w, plan=plan)
     tokens_per_step = cfg.tokens * len(mbs)
 
-    def timed(fn):
+    def timed(fn, runner=runner):
+        # A step is what lies between two optimizer steps: the weights have just changed, so their resident
+        # transposes (used by the data-gradient GEMMs) are rebuilt inside the timed region, once per step.
         for _ in range(args.warmup):
+            runner.refresh_weight_transposes()
             fn(mbs)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
+            runner.refresh_weight_transposes()
             fn(mbs)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps * 1e3
@@ -528,10 +536,10 @@ def main():
     if args.emulate_comm_us > 0:
         import dataclasses
         runner_c = LayerRunner(dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us), w, plan=plan)
-        ser_c, dbl_c = timed(runner_c.run_serial), timed(runner_c.run_double_strand)
+        ser_c, dbl_c = timed(runner_c.run_serial, runner_c), timed(runner_c.run_double_strand, runner_c)
         runner_l = LayerRunner(dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us, lockstep_blocks=True), w,
                                plan=plan)
-        dbl_l = timed(runner_l.run_double_strand)
+        dbl_l = timed(runner_l.run_double_strand, runner_l)
         emulated = {"standin_us_per_collective": args.emulate_comm_us, "collectives_per_microbatch": 8,
                     "serial_ms": round(ser_c, 4), "double_strand_ms": round(dbl_c, 4),
                     "double_strand_lockstep_ms": round(dbl_l, 4),

@@ -23,6 +23,7 @@ from typing import Dict, Optional
 
 import torch
 
+from .._Clib import keep_transposed
 from ..operators.embedding import word_embedding_bwd, word_embedding_fwd
 from ..operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
 from ..operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
@@ -186,6 +187,8 @@ class DSHB(torch.nn.Module):
         self.ln_bias = None
         for p in (self.word_embeddings, self.ln_weight):
             p.main_grad = torch.zeros_like(p)
+        if getattr(config, "resident_weight_transposes", False):
+            keep_transposed(self.word_embeddings)      # the logits product's data gradient in the forward's layout
         self.logits_weight = self.word_embeddings
 
     def forward(self, placeholder):

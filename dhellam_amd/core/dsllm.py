@@ -24,6 +24,7 @@ from typing import Dict, List, Optional
 import torch
 
 from . import dshb
+from .._Clib import keep_transposed
 from .dstb import DCoperation, LayerConfig, Plan, exec as exec_blocks, init_DCBlocks
 from .layer import make_weights
 
@@ -55,6 +56,8 @@ class DSLLMStep:
         self.final_ln_weight = torch.ones(cfg.hidden_size, dtype=dt, device=device)
         for t in (self.word_embeddings, self.final_ln_weight):
             t.main_grad = torch.zeros_like(t)
+        if cfg.resident_weight_transposes:
+            keep_transposed(self.word_embeddings)
         self.stream1 = stream1 or torch.cuda.Stream()
         self.stream2 = stream2 or torch.cuda.Stream()
         self.plan: Plan = init_DCBlocks(plan, self.stream1, self.stream2)

@@ -47,7 +47,7 @@ import torch
 
 from .. import _lib
 from ..common.global_variables import GLOBAL_VARIABLES
-from .._Clib import pymha_varlen_bwd, pymha_varlen_fwd, _attn_bwd_raw
+from .._Clib import keep_transposed, pymha_varlen_bwd, pymha_varlen_fwd, _attn_bwd_raw
 from ..operators.bda import bda_bwd, bda_fwd
 from ..operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
 from ..operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
@@ -119,6 +119,7 @@ class LayerConfig:
     # to and from the strand's own stream, instead of on the strand's stream itself
     comm_streams: Optional[tuple] = None
     fuse_adjacent: bool = True        # ops a plan lists next to each other run as one kernel where one exists (bda_attn + ln_mlp)
+    resident_weight_transposes: bool = True   # projection weights are kept as W and W^T: the data-gradient GEMMs then run in the forward's layout
 
     @property
     def head_dim(self) -> int:
@@ -1142,6 +1143,8 @@ class DSTB(torch.nn.Module):
             for k in names:
                 p = torch.nn.Parameter(w[k])
                 p.main_grad = torch.zeros_like(w[k])
+                if config.resident_weight_transposes and k in _DGRAD_WEIGHT.values():
+                    keep_transposed(p)
                 if k.startswith("ln_"):
                     p.sequence_parallel = config.tensor_model_parallel_size > 1
                 setattr(self, f"{k}_{tag}", p)

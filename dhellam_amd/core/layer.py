@@ -13,6 +13,7 @@ from typing import Dict, List, Optional
 
 import torch
 
+from .._Clib import keep_transposed
 from .dstb import DCoperation, LayerConfig, Plan, exec as exec_blocks, init_DCBlocks
 
 
@@ -60,6 +61,9 @@ def make_weights(cfg: LayerConfig, seed: int = 0, device="cuda", gen_device="cpu
         w["ln_mlp_bias"] = torch.zeros(h, dtype=dt, device=device)
     for t in w.values():
         t.main_grad = torch.zeros_like(t)
+    if cfg.resident_weight_transposes and device != "cpu":
+        for k in ("column_attn_weight", "linear_attn_weight", "column_mlp_weight", "linear_mlp_weight"):
+            keep_transposed(w[k])
     s = cfg.seq_length
     cu = torch.arange(0, (cfg.micro_batch_size + 1) * s, s, dtype=torch.int32, device=device)
     w["cu_seqlens_q"] = cu
@@ -110,6 +114,13 @@ class LayerRunner:
         return exec_blocks(self.cfg, DCoperation, self.weights if act_new is not None else None,
                            self.weights if act_prev is not None else None, x, dy, blocks, s1, s2, act_prev, act_new,
                            movable=self.plan.movable)
+
+    def refresh_weight_transposes(self):
+        """Rebuilds W^T of every projection weight on the current stream: what follows an optimizer step when the
+        weights are kept in both layouts (a step that goes through torch's in-place ops triggers it by itself)."""
+        if self.cfg.resident_weight_transposes:
+            for k in ("column_attn_weight", "linear_attn_weight", "column_mlp_weight", "linear_mlp_weight"):
+                keep_transposed(self.weights[k], refresh=True)
 
     def run_serial(self, mbs: List[dict]):
         """F0 B0 F1 B1 ... on ONE stream with the fwd_only / bwd_only plans."""

@@ -18,7 +18,7 @@ from typing import Optional
 
 import torch
 
-from .._Clib import dense_gemm, dense_ok
+from .._Clib import dense_gemm, dense_ok, dgrad_gemm, transposed_of
 from .._Clib import pygemm as gemm
 from .._Clib import wgrad_gemm
 from ._util import on_stream
@@ -72,13 +72,17 @@ def dgrad_bwd(args, input_grad: torch.Tensor, weight: torch.Tensor, dgrad_output
         if is_matmul:
             if (not transa and not transb and dense_ok(weight, input_grad, dgrad_output)
                     and weight.dtype == input_grad.dtype == dgrad_output.dtype):
-                dense_gemm(weight, input_grad, dgrad_output, False, False, False)
+                dgrad_gemm(input_grad, weight, dgrad_output)
             else:
                 w = weight.t() if transa else weight
                 g = input_grad.t() if transb else input_grad
                 torch.matmul(g, w, out=dgrad_output)
         else:
-            gemm(weight, input_grad, dgrad_output, None, 0, transa, transb, False, math_sm_count, False)
+            wt = transposed_of(weight) if not (transa or transb) else None
+            if wt is not None and wt.dtype == input_grad.dtype:      # same product in the forward's layout
+                gemm(wt, input_grad, dgrad_output, None, 0, True, False, False, math_sm_count, False)
+            else:
+                gemm(weight, input_grad, dgrad_output, None, 0, transa, transb, False, math_sm_count, False)
     return dgrad_output, el[0]
 
 

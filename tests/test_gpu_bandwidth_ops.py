@@ -293,6 +293,39 @@ def test_dense_gemm_layouts(dtype, t, n, k):
     assert_close(y5, ref_y, dtype, "strided weight")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,n,k", [(256, 384, 512), (4096, 1280, 1024), (100, 72, 40)])
+def test_dgrad_against_resident_transpose(dtype, t, n, k):
+    """A weight registered with keep_transposed: the data gradient runs against W^T in the forward's layout and equals
+    the NN product; the copy follows the weight through in-place updates (version counter), is usable from another
+    stream, and an explicit refresh covers writers that go around the counter."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.layernorm_column import dgrad_bwd
+    w, dy = randn((n, k), dtype, 1, std=0.1).cuda(), randn((t, n), dtype, 2).cuda()
+    plain, _ = dgrad_bwd(None, dy, w, None, "NN", False, 0, True, None)           # not registered: NN as given
+    assert _Clib.transposed_of(w) is None
+    assert_close(plain, dy.double().cpu() @ w.double().cpu(), dtype, "NN")
+    wt = _Clib.keep_transposed(w)
+    assert torch.equal(wt, w.t().contiguous()) and _Clib.transposed_of(w) is wt
+    for is_matmul in (True, False):
+        got, _ = dgrad_bwd(None, dy, w, None, "NN", False, 0, is_matmul, None)
+        assert_close(got, dy.double().cpu() @ w.double().cpu(), dtype, "against W^T")
+        assert_close(got, plain.double().cpu(), dtype, "both layouts agree")
+    w.mul_(0.5)                                                                   # an optimizer step: version moves
+    got, _ = dgrad_bwd(None, dy, w, None, "NN", False, 0, True, None)
+    assert torch.equal(_Clib.transposed_of(w), w.t().contiguous())
+    assert_close(got, dy.double().cpu() @ w.double().cpu(), dtype, "after an in-place update")
+    w.data.copy_(randn((n, k), dtype, 3, std=0.1))                                # around the counter: caller refreshes
+    _Clib.keep_transposed(w, refresh=True)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):                                                 # another stream than the one that built it
+        got, _ = dgrad_bwd(None, dy, w, None, "NN", False, 0, True, None)
+    side.synchronize()
+    assert_close(got, dy.double().cpu() @ w.double().cpu(), dtype, "from another stream")
+    odd = randn((n, k + 4), dtype, 4).cuda()[:, :k]                               # not a tensor the transpose takes
+    assert _Clib.keep_transposed(odd) is None and _Clib.transposed_of(odd) is None
+
+
 def test_dense_gemm_argument_errors():
     import ctypes
     from dhellam_amd import _Clib, _lib

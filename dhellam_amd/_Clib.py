@@ -366,19 +366,21 @@ def _attn_bwd_workspace(nbytes: int, device, stream_ptr: int) -> torch.Tensor:
     return ws
 
 
-def _attn_bwd_raw(dout, q, k, v, out, lse, dq, dk, dv, delta, cu_q, cu_k, max_q, max_k, scale, causal, stream_ptr):
+def _attn_bwd_raw(dout, q, k, v, out, lse, dq, dk, dv, delta, cu_q, cu_k, max_q, max_k, scale, causal, stream_ptr,
+                  accumulate_dq=False):
+    """``dh_attn_bwd``; with ``accumulate_dq`` the call's dq is added to the contents of ``dq`` inside the kernel."""
     lib = _lib.load()
     b = cu_q.numel() - 1
     nbytes = lib.dh_attn_bwd_workspace_bytes(q.shape[0], k.shape[0], b, int(max_q), q.shape[1], k.shape[1],
                                              q.shape[2], _lib.dt(q))
     ws = _attn_bwd_workspace(nbytes, q.device, stream_ptr)
-    _lib.check(lib.dh_attn_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-                               lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.ptr(delta),
-                               ws.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(), b, int(max_q), int(max_k),
-                               q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2], _tok_stride(q),
-                               _tok_stride(k), _tok_stride(v), _tok_stride(out), _tok_stride(dout),
-                               _tok_stride(dq), _tok_stride(dk), _tok_stride(dv), float(scale), int(bool(causal)),
-                               _lib.dt(q), stream_ptr))
+    _lib.check(lib.dh_attn_bwd_acc(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                   lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.ptr(delta),
+                                   ws.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(), b, int(max_q), int(max_k),
+                                   q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2], _tok_stride(q),
+                                   _tok_stride(k), _tok_stride(v), _tok_stride(out), _tok_stride(dout),
+                                   _tok_stride(dq), _tok_stride(dk), _tok_stride(dv), float(scale), int(bool(causal)),
+                                   int(bool(accumulate_dq)), _lib.dt(q), stream_ptr))
 
 
 def pymha_varlen_bwd(dout, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,

@@ -41,6 +41,7 @@ struct AttnBwdParams {
   int64_t q_stride, k_stride, v_stride, do_stride, dq_stride, dk_stride, dv_stride;
   float scale, scale_log2;
   int causal;
+  int dq_accumulate;         // dq += this call's gradient (read, add in fp32, round once) instead of dq =
 };
 
 // ---- delta = rowsum(dO * O) ---------------------------------------------------------------
@@ -454,8 +455,14 @@ __global__ void __launch_bounds__(64 * NW) attn_bwd_dq_kernel(const AttnBwdParam
 #pragma unroll
       for (int vb = 0; vb < 4; ++vb) {
         struct alignas(8) { T v[4]; } a;
+        if (p.dq_accumulate) {
+          a = *reinterpret_cast<const decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+          for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(static_cast<float>(a.v[e]) + dQt[t][4 * vb + e] * p.scale);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+        }
         *reinterpret_cast<decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh) = a;
       }
   }
@@ -750,8 +757,14 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
 #pragma unroll
           for (int vb = 0; vb < 4; ++vb) {
             struct alignas(8) { T v[4]; } a;
+            if (p.dq_accumulate) {
+              a = *reinterpret_cast<const decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+              for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(static_cast<float>(a.v[e]) + dQt[t][4 * vb + e] * p.scale);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+            }
             *reinterpret_cast<decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh) = a;
           }
       }
@@ -1199,7 +1212,7 @@ int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, 
                  void *dq, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k, int batch, int max_sq,
                  int max_sk, int hq, int hk, int d, int64_t q_stride, int64_t k_stride, int64_t v_stride,
                  int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int causal,
-                 hipStream_t st);
+                 int dq_accumulate, hipStream_t st);
 
 constexpr int DKV_NW = 2;  // wavefronts per dK/dV workgroup (64 key rows)
 
@@ -1218,13 +1231,13 @@ extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, 
   return n + 256;
 }
 
-extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
-                           const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
-                           const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
-                           int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
-                           int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
-                           int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
-                           float softmax_scale, int causal, int dtype, void *stream) {
+static int attn_bwd_entry(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                          const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
+                          const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
+                          int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                          int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                          int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                          float softmax_scale, int causal, int dq_accumulate, int dtype, void *stream) {
   using namespace dh;
   DH_CHECK(batch >= 0 && max_seqlen_q >= 0 && max_seqlen_k >= 0 && total_q >= 0 && total_k >= 0, "negative size");
   DH_CHECK(hq > 0 && hk > 0 && hq % hk == 0, "hq=%d must be a positive multiple of hk=%d", hq, hk);
@@ -1262,7 +1275,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
     DH_CHECK(d > 0 && d <= 256 && d % 4 == 0, "fp32 attention needs d %% 4 == 0 and d <= 256 (got %d)", d);
     return attn_bwd_f32(dout, q, k, v, lse, delta, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, batch, max_seqlen_q,
                         max_seqlen_k, hq, hk, d, q_stride, k_stride, v_stride, do_stride, dq_stride, dk_stride,
-                        dv_stride, softmax_scale, causal, st);
+                        dv_stride, softmax_scale, causal, dq_accumulate, st);
   }
   DH_CHECK(d == 64 || d == 128, "bf16/fp16 attention supports head dim 64 or 128 (got %d)", d);
   DH_CHECK(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && dq_stride % 4 == 0 && dk_stride % 4 == 0 &&
@@ -1283,6 +1296,7 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   p.scale = softmax_scale;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.causal = causal;
+  p.dq_accumulate = dq_accumulate ? 1 : 0;
   p.hsplit = pick_hsplit(d == 128 && causal ? (max_seqlen_k + 1) / 2 : max_seqlen_k, batch, hq, hk, 32 * DKV_NW);
   p.dk_part = nullptr;
   p.dv_part = nullptr;
@@ -1320,4 +1334,28 @@ extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const
   if (rc != DH_OK) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;
+}
+
+extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                           const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
+                           const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
+                           int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                           int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                           int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                           float softmax_scale, int causal, int dtype, void *stream) {
+  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, cu_seqlens_q, cu_seqlens_k, batch,
+                        max_seqlen_q, max_seqlen_k, total_q, total_k, hq, hk, d, q_stride, k_stride, v_stride, o_stride,
+                        do_stride, dq_stride, dk_stride, dv_stride, softmax_scale, causal, 0, dtype, stream);
+}
+
+extern "C" int dh_attn_bwd_acc(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                               const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
+                               const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
+                               int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                               int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                               int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
+                               float softmax_scale, int causal, int accumulate_dq, int dtype, void *stream) {
+  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, cu_seqlens_q, cu_seqlens_k, batch,
+                        max_seqlen_q, max_seqlen_k, total_q, total_k, hq, hk, d, q_stride, k_stride, v_stride, o_stride,
+                        do_stride, dq_stride, dk_stride, dv_stride, softmax_scale, causal, accumulate_dq, dtype, stream);
 }

@@ -95,7 +95,7 @@ attn_bwd_dq_f32_kernel(const float *__restrict__ dout, const float *__restrict__
                        const float *__restrict__ v, const float *__restrict__ lse, const float *__restrict__ delta,
                        float *__restrict__ dq, const int32_t *__restrict__ cu_q, const int32_t *__restrict__ cu_k,
                        int max_sq, int hq, int hk, int d, int64_t q_stride, int64_t k_stride, int64_t v_stride,
-                       int64_t do_stride, int64_t dq_stride, float scale, int causal) {
+                       int64_t do_stride, int64_t dq_stride, float scale, int causal, int accumulate) {
   __shared__ float sq_row[256], sdo_row[256];
   __shared__ float sds[F32_NT];
   const int b = blockIdx.z, h = blockIdx.y, i = blockIdx.x;
@@ -143,7 +143,7 @@ attn_bwd_dq_f32_kernel(const float *__restrict__ dout, const float *__restrict__
 #pragma unroll
   for (int ci = 0; ci < F32_MAXC; ++ci) {
     const int c = tid + ci * F32_NT;
-    if (c < d) dqr[c] = acc[ci] * scale;
+    if (c < d) dqr[c] = accumulate ? dqr[c] + acc[ci] * scale : acc[ci] * scale;
   }
 }
 
@@ -234,7 +234,7 @@ int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, 
                  void *dq, void *dk, void *dv, const int32_t *cu_q, const int32_t *cu_k, int batch, int max_sq,
                  int max_sk, int hq, int hk, int d, int64_t q_stride, int64_t k_stride, int64_t v_stride,
                  int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride, float scale, int causal,
-                 hipStream_t st) {
+                 int dq_accumulate, hipStream_t st) {
   DH_CHECK(q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 && do_stride % 4 == 0 && aligned16(q) &&
                aligned16(k) && aligned16(v) && aligned16(dout),
            "fp32 attention needs 16-byte aligned rows");
@@ -242,7 +242,7 @@ int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, 
     hipLaunchKernelGGL(attn_bwd_dq_f32_kernel, dim3((unsigned)max_sq, (unsigned)hq, (unsigned)batch), dim3(F32_NT), 0,
                        st, (const float *)dout, (const float *)q, (const float *)k, (const float *)v, lse, delta,
                        (float *)dq, cu_q, cu_k, max_sq, hq, hk, d, q_stride, k_stride, v_stride, do_stride, dq_stride,
-                       scale, causal);
+                       scale, causal, dq_accumulate);
   if (max_sk > 0)
     hipLaunchKernelGGL(attn_bwd_dkv_f32_kernel, dim3((unsigned)max_sk, (unsigned)hk, (unsigned)batch), dim3(F32_NT),
                        0, st, (const float *)dout, (const float *)q, (const float *)k, (const float *)v, lse, delta,

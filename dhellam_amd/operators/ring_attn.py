@@ -214,20 +214,26 @@ def fa_cp_block_bwd(dout, out, q, dq, kv, dkv_, softmax_lse, rng_states, cu_seql
         # With batch > 1 the first-half views of an 'L' step are not contiguous: _rows() then hands out
         # packed temporaries, and the results are copied back into the views.
         dkv_is_temp = dk_.data_ptr() != dkv[0].data_ptr()
-        dq_step = torch.empty(q_.shape, dtype=q.dtype, device=q.device)
-        _Clib._attn_bwd_raw(do_, q_, k_, v_, o_, lse_, dq_step, dk_, dv_, None, cq, ck, mq, mk, scale, cz, sp)
+        # dq: the first contribution to a row is a store, later ones add (ring_attn.py:391-408), both inside the
+        # kernel when the rows form one packed run (always for batch 1): no temporary and no extra pass over dq.
+        first_store = first_touch_all or (causal and i == 0)
+        if causal and i == 0 and not first_touch_all:      # first call is a 'U' step: only the second half exists yet
+            dq[:, 0].zero_()
+        if dq_rows.is_contiguous() or dq_rows.shape[0] == 1:
+            tgt = dq_rows.reshape(-1, hq, d) if dq_rows.is_contiguous() else dq_rows[0]
+            _Clib._attn_bwd_raw(do_, q_, k_, v_, o_, lse_, tgt, dk_, dv_, None, cq, ck, mq, mk, scale, cz, sp,
+                                accumulate_dq=not first_store)
+        else:
+            dq_step = torch.empty(q_.shape, dtype=q.dtype, device=q.device)
+            _Clib._attn_bwd_raw(do_, q_, k_, v_, o_, lse_, dq_step, dk_, dv_, None, cq, ck, mq, mk, scale, cz, sp)
+            dq_step = dq_step.view(dq_rows.shape)
+            if first_store:
+                dq_rows.copy_(dq_step)
+            else:
+                dq_rows.add_(dq_step)
         if dkv_is_temp:
             assert causal and case == "L"
             dkv[0][:, 0].copy_(dk_.view(b, c, hk, d))
             dkv[1][:, 0].copy_(dv_.view(b, c, hk, d))
-        dq_step = dq_step.view(dq_rows.shape)
-        # dq: the first contribution to a row is a copy, later ones add (ring_attn.py:391-408).
-        if first_touch_all:
-            dq_rows.copy_(dq_step)
-        elif causal and i == 0:             # first call is a 'U' step: only the second half exists yet
-            dq[:, 0].zero_()
-            dq_rows.copy_(dq_step)
-        else:
-            dq_rows.add_(dq_step)
         dkv_[step] = dkv
     return [dout, dq, dkv_, p2p_comm_buffers, i + 1], []

@@ -158,6 +158,22 @@ int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v,
                 int64_t dk_stride, int64_t dv_stride, float softmax_scale,
                 int causal, int dtype, void *stream);
 
+/* dh_attn_bwd with one more argument: accumulate_dq != 0 adds this call's dq
+ * to the values already in `dq` (read, added in fp32, rounded once) instead of
+ * overwriting them: a ring step's `dq.add_(dq_)` of
+ * dhellam/operators/ring_attn.py:391-408 without the temporary and the extra
+ * pass.  dk/dv are written as in dh_attn_bwd. */
+int dh_attn_bwd_acc(const void *dout, const void *q, const void *k,
+                    const void *v, const void *out, const float *lse, void *dq,
+                    void *dk, void *dv, float *delta_out, void *workspace,
+                    const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                    int batch, int max_seqlen_q, int max_seqlen_k,
+                    int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                    int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                    int64_t o_stride, int64_t do_stride, int64_t dq_stride,
+                    int64_t dk_stride, int64_t dv_stride, float softmax_scale,
+                    int causal, int accumulate_dq, int dtype, void *stream);
+
 /* ------------------------------------------------------------------------
  * Ring-attention merge of per-step partial results.
  * dhellam/operators/ring_attn.py:26-40 (lse and out correction) applied as in

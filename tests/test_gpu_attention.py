@@ -103,6 +103,33 @@ def test_attention_fp32(lens_q, lens_k, hq, hk, d, causal):
     _run_fwd_bwd(torch.float32, lens_q, lens_k, hq, hk, d, causal)
 
 
+@pytest.mark.parametrize("dtype,hq,hk,d", [(torch.bfloat16, 4, 2, 128), (torch.float16, 32, 8, 128), (torch.bfloat16, 2, 2, 64),
+                                         (torch.float32, 2, 1, 32)])
+def test_attention_backward_accumulates_dq(dtype, hq, hk, d):
+    """dh_attn_bwd_acc with accumulate_dq: dq += the call's gradient (one rounding of the fp32 sum); dk, dv and a
+    call without the flag are those of dh_attn_bwd."""
+    from dhellam_amd import _Clib
+    lens = [200, 56] if hq < 32 else [640]
+    cu = _cu(lens).cuda()
+    t, m, scale = sum(lens), max(lens), 1.0 / math.sqrt(d)
+    q, k, v, do = (randn((t, h, d), dtype, 10 + i).cuda() for i, h in enumerate((hq, hk, hk, hq)))
+    res = _Clib.pymha_varlen_fwd(q, k, v, cu, cu, m, m, 0.0, scale, True, False, 0, False)
+    out, lse = res[0], res[5]
+    sp = torch.cuda.current_stream().cuda_stream
+    dq0, dk0, dv0 = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _Clib._attn_bwd_raw(do, q, k, v, out, lse, dq0, dk0, dv0, None, cu, cu, m, m, scale, True, sp)
+    base = randn((t, hq, d), dtype, 20).cuda()
+    dq1, dk1, dv1 = base.clone(), torch.empty_like(k), torch.empty_like(v)
+    _Clib._attn_bwd_raw(do, q, k, v, out, lse, dq1, dk1, dv1, None, cu, cu, m, m, scale, True, sp, accumulate_dq=True)
+    assert torch.equal(dk1, dk0) and torch.equal(dv1, dv0)
+    # the kernel adds its fp32 gradient before rounding, so it is at least as close to the exact sum as adding the
+    # rounded gradient: compare with base + dq0 at the operator tolerance, and bit for bit where nothing was there
+    assert_close(dq1, base.double().cpu() + dq0.double().cpu(), dtype, "dq accumulated")
+    dq2 = torch.zeros_like(q)
+    _Clib._attn_bwd_raw(do, q, k, v, out, lse, dq2, dk1, dv1, None, cu, cu, m, m, scale, True, sp, accumulate_dq=True)
+    assert torch.equal(dq2, dq0)
+
+
 def test_attention_is_deterministic():
     a = _run_fwd_bwd(torch.bfloat16, [700], [700], 8, 2, 128, True)
     b = _run_fwd_bwd(torch.bfloat16, [700], [700], 8, 2, 128, True)

@@ -29,36 +29,65 @@ rope_kernel(const T *__restrict__ q, const T *__restrict__ k, T *__restrict__ qo
     int64_t pos;
     if (positions) pos = positions[t];
     else pos = seq_len > 0 ? t % seq_len : t;
+    // Heads are handled in groups of up to HG with all loads of a group issued first; the first group's loads go
+    // out before the cos/sin evaluation (a few hundred instructions), which then runs in their shadow.
+    constexpr int HG = 4;
+    const int h0 = hs * hper;
+    const int h1 = h0 + hper < heads ? h0 + hper : heads;
+    Vec<T> lo[HG], hi[HG];
+    auto src_of = [&](int h) {
+      return h < hq ? q + t * q_stride + (int64_t)h * d : k + t * k_stride + (int64_t)(h - hq) * d;
+    };
+    auto dst_of = [&](int h) {
+      return h < hq ? qo + t * qo_stride + (int64_t)h * d : ko + t * ko_stride + (int64_t)(h - hq) * d;
+    };
+    auto load_group = [&](int hb) {
+#pragma unroll
+      for (int g = 0; g < HG; ++g)
+        if (hb + g < h1) {
+          const T *src = src_of(hb + g);
+          lo[g] = ldg(src + c * N);
+          hi[g] = ldg(src + half + c * N);
+        }
+    };
+    load_group(h0);
     float cs[N], sn[N];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       const float ang = (float)pos * inv_freq[c * N + j];
-      sincosf(ang, &sn[j], &cs[j]);
+      if (sizeof(T) == 4) {
+        sincosf(ang, &sn[j], &cs[j]);
+      } else {
+        // 16-bit results: the hardware's sin / cos (argument in revolutions) after an exact reduction of the fp32
+        // angle: ang / 2pi as a two-term product whose rounding error is recovered with an fma, so the fraction
+        // of a revolution is good to ~1e-7 for angles of 1e5 rad; the routine's own error (~1e-6) is a thousand
+        // times below the rounding of the result.
+        const float c_hi = 0.15915494f, c_lo = 6.4206382e-9f;   // 1 / 2pi = c_hi + c_lo
+        float r_hi = ang * c_hi;
+        asm volatile("" : "+v"(r_hi));     // opaque to the compiler, which otherwise folds fma(a, b, -(a * b)) to zero
+        const float r_lo = fmaf(ang, c_lo, fmaf(ang, c_hi, -r_hi));   // that fma recovers the product's rounding error
+        const float rev = (r_hi - floorf(r_hi)) + r_lo;
+        sn[j] = __builtin_amdgcn_sinf(rev);
+        cs[j] = __builtin_amdgcn_cosf(rev);
+      }
       sn[j] *= sign;
     }
-    const int h0 = hs * hper;
-    const int h1 = h0 + hper < heads ? h0 + hper : heads;
-    for (int h = h0; h < h1; ++h) {
-      const T *src;
-      T *dst;
-      if (h < hq) {
-        src = q + t * q_stride + (int64_t)h * d;
-        dst = qo + t * qo_stride + (int64_t)h * d;
-      } else {
-        src = k + t * k_stride + (int64_t)(h - hq) * d;
-        dst = ko + t * ko_stride + (int64_t)(h - hq) * d;
-      }
-      const Vec<T> lo = ldg(src + c * N);
-      const Vec<T> hi = ldg(src + half + c * N);
-      Vec<T> olo, ohi;
+    for (int hb = h0; hb < h1; hb += HG) {
+      if (hb != h0) load_group(hb);
 #pragma unroll
-      for (int j = 0; j < N; ++j) {
-        const float a = to_f(lo.v[j]), b = to_f(hi.v[j]);
-        olo.v[j] = from_f<T>(a * cs[j] - b * sn[j]);
-        ohi.v[j] = from_f<T>(b * cs[j] + a * sn[j]);
-      }
-      stg(dst + c * N, olo);
-      stg(dst + half + c * N, ohi);
+      for (int g = 0; g < HG; ++g)
+        if (hb + g < h1) {
+          Vec<T> olo, ohi;
+#pragma unroll
+          for (int j = 0; j < N; ++j) {
+            const float a = to_f(lo[g].v[j]), b = to_f(hi[g].v[j]);
+            olo.v[j] = from_f<T>(a * cs[j] - b * sn[j]);
+            ohi.v[j] = from_f<T>(b * cs[j] + a * sn[j]);
+          }
+          T *dst = dst_of(hb + g);
+          stg(dst + c * N, olo);
+          stg(dst + half + c * N, ohi);
+        }
     }
   }
 }

@@ -193,6 +193,24 @@ def test_wgrad_product(dtype, T, N, K, accumulate):
     assert_close(d2, ref, dtype, "wgrad_bwd")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rope_large_positions(dtype):
+    """Positions up to 2^19: the 16-bit path evaluates cos / sin with the hardware's routines after its own range
+    reduction, which must keep the fraction of a revolution exact although angle / 2 pi has only 7 fractional
+    bits left in fp32.  Against cos / sin in fp64 of the fp32 angle, the error is the rounding of the result."""
+    from dhellam_amd.operators.rope import rope_fwd, rope_inv_freq
+    T, d = 4096, 128
+    inv = rope_inv_freq(5e5, d, "cuda")
+    pos = (torch.arange(T, device="cuda", dtype=torch.int32) * 128 + 77)
+    ang = (pos.float()[:, None] * inv[None, :]).double()
+    ref = torch.cat([torch.cos(ang) - torch.sin(ang), torch.cos(ang) + torch.sin(ang)], 1)
+    q, k = torch.ones(T, 2, d, device="cuda", dtype=dtype), torch.ones(T, 1, d, device="cuda", dtype=dtype)
+    qo, ko, _ = rope_fwd(q, k, pos, 5e5, 0, None, False)
+    ulp = {torch.float32: 2.0 ** -22, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[dtype]
+    for got in (qo[:, 0], qo[:, 1], ko[:, 0]):
+        assert (got.double() - ref).abs().max().item() <= 0.51 * ulp + 2e-6
+
+
 def test_bandwidth_ops_are_deterministic():
     """Norm backward (staged column sums), SwiGLU, RoPE: two runs, same bits."""
     from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd

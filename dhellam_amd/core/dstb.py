@@ -119,6 +119,7 @@ class LayerConfig:
     # to and from the strand's own stream, instead of on the strand's stream itself
     comm_streams: Optional[tuple] = None
     fuse_adjacent: bool = True        # ops a plan lists next to each other run as one kernel where one exists (bda_attn + ln_mlp)
+    gather_in_place: bool = True      # the op in front of a sequence-parallel all-gather writes straight into its rows of the gathered buffer
     resident_weight_transposes: bool = True   # projection weights are kept as W and W^T: the data-gradient GEMMs then run in the forward's layout
 
     @property
@@ -183,24 +184,26 @@ class DCFunc:
 
     # ---- forward ----------------------------------------------------------------------
     @staticmethod
-    def ln_attn(config, data, stream):
+    def ln_attn(config, data, stream, out=None):
+        """``out``: where the result goes when it is not a new tensor (the rank's rows of the buffer that the
+        sequence-parallel all-gather after this op fills, so that the gather has nothing left to copy)."""
         input, ln_weight, ln_bias = data
         inputmat = input.view((-1, ln_weight.numel()))
         output, mu, rsigma, _ = pylayernorm_fwd(inputmat, ln_weight, ln_bias, config.layernorm_epsilon, 0, False,
-                                                stream, profiling=False)
+                                                stream, profiling=False, ln_out=out)
         return output, mu, rsigma, inputmat, input, output
 
     ln_mlp = ln_attn
 
     @staticmethod
-    def bda_attn_ln_mlp(config, data, stream):
+    def bda_attn_ln_mlp(config, data, stream, out=None):
         """``bda_attn`` and ``ln_mlp`` (dstb.py:273-277, 73-78), adjacent in the layer, in one kernel: the residual
         sum is written once and normalised from registers.  Returns (ln output, mu, rsigma, norm input as a
         matrix, the residual sum in the layer's [b, s/tp, h] shape)."""
         input, residual, ln_weight, ln_bias = data
         input = input.view(config.micro_batch_size, config.seq_length // config.tensor_model_parallel_size, -1)
         output, mu, rsigma, _, x2 = pylayernorm_fwd(input, ln_weight, ln_bias, config.layernorm_epsilon, 0, False,
-                                                    stream, profiling=False, residual=residual)
+                                                    stream, profiling=False, residual=residual, ln_out=out)
         x2 = x2.view(input.shape)
         return output.view(-1, ln_weight.numel()), mu, rsigma, x2.view(-1, ln_weight.numel()), x2
 
@@ -394,11 +397,11 @@ class DCFunc:
         return dqkv
 
     @staticmethod
-    def ln_mlp_bwd(config, data, stream):
+    def ln_mlp_bwd(config, data, stream, out=None):
         output, ln_input, ln_mu, ln_rsigma, ln_weight, ln_bias, residual, w_main_grad, b_main_grad = data
         dgrad, _, _, _ = pylayernorm_bwd(output, ln_input, ln_mu, ln_rsigma, ln_weight, 0, False, stream, False,
                                          add_to_dgrad=residual, dgamma_out=w_main_grad,
-                                         dbeta_out=b_main_grad if ln_mu is not None else None)
+                                         dbeta_out=b_main_grad if ln_mu is not None else None, dgrad_out=out)
         return dgrad
 
     @staticmethod
@@ -440,9 +443,10 @@ class DCFunc:
         dst = peer[config.tp_rank * rows:(config.tp_rank + 1) * rows]
         src = input.view(rows, -1)
         assert dst.is_contiguous() and src.is_contiguous() and dst.dtype == src.dtype and dst.shape == src.shape
-        st = stream if stream is not None else torch.cuda.current_stream()
-        _lib.check(_lib.load().dh_copy_bytes(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(),
-                                             st.cuda_stream))
+        if src.data_ptr() != dst.data_ptr():        # else the producer wrote the rows in place (an in-place gather)
+            st = stream if stream is not None else torch.cuda.current_stream()
+            _lib.check(_lib.load().dh_copy_bytes(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(),
+                                                 st.cuda_stream))
         return peer, None
 
     @staticmethod
@@ -488,12 +492,25 @@ class _Ctx:
         return _use(self.act[key], self.stream)
 
 
+def _gather_slot(c, gather_name):
+    """This rank's rows of the buffer that the stand-in all-gather ``gather_name`` fills, or None: the op in front
+    of the gather writes its result there, as the producer of an in-place all-gather does."""
+    cfg = c.config
+    tp = cfg.tensor_model_parallel_size
+    peer = c.act.get(_PEER_KEY[gather_name]) if c.act is not None else None
+    if tp == 1 or peer is None or not cfg.gather_in_place:
+        return None
+    rows = peer.shape[0] // tp
+    return _use(peer, c.stream)[cfg.tp_rank * rows:(cfg.tp_rank + 1) * rows]
+
+
 def _h_norm(c):
     p = "attn" if c.op == 1 else "mlp"
     fn = c.dcfunc.ln_attn if c.op == 1 else c.dcfunc.ln_mlp
     act = c.act
     output, act[f"{p}_mu"], act[f"{p}_rsigma"], act[f"ln_{p}_input"], act[f"ln_{p}_residual"], _ = fn(
-        c.config, (c.x, c.weight[f"ln_{p}_weight"], c.weight.get(f"ln_{p}_bias")), c.stream)
+        c.config, (c.x, c.weight[f"ln_{p}_weight"], c.weight.get(f"ln_{p}_bias")), c.stream,
+        out=_gather_slot(c, f"allgather_{p}"))
     return output
 
 
@@ -657,14 +674,17 @@ def _h_norm_bwd(c):
     mu = c.act.get(f"{p}_mu")
     data = (c.x, c.g(f"ln_{p}_input"), _use(mu, c.stream), c.g(f"{p}_rsigma"), lw, lb, c.g(f"{p}_residual_bwd"),
             lw.main_grad, lb.main_grad if lb is not None else None)
-    return (c.dcfunc.ln_mlp_bwd if c.op == 25 else c.dcfunc.ln_attn_bwd)(c.config, data, c.stream)
+    if c.op == 25:       # its result is what allgather_attn_bwd gathers (bda_attn_bwd in between passes it through)
+        return c.dcfunc.ln_mlp_bwd(c.config, data, c.stream, out=_gather_slot(c, "allgather_attn_bwd"))
+    return c.dcfunc.ln_attn_bwd(c.config, data, c.stream)
 
 
 def _h_bda_attn_ln_mlp(c):
     """bda_attn followed by ln_mlp in one column of a plan: what the two handlers would save, from one kernel."""
     act = c.act
     output, act["mlp_mu"], act["mlp_rsigma"], act["ln_mlp_input"], act["ln_mlp_residual"] = c.dcfunc.bda_attn_ln_mlp(
-        c.config, (c.x, c.g("ln_attn_residual"), c.weight["ln_mlp_weight"], c.weight.get("ln_mlp_bias")), c.stream)
+        c.config, (c.x, c.g("ln_attn_residual"), c.weight["ln_mlp_weight"], c.weight.get("ln_mlp_bias")), c.stream,
+        out=_gather_slot(c, "allgather_mlp"))
     act["attn_mask"] = None
     act.pop("ln_attn_residual", None)
     return output

@@ -26,10 +26,12 @@ def _workspace(nbytes: int, device, stream) -> torch.Tensor:
 
 
 def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_gamma, stream, profiling=False,
-                    residual=None, sum_out=None):
+                    residual=None, sum_out=None, ln_out=None):
     """Returns (ln_out, mu, rsigma, ms).  Extension over the reference signature: with ``residual`` the row that
     is normalised is ``inp + residual``, which is also stored in ``sum_out`` (default: a new tensor, returned
-    as a fifth value) -- the reference's bda op and the norm after it (dstb.py:273-277, 73-78) in one pass."""
+    as a fifth value) -- the reference's bda op and the norm after it (dstb.py:273-277, 73-78) in one pass.
+    ``ln_out``: a contiguous tensor of the input's size to write the result into (e.g. this rank's rows of the
+    buffer a sequence-parallel all-gather fills) instead of a new one."""
     in_features = ln_weight.numel()
     assert inp.is_cuda, "dhellam needs a GPU."
     assert inp.shape[-1] == in_features, "LayerNorm not possible"
@@ -39,7 +41,10 @@ def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_g
     rows = inputmat.shape[0]
     el: list = []
     with on_stream(stream, profiling, el) as st:
-        ln_out = torch.empty_like(inputmat)
+        if ln_out is None:
+            ln_out = torch.empty_like(inputmat)
+        else:
+            assert ln_out.is_contiguous() and ln_out.numel() == inputmat.numel() and ln_out.dtype == inputmat.dtype
         rsigma = torch.empty(rows, dtype=torch.float32, device=inp.device)
         mu = torch.empty(rows, dtype=torch.float32, device=inp.device) if ln_bias is not None else None
         if residual is None:
@@ -61,13 +66,14 @@ def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_g
 
 
 def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_centered_gamma, stream,
-                    profiling=False, add_to_dgrad=None, dgamma_out=None, dbeta_out=None):
+                    profiling=False, add_to_dgrad=None, dgamma_out=None, dbeta_out=None, dgrad_out=None):
     """Returns (dinp, dgamma, dbeta, ms).
 
     Extensions over the reference signature (all optional): ``add_to_dgrad`` is
     added to dinp inside the kernel (the residual-branch gradient the reference
     adds afterwards, dstb.py:391,401); ``dgamma_out`` / ``dbeta_out`` are
-    accumulated into in place (the reference's ``main_grad.add_``, dstb.py:392-393).
+    accumulated into in place (the reference's ``main_grad.add_``, dstb.py:392-393);
+    ``dgrad_out`` is a contiguous tensor of the input's size that receives dinp instead of a new one.
     """
     in_features = ln_weight.numel()
     assert inp.is_cuda, "dhellam needs a GPU."
@@ -79,7 +85,11 @@ def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_ce
     rows = inputmat.shape[0]
     el: list = []
     with on_stream(stream, profiling, el) as st:
-        dinp = torch.empty_like(inputmat)
+        if dgrad_out is None:
+            dinp = torch.empty_like(inputmat)
+        else:
+            assert dgrad_out.is_contiguous() and dgrad_out.numel() == inputmat.numel() and dgrad_out.dtype == inputmat.dtype
+            dinp = dgrad_out.view(inputmat.shape)
         accumulate = dgamma_out is not None
         assert not accumulate or dgamma_out.dtype == ln_weight.dtype, "dgamma_out must have the weight's dtype"
         assert dbeta_out is None or dbeta_out.dtype == ln_weight.dtype, "dbeta_out must have the weight's dtype"

@@ -159,7 +159,7 @@ def kernel_rooflines(cfg):
     dq, dk, dv = torch.empty_like(do), torch.empty(T, hk, d, device=dev, dtype=dt), torch.empty(T, hk, d, device=dev, dtype=dt)
     bw = lambda: _Clib._attn_bwd_raw(do, q, k, v, out_l[0], out_l[5], dq, dk, dv, None, cu, cu, T, T, sc, True, sp)
     ms_bwd = time_gpu(bw)
-    add(f"attn_bwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", 2.5 * fl_fwd, ms_bwd, "2.5 * fwd flop (dQ incl. delta, dK/dV and head-split sum kernels)")
+    add(f"attn_bwd[causal S={T} {hq}q/{hk}kv d={d}]", "mfma", 2.5 * fl_fwd, ms_bwd, "2.5 * fwd flop (delta, dK/dV keeping dS, head-split sum and dQ-from-dS kernels)")
     # --- ring step (32q/8kv, d=128, q 4096, kv chunk 4096): one causal and one full-block step -------
     hq1, hk1, S1 = 32, 8, 4096
     q1, k1, v1, do1 = rn(S1, hq1, d), rn(S1, hk1, d), rn(S1, hk1, d), rn(S1, hq1, d)

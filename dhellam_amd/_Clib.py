@@ -357,6 +357,15 @@ def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
 _bwd_ws: dict = {}
 
 
+ATTN_BWD_DS_LIMIT_DEFAULT = 1280 << 20
+
+
+def set_attn_bwd_ds_limit(nbytes: int = ATTN_BWD_DS_LIMIT_DEFAULT) -> None:
+    """Workspace bytes up to which the attention backward keeps dS for its dQ product (``dh_attn_bwd_set_ds_limit``;
+    0: always recompute).  Process-wide."""
+    _lib.load().dh_attn_bwd_set_ds_limit(int(nbytes))
+
+
 def _attn_bwd_workspace(nbytes: int, device, stream_ptr: int) -> torch.Tensor:
     key = (str(device), stream_ptr)
     ws = _bwd_ws.get(key)

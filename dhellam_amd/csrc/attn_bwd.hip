@@ -19,6 +19,8 @@
 //             dS^T feeds dQ^T += K^T dS^T.
 // Recomputing S and dP in both passes costs 7 matrix products instead of 5 but
 // needs no fp32 dQ accumulator in memory and no atomics.
+#include <atomic>
+
 #include "mma.h"
 
 
@@ -42,6 +44,12 @@ struct AttnBwdParams {
   float scale, scale_log2;
   int causal;
   int dq_accumulate;         // dq += this call's gradient (read, add in fp32, round once) instead of dq =
+  // dS = P * (dP - delta) kept for the dQ product (head dim 128, 16 bits, when the workspace allows): 2 KB blocks of
+  // 32 keys x 32 query rows, block (b, h, query tile, key block); inside a block the 16-byte piece (s, hh, key)
+  // holds the query rows 16 s + 8 u + 4 hh + x of that key (u = 0, 1; x = 0..3): what a lane of the dK/dV kernel
+  // has in its packed dS fragment s.
+  void *ds;
+  int ds_nqt, ds_nkb;        // query tiles and key blocks (of 32) per (batch, head)
 };
 
 // ---- delta = rowsum(dO * O) ---------------------------------------------------------------
@@ -773,6 +781,236 @@ __global__ void __launch_bounds__(512) attn_bwd_dq_d128_kernel(const AttnBwdPara
   }
 }
 
+// dQ from the dS blocks that the dK/dV kernel left in the workspace: dQ^T[d, q] += K^T[d, key] dS^T[key, q], one
+// matrix product instead of the three of the recomputing kernel above (which stays for shapes whose dS would not
+// fit the workspace).  Same workgroup shape: 2 query row groups x 4 key splits, 32-key steps, the splits' partial
+// sums added through LDS in split order.  A step needs the K tile of its split (8 KB, swizzled rows, transpose
+// reads as above) and one 2 KB dS block per row group, copied as it lies in memory; its transpose reads pick,
+// for a 16-lane group of query columns, the 8-byte pieces (u, hh) of four consecutive keys, which puts query
+// row n of the tile on lane n.  The kernel streams 2 bytes of dS per 256 flops: it is bound by memory.
+template <typename T>
+__global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int D = 128, RG = 2, SPLIT = 4, BN = 32, BM = 32 * RG, NS = BN / 16;
+  constexpr int TILE = BN * D;                         // elements of one K tile
+  constexpr int TILEB = TILE * (int)sizeof(T);
+  constexpr int SLOTB = SPLIT * TILEB;                 // the K tiles of all splits: one stage
+  constexpr int DSB = RG * 2048;                       // the dS blocks of one split (one per row group)
+  constexpr int DSLOTB = SPLIT * DSB;
+  constexpr int NST = 3;                               // stages: the copies of a step go out two steps ahead of it
+  __shared__ __attribute__((aligned(1024))) char sAll[NST * SLOTB + NST * DSLOTB];   // 144 KB
+
+  const int b = blockIdx.y;
+  // a head's dS blocks were written from one XCD (the dK/dV kernel keeps a head group there): read them from the
+  // same one; the K rows of the kv head are small next to them
+  const int ratio = p.hq / p.hk, P = gridDim.x / p.hq;
+  int h, px;
+  xcd_group_item(blockIdx.x, p.hq, P, h, px);
+  const int hkv = h / ratio;
+  const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
+  const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
+  const int nqt = (sq + BM - 1) / BM;
+  const int causal = p.causal;
+  const int k_stride = (int)p.k_stride;
+  int qt[2], nq;
+  if (causal) {
+    if (2 * px >= nqt) return;
+    qt[0] = nqt - 1 - px; qt[1] = px;
+    nq = (qt[0] == qt[1]) ? 1 : 2;
+  } else {
+    if (px >= nqt) return;
+    qt[0] = px; qt[1] = 0; nq = 1;
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, hh = lane >> 5;
+  const int rg = w % RG, sp = w / RG;
+  const T *kg = reinterpret_cast<const T *>(p.k) + (int64_t)k0 * p.k_stride + (int64_t)hkv * D;
+  const char *kg_b = reinterpret_cast<const char *>(kg);
+  const uint32_t ldsK = (uint32_t)(uintptr_t)sAll, ldsD = ldsK + NST * SLOTB;
+
+  // ---- copies of wavefront w: rows [16 half, 16 half + 16) of the K tile of split w / 2 (four 1 KB blocks) and the
+  // dS block of row group `half` of that split (two 1 KB blocks) -------------------------------------------------
+  CopyLane cl0;
+  cl0.l16 = lane & 15;
+  cl0.lrow = lane >> 4;
+  const int csp = w >> 1, half = w & 1;
+  const uint32_t cp_step = (uint32_t)(4 * k_stride) * (uint32_t)sizeof(T);
+  uint32_t cp_off[4];
+  {
+    const uint32_t rowb = (uint32_t)(cl0.lrow * k_stride) * (uint32_t)sizeof(T);
+    const uint32_t chunk = (uint32_t)(cl0.l16 ^ (4 * cl0.lrow)) << 4;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
+  }
+  const uint32_t ds_lane = (uint32_t)lane * 16u;
+  const int64_t ds_head = ((int64_t)b * p.hq + h) * p.ds_nqt;
+  const char *ds_b = reinterpret_cast<const char *>(p.ds);
+
+  // ---- fragment reads ------------------------------------------------------------------------------------------
+  const int r = lane & 15;
+  const int ta_x = 4 * (r >> 2) + hh;                 // transpose reads of K: swz of rows 4*hh + r/4 (+8)
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r & 3) >> 1);
+  const uint32_t t_row = (uint32_t)(sp * TILEB + (4 * hh + (r >> 2)) * 256 + ((r & 3) & 1) * 8);
+  const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
+  const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
+  // dS block: piece (s = 16-lane group, hh_p = r % 2) of key 4 hh + r / 4, half u = (r % 4) / 2 of the piece
+  const uint32_t db_lane = (uint32_t)(sp * DSB + rg * 2048 + ((((lane >> 4) & 1) * 64 + (r & 1) * 32 + 4 * hh + (r >> 2)) * 16) +
+                                      ((r & 3) >> 1) * 8);
+
+  for (int qi = 0; qi < nq; ++qi) {
+    const int m0 = qt[qi] * BM;
+    const int wrow0 = m0 + rg * 32;
+    const int row_q = wrow0 + c;
+    const bool row_ok = row_q < sq;
+    int nk_end = sk;
+    if (causal && m0 + BM < nk_end) nk_end = m0 + BM;
+    const int ntiles = (nk_end + BN - 1) / BN;
+    const int niter = (ntiles + SPLIT - 1) / SPLIT;
+    const int n_fast = sk / (SPLIT * BN);          // iterations whose K tiles lie wholly inside the keys
+    const int64_t ds_row = (ds_head + (m0 >> 5) + half) * p.ds_nkb;   // the copied block row: query tile of row group `half`
+
+    floatx16 dQt[D / 32];
+#pragma unroll
+    for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dQt[t][v] = 0.f;
+
+    auto issue = [&](int it) {
+      const int tile = it * SPLIT + csp;
+      if (tile >= ntiles) return;
+      const uint32_t stK = (uint32_t)((it % NST) * SLOTB), stD = (uint32_t)((it % NST) * DSLOTB);
+      if (it < n_fast) {
+        const char *src = kg_b + (int64_t)(tile * BN + 16 * half) * k_stride * (int)sizeof(T);
+        uint32_t dst = ldsK + stK + (uint32_t)(csp * TILEB + 16 * half * 256);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          dma_block_fast(src, cp_off[x], dst);
+          src += cp_step;
+          dst += 1024;
+        }
+      } else {
+        dma_tile32_general<T, 4>(reinterpret_cast<T *>(sAll + stK + csp * TILEB) + 16 * half * D, kg, k_stride, 1,
+                                 tile * BN + 16 * half, 16 * half, sk, cl0);
+      }
+      const char *dsrc = ds_b + (ds_row + tile) * 2048;
+      const uint32_t ddst = ldsD + stD + (uint32_t)(csp * DSB + half * 2048);
+      dma_block_fast(dsrc, ds_lane, ddst);
+      dma_block_fast(dsrc + 1024, ds_lane, ddst + 1024);
+    };
+
+    // Steps 0 and 1 go out now; in the loop, step it + 2 goes out at the top of step it and the wait at the bottom
+    // leaves the newest step's copies in flight (6 per wavefront, or none: vmcnt counts in issue order).
+    if (niter > 0) issue(0);
+    if (niter > 1) issue(1);
+    if (niter > 1 && 1 * SPLIT + csp < ntiles && 1 < n_fast) {
+      asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
+      dma_wait_all();
+      __syncthreads();
+    }
+
+#pragma unroll 1
+    for (int it = 0; it < niter; ++it) {
+      if (it + 2 < niter) issue(it + 2);              // has two steps to land
+      const int tile_g = it * SPLIT + sp;
+      const int n0 = tile_g * BN;
+      const bool act = tile_g < ntiles && !(causal && n0 > wrow0 + 31);
+      if (act) {
+        const uint32_t curK = ldsK + (uint32_t)((it % NST) * SLOTB), curD = ldsD + (uint32_t)((it % NST) * DSLOTB);
+        uint32_t ta = curK + ta_lane, tb = curK + tb_lane, db = curD + db_lane;
+        asm volatile("" : "+v"(ta), "+v"(tb), "+v"(db));
+        // LDS reads in assembly (the compiler would hold them behind every copy in flight): the four dS pieces,
+        // the K^T fragments of the first 16 keys, then those of the second while the first multiply
+        uint32_t ad[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          ad[2 * t] = ta ^ (uint32_t)(t << 6);
+          ad[2 * t + 1] = tb ^ (uint32_t)(t << 6);
+        }
+        short4v bq[4], f0[8], f1[8];
+        lds_read_tr4<128>(bq, db);
+        lds_read_tr8<0>(f0, ad);
+        lds_wait<4>(bq[0], bq[1], bq[2], bq[3]);
+        lds_wait<4>(f0[0], f0[1], f0[2], f0[3]);
+        lds_read_tr8<16 * 256>(f1, ad);
+        const Frag dS0 = frag_join<T>(bq[0], bq[1]), dS1 = frag_join<T>(bq[2], bq[3]);
+        dQt[0] = M::mma(frag_join<T>(f0[0], f0[1]), dS0, dQt[0]);
+        dQt[1] = M::mma(frag_join<T>(f0[2], f0[3]), dS0, dQt[1]);
+        lds_wait<8>(f0[4], f0[5], f0[6], f0[7]);
+        dQt[2] = M::mma(frag_join<T>(f0[4], f0[5]), dS0, dQt[2]);
+        dQt[3] = M::mma(frag_join<T>(f0[6], f0[7]), dS0, dQt[3]);
+        lds_wait<4>(f1[0], f1[1], f1[2], f1[3]);
+        dQt[0] = M::mma(frag_join<T>(f1[0], f1[1]), dS1, dQt[0]);
+        dQt[1] = M::mma(frag_join<T>(f1[2], f1[3]), dS1, dQt[1]);
+        lds_wait<0>(f1[4], f1[5], f1[6], f1[7]);
+        dQt[2] = M::mma(frag_join<T>(f1[4], f1[5]), dS1, dQt[2]);
+        dQt[3] = M::mma(frag_join<T>(f1[6], f1[7]), dS1, dQt[3]);
+      }
+      // step it + 1 must have landed; the copies of step it + 2 (the newest 6 of this wavefront, if it issued them
+      // in the fast form) may stay in flight
+      // (__syncthreads() would drain them: it waits for every memory operation before its barrier)
+      if (it + 2 < niter && (it + 2) * SPLIT + csp < ntiles && it + 2 < n_fast) {
+        asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      } else {
+        dma_wait_all();
+        __syncthreads();
+      }
+    }
+
+    // add the splits' partial dQ through LDS, in split order: slot x = (s-1)*RG + g, 16 KB each
+    float *xo = reinterpret_cast<float *>(sAll);
+    static_assert(sizeof(sAll) >= (size_t)(SPLIT - 1) * RG * 4096 * sizeof(float), "exchange area");
+    if (sp > 0) {
+      float *dst = xo + ((sp - 1) * RG + rg) * 4096;
+#pragma unroll
+      for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(t * 16 + v) * 64 + lane] = dQt[t][v];
+    }
+    __syncthreads();
+    if (sp == 0) {
+#pragma unroll
+      for (int s2 = 1; s2 < SPLIT; ++s2) {
+        const float *src = xo + ((s2 - 1) * RG + rg) * 4096;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) dQt[t][v] += src[(t * 16 + v) * 64 + lane];
+      }
+      if (row_ok) {
+        T *dqp = reinterpret_cast<T *>(p.dq) + (int64_t)(q0 + row_q) * p.dq_stride + (int64_t)h * D;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t)
+#pragma unroll
+          for (int vb = 0; vb < 4; ++vb) {
+            struct alignas(8) { T v[4]; } a;
+            if (p.dq_accumulate) {
+              a = *reinterpret_cast<const decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(static_cast<float>(a.v[e]) + dQt[t][4 * vb + e] * p.scale);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) a.v[e] = static_cast<T>(dQt[t][4 * vb + e] * p.scale);
+            }
+            *reinterpret_cast<decltype(a) *>(dqp + 32 * t + 8 * vb + 4 * hh) = a;
+          }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+static int launch_dq2_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
+  constexpr int BM = 64;
+  const int nqt = (int)cdiv(p.max_sq, BM);
+  dim3 grid((unsigned)((p.causal ? (nqt + 1) / 2 : nqt) * p.hq), (unsigned)batch);
+  hipLaunchKernelGGL((attn_bwd_dq2_d128_kernel<T>), grid, dim3(512), 0, st, p);
+  return DH_OK;
+}
+
 template <typename T, int RG, int SPLIT, int BN>
 static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * RG;
@@ -791,7 +1029,7 @@ static int launch_dq_d128(const AttnBwdParams &p, int batch, hipStream_t st) {
 // order.  Causal: the workgroup owns key tiles j and n-1-j, so every workgroup does the same amount of
 // work.  The main loop is one rolled body; the Q / dO tiles of the next iteration come in with assembly
 // copies (scalar bases) issued between the matrix instructions.
-template <typename T>
+template <typename T, bool STORE_DS>
 __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
@@ -1001,12 +1239,13 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
             DH_DKV_COPY(ks);                          // one copy block per step: all eight are out before the softmax
           }
         }
-        if ((causal && i0 < jw0 + 31) || (i0 + BM > sq)) {
-          // masked scores become -inf, i.e. P = dS = 0 (lse and delta of rows past the sequence end are zeros)
+        if ((causal && i0 < jw0 + 31) || (i0 + BM > sq) || (STORE_DS && jw0 + 32 > sk)) {
+          // masked scores become -inf, i.e. P = dS = 0 (lse and delta of rows past the sequence end are zeros);
+          // keys past the end matter only when dS is kept: the dQ product would meet them
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int i = i0 + acc_row(v, hh);
-            if (i >= sq || (causal && jrow > i)) S[v] = -INFINITY;
+            if (i >= sq || (causal && jrow > i) || (STORE_DS && jrow >= sk)) S[v] = -INFINITY;
           }
         }
         Frag Pb[2], dSb[2];
@@ -1026,6 +1265,15 @@ __global__ void __launch_bounds__(512) attn_bwd_dkv_d128_kernel(const AttnBwdPar
           }
           Pb[s] = frag_pack<T>(pv);
           dSb[s] = frag_pack<T>(dsv);
+        }
+        if (STORE_DS) {
+          // the packed dS fragments go out as they are, 1 KB per fragment and wavefront
+          const int64_t blk = (((int64_t)b * p.hq + (h_first + g)) * p.ds_nqt + (i0 >> 5)) * p.ds_nkb + (jw0 >> 5);
+          int lx = lane;
+          asm volatile("" : "+v"(lx));
+          Frag *dst = reinterpret_cast<Frag *>(reinterpret_cast<char *>(p.ds) + blk * 2048) + lx;
+          dst[0] = dSb[0];
+          dst[64] = dSb[1];
         }
         if (have_next) load_ld(gn, tn);               // next tile's lse / delta, in flight across the barrier
         // dV^T += dO^T P and dK^T += Q^T dS; the eight copy blocks of this wavefront go out in between.
@@ -1144,7 +1392,8 @@ template <typename T>
 static int launch_dkv_d128(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
   const int nkt = (int)cdiv(max_sk, 64);
   dim3 grid((unsigned)((p.causal ? (nkt + 1) / 2 : nkt) * p.hk * p.hsplit), (unsigned)batch);
-  hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T>), grid, dim3(512), 0, st, p);
+  if (p.ds) hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T, true>), grid, dim3(512), 0, st, p);
+  else hipLaunchKernelGGL((attn_bwd_dkv_d128_kernel<T, false>), grid, dim3(512), 0, st, p);
   return DH_OK;
 }
 
@@ -1216,7 +1465,32 @@ int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, 
 
 constexpr int DKV_NW = 2;  // wavefronts per dK/dV workgroup (64 key rows)
 
+// Keeping dS for the dQ product costs 2 bytes per (head, query, key) of workspace, written once and read once.
+// It pays where the recomputing dQ kernel runs its small-grid form (fewer than 256 workgroups of 128 query rows:
+// the 8-head shard at 4096 tokens 181 -> 155 us, at 2048 tokens 95 -> 80 us); with the chip full the recomputing
+// kernel is the faster one (32 heads x 4096: 610 against 669 us; 16 heads: 321 against 329), as the extra
+// memory traffic then costs more than the two products saved.  Above the byte limit dS is never kept.
+static std::atomic<size_t> g_ds_limit{(size_t)1280 << 20};
+
+// Whether the recomputing dQ kernel would fill the chip (its 128-row form).
+static bool dq_big_grid(int batch, int max_sq, int hq, int causal) {
+  const int64_t t = cdiv(max_sq, 128);
+  return (causal ? (t + 1) / 2 : t) * hq * batch >= 256;
+}
+
+// Bytes of the dS blocks for these sizes (key count as an upper bound of the longest sequence), 0 if not kept.
+static size_t ds_bytes(int batch, int max_sq, int64_t max_sk, int hq, int d, int dtype, int causal) {
+  if (dtype == DH_F32 || d != 128 || batch <= 0 || max_sq <= 0 || max_sk <= 0) return 0;
+  if (dq_big_grid(batch, max_sq, hq, causal)) return 0;
+  // one block more per row than needed: rows a power of two apart would meet on the same memory channels
+  const size_t nqt = 2 * (size_t)cdiv(max_sq, 64), nkb = 2 * (size_t)cdiv(max_sk, 64) + 1;
+  const size_t n = (size_t)batch * hq * nqt * nkb * 2048;
+  return n <= g_ds_limit.load() ? n : 0;
+}
+
 }  // namespace dh
+
+extern "C" void dh_attn_bwd_set_ds_limit(size_t bytes) { dh::g_ds_limit.store(bytes); }
 
 extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch, int max_seqlen_q, int hq,
                                               int hk, int d, int dtype) {
@@ -1226,6 +1500,9 @@ extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, 
   size_t n = plane;                               // delta
   const size_t plane2 = align256((size_t)batch * hq * (size_t)(((max_seqlen_q > 0 ? max_seqlen_q : 0) + 31) / 32 * 32) * sizeof(float));
   if (dtype != DH_F32 && d == 128) n += 2 * plane2;  // lse (exp2 units) and delta side by side for the d = 128 kernels
+  // dS blocks, if a call of these sizes may keep them (causal or not is not known here: the causal grid is the smaller
+  // one; the longest sequence has at most total_k keys)
+  n += align256(ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, 1));
   if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
     n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
   return n + 256;
@@ -1263,8 +1540,14 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
   DH_CHECK(d % n == 0 || dtype == DH_F32, "head dim %d must be a multiple of %d", d, n);
   DH_CHECK(do_stride % n == 0 && o_stride % n == 0 && aligned16(dout) && aligned16(out),
            "dout/out rows must be 16-byte aligned");
-  // head dim 128 in 16 bits: the dQ kernel forms delta itself (and runs first); everything else uses the delta kernel
-  const bool delta_in_dq = dtype != DH_F32 && d == 128;
+  // head dim 128 in 16 bits, two ways: with room for dS in the workspace the dK/dV kernel keeps it and dQ is one
+  // product over it (delta from the delta kernel, which runs first); otherwise the dQ kernel recomputes S and dP,
+  // forms delta itself and runs first.  Everything else uses the delta kernel.
+  const size_t dsb = ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, causal);
+  const bool keep_ds = dsb > 0 && max_seqlen_k > 0;
+  uint8_t *ds_ws = ws;
+  ws += align256(dsb);
+  const bool delta_in_dq = dtype != DH_F32 && d == 128 && !keep_ds;
   if (max_seqlen_q > 0 && !delta_in_dq) {
     DH_DISPATCH_DTYPE(dtype, {
       launch_delta<T>(dout, out, delta, lse, ld2, (int64_t)(plane2 / sizeof(float)), ld2_pitch, cu_seqlens_q, batch, max_seqlen_q, hq, d,
@@ -1297,6 +1580,9 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.causal = causal;
   p.dq_accumulate = dq_accumulate ? 1 : 0;
+  p.ds = keep_ds ? (void *)ds_ws : nullptr;
+  p.ds_nqt = 2 * (int)cdiv(max_seqlen_q, 64);
+  p.ds_nkb = 2 * (int)cdiv(max_seqlen_k < total_k ? max_seqlen_k : total_k, 64) + 1;
   p.hsplit = pick_hsplit(d == 128 && causal ? (max_seqlen_k + 1) / 2 : max_seqlen_k, batch, hq, hk, 32 * DKV_NW);
   p.dk_part = nullptr;
   p.dv_part = nullptr;
@@ -1306,13 +1592,13 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
     p.dv_part = (float *)(ws + part);
   }
   const bool small_q = cdiv(max_seqlen_q, 128) * hq * batch < 2 * 256;
-  const bool big_q = (causal ? (cdiv(max_seqlen_q, 128) + 1) / 2 : cdiv(max_seqlen_q, 128)) * hq * batch >= 256;
+  const bool big_q = dq_big_grid(batch, max_seqlen_q, hq, causal);
   DH_CHECK(k_stride < (1ll << 31) && v_stride < (1ll << 31) && q_stride < (1ll << 31) && do_stride < (1ll << 31),
            "token stride too large");
   int rc = DH_OK;
 #define DH_BWD(TT, DD)                                                                         \
   do {                                                                                         \
-    if (DD == 128 && max_seqlen_q > 0)                                                         \
+    if (DD == 128 && max_seqlen_q > 0 && !keep_ds)                                             \
       rc = big_q ? launch_dq_d128<TT, 4, 2, 32>(p, batch, st) : launch_dq_d128<TT, 2, 4, 32>(p, batch, st); \
     if (rc == DH_OK && max_seqlen_k > 0)                                                       \
       rc = DD == 128 ? launch_dkv_d128<TT>(p, batch, max_seqlen_k, st) : launch_dkv<TT, DD, DKV_NW>(p, batch, max_seqlen_k, st); \
@@ -1324,6 +1610,7 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
     }                                                                                          \
     if (rc == DH_OK && max_seqlen_q > 0 && DD != 128)                                          \
       rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st);  \
+    if (rc == DH_OK && max_seqlen_q > 0 && DD == 128 && keep_ds) rc = launch_dq2_d128<TT>(p, batch, st); \
   } while (0)
   if (dtype == DH_BF16) {
     if (d == 128) DH_BWD(bf16_t, 128); else DH_BWD(bf16_t, 64);

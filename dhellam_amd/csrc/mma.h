@@ -168,6 +168,14 @@ template <int OFF> __device__ __forceinline__ void lds_read_tr8(short4v (&f)[8],
                : "v"(ad[0]), "v"(ad[1]), "v"(ad[2]), "v"(ad[3]), "v"(ad[4]), "v"(ad[5]), "v"(ad[6]), "v"(ad[7]), "n"(OFF)
                : "memory");
 }
+// Four transpose reads from one lane address plus the byte offsets 0, S, 2 S, 3 S.
+template <int S> __device__ __forceinline__ void lds_read_tr4(short4v (&f)[4], uint32_t addr) {
+  asm volatile("ds_read_b64_tr_b16 %0, %4\n\tds_read_b64_tr_b16 %1, %4 offset:%5\n\t"
+               "ds_read_b64_tr_b16 %2, %4 offset:%6\n\tds_read_b64_tr_b16 %3, %4 offset:%7"
+               : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3])
+               : "v"(addr), "n"(S), "n"(2 * S), "n"(3 * S)
+               : "memory");
+}
 template <int N> __device__ __forceinline__ void lds_wait(int4v &d) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(d) : "n"(N));
 }

@@ -143,6 +143,17 @@ size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
                                    int max_seqlen_q, int hq, int hk, int d,
                                    int dtype);
 
+/* Head dim 128 in 16 bits, calls too small to fill the chip with 128-row
+ * query tiles (fewer than 256 of them, halved for causal): when 2 bytes per
+ * (head, query, key) fit into this many bytes of workspace (default 1280 MiB)
+ * the backward keeps dS = P * (dP - delta) from its dK/dV pass and forms dQ
+ * from it in one product; otherwise (0: never) its dQ pass recomputes S and dP
+ * and needs no such space.  No counterpart in the reference (flash-attention
+ * always recomputes); a process-wide setting, read by
+ * dh_attn_bwd_workspace_bytes and dh_attn_bwd alike: change it only between a
+ * sizing call and the calls it sizes for. */
+void dh_attn_bwd_set_ds_limit(size_t bytes);
+
 /* dq like q, dk/dv like k/v (GQA groups are reduced inside the kernel; the
  * reference sums an expanded buffer afterwards, flash_atten.cu:646-652).
  * delta_out (fp32 [b, hq, max_seqlen_q], may be NULL) receives rowsum(dO*O),

@@ -67,6 +67,15 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     return out, lse, dq, dk, dv
 
 
+@pytest.fixture(params=[True, False], ids=["keep_ds", "recompute"])
+def ds_path(request):
+    """Head dim 128 has two backward paths: dQ from the dS that the dK/dV pass keeps, or from recomputed S and dP."""
+    from dhellam_amd import _Clib
+    _Clib.set_attn_bwd_ds_limit(_Clib.ATTN_BWD_DS_LIMIT_DEFAULT if request.param else 0)
+    yield request.param
+    _Clib.set_attn_bwd_ds_limit()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("lens_q,lens_k,hq,hk,d,causal", [
     ([1024], [1024], 8, 1, 128, True),          # the 70B shard's head layout, shortened
@@ -80,8 +89,41 @@ def _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal, oracle_dtype=torch.fl
     ([128] * 4, [512] * 4, 64, 16, 128, False),  # many kv heads: two query heads per dK/dV workgroup
     ([0, 65, 33], [0, 65, 33], 4, 2, 128, True),   # an empty sequence in the batch
 ])
-def test_attention_16bit(dtype, lens_q, lens_k, hq, hk, d, causal):
+def test_attention_16bit(dtype, lens_q, lens_k, hq, hk, d, causal, ds_path):
+    if d != 128 and not ds_path:
+        pytest.skip("one backward path at this head dim")
     _run_fwd_bwd(dtype, lens_q, lens_k, hq, hk, d, causal)
+
+
+@pytest.mark.parametrize("lens_q,lens_k,hq,hk,causal", [
+    ([1024], [1024], 8, 1, True), ([100, 257, 64, 1], [100, 257, 64, 1], 4, 2, True), ([300, 40], [200, 97], 4, 2, False),
+    ([2048], [1000], 8, 2, False),
+])
+def test_attention_backward_paths_agree(lens_q, lens_k, hq, hk, causal):
+    """The two backward paths at head dim 128 on the same inputs: dV comes from the same kernel arithmetic
+    (bit-identical); dK and dQ use delta = rowsum(dO * O), which the two paths sum in a different order (the delta
+    kernel / the prologue of the recomputing dQ kernel), so a few of their elements differ in the last place."""
+    from dhellam_amd import _Clib
+    dtype, d = torch.bfloat16, 128
+    cq, ck = _cu(lens_q).cuda(), _cu(lens_k).cuda()
+    tq, tk, mq, mk = sum(lens_q), sum(lens_k), max(lens_q), max(lens_k)
+    scale = 1.0 / math.sqrt(d)
+    q, k, v, do = (randn((t, h, d), dtype, 30 + i).cuda() for i, (t, h) in enumerate(((tq, hq), (tk, hk), (tk, hk), (tq, hq))))
+    res = _Clib.pymha_varlen_fwd(q, k, v, cq, ck, mq, mk, 0.0, scale, causal, False, 0, False)
+    out, lse = res[0], res[5]
+    sp = torch.cuda.current_stream().cuda_stream
+    got = []
+    try:
+        for limit in (_Clib.ATTN_BWD_DS_LIMIT_DEFAULT, 0):
+            _Clib.set_attn_bwd_ds_limit(limit)
+            dq, dk, dv = torch.full_like(q, float("nan")), torch.full_like(k, float("nan")), torch.full_like(v, float("nan"))
+            _Clib._attn_bwd_raw(do, q, k, v, out, lse, dq, dk, dv, None, cq, ck, mq, mk, scale, causal, sp)
+            got.append((dq, dk, dv))
+    finally:
+        _Clib.set_attn_bwd_ds_limit()
+    assert torch.equal(got[0][2], got[1][2])
+    assert_close(got[0][1], got[1][1].double().cpu(), dtype, "dk of the two paths", scale=0.25)
+    assert_close(got[0][0], got[1][0].double().cpu(), dtype, "dq of the two paths", scale=0.25)
 
 
 def test_attention_packed_qkv_views():
@@ -105,7 +147,7 @@ def test_attention_fp32(lens_q, lens_k, hq, hk, d, causal):
 
 @pytest.mark.parametrize("dtype,hq,hk,d", [(torch.bfloat16, 4, 2, 128), (torch.float16, 32, 8, 128), (torch.bfloat16, 2, 2, 64),
                                          (torch.float32, 2, 1, 32)])
-def test_attention_backward_accumulates_dq(dtype, hq, hk, d):
+def test_attention_backward_accumulates_dq(dtype, hq, hk, d, ds_path):
     """dh_attn_bwd_acc with accumulate_dq: dq += the call's gradient (one rounding of the fp32 sum); dk, dv and a
     call without the flag are those of dh_attn_bwd."""
     from dhellam_amd import _Clib

@@ -228,15 +228,22 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
 # kernel) must call ``keep_transposed(weight, refresh=True)`` itself; weights that were never registered take the NN
 # product as before.
 def keep_transposed(weight: torch.Tensor, refresh: bool = False) -> Optional[torch.Tensor]:
-    """Registers ``weight`` [N, K] for a resident transpose [K, N] (built now, on the current stream) and returns
-    it; None if the tensor is not one ``dh_transpose_2d`` takes (then nothing is registered)."""
-    if not (weight.is_cuda and _can_transpose(weight)):
+    """Registers ``weight`` [N, K] (or a stack of them, [G, N, K]: the experts of a rank) for a resident transpose
+    [K, N] ([G, K, N]) built now, on the current stream, and returns it; None if the tensor is not one
+    ``dh_transpose_2d`` takes (then nothing is registered)."""
+    if not (weight.is_cuda and weight.dim() in (2, 3) and weight.is_contiguous() and _can_transpose(weight[0] if weight.dim() == 3 else weight)):
         return None
     held = getattr(weight, "_dh_transposed", None)
     if held is not None and not refresh and held[0] == weight._version:
         return held[1]
     with torch.no_grad():
-        wt = transpose_2d(weight.detach(), held[1] if held is not None else None)
+        w = weight.detach()
+        if w.dim() == 2:
+            wt = transpose_2d(w, held[1] if held is not None else None)
+        else:
+            wt = held[1] if held is not None else torch.empty((w.shape[0], w.shape[2], w.shape[1]), dtype=w.dtype, device=w.device)
+            for g in range(w.shape[0]):
+                transpose_2d(w[g], wt[g])
     stream = torch.cuda.current_stream()
     ev = torch.cuda.Event()
     ev.record(stream)

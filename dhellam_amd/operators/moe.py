@@ -14,6 +14,7 @@ from dataclasses import dataclass
 import torch
 
 from .. import _lib
+from .._Clib import transposed_of
 from ._util import on_stream
 
 
@@ -193,9 +194,12 @@ def expert_ffn_bwd(dy, xp, w1, w2, offs, saved, dw1=None, dw2=None, stream=None,
     h, a = saved
     el: list = []
     with on_stream(stream, profiling, el) as st:
-        da = grouped_gemm_nn(dy, w2, offs, stream=st)                    # [R, F] = dy @ w2[g]
+        # data gradients: against the resident transposes of the expert weights where the caller keeps them
+        # (``_Clib.keep_transposed``): the same products in the forward's layout, which the grouped kernel runs faster
+        w2t, w1t = transposed_of(w2), transposed_of(w1)
+        da = grouped_gemm_nt(dy, w2t, offs, stream=st) if w2t is not None else grouped_gemm_nn(dy, w2, offs, stream=st)   # [R, F] = dy @ w2[g]
         dw2 = grouped_gemm_tn(dy, a, offs, out=dw2, accumulate=dw2 is not None, stream=st)   # [G, H, F]
         dh, _ = swiglu_back(da, h, None, st)
-        dxp = grouped_gemm_nn(dh, w1, offs, stream=st)                   # [R, H] = dh @ w1[g]
+        dxp = grouped_gemm_nt(dh, w1t, offs, stream=st) if w1t is not None else grouped_gemm_nn(dh, w1, offs, stream=st)   # [R, H] = dh @ w1[g]
         dw1 = grouped_gemm_tn(dh, xp, offs, out=dw1, accumulate=dw1 is not None, stream=st)  # [G, 2F, H]
     return dxp, dw1, dw2, el[0]

@@ -295,3 +295,23 @@ def test_sort_leaves_out_expert_ids_outside_the_range():
     dest = plan.dest_row.cpu().numpy()
     assert (dest[~keep] == -1).all()
     assert np.array_equal(dest[order], np.arange(n_good))
+
+def test_expert_ffn_bwd_with_resident_weight_transposes():
+    """Expert weights registered with keep_transposed: the data gradients run as NT products against [G, K, N]
+    copies and give the bits of the NN products; the copies follow an in-place update of the weights."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators import moe
+    dt = torch.bfloat16
+    G, H, F, R = 3, 256, 512, 700
+    offs = torch.tensor([0, 300, 300, 700], dtype=torch.int32).cuda()           # one empty expert
+    xp, dy = randn((R, H), dt, 1).cuda(), randn((R, H), dt, 2).cuda()
+    w1, w2 = randn((G, 2 * F, H), dt, 3, std=0.05).cuda(), randn((G, H, F), dt, 4, std=0.05).cuda()
+    y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
+    ref = moe.expert_ffn_bwd(dy, xp, w1, w2, offs, saved)
+    w1t, w2t = _Clib.keep_transposed(w1), _Clib.keep_transposed(w2)
+    assert w1t.shape == (G, H, 2 * F) and torch.equal(w2t, w2.transpose(1, 2).contiguous())
+    got = moe.expert_ffn_bwd(dy, xp, w1, w2, offs, saved)
+    for a, b in zip(ref[:3], got[:3]):
+        assert torch.equal(a, b)
+    w2.mul_(0.5)
+    assert torch.equal(_Clib.transposed_of(w2), w2.transpose(1, 2).contiguous())

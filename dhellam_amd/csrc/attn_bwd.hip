@@ -792,7 +792,7 @@ template <typename T>
 __global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
-  constexpr int D = 128, RG = 2, SPLIT = 4, BN = 32, BM = 32 * RG, NS = BN / 16;
+  constexpr int D = 128, RG = 2, SPLIT = 4, BN = 32, BM = 32 * RG;
   constexpr int TILE = BN * D;                         // elements of one K tile
   constexpr int TILEB = TILE * (int)sizeof(T);
   constexpr int SLOTB = SPLIT * TILEB;                 // the K tiles of all splits: one stage

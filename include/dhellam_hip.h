@@ -137,8 +137,9 @@ int dh_attn_fwd(const void *q, const void *k, const void *v, void *out,
                 int64_t k_stride, int64_t v_stride, int64_t o_stride,
                 float softmax_scale, int causal, int dtype, void *stream);
 
-/* Bytes of scratch dh_attn_bwd needs (delta = rowsum(dO*O), and fp32 dK/dV
- * partials when a GQA group is split over workgroups). */
+/* Bytes of scratch dh_attn_bwd needs (delta = rowsum(dO*O), fp32 dK/dV
+ * partials when a GQA group is split over workgroups, and the dS blocks of
+ * calls that keep them: see dh_attn_bwd_set_ds_limit). */
 size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
                                    int max_seqlen_q, int hq, int hk, int d,
                                    int dtype);

@@ -212,7 +212,10 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
                workspace_bytes: int = 0) -> None:
     """out [N, K] (+)= grad [T, N]^T @ data [T, K] through ``dh_gemm``, in the layout ``wgrad_layout`` picks."""
     if wgrad_layout(grad, data) == "NN":
-        dense_gemm(data, transpose_2d(grad), out, False, False, accumulate, workspace, workspace_bytes)
+        gt = getattr(grad, "_dh_rows_transposed", None)       # left there by the kernel that produced ``grad``
+        if gt is None or gt.shape != (grad.shape[1], grad.shape[0]) or gt.dtype != grad.dtype:
+            gt = transpose_2d(grad)
+        dense_gemm(data, gt, out, False, False, accumulate, workspace, workspace_bytes)
     else:
         dense_gemm(data, grad, out, False, True, accumulate, workspace, workspace_bytes)
 

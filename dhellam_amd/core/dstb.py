@@ -47,7 +47,8 @@ import torch
 
 from .. import _lib
 from ..common.global_variables import GLOBAL_VARIABLES
-from .._Clib import keep_transposed, pymha_varlen_bwd, pymha_varlen_fwd, _attn_bwd_raw
+from .._Clib import (WGRAD_TRANSPOSE_GRAD_MIN_K, WGRAD_TRANSPOSE_MIN_ELEMS, keep_transposed, pymha_varlen_bwd,
+                      pymha_varlen_fwd, _attn_bwd_raw)
 from ..operators.bda import bda_bwd, bda_fwd
 from ..operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
 from ..operators.layernorm_column import dgrad_bwd, gemm_fwd, wgrad_bwd
@@ -363,7 +364,11 @@ class DCFunc:
     def swiglu_bwd(config, data, stream):
         swiglu_input, grad_output = data
         swiglu_input = swiglu_input.view(-1, swiglu_input.shape[-1])
-        dgrad, _ = swiglu_back(grad_output, swiglu_input, None, stream, profiling=False)
+        # the weight-gradient product of the column projection wants this gradient transposed when the layer is
+        # wide enough for that layout to pay (``_Clib.wgrad_layout``): the kernel then writes it alongside
+        rows, n2 = swiglu_input.shape
+        want_t = (config.hidden_size >= WGRAD_TRANSPOSE_GRAD_MIN_K and rows * n2 >= WGRAD_TRANSPOSE_MIN_ELEMS)
+        dgrad, _ = swiglu_back(grad_output, swiglu_input, None, stream, profiling=False, with_transposed=want_t)
         return dgrad
 
     @staticmethod

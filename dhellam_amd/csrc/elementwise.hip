@@ -7,6 +7,18 @@
 namespace dh {
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// d(gate) and d(up) of out = silu(gate) * up for one element, every operation rounded by itself (no fused multiply-add: the
+// kernels that use it must give the same bits, whatever the compiler would fuse around each call).
+__device__ __forceinline__ void swiglu_grad(float y1, float y2, float gg, float &d1, float &d2) {
+#pragma clang fp contract(off)
+  const float s = sigmoidf_(y1);
+  const float u = 1.0f + y1 * (1.0f - s);
+  d1 = gg * s * u * y2;
+  d2 = gg * (y1 * s);
+  // keeps the last product apart from the caller's conversion to 16 bits (one instruction can do both, rounding
+  // once instead of twice, and whether the compiler picks it depends on the code around the call)
+  asm("" : "+v"(d1), "+v"(d2));
+}
 
 // One "item" = one 16-byte vector of the output row; rows x fv items in total.
 // Item mapping of the streaming kernels: blocked = a workgroup's UNROLL vectors per lane are 256
@@ -84,10 +96,10 @@ swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restric
         Vec<T> d1, d2;
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-          const float y1 = to_f(a[u].v[j]), y2 = to_f(b[u].v[j]), gg = to_f(gv[u].v[j]);
-          const float s = sigmoidf_(y1);
-          d1.v[j] = from_f<T>(gg * s * (1.0f + y1 * (1.0f - s)) * y2);
-          d2.v[j] = from_f<T>(gg * (y1 * s));
+          float v1, v2;
+          swiglu_grad(to_f(a[u].v[j]), to_f(b[u].v[j]), to_f(gv[u].v[j]), v1, v2);
+          d1.v[j] = from_f<T>(v1);
+          d2.v[j] = from_f<T>(v2);
         }
         T *row = dy + r * (2 * (int64_t)fv * N);
         stg_s<NT>(row + (int64_t)c * N, d1);
@@ -95,6 +107,80 @@ swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restric
       }
     }
   }
+}
+
+// SwiGLU backward that also writes the gradient transposed: dy [rows, 2f] and dyT [2f, rows] from one read of g and
+// y.  The transpose feeds the weight-gradient GEMM of the projection in front of the activation (dW = dy^T x runs
+// fastest with dy^T row-major); produced here it costs one more write instead of a read and a write of its own.
+// A workgroup takes 64 rows x 128 columns of g: it computes the 64 x 128 tiles of d(gate) and d(up), stores them
+// as rows, and passes them through LDS (rows of 65 dwords, so 8-row steps land 8 banks apart) to store them as
+// columns: every lane gathers 8 consecutive rows of one column and writes them as 16 contiguous bytes, the 8
+// lanes of a column adjacent, i.e. whole 128-byte lines of dyT per store instruction.
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_bwd_t_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, T *__restrict__ dyt,
+                    int64_t rows, int64_t f, int64_t ld_t) {
+  constexpr int N = Vec<T>::N;                      // 8
+  constexpr int TR = 64, TC = 128, PITCH = TC * 2 + 4;
+  __shared__ __attribute__((aligned(16))) unsigned char tile[2][TR * PITCH];
+  const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
+  const int tid = threadIdx.x;
+  {
+    const int lr = tid >> 4, ch = tid & 15;
+    Vec<T> a[4], b[4], gv[4];
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t r = r0 + lr + 16 * i, c = c0 + ch * N;
+      ok[i] = r < rows && c < f;
+      if (ok[i]) {
+        const T *row = y + r * (2 * f);
+        a[i] = ldg(row + c);
+        b[i] = ldg(row + f + c);
+        gv[i] = ldg(g + r * f + c);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int rl = lr + 16 * i;
+      Vec<T> d1, d2;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        float v1 = 0.f, v2 = 0.f;
+        if (ok[i]) swiglu_grad(to_f(a[i].v[j]), to_f(b[i].v[j]), to_f(gv[i].v[j]), v1, v2);
+        d1.v[j] = from_f<T>(v1);
+        d2.v[j] = from_f<T>(v2);
+      }
+      if (ok[i]) {
+        T *row = dy + (r0 + rl) * (2 * f);
+        stg(row + c0 + ch * N, d1);
+        stg(row + f + c0 + ch * N, d2);
+      }
+      // rows are 4-byte aligned only: dword stores
+      const uint32_t *s1 = reinterpret_cast<const uint32_t *>(&d1), *s2 = reinterpret_cast<const uint32_t *>(&d2);
+      uint32_t *t1 = reinterpret_cast<uint32_t *>(tile[0] + rl * PITCH + ch * 16);
+      uint32_t *t2 = reinterpret_cast<uint32_t *>(tile[1] + rl * PITCH + ch * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        t1[q] = s1[q];
+        t2[q] = s2[q];
+      }
+    }
+  }
+  __syncthreads();
+  const int lane = tid & 63, w = tid >> 6;
+  const int rb = lane & 7, cl = lane >> 3;            // 8-row block, column within the step
+#pragma unroll
+  for (int part = 0; part < 2; ++part)
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+      const int col = 32 * w + 8 * s2 + cl;
+      const unsigned char *src = tile[part] + (8 * rb) * PITCH + col * 2;
+      Vec<T> o;
+#pragma unroll
+      for (int j = 0; j < N; ++j) o.v[j] = *reinterpret_cast<const T *>(src + j * PITCH);
+      if (c0 + col < f && r0 + 8 * rb < rows) stg(dyt + ((int64_t)part * f + c0 + col) * ld_t + r0 + 8 * rb, o);
+    }
 }
 
 // Scalar fallbacks (f not a multiple of the vector width, or unaligned pointers).
@@ -114,9 +200,10 @@ swiglu_bwd_scalar_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / f, c = i - r * f;
     const float y1 = to_f(y[r * 2 * f + c]), y2 = to_f(y[r * 2 * f + f + c]), gg = to_f(g[i]);
-    const float s = sigmoidf_(y1);
-    dy[r * 2 * f + c] = from_f<T>(gg * s * (1.0f + y1 * (1.0f - s)) * y2);
-    dy[r * 2 * f + f + c] = from_f<T>(gg * (y1 * s));
+    float v1, v2;
+    swiglu_grad(y1, y2, gg, v1, v2);
+    dy[r * 2 * f + c] = from_f<T>(v1);
+    dy[r * 2 * f + f + c] = from_f<T>(v2);
   }
 }
 
@@ -257,6 +344,28 @@ extern "C" int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t row
                          (const T *)g, (const T *)y, (T *)dy, rows * f, f);
     }
   });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_swiglu_bwd_t(const void *g, const void *y, void *dy, void *dy_t, int64_t rows, int64_t f, int dtype,
+                               void *stream) {
+  using namespace dh;
+  DH_CHECK(rows >= 0 && f >= 0, "bad shape rows=%lld f=%lld", (long long)rows, (long long)f);
+  if (rows == 0 || f == 0) return DH_OK;
+  DH_CHECK(g && y && dy && dy_t, "null pointer");
+  DH_CHECK(dtype == DH_BF16 || dtype == DH_F16, "16-bit element types only (dtype %d)", dtype);
+  DH_CHECK(rows % 8 == 0 && f % 8 == 0, "rows=%lld and f=%lld must be multiples of 8", (long long)rows, (long long)f);
+  DH_CHECK(aligned16(y) && aligned16(g) && aligned16(dy) && aligned16(dy_t), "pointers must be 16-byte aligned");
+  const dim3 grid((unsigned)cdiv(f, 128), (unsigned)cdiv(rows, 64));
+  DH_CHECK(grid.y < 65536, "too many rows for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == DH_BF16)
+    hipLaunchKernelGGL((swiglu_bwd_t_kernel<bf16_t>), grid, dim3(256), 0, st, (const bf16_t *)g, (const bf16_t *)y,
+                       (bf16_t *)dy, (bf16_t *)dy_t, rows, f, rows);
+  else
+    hipLaunchKernelGGL((swiglu_bwd_t_kernel<f16_t>), grid, dim3(256), 0, st, (const f16_t *)g, (const f16_t *)y,
+                       (f16_t *)dy, (f16_t *)dy_t, rows, f, rows);
   DH_LAUNCH_CHECK();
   return DH_OK;
 }

@@ -23,9 +23,11 @@ def swiglu(y, stream=None, profiling=False):
     return out, el[0]
 
 
-def swiglu_back(g, y, o=None, stream=None, profiling=False):
+def swiglu_back(g, y, o=None, stream=None, profiling=False, with_transposed=False):
     """``o`` (optional) receives the result; the reference allocates it but its kernel
-    ignores it (swiglu.py:48-55)."""
+    ignores it (swiglu.py:48-55).  ``with_transposed``: the kernel also writes the result transposed
+    ([2f, rows], for the weight-gradient product of the projection in front of the activation) and hangs it on the
+    returned tensor, where ``_Clib.wgrad_gemm`` finds it; ignored for shapes or types the kernel does not take."""
     assert y.is_cuda and y.is_contiguous() and g.is_contiguous() and y.shape[-1] % 2 == 0
     lib = _lib.load()
     f = y.shape[-1] // 2
@@ -36,5 +38,12 @@ def swiglu_back(g, y, o=None, stream=None, profiling=False):
         if o is None:
             o = torch.empty_like(y)
         assert o.is_contiguous() and o.shape == y.shape
-        _lib.check(lib.dh_swiglu_bwd(g.data_ptr(), y.data_ptr(), o.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
+        if (with_transposed and y.dtype in (torch.bfloat16, torch.float16) and rows % 8 == 0 and f % 8 == 0 and rows > 0
+                and f > 0 and g.dtype == y.dtype):
+            ot = torch.empty((2 * f, rows), dtype=y.dtype, device=y.device)
+            _lib.check(lib.dh_swiglu_bwd_t(g.data_ptr(), y.data_ptr(), o.data_ptr(), ot.data_ptr(), rows, f, _lib.dt(y),
+                                           st.cuda_stream))
+            o._dh_rows_transposed = ot
+        else:
+            _lib.check(lib.dh_swiglu_bwd(g.data_ptr(), y.data_ptr(), o.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
     return o, el[0]

@@ -86,6 +86,14 @@ int dh_swiglu_fwd(const void *y, void *out, int64_t rows, int64_t f, int dtype,
 int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t rows,
                   int64_t f, int dtype, void *stream);
 
+/* dh_swiglu_bwd that also writes the gradient transposed: dy_t [2f, rows]
+ * (row-major) next to dy [rows, 2f], for the weight-gradient product of the
+ * projection in front of the activation (csrc/operators/gemm.cu:3-170 with
+ * transb; dhellam/core/dstb.py:543-598).  16-bit types; rows and f multiples
+ * of 8.  No counterpart in the reference. */
+int dh_swiglu_bwd_t(const void *g, const void *y, void *dy, void *dy_t,
+                    int64_t rows, int64_t f, int dtype, void *stream);
+
 /* ------------------------------------------------------------------------
  * Residual add (bias-dropout-add with dropout disabled).
  * dhellam/operators/bda.py:3-12.  out = x + residual (out may alias x: the

@@ -211,6 +211,31 @@ def test_rope_large_positions(dtype):
         assert (got.double() - ref).abs().max().item() <= 0.51 * ulp + 2e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,f", [(4096, 3584), (72, 200), (8, 8), (136, 1032)])
+def test_swiglu_backward_with_transposed_output(dtype, rows, f):
+    """dh_swiglu_bwd_t: the same gradient as dh_swiglu_bwd, bit for bit, plus its transpose; the weight-gradient
+    helper picks the transpose up from the tensor."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.swiglu import swiglu_back
+    y, g = randn((rows, 2 * f), dtype, 1).cuda(), randn((rows, f), dtype, 2).cuda()
+    ref, _ = swiglu_back(g, y)
+    got, _ = swiglu_back(g, y, with_transposed=True)
+    assert torch.equal(got, ref)
+    gt = got._dh_rows_transposed
+    assert gt.shape == (2 * f, rows) and torch.equal(gt, ref.t().contiguous())
+    x = randn((rows, 3080), dtype, 3).cuda()                     # wide enough for the transposed layout
+    if rows * 2 * f >= _Clib.WGRAD_TRANSPOSE_MIN_ELEMS:
+        d1 = torch.zeros(2 * f, 3080, dtype=dtype, device="cuda")
+        d2 = torch.zeros_like(d1)
+        _Clib.wgrad_gemm(got, x, d1, False)                      # uses the kernel's transpose
+        _Clib.wgrad_gemm(ref, x, d2, False)                      # transposes by itself
+        assert torch.equal(d1, d2)
+    odd, _ = swiglu_back(g[:, : f - 4].contiguous(), torch.cat([y[:, : f - 4], y[:, f: 2 * f - 4]], 1).contiguous(),
+                         with_transposed=True)                   # f not a multiple of 8: plain kernel, no transpose
+    assert not hasattr(odd, "_dh_rows_transposed")
+
+
 def test_bandwidth_ops_are_deterministic():
     """Norm backward (staged column sums), SwiGLU, RoPE: two runs, same bits."""
     from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd

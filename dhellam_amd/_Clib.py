@@ -212,8 +212,10 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
                workspace_bytes: int = 0) -> None:
     """out [N, K] (+)= grad [T, N]^T @ data [T, K] through ``dh_gemm``, in the layout ``wgrad_layout`` picks."""
     if wgrad_layout(grad, data) == "NN":
-        gt = getattr(grad, "_dh_rows_transposed", None)       # left there by the kernel that produced ``grad``
-        if gt is None or gt.shape != (grad.shape[1], grad.shape[0]) or gt.dtype != grad.dtype:
+        # the kernel that produced ``grad`` may have left its transpose on it, stamped with the tensor's version
+        version, gt = getattr(grad, "_dh_rows_transposed", None) or (None, None)
+        if (gt is None or version != grad._version or gt.shape != (grad.shape[1], grad.shape[0])
+                or gt.dtype != grad.dtype):
             gt = transpose_2d(grad)
         dense_gemm(data, gt, out, False, False, accumulate, workspace, workspace_bytes)
     else:

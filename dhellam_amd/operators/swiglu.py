@@ -43,7 +43,7 @@ def swiglu_back(g, y, o=None, stream=None, profiling=False, with_transposed=Fals
             ot = torch.empty((2 * f, rows), dtype=y.dtype, device=y.device)
             _lib.check(lib.dh_swiglu_bwd_t(g.data_ptr(), y.data_ptr(), o.data_ptr(), ot.data_ptr(), rows, f, _lib.dt(y),
                                            st.cuda_stream))
-            o._dh_rows_transposed = ot
+            o._dh_rows_transposed = (o._version, ot)    # valid while nothing has written ``o`` since
         else:
             _lib.check(lib.dh_swiglu_bwd(g.data_ptr(), y.data_ptr(), o.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
     return o, el[0]

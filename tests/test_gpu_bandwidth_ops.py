@@ -222,14 +222,18 @@ def test_swiglu_backward_with_transposed_output(dtype, rows, f):
     ref, _ = swiglu_back(g, y)
     got, _ = swiglu_back(g, y, with_transposed=True)
     assert torch.equal(got, ref)
-    gt = got._dh_rows_transposed
-    assert gt.shape == (2 * f, rows) and torch.equal(gt, ref.t().contiguous())
+    version, gt = got._dh_rows_transposed
+    assert version == got._version and gt.shape == (2 * f, rows) and torch.equal(gt, ref.t().contiguous())
     x = randn((rows, 3080), dtype, 3).cuda()                     # wide enough for the transposed layout
     if rows * 2 * f >= _Clib.WGRAD_TRANSPOSE_MIN_ELEMS:
         d1 = torch.zeros(2 * f, 3080, dtype=dtype, device="cuda")
         d2 = torch.zeros_like(d1)
         _Clib.wgrad_gemm(got, x, d1, False)                      # uses the kernel's transpose
         _Clib.wgrad_gemm(ref, x, d2, False)                      # transposes by itself
+        assert torch.equal(d1, d2)
+        got.mul_(2)                                              # a write to the gradient retires its transpose
+        _Clib.wgrad_gemm(got, x, d1, False)
+        _Clib.wgrad_gemm(ref * 2, x, d2, False)
         assert torch.equal(d1, d2)
     odd, _ = swiglu_back(g[:, : f - 4].contiguous(), torch.cat([y[:, : f - 4], y[:, f: 2 * f - 4]], 1).contiguous(),
                          with_transposed=True)                   # f not a multiple of 8: plain kernel, no transpose

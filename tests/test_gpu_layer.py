@@ -180,15 +180,16 @@ def test_delay_and_emulated_collectives():
                       micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
                       params_dtype=torch.bfloat16)
     res = []
-    for us in (0.0, 40.0):
-        c = dataclasses.replace(cfg, comm_standin_us=us)
+    for us, engine in ((0.0, "kernel"), (40.0, "kernel"), (40.0, "dma")):   # "dma": a copy-engine stand-in
+        c = dataclasses.replace(cfg, comm_standin_us=us, comm_standin_engine=engine)
         w = make_weights(c, 0)
         mbs = [make_microbatch(c, i) for i in range(2)]
         outs, dxs = LayerRunner(c, w).run_double_strand(mbs)
         torch.cuda.synchronize()
         res.append((outs, dxs, [w[k].main_grad.clone() for k in GRAD_KEYS]))
-    for x, y in zip(res[0][0] + res[0][1] + res[0][2], res[1][0] + res[1][1] + res[1][2]):
-        assert torch.equal(x, y)
+    for other in res[1:]:
+        for x, y in zip(res[0][0] + res[0][1] + res[0][2], other[0] + other[1] + other[2]):
+            assert torch.equal(x, y)
 
 
 def test_cu_partitioned_streams():

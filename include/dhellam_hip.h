@@ -159,8 +159,10 @@ size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
  * from it in one product; otherwise (0: never) its dQ pass recomputes S and dP
  * and needs no such space.  No counterpart in the reference (flash-attention
  * always recomputes); a process-wide setting, read by
- * dh_attn_bwd_workspace_bytes and dh_attn_bwd alike: change it only between a
- * sizing call and the calls it sizes for. */
+ * dh_attn_bwd_workspace_bytes and dh_attn_bwd alike: dh_attn_bwd takes no
+ * workspace size, so a workspace must be sized AFTER the last change of this
+ * limit (raising it between a sizing call and the dh_attn_bwd call that uses
+ * the result would let the kernels write past the workspace). */
 void dh_attn_bwd_set_ds_limit(size_t bytes);
 
 /* dq like q, dk/dv like k/v (GQA groups are reduced inside the kernel; the

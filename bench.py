@@ -543,24 +543,9 @@ def main():
         emulated = {"standin_us_per_collective": args.emulate_comm_us, "collectives_per_microbatch": 8,
                     "serial_ms": round(ser_c, 4), "double_strand_ms": round(dbl_c, 4),
                     "double_strand_lockstep_ms": round(dbl_l, 4),
-                    "double_strand_speedup": round(ser_c / min(dbl_c, dbl_l), 4)}
-        # the same with the stand-ins carried by the copy engines (a copy to pinned host memory of that duration)
-        # instead of a kernel: a collective that needs no compute unit starts while a GEMM fills the chip
-        dma = dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us, comm_standin_engine="dma")
-        runner_d = LayerRunner(dma, w, plan=plan)
-        ser_d, dbl_d = timed(runner_d.run_serial, runner_d), timed(runner_d.run_double_strand, runner_d)
-        runner_dl = LayerRunner(dataclasses.replace(dma, lockstep_blocks=True), w, plan=plan)
-        dbl_dl = timed(runner_dl.run_double_strand, runner_dl)
-        from dhellam_amd.core.dstb import dma_standin_calibration
-        n_standins = 8 * len(mbs)
-        emulated["serial_cost_us_per_standin"] = round((ser_c - ms_serial) * 1e3 / n_standins, 1)
-        emulated["copy_engine_standins"] = {"calibration": dma_standin_calibration(),
-                                            # what one stand-in adds to the serial schedule: the copy itself plus the
-                                            # hand-over between the compute queue and the copy engine, both ways
-                                            "serial_cost_us_per_standin": round((ser_d - ms_serial) * 1e3 / n_standins, 1),
-                                            "serial_ms": round(ser_d, 4), "double_strand_ms": round(dbl_d, 4),
-                                            "double_strand_lockstep_ms": round(dbl_dl, 4),
-                                            "double_strand_speedup": round(ser_d / min(dbl_d, dbl_dl), 4)}
+                    "double_strand_speedup": round(ser_c / min(dbl_c, dbl_l), 4),
+                    # what one stand-in adds to the serial schedule
+                    "serial_cost_us_per_standin": round((ser_c - ms_serial) * 1e3 / (8 * len(mbs)), 1)}
     layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
 
     measured = _measured()

@@ -115,10 +115,6 @@ class LayerConfig:
     params_dtype: torch.dtype = torch.bfloat16
     layernorm_bias: bool = False      # False: RMSNorm (Llama); True: LayerNorm with bias (the reference's TE call)
     comm_standin_us: float = 0.0      # > 0: every sequence-parallel stand-in also occupies its stream this long
-    # what occupies the stream: "kernel" = a one-wavefront delay kernel (a collective made of kernels: it competes
-    # for compute units with whatever else runs), "dma" = a copy to pinned host memory sized to last that long (a
-    # collective carried by the copy engines: needs no compute unit)
-    comm_standin_engine: str = "kernel"
     lockstep_blocks: bool = False     # the two strands enter every plan block together (events between the streams)
     # (forward strand's, backward strand's) communication streams: the stand-ins' delays run there, with events
     # to and from the strand's own stream, instead of on the strand's stream itself
@@ -182,57 +178,6 @@ def _split_qkv(config: LayerConfig, qkv: torch.Tensor):
     k = g[:, :, r * d:(r + 1) * d].contiguous()
     v = g[:, :, (r + 1) * d:].contiguous()
     return q, k, v
-
-
-_DMA_STANDIN: dict = {}
-
-
-def _dma_standin(us: float, stream, bwd_strand: bool) -> None:
-    """Keeps ``stream`` busy for about ``us`` microseconds with a device-to-pinned-host copy, which the copy engines
-    carry without occupying a compute unit.  What a copy costs its stream is measured once per device, between two
-    small kernels on an otherwise idle GPU (the hand-over between the compute queue and the copy engine is part of
-    it): the fixed part from a 4 KiB copy, the rate from a 16 MiB one, best of five each.  A request below the fixed
-    part gets the smallest copy.  Each strand has its own pair of buffers."""
-    dev = torch.cuda.current_device()
-    state = _DMA_STANDIN.get(dev)
-    if state is None:
-        n = 64 << 20
-        bufs = [(torch.empty(n, dtype=torch.uint8, device="cuda"), torch.empty(n, dtype=torch.uint8, pin_memory=True))
-                for _ in range(2)]
-        cal = torch.cuda.Stream()
-        cal.wait_stream(torch.cuda.current_stream())
-        tick = torch.zeros(64, device="cuda")
-
-        def occupied_us(nbytes: int) -> float:
-            best = None
-            for _ in range(5):
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                tick.add_(1.0)
-                if nbytes:
-                    bufs[0][1][:nbytes].copy_(bufs[0][0][:nbytes], non_blocking=True)
-                tick.add_(1.0)
-                b.record()
-                b.synchronize()
-                t = a.elapsed_time(b) * 1e3
-                best = t if best is None else min(best, t)
-            return best
-
-        with torch.cuda.stream(cal):
-            base = occupied_us(0)
-            fixed = max(0.0, occupied_us(4096) - base)
-            big = max(fixed + 1.0, occupied_us(16 << 20) - base)
-        state = _DMA_STANDIN[dev] = {"bufs": bufs, "fixed_us": fixed, "bytes_per_us": (16 << 20) / (big - fixed), "max": n}
-    nbytes = int(min(state["max"], max(4096.0, (us - state["fixed_us"]) * state["bytes_per_us"]))) & ~255
-    d, h = state["bufs"][1 if bwd_strand else 0]
-    with torch.cuda.stream(stream):
-        h[:nbytes].copy_(d[:nbytes], non_blocking=True)
-
-
-def dma_standin_calibration() -> Optional[dict]:
-    """{"fixed_us", "bytes_per_us"} of the current device's copy stand-in once it has been used, else None."""
-    st = _DMA_STANDIN.get(torch.cuda.current_device())
-    return None if st is None else {"fixed_us": round(st["fixed_us"], 2), "bytes_per_us": round(st["bytes_per_us"], 1)}
 
 
 class DCFunc:
@@ -477,9 +422,6 @@ class DCFunc:
         us = getattr(config, "comm_standin_us", 0.0)
         if us > 0:
             st = stream if stream is not None else torch.cuda.current_stream()
-            if getattr(config, "comm_standin_engine", "kernel") == "dma":
-                _dma_standin(us, st, bwd_strand)
-                return
             comm = getattr(config, "comm_streams", None)
             if comm is None:
                 _lib.check(_lib.load().dh_delay(int(us * 1000), st.cuda_stream))

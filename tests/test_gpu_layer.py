@@ -180,8 +180,8 @@ def test_delay_and_emulated_collectives():
                       micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
                       params_dtype=torch.bfloat16)
     res = []
-    for us, engine in ((0.0, "kernel"), (40.0, "kernel"), (40.0, "dma")):   # "dma": a copy-engine stand-in
-        c = dataclasses.replace(cfg, comm_standin_us=us, comm_standin_engine=engine)
+    for us in (0.0, 40.0):
+        c = dataclasses.replace(cfg, comm_standin_us=us)
         w = make_weights(c, 0)
         mbs = [make_microbatch(c, i) for i in range(2)]
         outs, dxs = LayerRunner(c, w).run_double_strand(mbs)

@@ -546,6 +546,18 @@ def main():
                     "double_strand_speedup": round(ser_c / min(dbl_c, dbl_l), 4),
                     # what one stand-in adds to the serial schedule
                     "serial_cost_us_per_standin": round((ser_c - ms_serial) * 1e3 / (8 * len(mbs)), 1)}
+        # The same with stand-ins that need no compute unit (a host function of the stream: a transfer carried by a
+        # copy engine or a network adapter).  Its cost to a stream includes the runtime's hand-over to a host
+        # thread and back, so both costs are reported: per stand-in in the serial schedule and in the double strand.
+        host = dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us, comm_standin_engine="host")
+        runner_h = LayerRunner(host, w, plan=plan)
+        ser_h, dbl_h = timed(runner_h.run_serial, runner_h), timed(runner_h.run_double_strand, runner_h)
+        n_standins = 8 * len(mbs)
+        emulated["host_function_standins"] = {
+            "serial_ms": round(ser_h, 4), "double_strand_ms": round(dbl_h, 4),
+            "double_strand_speedup": round(ser_h / dbl_h, 4),
+            "serial_cost_us_per_standin": round((ser_h - ms_serial) * 1e3 / n_standins, 1),
+            "double_strand_cost_us_per_standin": round((dbl_h - ms_double) * 1e3 / n_standins, 1)}
     layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
 
     measured = _measured()

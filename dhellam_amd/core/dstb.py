@@ -115,6 +115,10 @@ class LayerConfig:
     params_dtype: torch.dtype = torch.bfloat16
     layernorm_bias: bool = False      # False: RMSNorm (Llama); True: LayerNorm with bias (the reference's TE call)
     comm_standin_us: float = 0.0      # > 0: every sequence-parallel stand-in also occupies its stream this long
+    # what occupies the stream: "kernel" = a one-wavefront delay kernel (a collective made of kernels: it has to find
+    # a free wavefront slot next to whatever else runs), "host" = a host function of the stream (a transfer carried
+    # by a copy engine or a network adapter: needs no compute unit)
+    comm_standin_engine: str = "kernel"
     lockstep_blocks: bool = False     # the two strands enter every plan block together (events between the streams)
     # (forward strand's, backward strand's) communication streams: the stand-ins' delays run there, with events
     # to and from the strand's own stream, instead of on the strand's stream itself
@@ -423,14 +427,16 @@ class DCFunc:
         if us > 0:
             st = stream if stream is not None else torch.cuda.current_stream()
             comm = getattr(config, "comm_streams", None)
+            delay = _lib.load().dh_host_delay if getattr(config, "comm_standin_engine", "kernel") == "host" \
+                else _lib.load().dh_delay
             if comm is None:
-                _lib.check(_lib.load().dh_delay(int(us * 1000), st.cuda_stream))
+                _lib.check(delay(int(us * 1000), st.cuda_stream))
                 return
             cs = comm[1] if bwd_strand else comm[0]
             posted, done = torch.cuda.Event(), torch.cuda.Event()
             posted.record(st)
             cs.wait_event(posted)
-            _lib.check(_lib.load().dh_delay(int(us * 1000), cs.cuda_stream))
+            _lib.check(delay(int(us * 1000), cs.cuda_stream))
             done.record(cs)
             st.wait_event(done)
 

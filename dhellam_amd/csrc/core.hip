@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 #include <algorithm>
 #include <mutex>
 #include <vector>
@@ -67,6 +68,31 @@ extern "C" int dh_delay(int64_t nanoseconds, void *stream) {
   const unsigned long long max_iters = (unsigned long long)(nanoseconds / 200) + 1024;
   hipLaunchKernelGGL(delay_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, ticks, max_iters);
   DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+// The same stretch of stream time without a compute unit: a host function in the stream, which the runtime calls on
+// one of its own threads once the stream's earlier work is done and whose return releases the work behind it.  It
+// stands for a transfer that an agent other than the compute units carries (a copy engine, a network adapter):
+// unlike the delay kernel it needs no free wavefront slot, so it starts while a kernel of another stream owns every
+// compute unit.  What it costs the stream beyond the requested time is the runtime's hand-over to its thread and
+// back (measured by the caller, not assumed).
+namespace dh {
+static void host_spin_entry(void *arg) {
+  const int64_t ns = (int64_t)(intptr_t)arg;
+  timespec t0, t;
+  clock_gettime(CLOCK_MONOTONIC, &t0);
+  for (;;) {
+    clock_gettime(CLOCK_MONOTONIC, &t);
+    if ((int64_t)(t.tv_sec - t0.tv_sec) * 1000000000ll + (t.tv_nsec - t0.tv_nsec) >= ns) break;
+  }
+}
+}  // namespace dh
+
+extern "C" int dh_host_delay(int64_t nanoseconds, void *stream) {
+  DH_CHECK(nanoseconds >= 0 && nanoseconds <= 1000000000ll, "delay of %lld ns outside [0, 1 s]", (long long)nanoseconds);
+  if (nanoseconds == 0) return DH_OK;
+  DH_HIP(hipLaunchHostFunc((hipStream_t)stream, dh::host_spin_entry, (void *)(intptr_t)nanoseconds));
   return DH_OK;
 }
 

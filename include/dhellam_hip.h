@@ -307,6 +307,12 @@ int dh_copy_bytes(const void *src, void *dst, int64_t nbytes, void *stream);
  * (dhellam/common/comm.py) in scheduler experiments, so that the double-strand runtime has something to hide. */
 int dh_delay(int64_t nanoseconds, void *stream);
 
+/* The same stretch of stream time spent in a host function of the stream
+ * (hipLaunchHostFunc) instead of a kernel: stands for a transfer that needs no
+ * compute unit (copy engine, network adapter), so it starts while kernels of
+ * another stream fill the device.  No counterpart in the reference. */
+int dh_host_delay(int64_t nanoseconds, void *stream);
+
 /* Dense GEMM through hipBLASLt: cublas_gemm / pygemm, csrc/operators/gemm.cu:3-170 (csrc/operators/ops.h:54-65).
  * The reference's convention is kept: A [a_rows, a_cols], B [b_rows, b_cols] and D are contiguous row-major
  * arrays given to a column-major library, so with m = transa ? a_rows : a_cols, k = transa ? a_cols : a_rows,

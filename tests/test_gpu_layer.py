@@ -159,8 +159,8 @@ def test_plan_with_deferred_wgrad_placeholders():
 
 
 def test_delay_and_emulated_collectives():
-    """dh_delay keeps a stream busy for at least the requested time, and a layer whose sequence-parallel
-    stand-ins carry such delays computes the same bits."""
+    """dh_delay / dh_host_delay keep a stream busy for at least the requested time, and a layer whose
+    sequence-parallel stand-ins carry such delays computes the same bits."""
     import dataclasses
     from dhellam_amd import _lib
     from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
@@ -180,8 +180,15 @@ def test_delay_and_emulated_collectives():
                       micro_batch_size=1, tensor_model_parallel_size=4, tp_rank=1, rope_theta=10000.0,
                       params_dtype=torch.bfloat16)
     res = []
-    for us in (0.0, 40.0):
-        c = dataclasses.replace(cfg, comm_standin_us=us)
+    a.record()
+    _lib.check(lib.dh_host_delay(2_000_000, st.cuda_stream))      # the same in a host function of the stream
+    b.record()
+    b.synchronize()
+    assert 1.9 <= a.elapsed_time(b) <= 50.0, a.elapsed_time(b)
+    with pytest.raises(RuntimeError):
+        _lib.check(lib.dh_host_delay(-1, st.cuda_stream))
+    for us, engine in ((0.0, "kernel"), (40.0, "kernel"), (40.0, "host")):
+        c = dataclasses.replace(cfg, comm_standin_us=us, comm_standin_engine=engine)
         w = make_weights(c, 0)
         mbs = [make_microbatch(c, i) for i in range(2)]
         outs, dxs = LayerRunner(c, w).run_double_strand(mbs)

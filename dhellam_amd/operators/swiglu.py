@@ -39,7 +39,8 @@ def swiglu_back(g, y, o=None, stream=None, profiling=False, with_transposed=Fals
             o = torch.empty_like(y)
         assert o.is_contiguous() and o.shape == y.shape
         if (with_transposed and y.dtype in (torch.bfloat16, torch.float16) and rows % 8 == 0 and f % 8 == 0 and rows > 0
-                and f > 0 and g.dtype == y.dtype and rows < 64 * 65535):
+                and f > 0 and g.dtype == y.dtype and rows < 64 * 65535
+                and g.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0 and o.data_ptr() % 16 == 0):
             ot = torch.empty((2 * f, rows), dtype=y.dtype, device=y.device)
             _lib.check(lib.dh_swiglu_bwd_t(g.data_ptr(), y.data_ptr(), o.data_ptr(), ot.data_ptr(), rows, f, _lib.dt(y),
                                            st.cuda_stream))

@@ -27,9 +27,15 @@ not vendored: transformer-engine 1.4.0, flash-attn >= 2.0.6, Megatron-core
   pinned by equality with ONE dense causal attention over the zig-zag token order.
 * ``moe.*``                           numpy index arithmetic; pinned by brute force,
   ``numpy.argsort(kind="stable")``, bijection and round-trip invariants.
-* ``layer.*``                         the decoder layer of configs 0 and 2 with autograd.
+* ``layer.*``                         the decoder layer of configs 0 and 2 with autograd; pinned by an
+  independently written forward from library routines (``F.rms_norm``, ``F.linear``,
+  ``F.scaled_dot_product_attention``, ``F.silu``) with fp64 autograd at 1e-12, and the
+  sequence-parallel gather / scatter stand-ins by explicit slicing.
+* ``head.*``                          dhellam/operators/loss.py:15-164 and embedding.py:16-49, restated
+  line by line; pinned by ``F.cross_entropy`` / ``F.embedding`` and their autograd, one rank and four.
 
-Parity against the REFERENCE's own numerical output is unpinned for every
-function here: the reference cannot run without CUDA, TransformerEngine,
-flash-attn and Megatron, and holds no recorded outputs.
+Every function above is pinned by the checks named with it (``tests/test_oracle_pins.py``,
+``tests/test_golden.py``).  None of them could be held against numbers produced by the
+reference itself: it cannot run without CUDA, TransformerEngine, flash-attn and Megatron,
+and it holds no recorded outputs.
 """

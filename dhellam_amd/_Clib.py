@@ -84,6 +84,11 @@ def dense_gemm(A, B, D, transa: bool, transb: bool, accumulate: bool, workspace=
         if not accumulate:
             D.zero_()
         return
+    if transa and transb:      # refused by dh_gemm as by the reference's cublas_gemm; the library's own entry for it
+        _lib.check(_lib.load().dh_gemm_tt(A.data_ptr(), B.data_ptr(), D.data_ptr(), A.shape[0], A.shape[1], B.shape[0],
+                                          B.shape[1], int(accumulate), _lib.dt(A), _lib.dt(D), workspace.data_ptr(),
+                                          workspace_bytes, stream.cuda_stream))
+        return
     _lib.check(_lib.load().dh_gemm(A.data_ptr(), B.data_ptr(), D.data_ptr(), A.shape[0], A.shape[1], B.shape[0],
                                    B.shape[1], int(transa), int(transb), int(accumulate), _lib.dt(A), _lib.dt(D),
                                    workspace.data_ptr(), workspace_bytes, stream.cuda_stream))
@@ -105,12 +110,15 @@ def pygemm(inputA, inputB, outputD, input_workspace, workspaceSize, transa, tran
     ``math_sm_count`` > 0 confines the product to that many compute units, as the reference's libsmctrl
     mask does (csrc/operators/gemm.cu:66-70, smctrl.cpp:135-160): it runs on a stream created with that
     compute-unit mask (cached per device and count), ordered after and before the current stream by events;
-    a count above the device's compute units is refused.  For the weight gradient, B^T is materialised first
-    where that makes the product faster by more than it costs (``wgrad_layout``).
+    a count above the device's compute units is refused.  For the weight gradient, the smaller operand is
+    materialised transposed first where that makes the product faster by more than it costs (``wgrad_layout``).
     """
     _lib.need_cuda(inputA, inputB, outputD)
     stream = torch.cuda.current_stream()
     ws_bytes = int(workspaceSize or 0)
+
+    if transa and transb:
+        raise RuntimeError("pygemm: TT layout not allowed")     # as the reference (csrc/operators/gemm.cu)
 
     def product():
         if transb and not transa:
@@ -172,10 +180,13 @@ def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
 
 # The weight-gradient product dW[N, K] = dY[T, N]^T X[T, K] reads both operands along their strided dimension, the
 # GEMM library's slowest layout here.  Measured at T = 4096, bf16, accumulating (us; N, K = 7168, 8192 / 8192, 3584 /
-# 1280, 8192 / 8192, 1024):   as given 484 / 233-257 / 95 / 76;   dY^T row-major 409 / 203 / 82 / 67;
-# dY^T and X^T both row-major (the forward's layout) 343 / 171 / 73 / 61.  dh_transpose_2d moves 5.5-6 TB/s (a
-# [4096, 8192] matrix in 24 us), so materialising dY^T pays from K of about 3000.  X^T as well would pay from N of
-# about 4000, but for that layout the library picks a kernel that splits tiles over workgroups, and its
+# 1280, 8192 / 8192, 1024):   as given 464 / 233 / 105 / 85;   dY^T row-major 380 / 190 / 87 / 72;   X^T row-major
+# (the layout ``dh_gemm`` refuses, ``dh_gemm_tt``) 383 / 188 / 95 / 70;   both row-major (the forward's layout)
+# 335 / 165 / 76 / 61.  One transposed operand is worth 15-20 % whichever it is, so the SMALLER one is transposed
+# (dh_transpose_2d moves 5.5-6 TB/s: [4096, 8192] in 24 us, [4096, 3584] in 11 us, [4096, 1024] in 8 us): X when the
+# weight has fewer inputs than outputs (fc2, the attention output projection, the vocabulary projection), dY
+# otherwise (qkv, fc1 -- where the kernel that produces dY writes the transpose alongside).  Both transposed would
+# be faster still, but for that layout the library picks a kernel that splits tiles over workgroups, and its
 # accumulation into dW does not always give the same bits when another kernel shares the GPU (1 step in 40-100
 # of the double-strand schedule differed from the serial one in the last bits of one weight gradient; giving each
 # stream its own workspace does not change that), while the two schedules are required to agree bit for bit: not
@@ -189,35 +200,41 @@ def _can_transpose(t: torch.Tensor) -> bool:
             and t.shape[0] % 8 == 0 and t.shape[1] % 8 == 0 and t.data_ptr() % 16 == 0)
 
 
-def wgrad_operands(grad: torch.Tensor, data: torch.Tensor):
-    """(lhs, rhs) with lhs @ rhs = grad^T @ data for grad = dY [T, N], data = X [T, K]: the strided view of dY,
-    or its materialised row-major transpose where that makes the product faster by more than it costs."""
-    (t, n), k = grad.shape, data.shape[1]
-    if (k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad)
-            and grad.dtype == data.dtype):
-        return transpose_2d(grad), data
-    return grad.t(), data
-
-
 def wgrad_layout(grad: torch.Tensor, data: torch.Tensor) -> str:
-    """Which operand of dW = dY^T X is materialised transposed before the library call: "NT" (none) or "NN" (dY^T)."""
+    """Which operand of dW = dY^T X is materialised transposed before the library call: "NT" (none), "NN" (dY^T)
+    or "TT" (X^T)."""
     (t, n), k = grad.shape, data.shape[1]
-    if (k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad)
-            and grad.dtype == data.dtype):
+    if grad.dtype != data.dtype:
+        return "NT"
+    if k < n and t * k >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(data) and _can_transpose(grad):
+        return "TT"
+    if k >= WGRAD_TRANSPOSE_GRAD_MIN_K and t * n >= WGRAD_TRANSPOSE_MIN_ELEMS and _can_transpose(grad):
         return "NN"
     return "NT"
 
 
+def wgrad_operands(grad: torch.Tensor, data: torch.Tensor):
+    """(lhs, rhs) with lhs @ rhs = grad^T @ data for grad = dY [T, N], data = X [T, K]: the strided view of dY,
+    or its materialised row-major transpose where ``wgrad_layout`` says "NN" (a product through torch has no use
+    for X^T)."""
+    if wgrad_layout(grad, data) == "NN":
+        return transpose_2d(grad), data
+    return grad.t(), data
+
+
 def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumulate: bool, workspace=None,
                workspace_bytes: int = 0) -> None:
-    """out [N, K] (+)= grad [T, N]^T @ data [T, K] through ``dh_gemm``, in the layout ``wgrad_layout`` picks."""
-    if wgrad_layout(grad, data) == "NN":
+    """out [N, K] (+)= grad [T, N]^T @ data [T, K] through the GEMM library, in the layout ``wgrad_layout`` picks."""
+    layout = wgrad_layout(grad, data)
+    if layout == "NN":
         # the kernel that produced ``grad`` may have left its transpose on it, stamped with the tensor's version
         version, gt = getattr(grad, "_dh_rows_transposed", None) or (None, None)
         if (gt is None or version != grad._version or gt.shape != (grad.shape[1], grad.shape[0])
                 or gt.dtype != grad.dtype):
             gt = transpose_2d(grad)
         dense_gemm(data, gt, out, False, False, accumulate, workspace, workspace_bytes)
+    elif layout == "TT":
+        dense_gemm(transpose_2d(data), grad, out, True, True, accumulate, workspace, workspace_bytes)
     else:
         dense_gemm(data, grad, out, False, True, accumulate, workspace, workspace_bytes)
 

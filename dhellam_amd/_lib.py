@@ -26,6 +26,7 @@ SIGNATURES = {
     "dh_delay": (_i32, [_i64, _vp]),
     "dh_host_delay": (_i32, [_i64, _vp]),
     "dh_gemm": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _sz, _vp]),
+    "dh_gemm_tt": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _sz, _vp]),
     "dh_stream_create_cu_mask": (_i32, [_vp, _i32, _vp]),
     "dh_stream_destroy": (_i32, [_vp]),
     "dh_transpose_2d": (_i32, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp]),

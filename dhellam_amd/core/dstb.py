@@ -371,7 +371,8 @@ class DCFunc:
         # the weight-gradient product of the column projection wants this gradient transposed when the layer is
         # wide enough for that layout to pay (``_Clib.wgrad_layout``): the kernel then writes it alongside
         rows, n2 = swiglu_input.shape
-        want_t = (config.hidden_size >= WGRAD_TRANSPOSE_GRAD_MIN_K and rows * n2 >= WGRAD_TRANSPOSE_MIN_ELEMS)
+        want_t = (config.hidden_size >= WGRAD_TRANSPOSE_GRAD_MIN_K and rows * n2 >= WGRAD_TRANSPOSE_MIN_ELEMS
+                  and config.hidden_size >= n2)     # (fewer inputs than outputs: the input is the operand transposed)
         dgrad, _ = swiglu_back(grad_output, swiglu_input, None, stream, profiling=False, with_transposed=want_t)
         return dgrad
 

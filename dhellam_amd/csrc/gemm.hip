@@ -91,12 +91,11 @@ int make_plan(hipblasLtHandle_t h, const Key &key, int transa, int transb, int d
 
 }  // namespace
 
-extern "C" int dh_gemm(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows,
-                       int64_t b_cols, int transa, int transb, int accumulate, int dtype, int out_dtype,
-                       void *workspace, size_t workspace_bytes, void *stream) {
+static int gemm_entry(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows,
+                      int64_t b_cols, int transa, int transb, int accumulate, int dtype, int out_dtype,
+                      void *workspace, size_t workspace_bytes, void *stream) {
   DH_CHECK(dtype == DH_BF16 || dtype == DH_F16 || dtype == DH_F32, "unknown dtype %d", dtype);
   DH_CHECK(out_dtype == dtype || out_dtype == DH_F32, "the result is of the operands' type or fp32");
-  DH_CHECK(!(transa && transb), "TT layout not allowed");
   DH_CHECK(a_rows >= 0 && a_cols >= 0 && b_rows >= 0 && b_cols >= 0, "negative size");
   const int64_t m = transa ? a_rows : a_cols, k = transa ? a_cols : a_rows;
   const int64_t n = transb ? b_cols : b_rows, kb = transb ? b_rows : b_cols;
@@ -133,4 +132,21 @@ extern "C" int dh_gemm(const void *a, const void *b, void *d, int64_t a_rows, in
   DH_BLAS(hipblasLtMatmul(h, pl.op, &one, a, pl.a, b, pl.b, accumulate ? &one : &zero, d, pl.d, d, pl.d, &pl.algo,
                           workspace, workspace_bytes, (hipStream_t)stream));
   return DH_OK;
+}
+
+extern "C" int dh_gemm(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows,
+                       int64_t b_cols, int transa, int transb, int accumulate, int dtype, int out_dtype,
+                       void *workspace, size_t workspace_bytes, void *stream) {
+  DH_CHECK(!(transa && transb), "TT layout not allowed");
+  return gemm_entry(a, b, d, a_rows, a_cols, b_rows, b_cols, transa, transb, accumulate, dtype, out_dtype, workspace,
+                    workspace_bytes, stream);
+}
+
+// The layout dh_gemm refuses: D [n, m] = B^T @ A^T for A [m, k] and B [k, n], i.e. the weight-gradient product
+// dW = dY^T X with X handed over transposed (A = X^T) and dY as it is.
+extern "C" int dh_gemm_tt(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows,
+                          int64_t b_cols, int accumulate, int dtype, int out_dtype, void *workspace,
+                          size_t workspace_bytes, void *stream) {
+  return gemm_entry(a, b, d, a_rows, a_cols, b_rows, b_cols, 1, 1, accumulate, dtype, out_dtype, workspace,
+                    workspace_bytes, stream);
 }

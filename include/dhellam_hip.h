@@ -328,6 +328,13 @@ int dh_gemm(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_col
             int transa, int transb, int accumulate, int dtype, int out_dtype, void *workspace,
             size_t workspace_bytes, void *stream);
 
+/* The one layout dh_gemm refuses (as the reference does, "TT layout not allowed", csrc/operators/gemm.cu:3-170):
+ * D [n, m] = B^T @ A^T for A [m, k] and B [k, n], both row-major.  It is the weight-gradient product dW = dY^T X
+ * with X handed over transposed (A = X^T [K, T]) and dY [T, N] as it is: the cheaper of the two operands to
+ * transpose when the weight has fewer inputs than outputs.  No counterpart in the reference. */
+int dh_gemm_tt(const void *a, const void *b, void *d, int64_t a_rows, int64_t a_cols, int64_t b_rows, int64_t b_cols,
+               int accumulate, int dtype, int out_dtype, void *workspace, size_t workspace_bytes, void *stream);
+
 /* A stream whose kernels run only on the compute units named in `mask` (bit i of word i / 32; `words` x 32
  * bits must cover the device; with several XCDs bit i is compute unit i / n_xcd of XCD i % n_xcd).  The
  * MI355X form of the reference's libsmctrl partitioning (csrc/operators/smctrl.cpp:135-160, the `math_sm_count`

@@ -180,11 +180,19 @@ def test_wgrad_product(dtype, T, N, K, accumulate):
     dy, x = randn((T, N), dtype, 11, std=0.5), randn((T, K), dtype, 12, std=0.5)
     w0 = randn((N, K), dtype, 13)
     ref = dy.double().t() @ x.double() + (w0.double() if accumulate else 0)
+    # the smaller operand is the one transposed: X when the weight has fewer inputs than outputs ("TT"), else dY ("NN")
+    if dtype == torch.float32:
+        want = "NT"
+    elif K < N and T * K >= 1 << 20:
+        want = "TT"
+    elif K >= 3072 and T * N >= 1 << 20:
+        want = "NN"
+    else:
+        want = "NT"
+    assert _Clib.wgrad_layout(dy.cuda(), x.cuda()) == want
     lhs, rhs = _Clib.wgrad_operands(dy.cuda(), x.cuda())
-    assert lhs.is_contiguous() == (dtype != torch.float32 and K >= 3072 and T * N >= 1 << 20)
-    assert rhs.is_contiguous()
+    assert lhs.is_contiguous() == (want == "NN") and rhs.is_contiguous()
     assert torch.equal(lhs, dy.cuda().t()) and torch.equal(rhs, x.cuda())
-    assert _Clib.wgrad_layout(dy.cuda(), x.cuda()) == ("NN" if lhs.is_contiguous() else "NT")
     d = w0.clone().cuda()
     _Clib.pygemm(x.cuda(), dy.cuda(), d, None, 0, False, True, accumulate, 0, False)
     assert_close(d, ref, dtype, "pygemm wgrad")
@@ -386,7 +394,7 @@ def test_dense_gemm_argument_errors():
         return lib.dh_gemm(a.data_ptr(), b.data_ptr(), d.data_ptr(), ar, ac, br, bc, ta, tb, acc, dt, odt, ws, wsb, st)
 
     assert call(16, 32, 8, 32, 1, 0) == 0                                  # TN, no workspace
-    for bad in (call(16, 32, 8, 32, 1, 1),                                # TT
+    for bad in (call(16, 32, 8, 32, 1, 1),                                # TT: refused here as in the reference
                 call(16, 32, 8, 24, 1, 0),                                # inner sizes differ
                 call(16, 32, 8, 32, 1, 0, dt=7, odt=7),                   # unknown type
                 call(16, 32, 8, 32, 1, 0, dt=1, odt=2),                   # bf16 operands, fp16 result

@@ -234,7 +234,11 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
             gt = transpose_2d(grad)
         dense_gemm(data, gt, out, False, False, accumulate, workspace, workspace_bytes)
     elif layout == "TT":
-        dense_gemm(transpose_2d(data), grad, out, True, True, accumulate, workspace, workspace_bytes)
+        version, xt = getattr(data, "_dh_rows_transposed", None) or (None, None)
+        if (xt is None or version != data._version or xt.shape != (data.shape[1], data.shape[0])
+                or xt.dtype != data.dtype):
+            xt = transpose_2d(data)
+        dense_gemm(xt, grad, out, True, True, accumulate, workspace, workspace_bytes)
     else:
         dense_gemm(data, grad, out, False, True, accumulate, workspace, workspace_bytes)
 

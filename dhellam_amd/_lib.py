@@ -45,6 +45,7 @@ SIGNATURES = {
     "dh_swiglu_fwd": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp]),
     "dh_swiglu_bwd": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
     "dh_swiglu_bwd_t": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp]),
+    "dh_swiglu_fwd_t": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
     "dh_residual_add": (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     "dh_gelu": (_i32, [_vp, _vp, _i64, _i32, _vp]),
     "dh_bias_mask_add": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp]),

@@ -164,6 +164,9 @@ def _use(t, stream):
     """Tell the caching allocator that ``t`` is consumed on ``stream``."""
     if isinstance(t, torch.Tensor) and t.is_cuda:
         t.record_stream(stream)
+        kept = getattr(t, "_dh_rows_transposed", None)     # the transpose its producer left on it is consumed there too
+        if kept is not None:
+            kept[1].record_stream(stream)
     return t
 
 
@@ -230,7 +233,10 @@ class DCFunc:
     @staticmethod
     def gemm_mlp_linear(config, data, stream):
         input, weight = data
+        kept = getattr(input, "_dh_rows_transposed", None)
         input = input.view(config.tokens, -1)
+        if kept is not None:        # the transpose its producer wrote stays with the saved view (views share the version)
+            input._dh_rows_transposed = kept
         output, _ = gemm_fwd(config, input, weight, None, "TN", False, 0, True, stream)
         return output, input
 
@@ -327,7 +333,11 @@ class DCFunc:
     def swiglu(config, data, stream):
         (input,) = data
         input = input.view(config.micro_batch_size, config.seq_length, -1)
-        output, _ = swiglu(input, stream, False)
+        # the weight-gradient product of the row projection behind the activation takes this result transposed when
+        # the projection has fewer inputs than outputs (``_Clib.wgrad_layout``): the kernel then writes it alongside
+        f = input.shape[-1] // 2
+        want_t = f < config.hidden_size and config.tokens * f >= WGRAD_TRANSPOSE_MIN_ELEMS
+        output, _ = swiglu(input, stream, False, with_transposed=want_t)
         return output
 
     # ---- backward ---------------------------------------------------------------------

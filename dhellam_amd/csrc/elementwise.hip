@@ -7,6 +7,14 @@
 namespace dh {
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// out = silu(gate) * up for one element, every operation rounded by itself and the last product kept apart from
+// the caller's conversion (the kernels that use it must give the same bits).
+__device__ __forceinline__ float swiglu_value(float g, float u) {
+#pragma clang fp contract(off)
+  float o = g * sigmoidf_(g) * u;
+  asm("" : "+v"(o));
+  return o;
+}
 // d(gate) and d(up) of out = silu(gate) * up for one element, every operation rounded by itself (no fused multiply-add: the
 // kernels that use it must give the same bits, whatever the compiler would fuse around each call).
 __device__ __forceinline__ void swiglu_grad(float y1, float y2, float gg, float &d1, float &d2) {
@@ -57,8 +65,7 @@ swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems, 
         Vec<T> o;
 #pragma unroll
         for (int j = 0; j < N; ++j) {
-          const float g = to_f(a[u].v[j]);
-          o.v[j] = from_f<T>(g * sigmoidf_(g) * to_f(b[u].v[j]));
+          o.v[j] = from_f<T>(swiglu_value(to_f(a[u].v[j]), to_f(b[u].v[j])));
         }
         stg_s<NT>(out + id * N, o);
       }
@@ -106,6 +113,61 @@ swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restric
         stg_s<NT>(row + ((int64_t)fv + c) * N, d2);
       }
     }
+  }
+}
+
+// SwiGLU forward that also writes its result transposed: out [rows, f] and outT [f, rows] from one read of y.  The
+// transpose feeds the weight-gradient GEMM of the projection BEHIND the activation (dW = dY^T out runs fastest with
+// one operand transposed, and out is the smaller one there); produced here it costs one more write instead of a
+// read and a write of its own.  Same tiling as the backward below: a workgroup takes 64 rows x 128 columns,
+// stores them as rows, and passes them through LDS to store them as columns, 8 rows per lane.
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_fwd_t_kernel(const T *__restrict__ y, T *__restrict__ out, T *__restrict__ outt, int64_t rows, int64_t f,
+                    int64_t ld_t) {
+  constexpr int N = Vec<T>::N;                      // 8
+  constexpr int TR = 64, TC = 128, PITCH = TC * 2 + 4;
+  __shared__ __attribute__((aligned(16))) unsigned char tile[TR * PITCH];
+  const int64_t r0 = (int64_t)blockIdx.y * TR, c0 = (int64_t)blockIdx.x * TC;
+  const int tid = threadIdx.x;
+  {
+    const int lr = tid >> 4, ch = tid & 15;
+    Vec<T> a[4], b[4];
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t r = r0 + lr + 16 * i, c = c0 + ch * N;
+      ok[i] = r < rows && c < f;
+      if (ok[i]) {
+        const T *row = y + r * (2 * f);
+        a[i] = ldg(row + c);
+        b[i] = ldg(row + f + c);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int rl = lr + 16 * i;
+      Vec<T> o;
+#pragma unroll
+      for (int j = 0; j < N; ++j) o.v[j] = from_f<T>(ok[i] ? swiglu_value(to_f(a[i].v[j]), to_f(b[i].v[j])) : 0.f);
+      if (ok[i]) stg(out + (r0 + rl) * f + c0 + ch * N, o);
+      const uint32_t *s1 = reinterpret_cast<const uint32_t *>(&o);      // rows are 4-byte aligned only: dword stores
+      uint32_t *t1 = reinterpret_cast<uint32_t *>(tile + rl * PITCH + ch * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) t1[q] = s1[q];
+    }
+  }
+  __syncthreads();
+  const int lane = tid & 63, w = tid >> 6;
+  const int rb = lane & 7, cl = lane >> 3;            // 8-row block, column within the step
+#pragma unroll
+  for (int s2 = 0; s2 < 4; ++s2) {
+    const int col = 32 * w + 8 * s2 + cl;
+    const unsigned char *src = tile + (8 * rb) * PITCH + col * 2;
+    Vec<T> o;
+#pragma unroll
+    for (int j = 0; j < N; ++j) o.v[j] = *reinterpret_cast<const T *>(src + j * PITCH);
+    if (c0 + col < f && r0 + 8 * rb < rows) stg(outt + (c0 + col) * ld_t + r0 + 8 * rb, o);
   }
 }
 
@@ -190,7 +252,7 @@ swiglu_fwd_scalar_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t n
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / f, c = i - r * f;
     const float g = to_f(y[r * 2 * f + c]);
-    out[i] = from_f<T>(g * sigmoidf_(g) * to_f(y[r * 2 * f + f + c]));
+    out[i] = from_f<T>(swiglu_value(g, to_f(y[r * 2 * f + f + c])));
   }
 }
 template <typename T>
@@ -344,6 +406,27 @@ extern "C" int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t row
                          (const T *)g, (const T *)y, (T *)dy, rows * f, f);
     }
   });
+  DH_LAUNCH_CHECK();
+  return DH_OK;
+}
+
+extern "C" int dh_swiglu_fwd_t(const void *y, void *out, void *out_t, int64_t rows, int64_t f, int dtype, void *stream) {
+  using namespace dh;
+  DH_CHECK(rows >= 0 && f >= 0, "bad shape rows=%lld f=%lld", (long long)rows, (long long)f);
+  if (rows == 0 || f == 0) return DH_OK;
+  DH_CHECK(y && out && out_t, "null pointer");
+  DH_CHECK(dtype == DH_BF16 || dtype == DH_F16, "16-bit element types only (dtype %d)", dtype);
+  DH_CHECK(rows % 8 == 0 && f % 8 == 0, "rows=%lld and f=%lld must be multiples of 8", (long long)rows, (long long)f);
+  DH_CHECK(aligned16(y) && aligned16(out) && aligned16(out_t), "pointers must be 16-byte aligned");
+  const dim3 grid((unsigned)cdiv(f, 128), (unsigned)cdiv(rows, 64));
+  DH_CHECK(grid.y < 65536, "too many rows for one launch");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == DH_BF16)
+    hipLaunchKernelGGL((swiglu_fwd_t_kernel<bf16_t>), grid, dim3(256), 0, st, (const bf16_t *)y, (bf16_t *)out,
+                       (bf16_t *)out_t, rows, f, rows);
+  else
+    hipLaunchKernelGGL((swiglu_fwd_t_kernel<f16_t>), grid, dim3(256), 0, st, (const f16_t *)y, (f16_t *)out,
+                       (f16_t *)out_t, rows, f, rows);
   DH_LAUNCH_CHECK();
   return DH_OK;
 }

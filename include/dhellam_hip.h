@@ -86,6 +86,15 @@ int dh_swiglu_fwd(const void *y, void *out, int64_t rows, int64_t f, int dtype,
 int dh_swiglu_bwd(const void *g, const void *y, void *dy, int64_t rows,
                   int64_t f, int dtype, void *stream);
 
+/* dh_swiglu_fwd that also writes its result transposed: out_t [f, rows]
+ * (row-major) next to out [rows, f], for the weight-gradient product of the
+ * projection behind the activation (dhellam/core/dstb.py:543-598), which runs
+ * with the activation handed over transposed (dh_gemm_tt).  16-bit types; rows
+ * and f multiples of 8; out is bit for bit that of dh_swiglu_fwd.  No
+ * counterpart in the reference. */
+int dh_swiglu_fwd_t(const void *y, void *out, void *out_t, int64_t rows,
+                    int64_t f, int dtype, void *stream);
+
 /* dh_swiglu_bwd that also writes the gradient transposed: dy_t [2f, rows]
  * (row-major) next to dy [rows, 2f], for the weight-gradient product of the
  * projection in front of the activation (csrc/operators/gemm.cu:3-170 with

@@ -248,6 +248,33 @@ def test_swiglu_backward_with_transposed_output(dtype, rows, f):
     assert not hasattr(odd, "_dh_rows_transposed")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,f", [(4096, 3584), (72, 200), (8, 8), (136, 1032)])
+def test_swiglu_forward_with_transposed_output(dtype, rows, f):
+    """dh_swiglu_fwd_t: the same result as dh_swiglu_fwd, bit for bit, plus its transpose; the weight-gradient
+    helper picks the transpose up from the tensor (the layout that hands X over transposed)."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.swiglu import swiglu
+    y = randn((rows, 2 * f), dtype, 1).cuda()
+    ref, _ = swiglu(y)
+    got, _ = swiglu(y, with_transposed=True)
+    assert torch.equal(got, ref)
+    version, gt = got._dh_rows_transposed
+    assert version == got._version and gt.shape == (f, rows) and torch.equal(gt, ref.t().contiguous())
+    n = 2 * f + 8                                                # more outputs than inputs: X is the operand transposed
+    dy = randn((rows, n), dtype, 3).cuda()
+    if rows * f >= _Clib.WGRAD_TRANSPOSE_MIN_ELEMS:
+        assert _Clib.wgrad_layout(dy, got) == "TT"
+        d1 = torch.zeros(n, f, dtype=dtype, device="cuda")
+        d2 = torch.zeros_like(d1)
+        _Clib.wgrad_gemm(dy, got, d1, False)                     # uses the kernel's transpose
+        _Clib.wgrad_gemm(dy, ref, d2, False)                     # transposes by itself
+        assert torch.equal(d1, d2)
+        assert_close(d1, dy.double().cpu().t() @ ref.double().cpu(), dtype, "wgrad through X^T")
+    odd, _ = swiglu(torch.cat([y[:, : f - 4], y[:, f: 2 * f - 4]], 1).contiguous(), with_transposed=True)
+    assert not hasattr(odd, "_dh_rows_transposed")              # f not a multiple of 8: plain kernel
+
+
 def test_bandwidth_ops_are_deterministic():
     """Norm backward (staged column sums), SwiGLU, RoPE: two runs, same bits."""
     from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd

@@ -337,7 +337,7 @@ def profile_op(name: str, iters: int = 5):
             y, saved, _ = moe.expert_ffn_fwd(xp, w1, w2, offs)
             dyp = rn(Rm, Hm)
             fn = lambda: moe.expert_ffn_bwd(dyp, xp, w1, w2, offs, saved)
-    elif name in ("norm", "swiglu", "cross_entropy", "transpose"):
+    elif name in ("norm", "swiglu", "swiglu_t", "cross_entropy", "transpose"):
         # bandwidth kernels at sizes beyond the 256 MB last-level cache (norm, SwiGLU) / at the head-block and
         # weight-gradient shapes (cross entropy, transpose); forward then backward in each iteration
         from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
@@ -350,6 +350,9 @@ def profile_op(name: str, iters: int = 5):
         elif name == "swiglu":
             yy, gg = rn(16384, 7168), rn(16384, 3584)
             fn = lambda: (swiglu(yy), swiglu_back(gg, yy))
+        elif name == "swiglu_t":       # the kernels that write their result transposed as well
+            yy, gg = rn(16384, 7168), rn(16384, 3584)
+            fn = lambda: (swiglu(yy, with_transposed=True), swiglu_back(gg, yy, with_transposed=True))
         elif name == "cross_entropy":
             lg = rn(4096, 16032)
             ce_in = {"vocab_parallel_logits": lg, "target": torch.randint(0, 16032, (4096,), generator=g, device=dev)}
@@ -483,7 +486,7 @@ def main():
                     help="also time both schedules with each sequence-parallel stand-in taking this long (0: skip)")
     ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
     ap.add_argument("--profile-op", default=None,
-                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, swiglu_t, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
     ap.add_argument("--analyze-trace", default=None,
                     help="kernel-trace CSV of `rocprofv3 --kernel-trace -- python bench.py --profile-op layer`: print the "
                          "overlap headroom of the serial schedule and exit (no GPU needed)")

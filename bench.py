@@ -517,14 +517,13 @@ def main():
 
     def timed(fn, runner=runner):
         # A step is what lies between two optimizer steps: the weights have just changed, so their resident
-        # transposes (used by the data-gradient GEMMs) are rebuilt inside the timed region, once per step.
+        # transposes (used by the data-gradient GEMMs) are rebuilt inside the timed region, once per step
+        # (run_serial / run_double_strand do it on entry).
         for _ in range(args.warmup):
-            runner.refresh_weight_transposes()
             fn(mbs)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            runner.refresh_weight_transposes()
             fn(mbs)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps * 1e3

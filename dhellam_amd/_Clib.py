@@ -10,13 +10,14 @@ merge, MoE, grouped GEMM) are exported under ``py*`` names in the same style.
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Optional
 
 import torch
 
 from . import _lib
 
-__all__ = ["add_tensors", "pygemm", "dense_gemm", "dense_ok", "wgrad_gemm", "wgrad_layout", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
+__all__ = ["add_tensors", "pygemm", "dense_gemm", "dense_ok", "keep_transposed", "refresh_transposed", "wgrad_gemm", "wgrad_layout", "pygelu", "pybda", "pymha_varlen_fwd", "pymha_varlen_bwd", "pyattn_merge",
            "pyrmsnorm_fwd", "pyrmsnorm_bwd", "pyrope_fwd", "pyrope_bwd", "pyswiglu_fwd", "pyswiglu_bwd",
            "pymoe_route_topk", "pymoe_sort", "pymoe_permute", "pymoe_unpermute", "pygrouped_gemm_nt",
            "pygrouped_gemm_nn", "pygrouped_gemm_tn", "pycross_entropy_fwd", "pycross_entropy_bwd",
@@ -75,6 +76,7 @@ def dense_gemm(A, B, D, transa: bool, transb: bool, accumulate: bool, workspace=
     if tuple(D.shape) != (n, m):
         raise RuntimeError(f"dense_gemm: output is {tuple(D.shape)}, the product is {(n, m)}")
     stream = torch.cuda.current_stream()
+    _lib.mark_written(D)
     if workspace is None or not getattr(workspace, "is_cuda", False) or workspace_bytes <= 0:
         workspace = _gemm_workspace(A.device, stream.cuda_stream)
         workspace_bytes = workspace.numel()
@@ -249,46 +251,98 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
 # 8192, 1024 / 7168, 8192 / 8192, 3584)  90 -> 72 / 94 -> 73 / 366 -> 308 / 205 -> 174, results identical bit for
 # bit.  A weight changes once per optimizer step and is read by every micro-batch's backward in between, and the
 # transposes (9 / 7 / 38 / 20 us) cost less than one micro-batch saves, so a weight may be registered to be kept in
-# both layouts.  The copy lives on the tensor object and is rebuilt when the tensor's version counter has moved (any
-# in-place torch op on the tensor moves it).  A writer that goes around the counter (``weight.data.copy_()``, a raw
-# kernel) must call ``keep_transposed(weight, refresh=True)`` itself; weights that were never registered take the NN
-# product as before.
+# both layouts.  The copy lives on the tensor object.  Who keeps it current: the containers that run a step
+# (``LayerRunner.run_*``, ``DSLLMStep.step``, ``run_microbatches``) rebuild the copies of their weights at the START
+# of every step with ``refresh_transposed`` -- unconditionally, because the writers that matter do not announce
+# themselves: ``p.data.copy_()`` / ``p.data.add_()`` (Megatron's fp16 and distributed optimizers), collectives and raw
+# kernels writing into a parameter buffer all leave the tensor's version counter where it was.  In between, a moved
+# version counter (any in-place torch op on the tensor itself) also triggers a rebuild at the next use.  A caller
+# that drives ``dgrad_gemm`` by hand and updates weights around the counter calls ``refresh_transposed`` itself;
+# weights that were never registered take the NN product as before.
+_kept_weights: "weakref.WeakSet" = weakref.WeakSet()
+
+
+class _Held:
+    """What a registered weight carries: the transpose, the version it was built from, the event and stream of
+    the build, and one event per stream that has read the copy since (a rebuild waits for them)."""
+    __slots__ = ("version", "wt", "built", "stream_ptr", "readers")
+
+    def __init__(self, version, wt, built, stream_ptr):
+        self.version, self.wt, self.built, self.stream_ptr, self.readers = version, wt, built, stream_ptr, {}
+
+
 def keep_transposed(weight: torch.Tensor, refresh: bool = False) -> Optional[torch.Tensor]:
     """Registers ``weight`` [N, K] (or a stack of them, [G, N, K]: the experts of a rank) for a resident transpose
     [K, N] ([G, K, N]) built now, on the current stream, and returns it; None if the tensor is not one
-    ``dh_transpose_2d`` takes (then nothing is registered)."""
+    ``dh_transpose_2d`` takes (then nothing is registered).  ``refresh`` rebuilds the copy of a weight that is
+    already registered even if its version counter has not moved; the rebuild writes into the same buffer after
+    waiting for every stream that read the old copy."""
     if not (weight.is_cuda and weight.dim() in (2, 3) and weight.is_contiguous() and _can_transpose(weight[0] if weight.dim() == 3 else weight)):
         return None
     held = getattr(weight, "_dh_transposed", None)
-    if held is not None and not refresh and held[0] == weight._version:
-        return held[1]
+    if held is not None and not refresh and held.version == weight._version:
+        return held.wt
+    stream = torch.cuda.current_stream()
+    if held is not None:
+        for ptr, ev in held.readers.items():          # the old copy may still be read on another stream
+            if ptr != stream.cuda_stream:
+                stream.wait_event(ev)
+        if held.stream_ptr != stream.cuda_stream:
+            stream.wait_event(held.built)
     with torch.no_grad():
         w = weight.detach()
         if w.dim() == 2:
-            wt = transpose_2d(w, held[1] if held is not None else None)
+            wt = transpose_2d(w, held.wt if held is not None else None)
         else:
-            wt = held[1] if held is not None else torch.empty((w.shape[0], w.shape[2], w.shape[1]), dtype=w.dtype, device=w.device)
+            wt = held.wt if held is not None else torch.empty((w.shape[0], w.shape[2], w.shape[1]), dtype=w.dtype, device=w.device)
             for g in range(w.shape[0]):
                 transpose_2d(w[g], wt[g])
-    stream = torch.cuda.current_stream()
     ev = torch.cuda.Event()
     ev.record(stream)
-    weight._dh_transposed = (weight._version, wt, ev, stream.cuda_stream)
+    weight._dh_transposed = _Held(weight._version, wt, ev, stream.cuda_stream)
+    _kept_weights.add(weight)
     return wt
+
+
+def refresh_transposed(weights=None) -> int:
+    """Rebuilds the resident transposes of ``weights`` (default: every registered weight still alive) on the current
+    stream, whatever their version counters say: the call that follows an optimizer step.  Unregistered tensors in
+    ``weights`` are skipped.  Returns how many copies were rebuilt."""
+    n = 0
+    for w in (list(_kept_weights) if weights is None else weights):
+        if isinstance(w, torch.Tensor) and getattr(w, "_dh_transposed", None) is not None:
+            keep_transposed(w, refresh=True)
+            n += 1
+    return n
 
 
 def transposed_of(weight: torch.Tensor) -> Optional[torch.Tensor]:
     """The resident transpose of a registered weight, brought up to date and safe to read on the current stream;
-    None for a weight that was not registered with ``keep_transposed``."""
+    None for a weight that was not registered with ``keep_transposed``.  The reader calls ``_note_read`` after
+    it has queued its work."""
     held = getattr(weight, "_dh_transposed", None)
     if held is None:
         return None
-    if held[0] != weight._version:
+    if held.version != weight._version:
         return keep_transposed(weight, refresh=True)
     stream = torch.cuda.current_stream()
-    if held[3] != stream.cuda_stream:
-        stream.wait_event(held[2])
-    return held[1]
+    if held.stream_ptr != stream.cuda_stream:
+        stream.wait_event(held.built)
+    return held.wt
+
+
+def _note_read(weight: torch.Tensor) -> None:
+    """Marks the point on the current stream up to which the resident transpose of ``weight`` is being read."""
+    held = getattr(weight, "_dh_transposed", None)
+    if held is None:
+        return
+    stream = torch.cuda.current_stream()
+    if stream.cuda_stream == held.stream_ptr:
+        return                                        # same stream as the builder: already ordered
+    ev = held.readers.get(stream.cuda_stream)
+    if ev is None:
+        ev = held.readers[stream.cuda_stream] = torch.cuda.Event()
+    ev.record(stream)
 
 
 def dgrad_gemm(grad: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
@@ -297,6 +351,7 @@ def dgrad_gemm(grad: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> N
     wt = transposed_of(weight)
     if wt is not None and wt.dtype == grad.dtype:
         dense_gemm(wt, grad, out, True, False, False)
+        _note_read(weight)
     else:
         dense_gemm(weight, grad, out, False, False, False)
 
@@ -394,8 +449,9 @@ ATTN_BWD_DS_LIMIT_DEFAULT = 1280 << 20
 
 
 def set_attn_bwd_ds_limit(nbytes: int = ATTN_BWD_DS_LIMIT_DEFAULT) -> None:
-    """Workspace bytes up to which the attention backward keeps dS for its dQ product (``dh_attn_bwd_set_ds_limit``;
-    0: always recompute).  Process-wide."""
+    """Bytes of dS up to which the attention backward keeps dS for its dQ product (``dh_attn_bwd_set_ds_limit``;
+    0: always recompute).  Process-wide; it steers the sizing call and the choice inside the backward, which also
+    checks the size of the workspace it was handed."""
     _lib.load().dh_attn_bwd_set_ds_limit(int(nbytes))
 
 
@@ -418,7 +474,7 @@ def _attn_bwd_raw(dout, q, k, v, out, lse, dq, dk, dv, delta, cu_q, cu_k, max_q,
     ws = _attn_bwd_workspace(nbytes, q.device, stream_ptr)
     _lib.check(lib.dh_attn_bwd_acc(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                    lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _lib.ptr(delta),
-                                   ws.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(), b, int(max_q), int(max_k),
+                                   ws.data_ptr(), ws.numel(), cu_q.data_ptr(), cu_k.data_ptr(), b, int(max_q), int(max_k),
                                    q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2], _tok_stride(q),
                                    _tok_stride(k), _tok_stride(v), _tok_stride(out), _tok_stride(dout),
                                    _tok_stride(dq), _tok_stride(dk), _tok_stride(dv), float(scale), int(bool(causal)),

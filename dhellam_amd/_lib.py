@@ -41,7 +41,7 @@ SIGNATURES = {
     "dh_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _vp]),
     "dh_add_norm_fwd": (_i32, [_vp] * 8 + [_i64, _i64, _f32, _i32, _i32, _vp]),
     "dh_norm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
-    "dh_norm_bwd": (_i32, [_vp] * 10 + [_i64, _i64, _i32, _i32, _i32, _vp]),
+    "dh_norm_bwd": (_i32, [_vp] * 10 + [_sz, _i64, _i64, _i32, _i32, _i32, _vp]),
     "dh_swiglu_fwd": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp]),
     "dh_swiglu_bwd": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
     "dh_swiglu_bwd_t": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp]),
@@ -52,13 +52,14 @@ SIGNATURES = {
     "dh_rope": (_i32, [_vp] * 6 + [_i64, _i32, _i32, _i32, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _vp]),
     "dh_attn_fwd": (_i32, [_vp] * 7 + [_i32] * 6 + [_i64] * 4 + [_f32, _i32, _i32, _vp]),
     "dh_attn_bwd_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]),
-    "dh_attn_bwd": (_i32, [_vp] * 13 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _vp]),
+    "dh_attn_bwd_min_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]),
+    "dh_attn_bwd": (_i32, [_vp] * 11 + [_sz] + [_vp] * 2 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _vp]),
     "dh_attn_bwd_set_ds_limit": (None, [_sz]),
-    "dh_attn_bwd_acc": (_i32, [_vp] * 13 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _i32, _vp]),
+    "dh_attn_bwd_acc": (_i32, [_vp] * 11 + [_sz] + [_vp] * 2 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _i32, _vp]),
     "dh_attn_merge": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
     "dh_moe_route_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
     "dh_moe_sort_workspace_bytes": (_sz, [_i64, _i32]),
-    "dh_moe_sort": (_i32, [_vp] * 6 + [_i64, _i32, _vp]),
+    "dh_moe_sort": (_i32, [_vp] * 6 + [_sz, _i64, _i32, _vp]),
     "dh_moe_sort_static_max_assign": (_i64, []),
     "dh_moe_sort_static": (_i32, [_vp] * 5 + [_i64, _i32, _vp]),
     "dh_moe_gather_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
@@ -115,3 +116,12 @@ def need_cuda(*ts) -> None:
     for t in ts:
         if t is not None and not t.is_cuda:
             raise RuntimeError("dhellam operators need tensors on the GPU")
+
+
+def mark_written(*ts) -> None:
+    """A kernel of this library is about to write these tensors through their raw pointers, which does not move
+    torch's version counter: whatever a producer hung on them that described their OLD contents (the transposed
+    twin that the SwiGLU kernels leave for the weight-gradient GEMM) is dropped here."""
+    for t in ts:
+        if t is not None:
+            t.__dict__.pop("_dh_rows_transposed", None)

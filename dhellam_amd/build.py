@@ -82,6 +82,49 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     return LIB_PATH
 
 
+EXT_SRC = CSRC / "torchapi.cpp"
+EXT_PKG = ROOT / "dhellam"
+
+
+def torch_extension_path() -> Path:
+    import sysconfig
+    return EXT_PKG / ("_Clib" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_torch_extension(verbose: bool = False) -> Path:
+    """Compiles ``csrc/torchapi.cpp`` into the pybind11 torch extension ``dhellam._Clib`` (the reference builds a
+    module of that name from its csrc/torchapi.cpp, setup.py:234-244).  Host code only: the host compiler with
+    torch's headers, linked against ``libdhellam_hip.so`` (found at run time relative to the extension)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as E
+    if not LIB_PATH.exists():
+        raise RuntimeError(f"{LIB_PATH} must be built first")
+    rocm = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+    out = torch_extension_path()
+    tmp = out.with_suffix(".so.tmp")
+    torch_lib = E.library_paths()[0]
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_Clib", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{ROOT / 'include'}", *[f"-isystem{p}" for p in E.include_paths()], f"-isystem{rocm / 'include'}",
+           f"-I{sysconfig.get_paths()['include']}", str(EXT_SRC), "-o", str(tmp),
+           f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lamdhip64",
+           f"-L{LIB_DIR}", "-ldhellam_hip", "-Wl,-rpath,$ORIGIN/../dhellam_amd/lib", f"-Wl,-rpath,{torch_lib}"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building dhellam._Clib failed:\n{res.stderr}")
+    if res.stderr.strip() and verbose:
+        print(res.stderr, file=sys.stderr)
+    os.replace(tmp, out)
+    return out
+
+
 if __name__ == "__main__":
     path = build(verbose="-v" in sys.argv)
     print(path)
+    if "--no-ext" not in sys.argv:
+        print(build_torch_extension(verbose="-v" in sys.argv))

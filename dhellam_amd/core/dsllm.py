@@ -24,7 +24,7 @@ from typing import Dict, List, Optional
 import torch
 
 from . import dshb
-from .._Clib import keep_transposed
+from .._Clib import keep_transposed, refresh_transposed
 from .dstb import DCoperation, LayerConfig, Plan, exec as exec_blocks, init_DCBlocks
 from .layer import make_weights
 
@@ -105,10 +105,15 @@ class DSLLMStep:
             dshb.pre_process_bwd(ctx, dx, batch_first=True)
 
     # ---- schedules ----------------------------------------------------------------------------
-    def step(self, batches: List[dict], double_strand: bool = True, loss_scale: float = 1.0) -> List[torch.Tensor]:
+    def step(self, batches: List[dict], double_strand: bool = True, loss_scale: float = 1.0,
+             refresh_transposes: bool = True) -> List[torch.Tensor]:
         """Forward and backward of every micro-batch ({"token_ids", "labels", "loss_mask"}, each [b, s]);
         gradients accumulate into the parameters' ``main_grad``.  Returns the micro-batch losses
-        (each already divided by the number of micro-batches and multiplied by ``loss_scale``)."""
+        (each already divided by the number of micro-batches and multiplied by ``loss_scale``).  The resident
+        transposes of the weights are rebuilt first (the weights may have been updated by any means since the last
+        step); ``refresh_transposes=False`` is for several calls between two updates."""
+        if refresh_transposes and self.cfg.resident_weight_transposes:
+            refresh_transposed(t for _, t in self.named_parameters())
         n, L = len(batches), self.num_layers
         s1 = self.stream1
         s2 = self.stream2 if double_strand else self.stream1
@@ -259,11 +264,14 @@ class DSLLM(torch.nn.Module):
         return self.dctb(placeholder)
 
 
-def run_microbatches(model: DSLLM, batches: List[dict]) -> List[torch.Tensor]:
+def run_microbatches(model: DSLLM, batches: List[dict], refresh_transposes: bool = True) -> List[torch.Tensor]:
     """A whole step through the module shell: forward of micro-batch 0, then forward(i + 1) beside backward(i),
     then the last backward -- the order the reference's patched no-pipelining schedule produces.  Returns the
-    micro-batch losses; gradients are in the parameters' ``main_grad``."""
+    micro-batch losses; gradients are in the parameters' ``main_grad``.  The resident transposes of the model's
+    weights are rebuilt first: an optimizer that writes through ``p.data`` leaves nothing a lazy check could see."""
     from ..common.global_variables import GLOBAL_VARIABLES
+    if refresh_transposes:
+        refresh_transposed(model.parameters())
     GLOBAL_VARIABLES['loss'] = []
     prev = None
     for mb in list(batches) + [None]:

@@ -13,7 +13,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from .._Clib import keep_transposed
+from .._Clib import keep_transposed, refresh_transposed
 from .dstb import DCoperation, LayerConfig, Plan, exec as exec_blocks, init_DCBlocks
 
 
@@ -116,14 +116,17 @@ class LayerRunner:
                            movable=self.plan.movable)
 
     def refresh_weight_transposes(self):
-        """Rebuilds W^T of every projection weight on the current stream: what follows an optimizer step when the
-        weights are kept in both layouts (a step that goes through torch's in-place ops triggers it by itself)."""
+        """Rebuilds W^T of every projection weight on the current stream.  ``run_serial`` / ``run_double_strand``
+        call it at the start of every step: a step is what lies between two optimizer steps, and an optimizer that
+        writes through ``p.data`` (or a raw kernel, or a collective) leaves no trace a lazy check could see."""
         if self.cfg.resident_weight_transposes:
-            for k in ("column_attn_weight", "linear_attn_weight", "column_mlp_weight", "linear_mlp_weight"):
-                keep_transposed(self.weights[k], refresh=True)
+            refresh_transposed(self.weights.values())
 
-    def run_serial(self, mbs: List[dict]):
-        """F0 B0 F1 B1 ... on ONE stream with the fwd_only / bwd_only plans."""
+    def run_serial(self, mbs: List[dict], refresh_transposes: bool = True):
+        """F0 B0 F1 B1 ... on ONE stream with the fwd_only / bwd_only plans.  ``refresh_transposes=False`` is for a
+        caller that runs several such calls between two weight updates."""
+        if refresh_transposes:
+            self.refresh_weight_transposes()
         s = self.stream1
         s.wait_stream(torch.cuda.current_stream())
         outs, dxs = [], []
@@ -136,9 +139,11 @@ class LayerRunner:
         torch.cuda.current_stream().wait_stream(s)
         return outs, dxs
 
-    def run_double_strand(self, mbs: List[dict]):
+    def run_double_strand(self, mbs: List[dict], refresh_transposes: bool = True):
         """F0 . (F1 || B0) . (F2 || B1) ... B_last: forward strand on stream1, backward strand
         on stream2, paired steps following the plan's DCBlocks."""
+        if refresh_transposes:
+            self.refresh_weight_transposes()
         s1, s2 = self.stream1, self.stream2
         cur = torch.cuda.current_stream()
         s1.wait_stream(cur)

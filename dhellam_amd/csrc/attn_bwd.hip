@@ -1414,12 +1414,7 @@ template <typename T, int D, int NW>
 static int launch_dkv(const AttnBwdParams &p, int batch, int max_sk, hipStream_t st) {
   constexpr int BN = 32 * NW, BM = 32;
   constexpr size_t smem = 2 * 2 * BM * (D + 16) * sizeof(T) + 4 * BM * sizeof(float);
-  static bool attr_set = false;
-  if (!attr_set) {
-    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dkv_kernel<T, D, NW>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
-  }
+  DH_MAX_DYNAMIC_LDS_PER_DEVICE((&attn_bwd_dkv_kernel<T, D, NW>), smem);
   dim3 grid((unsigned)cdiv(max_sk, BN), (unsigned)(p.hk * p.hsplit), (unsigned)batch);
   hipLaunchKernelGGL((attn_bwd_dkv_kernel<T, D, NW>), grid, dim3(64 * NW), smem, st, p);
   return DH_OK;
@@ -1429,12 +1424,7 @@ template <typename T, int D, int NW>
 static int launch_dq(const AttnBwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * NW, BN = 32;
   constexpr size_t smem = 2 * BN * ((D + 16) + (D + 8)) * sizeof(T);
-  static bool attr_set = false;
-  if (!attr_set) {
-    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_bwd_dq_kernel<T, D, NW>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
-  }
+  DH_MAX_DYNAMIC_LDS_PER_DEVICE((&attn_bwd_dq_kernel<T, D, NW>), smem);
   dim3 grid((unsigned)cdiv(p.max_sq, BM), (unsigned)p.hq, (unsigned)batch);
   hipLaunchKernelGGL((attn_bwd_dq_kernel<T, D, NW>), grid, dim3(64 * NW), smem, st, p);
   return DH_OK;
@@ -1478,40 +1468,57 @@ static bool dq_big_grid(int batch, int max_sq, int hq, int causal) {
   return (causal ? (t + 1) / 2 : t) * hq * batch >= 256;
 }
 
-// Bytes of the dS blocks for these sizes (key count as an upper bound of the longest sequence), 0 if not kept.
-static size_t ds_bytes(int batch, int max_sq, int64_t max_sk, int hq, int d, int dtype, int causal) {
+// Bytes of the dS blocks for these sizes (key count as an upper bound of the longest sequence); 0 for calls that
+// never keep dS, whatever space there is (other head dims, fp32, a chip-filling recomputing kernel).
+static size_t ds_bytes_wanted(int batch, int max_sq, int64_t max_sk, int hq, int d, int dtype, int causal) {
   if (dtype == DH_F32 || d != 128 || batch <= 0 || max_sq <= 0 || max_sk <= 0) return 0;
   if (dq_big_grid(batch, max_sq, hq, causal)) return 0;
   // one block more per row than needed: rows a power of two apart would meet on the same memory channels
   const size_t nqt = 2 * (size_t)cdiv(max_sq, 64), nkb = 2 * (size_t)cdiv(max_sk, 64) + 1;
-  const size_t n = (size_t)batch * hq * nqt * nkb * 2048;
+  return (size_t)batch * hq * nqt * nkb * 2048;
+}
+
+// ... and under the process-wide limit: 0 if they exceed it.
+static size_t ds_bytes(int batch, int max_sq, int64_t max_sk, int hq, int d, int dtype, int causal) {
+  const size_t n = ds_bytes_wanted(batch, max_sq, max_sk, hq, d, dtype, causal);
   return n <= g_ds_limit.load() ? n : 0;
+}
+
+// Workspace bytes every call of these sizes needs: delta, the lse / delta planes of the head-dim-128 kernels and the
+// fp32 dK / dV partials of a split GQA group.  The dS blocks, where kept, lie behind them.
+static size_t bwd_base_bytes(int64_t total_k, int batch, int max_seqlen_q, int hq, int hk, int d, int dtype) {
+  const size_t sq = (size_t)(max_seqlen_q > 0 ? max_seqlen_q : 0);
+  size_t n = align256((size_t)batch * hq * sq * sizeof(float));            // delta
+  if (dtype != DH_F32 && d == 128) n += 2 * align256((size_t)batch * hq * ((sq + 31) / 32 * 32) * sizeof(float));
+  if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
+    n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
+  return n + 256;                                                          // the base pointer is rounded up to 256
 }
 
 }  // namespace dh
 
 extern "C" void dh_attn_bwd_set_ds_limit(size_t bytes) { dh::g_ds_limit.store(bytes); }
 
+extern "C" size_t dh_attn_bwd_min_workspace_bytes(int64_t total_q, int64_t total_k, int batch, int max_seqlen_q, int hq,
+                                                  int hk, int d, int dtype) {
+  (void)total_q;
+  return dh::bwd_base_bytes(total_k, batch, max_seqlen_q, hq, hk, d, dtype);
+}
+
 extern "C" size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch, int max_seqlen_q, int hq,
                                               int hk, int d, int dtype) {
   using namespace dh;
   (void)total_q;
-  const size_t plane = align256((size_t)batch * hq * (max_seqlen_q > 0 ? max_seqlen_q : 0) * sizeof(float));
-  size_t n = plane;                               // delta
-  const size_t plane2 = align256((size_t)batch * hq * (size_t)(((max_seqlen_q > 0 ? max_seqlen_q : 0) + 31) / 32 * 32) * sizeof(float));
-  if (dtype != DH_F32 && d == 128) n += 2 * plane2;  // lse (exp2 units) and delta side by side for the d = 128 kernels
   // dS blocks, if a call of these sizes may keep them (causal or not is not known here: the causal grid is the smaller
   // one; the longest sequence has at most total_k keys)
-  n += align256(ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, 1));
-  if (dtype != DH_F32 && hk > 0 && hq / hk > 1)
-    n += 2 * align256((size_t)(hq / hk) * (size_t)total_k * hk * d * sizeof(float));
-  return n + 256;
+  return bwd_base_bytes(total_k, batch, max_seqlen_q, hq, hk, d, dtype) +
+         align256(ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, 1));
 }
 
 static int attn_bwd_entry(const void *dout, const void *q, const void *k, const void *v, const void *out,
                           const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
-                          const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
-                          int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                          size_t workspace_bytes, const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch,
+                          int max_seqlen_q, int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
                           int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
                           int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
                           float softmax_scale, int causal, int dq_accumulate, int dtype, void *stream) {
@@ -1522,6 +1529,9 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
   DH_CHECK(dout && q && k && v && out && lse && dq && dk && dv && workspace && cu_seqlens_q && cu_seqlens_k,
            "null pointer");
   DH_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");
+  const size_t base_bytes = bwd_base_bytes(total_k, batch, max_seqlen_q, hq, hk, d, dtype);
+  DH_CHECK(workspace_bytes >= base_bytes, "workspace of %zu bytes is smaller than the %zu bytes this call needs "
+           "(dh_attn_bwd_min_workspace_bytes)", workspace_bytes, base_bytes);
   hipStream_t st = (hipStream_t)stream;
   uint8_t *ws = (uint8_t *)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   const size_t plane = align256((size_t)batch * hq * max_seqlen_q * sizeof(float));
@@ -1543,10 +1553,12 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
   // head dim 128 in 16 bits, two ways: with room for dS in the workspace the dK/dV kernel keeps it and dQ is one
   // product over it (delta from the delta kernel, which runs first); otherwise the dQ kernel recomputes S and dP,
   // forms delta itself and runs first.  Everything else uses the delta kernel.
-  const size_t dsb = ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, causal);
+  // dS is kept only if the blocks fit behind everything else in the workspace THIS call was given (and under the
+  // process-wide limit); they take the tail of the workspace
+  size_t dsb = ds_bytes(batch, max_seqlen_q, total_k, hq, d, dtype, causal);
+  if (dsb > 0 && base_bytes + align256(dsb) > workspace_bytes) dsb = 0;
   const bool keep_ds = dsb > 0 && max_seqlen_k > 0;
-  uint8_t *ds_ws = ws;
-  ws += align256(dsb);
+  uint8_t *ds_ws = (uint8_t *)(((uintptr_t)workspace + 255) & ~(uintptr_t)255) + (base_bytes - 256);
   const bool delta_in_dq = dtype != DH_F32 && d == 128 && !keep_ds;
   if (max_seqlen_q > 0 && !delta_in_dq) {
     DH_DISPATCH_DTYPE(dtype, {
@@ -1625,24 +1637,24 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
 
 extern "C" int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                            const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
-                           const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
-                           int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
+                           size_t workspace_bytes, const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch,
+                           int max_seqlen_q, int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
                            int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
                            int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
                            float softmax_scale, int causal, int dtype, void *stream) {
-  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, cu_seqlens_q, cu_seqlens_k, batch,
+  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, workspace_bytes, cu_seqlens_q, cu_seqlens_k, batch,
                         max_seqlen_q, max_seqlen_k, total_q, total_k, hq, hk, d, q_stride, k_stride, v_stride, o_stride,
                         do_stride, dq_stride, dk_stride, dv_stride, softmax_scale, causal, 0, dtype, stream);
 }
 
 extern "C" int dh_attn_bwd_acc(const void *dout, const void *q, const void *k, const void *v, const void *out,
                                const float *lse, void *dq, void *dk, void *dv, float *delta_out, void *workspace,
-                               const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k, int batch, int max_seqlen_q,
-                               int max_seqlen_k, int64_t total_q, int64_t total_k, int hq, int hk, int d,
-                               int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
+                               size_t workspace_bytes, const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                               int batch, int max_seqlen_q, int max_seqlen_k, int64_t total_q, int64_t total_k, int hq,
+                               int hk, int d, int64_t q_stride, int64_t k_stride, int64_t v_stride, int64_t o_stride,
                                int64_t do_stride, int64_t dq_stride, int64_t dk_stride, int64_t dv_stride,
                                float softmax_scale, int causal, int accumulate_dq, int dtype, void *stream) {
-  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, cu_seqlens_q, cu_seqlens_k, batch,
+  return attn_bwd_entry(dout, q, k, v, out, lse, dq, dk, dv, delta_out, workspace, workspace_bytes, cu_seqlens_q, cu_seqlens_k, batch,
                         max_seqlen_q, max_seqlen_k, total_q, total_k, hq, hk, d, q_stride, k_stride, v_stride, o_stride,
                         do_stride, dq_stride, dk_stride, dv_stride, softmax_scale, causal, accumulate_dq, dtype, stream);
 }

@@ -595,12 +595,7 @@ template <typename T, int D, int NW>
 static int launch_attn_fwd(const AttnFwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * NW, BN = 64;
   constexpr size_t smem = 2 * BN * ((D + 8) + (D + 32)) * sizeof(T);
-  static bool attr_set = false;
-  if (!attr_set) {
-    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&attn_fwd_kernel<T, D, NW>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set = true;
-  }
+  DH_MAX_DYNAMIC_LDS_PER_DEVICE((&attn_fwd_kernel<T, D, NW>), smem);
   dim3 grid((unsigned)cdiv(p.max_sq, BM), (unsigned)p.hq, (unsigned)batch);
   hipLaunchKernelGGL((attn_fwd_kernel<T, D, NW>), grid, dim3(64 * NW), smem, st, p);
   return DH_OK;

@@ -1,6 +1,7 @@
 // Shared device/host helpers for the gfx950 operator library.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include <stddef.h>
 #include "../../include/dhellam_hip.h"
@@ -29,6 +30,22 @@ void set_error(const char *file, int line, const char *func, const char *fmt, ..
   } while (0)
 
 #define DH_LAUNCH_CHECK() DH_HIP(hipGetLastError())
+
+// Raises a kernel's dynamic LDS limit once per (kernel, device): the attribute belongs to that pair, so the guard
+// is one bit per device, set by whichever thread gets there first (setting it twice is harmless).  Use inside a
+// function or function template that launches exactly this kernel; pass the kernel's address in parentheses.
+#define DH_MAX_DYNAMIC_LDS_PER_DEVICE(kernel_addr, bytes)                                          \
+  do {                                                                                             \
+    static std::atomic<uint64_t> dh_attr_done_{0};                                                 \
+    int dh_dev_ = 0;                                                                               \
+    DH_HIP(hipGetDevice(&dh_dev_));                                                                \
+    const uint64_t dh_bit_ = 1ull << (dh_dev_ & 63);                                               \
+    if (!(dh_attr_done_.load(std::memory_order_acquire) & dh_bit_)) {                              \
+      DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel_addr),                      \
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)));       \
+      dh_attr_done_.fetch_or(dh_bit_, std::memory_order_release);                                  \
+    }                                                                                              \
+  } while (0)
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

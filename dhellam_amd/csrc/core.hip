@@ -25,7 +25,7 @@ void set_error(const char *file, int line, const char *func, const char *fmt, ..
 }
 }  // namespace dh
 
-extern "C" int dh_version(void) { return 100; }
+extern "C" int dh_version(void) { return 200; }
 extern "C" const char *dh_last_error(void) { return dh::g_err; }
 
 // Grid-stride 16-byte copy; the tail (nbytes % 16) is copied bytewise by block 0.

@@ -583,16 +583,7 @@ static int launch_gg(GGParams p, int64_t m_extent, hipStream_t st) {
   using LB = TileLoader<T, BN, TB, NT>;
   constexpr size_t smem = 2 * (LA::ELEMS + LB::ELEMS) * sizeof(T);
   static_assert(smem <= 160 * 1024, "LDS budget");
-  // the attribute belongs to the (kernel, device) pair: one bit per device, set by whichever thread gets there first
-  static std::atomic<uint64_t> attr_set{0};
-  int dev = 0;
-  DH_HIP(hipGetDevice(&dev));
-  const uint64_t bit = 1ull << (dev & 63);
-  if (!(attr_set.load(std::memory_order_acquire) & bit)) {
-    DH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&grouped_gemm_kernel<T, TA, TB, WM, WN, WVN, GROUPED_OUT>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    attr_set.fetch_or(bit, std::memory_order_release);
-  }
+  DH_MAX_DYNAMIC_LDS_PER_DEVICE((&grouped_gemm_kernel<T, TA, TB, WM, WN, WVN, GROUPED_OUT>), smem);
   p.tiles_n = (int)cdiv(p.n_dim, BN);
   p.tiles_m = GROUPED_OUT ? (int)cdiv(m_extent, BM) : (int)(cdiv(m_extent, BM) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;

@@ -369,12 +369,15 @@ static int moe_sort_launch(const int32_t *topk_idx, int32_t *tokens_per_expert, 
 }
 
 extern "C" int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert, int32_t *expert_offsets,
-                           int32_t *sorted_idx, int32_t *dest_row, void *workspace, int64_t n_assign, int experts,
-                           void *stream) {
+                           int32_t *sorted_idx, int32_t *dest_row, void *workspace, size_t workspace_bytes,
+                           int64_t n_assign, int experts, void *stream) {
   using namespace dh;
   DH_CHECK(n_assign >= 0 && n_assign < (1ll << 31), "n_assign out of range");
   DH_CHECK(experts >= 1 && experts <= MOE_MAX_E, "experts=%d must be in [1, %d]", experts, MOE_MAX_E);
   DH_CHECK(tokens_per_expert && expert_offsets && workspace, "null pointer");
+  DH_CHECK(workspace_bytes >= dh_moe_sort_workspace_bytes(n_assign, experts),
+           "workspace of %zu bytes is smaller than dh_moe_sort_workspace_bytes(%lld, %d) = %zu", workspace_bytes,
+           (long long)n_assign, experts, dh_moe_sort_workspace_bytes(n_assign, experts));
   return moe_sort_launch(topk_idx, tokens_per_expert, expert_offsets, sorted_idx, dest_row, (int32_t *)workspace,
                          n_assign, experts, (hipStream_t)stream);
 }

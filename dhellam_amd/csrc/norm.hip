@@ -661,11 +661,14 @@ __global__ void __launch_bounds__(256) zero_bytes_kernel(uint8_t *p, int64_t n) 
 
 extern "C" int dh_norm_bwd(const void *dy, const void *x, const float *mu, const float *rsigma, const void *gamma,
                            const void *add_to_dx, void *dx, void *dgamma, void *dbeta, void *workspace,
-                           int64_t rows, int64_t cols, int zero_centered_gamma, int accumulate_wgrad, int dtype,
-                           void *stream) {
+                           size_t workspace_bytes, int64_t rows, int64_t cols, int zero_centered_gamma,
+                           int accumulate_wgrad, int dtype, void *stream) {
   using namespace dh;
   DH_CHECK(rows >= 0 && cols > 0, "bad shape rows=%lld cols=%lld", (long long)rows, (long long)cols);
   DH_CHECK(dy && x && rsigma && gamma && dx && dgamma && workspace, "null pointer");
+  DH_CHECK(workspace_bytes >= dh_norm_bwd_workspace_bytes(rows, cols),
+           "workspace of %zu bytes is smaller than dh_norm_bwd_workspace_bytes(%lld, %lld) = %zu", workspace_bytes,
+           (long long)rows, (long long)cols, dh_norm_bwd_workspace_bytes(rows, cols));
   DH_CHECK(mu == nullptr || dbeta != nullptr, "LayerNorm backward (mu given) needs a dbeta output");
   DH_CHECK(cols < (1ll << 31), "cols too large");
   DH_CHECK(aligned16(workspace), "workspace must be 16-byte aligned");

@@ -45,6 +45,7 @@ def pylayernorm_fwd(inp, ln_weight, ln_bias, eps, fwd_sm_margin, zero_centered_g
             ln_out = torch.empty_like(inputmat)
         else:
             assert ln_out.is_contiguous() and ln_out.numel() == inputmat.numel() and ln_out.dtype == inputmat.dtype
+            _lib.mark_written(ln_out)
         rsigma = torch.empty(rows, dtype=torch.float32, device=inp.device)
         mu = torch.empty(rows, dtype=torch.float32, device=inp.device) if ln_bias is not None else None
         if residual is None:
@@ -89,6 +90,7 @@ def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_ce
             dinp = torch.empty_like(inputmat)
         else:
             assert dgrad_out.is_contiguous() and dgrad_out.numel() == inputmat.numel() and dgrad_out.dtype == inputmat.dtype
+            _lib.mark_written(dgrad_out)
             dinp = dgrad_out.view(inputmat.shape)
         accumulate = dgamma_out is not None
         assert not accumulate or dgamma_out.dtype == ln_weight.dtype, "dgamma_out must have the weight's dtype"
@@ -103,6 +105,6 @@ def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_ce
         add = add_to_dgrad.view((-1, in_features)) if add_to_dgrad is not None else None
         _lib.check(lib.dh_norm_bwd(d_ln_out.data_ptr(), inputmat.data_ptr(), _lib.ptr(mu), rsigma.data_ptr(),
                                    ln_weight.data_ptr(), _lib.ptr(add), dinp.data_ptr(), dgamma.data_ptr(),
-                                   _lib.ptr(dbeta), ws.data_ptr(), rows, in_features,
+                                   _lib.ptr(dbeta), ws.data_ptr(), ws.numel(), rows, in_features,
                                    int(bool(zero_centered_gamma)), int(accumulate), _lib.dt(inp), st.cuda_stream))
     return dinp.view_as(inp), dgamma, dbeta, el[0]

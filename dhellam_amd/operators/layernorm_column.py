@@ -18,7 +18,7 @@ from typing import Optional
 
 import torch
 
-from .._Clib import dense_gemm, dense_ok, dgrad_gemm, transposed_of
+from .._Clib import _note_read, dense_gemm, dense_ok, dgrad_gemm, transposed_of
 from .._Clib import pygemm as gemm
 from .._Clib import wgrad_gemm
 from ._util import on_stream
@@ -81,6 +81,7 @@ def dgrad_bwd(args, input_grad: torch.Tensor, weight: torch.Tensor, dgrad_output
             wt = transposed_of(weight) if not (transa or transb) else None
             if wt is not None and wt.dtype == input_grad.dtype:      # same product in the forward's layout
                 gemm(wt, input_grad, dgrad_output, None, 0, True, False, False, math_sm_count, False)
+                _note_read(weight)
             else:
                 gemm(weight, input_grad, dgrad_output, None, 0, transa, transb, False, math_sm_count, False)
     return dgrad_output, el[0]

@@ -14,7 +14,7 @@ from dataclasses import dataclass
 import torch
 
 from .. import _lib
-from .._Clib import transposed_of
+from .._Clib import _note_read, transposed_of
 from ._util import on_stream
 
 
@@ -59,7 +59,7 @@ def sort_assignments(topk_idx, num_experts, stream=None, profiling=False):
         dest = torch.empty(n, dtype=torch.int32, device=dev)
         ws = torch.empty(lib.dh_moe_sort_workspace_bytes(n, num_experts), dtype=torch.uint8, device=dev)
         _lib.check(lib.dh_moe_sort(topk_idx.data_ptr(), tpe.data_ptr(), offs.data_ptr(), sorted_idx.data_ptr(),
-                                   dest.data_ptr(), ws.data_ptr(), n, num_experts, st.cuda_stream))
+                                   dest.data_ptr(), ws.data_ptr(), ws.numel(), n, num_experts, st.cuda_stream))
     return MoEPlan(t, k, num_experts, tpe, offs, sorted_idx, dest), el[0]
 
 
@@ -202,4 +202,7 @@ def expert_ffn_bwd(dy, xp, w1, w2, offs, saved, dw1=None, dw2=None, stream=None,
         dh, _ = swiglu_back(da, h, None, st)
         dxp = grouped_gemm_nt(dh, w1t, offs, stream=st) if w1t is not None else grouped_gemm_nn(dh, w1, offs, stream=st)   # [R, H] = dh @ w1[g]
         dw1 = grouped_gemm_tn(dh, xp, offs, out=dw1, accumulate=dw1 is not None, stream=st)  # [G, 2F, H]
+        with torch.cuda.stream(st):
+            _note_read(w2)
+            _note_read(w1)
     return dxp, dw1, dw2, el[0]

@@ -60,5 +60,6 @@ def swiglu_back(g, y, o=None, stream=None, profiling=False, with_transposed=Fals
                                            st.cuda_stream))
             o._dh_rows_transposed = (o._version, ot)    # valid while nothing has written ``o`` since
         else:
+            _lib.mark_written(o)            # a reused ``o`` may carry the transposed twin of an earlier call
             _lib.check(lib.dh_swiglu_bwd(g.data_ptr(), y.data_ptr(), o.data_ptr(), rows, f, _lib.dt(y), st.cuda_stream))
     return o, el[0]

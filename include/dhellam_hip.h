@@ -35,7 +35,9 @@ typedef enum {
   DH_ERR_UNSUPPORTED = -3
 } dh_status;
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Library version (major*100 + minor).  2.0: dh_attn_bwd, dh_attn_bwd_acc,
+ * dh_norm_bwd and dh_moe_sort take the size of the caller's workspace and
+ * check it (1.x trusted the caller). */
 int dh_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *dh_last_error(void);
@@ -69,12 +71,15 @@ size_t dh_norm_bwd_workspace_bytes(int64_t rows, int64_t cols);
  * reference adds in a separate launch, dhellam/core/dstb.py:387-405).
  * dgamma/dbeta [cols] in `dtype`; mu == NULL selects RMSNorm (dbeta may be
  * NULL).  accumulate_wgrad != 0: dgamma/dbeta are added to instead of
- * overwritten.  workspace: dh_norm_bwd_workspace_bytes() bytes. */
+ * overwritten.  workspace: workspace_bytes bytes, at least
+ * dh_norm_bwd_workspace_bytes(rows, cols) or the call is refused with
+ * DH_ERR_INVALID before anything is launched. */
 int dh_norm_bwd(const void *dy, const void *x, const float *mu,
                 const float *rsigma, const void *gamma, const void *add_to_dx,
                 void *dx, void *dgamma, void *dbeta, void *workspace,
-                int64_t rows, int64_t cols, int zero_centered_gamma,
-                int accumulate_wgrad, int dtype, void *stream);
+                size_t workspace_bytes, int64_t rows, int64_t cols,
+                int zero_centered_gamma, int accumulate_wgrad, int dtype,
+                void *stream);
 
 /* ------------------------------------------------------------------------
  * SwiGLU.  dhellam/operators/swiglu.py:13-16 (fwd) and :21-26 (bwd).
@@ -154,33 +159,42 @@ int dh_attn_fwd(const void *q, const void *k, const void *v, void *out,
                 int64_t k_stride, int64_t v_stride, int64_t o_stride,
                 float softmax_scale, int causal, int dtype, void *stream);
 
-/* Bytes of scratch dh_attn_bwd needs (delta = rowsum(dO*O), fp32 dK/dV
- * partials when a GQA group is split over workgroups, and the dS blocks of
- * calls that keep them: see dh_attn_bwd_set_ds_limit). */
+/* Bytes of scratch dh_attn_bwd works in.  dh_attn_bwd_min_workspace_bytes: what
+ * every call of these sizes needs (delta = rowsum(dO*O), the lse / delta planes
+ * of the head-dim-128 kernels, fp32 dK/dV partials when a GQA group is split
+ * over workgroups); a smaller workspace is refused.  dh_attn_bwd_workspace_bytes:
+ * that plus room for the dS blocks of calls that would keep them (below); with
+ * it the backward picks its faster form. */
+size_t dh_attn_bwd_min_workspace_bytes(int64_t total_q, int64_t total_k,
+                                       int batch, int max_seqlen_q, int hq,
+                                       int hk, int d, int dtype);
 size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
                                    int max_seqlen_q, int hq, int hk, int d,
                                    int dtype);
 
 /* Head dim 128 in 16 bits, calls too small to fill the chip with 128-row
- * query tiles (fewer than 256 of them, halved for causal): when 2 bytes per
- * (head, query, key) fit into this many bytes of workspace (default 1280 MiB)
- * the backward keeps dS = P * (dP - delta) from its dK/dV pass and forms dQ
- * from it in one product; otherwise (0: never) its dQ pass recomputes S and dP
- * and needs no such space.  No counterpart in the reference (flash-attention
- * always recomputes); a process-wide setting, read by
- * dh_attn_bwd_workspace_bytes and dh_attn_bwd alike: dh_attn_bwd takes no
- * workspace size, so a workspace must be sized AFTER the last change of this
- * limit (raising it between a sizing call and the dh_attn_bwd call that uses
- * the result would let the kernels write past the workspace). */
+ * query tiles (fewer than 256 of them, halved for causal): the backward keeps
+ * dS = P * (dP - delta) from its dK/dV pass and forms dQ from it in one
+ * product when 2 bytes per (head, query, key) (a) stay under this process-wide
+ * limit (default 1280 MiB; 0: never keep) and (b) fit into the workspace the
+ * call was given behind its minimum; otherwise its dQ pass recomputes S and dP
+ * and needs no such space.  The limit only steers the choice: a call never
+ * writes past workspace + workspace_bytes, whatever the limit is or was when
+ * the workspace was sized.  No counterpart in the reference (flash-attention
+ * always recomputes). */
 void dh_attn_bwd_set_ds_limit(size_t bytes);
 
 /* dq like q, dk/dv like k/v (GQA groups are reduced inside the kernel; the
  * reference sums an expanded buffer afterwards, flash_atten.cu:646-652).
  * delta_out (fp32 [b, hq, max_seqlen_q], may be NULL) receives rowsum(dO*O),
- * the reference's softmax_d. */
+ * the reference's softmax_d, for the rows of each sequence (entries past a
+ * sequence's length are left as they were).  workspace: workspace_bytes bytes,
+ * 16-byte aligned; fewer than dh_attn_bwd_min_workspace_bytes() is refused
+ * with DH_ERR_INVALID before anything is launched. */
 int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v,
                 const void *out, const float *lse, void *dq, void *dk,
                 void *dv, float *delta_out, void *workspace,
+                size_t workspace_bytes,
                 const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
                 int batch, int max_seqlen_q, int max_seqlen_k,
                 int64_t total_q, int64_t total_k, int hq, int hk, int d,
@@ -197,6 +211,7 @@ int dh_attn_bwd(const void *dout, const void *q, const void *k, const void *v,
 int dh_attn_bwd_acc(const void *dout, const void *q, const void *k,
                     const void *v, const void *out, const float *lse, void *dq,
                     void *dk, void *dv, float *delta_out, void *workspace,
+                    size_t workspace_bytes,
                     const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
                     int batch, int max_seqlen_q, int max_seqlen_k,
                     int64_t total_q, int64_t total_k, int hq, int hk, int d,
@@ -234,10 +249,13 @@ size_t dh_moe_sort_workspace_bytes(int64_t n_assign, int experts);
  * (assignment a = token*k + j) by expert id.  tokens_per_expert int32
  * [experts]; expert_offsets int32 [experts+1] (exclusive scan of the counts);
  * sorted_idx int32 [n_assign] (assignment ids in sorted order); dest_row int32
- * [n_assign] (position of each assignment in the sorted order). */
+ * [n_assign] (position of each assignment in the sorted order).  workspace:
+ * workspace_bytes bytes, at least dh_moe_sort_workspace_bytes(n_assign,
+ * experts) or the call is refused with DH_ERR_INVALID. */
 int dh_moe_sort(const int32_t *topk_idx, int32_t *tokens_per_expert,
                 int32_t *expert_offsets, int32_t *sorted_idx, int32_t *dest_row,
-                void *workspace, int64_t n_assign, int experts, void *stream);
+                void *workspace, size_t workspace_bytes, int64_t n_assign,
+                int experts, void *stream);
 
 /* dh_moe_sort for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same results as

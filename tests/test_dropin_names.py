@@ -48,23 +48,60 @@ def test_reference_import_line_resolves(line):
     assert len(ns) > 1
 
 
-def test_binding_signatures_are_the_references():
-    """Positional parameter names of the six pybind functions, csrc/operators/ops.h:18-81 / dhellam/_Clib/__init__.pyi."""
+WANT_PARAMS = {
+    "pygemm": ["inputA", "inputB", "outputD", "input_workspace", "workspaceSize", "transa", "transb",
+               "grad_accumulate", "math_sm_count", "profiling"],
+    "pygelu": ["input", "output", "profiling"],
+    "pybda": ["input", "bias", "residual", "output", "prob", "profiling"],
+    "add_tensors": ["a", "b"],
+    "pymha_varlen_fwd": ["q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout",
+                         "softmax_scale", "is_causal", "return_softmax", "math_sm_count", "profiling"],
+    "pymha_varlen_bwd": ["dout", "q", "k", "v", "out", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q",
+                         "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "rng_state", "deterministic",
+                         "math_sm_count", "profiling", "stream_ptr"],
+}
+WANT_RETURNS = {"pygemm": "float", "pygelu": "float", "pybda": "float", "add_tensors": "torch.Tensor",
+                "pymha_varlen_fwd": "list[torch.Tensor]", "pymha_varlen_bwd": "list[torch.Tensor]"}
+
+
+def test_compiled_binding_signatures_are_the_references():
+    """``dhellam._Clib`` is the compiled pybind11 extension (csrc/torchapi.cpp:2-9 in the reference): its six
+    functions take the positional parameters of csrc/operators/ops.h:18-81, in that order, and return what the
+    reference's do.  pybind11 puts the signature into the first line of the docstring."""
+    import re
     import dhellam._Clib as C
-    want = {
-        "pygemm": ["inputA", "inputB", "outputD", "input_workspace", "workspaceSize", "transa", "transb",
-                   "grad_accumulate", "math_sm_count", "profiling"],
-        "pygelu": ["input", "output", "profiling"],
-        "pymha_varlen_fwd": ["q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout",
-                             "softmax_scale", "is_causal", "return_softmax", "math_sm_count", "profiling"],
-        "pymha_varlen_bwd": ["dout", "q", "k", "v", "out", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q",
-                             "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "rng_state", "deterministic",
-                             "math_sm_count", "profiling", "stream_ptr"],
-    }
-    for name, params in want.items():
+    assert C.__file__.endswith(".so"), C.__file__
+    assert sorted(n for n in dir(C) if not n.startswith("_")) == sorted(WANT_PARAMS)
+    for name, params in WANT_PARAMS.items():
+        first = getattr(C, name).__doc__.splitlines()[0]
+        m = re.fullmatch(rf"{name}\((.*)\) -> (.*)", first)
+        assert m, first
+        got = [p.split(":")[0].strip() for p in m.group(1).split(", ")]
+        assert got == params, (name, got)
+        assert m.group(2) == WANT_RETURNS[name], (name, m.group(2))
+
+
+def test_ctypes_mirror_signatures_are_the_references():
+    """The Python mirror of the same module (``dhellam_amd._Clib``, ctypes over the C ABI) keeps the same names."""
+    import dhellam_amd._Clib as C
+    for name, params in WANT_PARAMS.items():
         got = list(inspect.signature(getattr(C, name)).parameters)
         assert got == params, (name, got)
-    assert len(inspect.signature(C.pybda).parameters) == 6
+
+
+def test_compiled_binding_refuses_what_the_library_does_not_do():
+    """Error paths that need no GPU: they surface as RuntimeError like the reference's TORCH_CHECKs."""
+    import torch
+    import dhellam._Clib as C
+    x = torch.zeros(4, 2, 8)
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="dropout"):
+        C.pymha_varlen_fwd(x, x, x, cu, cu, 4, 4, 0.1, 1.0, True, False, 0, False)
+    with pytest.raises(RuntimeError, match="GPU"):
+        C.pymha_varlen_fwd(x, x, x, cu, cu, 4, 4, 0.0, 1.0, True, False, 0, False)
+    with pytest.raises(RuntimeError, match="TT layout"):
+        C.pygemm(x[0], x[0], x[0], x[0], 0, True, True, False, 0, False)
+    assert torch.equal(C.add_tensors(torch.ones(3), torch.ones(3)), torch.full((3,), 2.0))
 
 
 def test_one_rank_collectives_and_refusals():

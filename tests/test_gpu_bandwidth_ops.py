@@ -520,3 +520,23 @@ def test_residual_add_fused_into_norm_is_the_two_ops_bit_for_bit(dtype, rows, co
     x2 = x.clone()
     y2, _, _, _, s2 = pylayernorm_fwd(x2, g, b, 1e-5, 0, False, None, residual=r, sum_out=x2)
     assert s2 is x2 and torch.equal(x2, s_ref) and torch.equal(y2, y_ref)
+
+
+def test_reused_swiglu_gradient_buffer_drops_the_transposed_twin():
+    """``swiglu_back(..., with_transposed=True)`` hangs dY^T on its result for the weight-gradient GEMM.  The
+    library's kernels write through raw pointers, so the tensor's version counter does not move when the same buffer
+    is written again by the plain kernel: the stale twin must be dropped, or ``wgrad_gemm`` multiplies the old one."""
+    from dhellam_amd import _Clib
+    from dhellam_amd.operators.swiglu import swiglu_back
+    dtype, rows, f, k = torch.bfloat16, 4096, 512, 4096
+    y1, g1, y2, g2 = (randn(s, dtype, i).cuda() for i, s in enumerate(((rows, 2 * f), (rows, f), (rows, 2 * f), (rows, f))))
+    x = randn((rows, k), dtype, 9).cuda()
+    buf = torch.empty_like(y1)
+    d1, _ = swiglu_back(g1, y1, buf, None, False, with_transposed=True)
+    assert d1 is buf and torch.equal(buf._dh_rows_transposed[1], buf.t().contiguous())
+    assert _Clib.wgrad_layout(buf, x) == "NN"                  # the layout that picks the twin up
+    d2, _ = swiglu_back(g2, y2, buf, None, False, with_transposed=False)
+    assert d2 is buf and not hasattr(buf, "_dh_rows_transposed")
+    out = torch.empty((2 * f, k), dtype=dtype, device="cuda")
+    _Clib.wgrad_gemm(buf, x, out, False)
+    assert_close(out, (buf.double().t() @ x.double()).cpu(), dtype, "wgrad of the rewritten buffer")

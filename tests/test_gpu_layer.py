@@ -315,3 +315,44 @@ def test_fused_adjacent_ops_give_the_bits_of_the_separate_ops():
         res.append(outs + dxs + [w[k].main_grad.clone() for k in GRAD_KEYS])
     for a, b in zip(*res):
         assert torch.equal(a, b)
+
+
+def test_weights_updated_around_the_version_counter_are_seen_by_the_next_step():
+    """The projection weights are kept resident as W and W^T, and the data-gradient GEMMs read W^T.  An optimizer
+    that writes through ``p.data`` (Megatron's do) does not move the tensor's version counter, so only an
+    unconditional rebuild at the step boundary keeps W^T current: the step after such an update must give the
+    gradients of the NEW weights, bit for bit those of a layer that holds no resident transposes."""
+    import dataclasses
+    from dhellam_amd.core.dstb import LayerConfig
+    from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
+    cfg = LayerConfig(hidden_size=1024, num_attention_heads=16, num_query_groups=2, ffn_hidden_size=2048,
+                      seq_length=256, micro_batch_size=1, tensor_model_parallel_size=2, tp_rank=0,
+                      rope_theta=500000.0, params_dtype=torch.bfloat16)
+    assert cfg.resident_weight_transposes
+    w = make_weights(cfg, 0)
+    mbs = [make_microbatch(cfg, i) for i in range(2)]
+    runner = LayerRunner(cfg, w)
+    runner.run_double_strand(mbs)                                    # a first step with the initial weights
+    new = make_weights(dataclasses.replace(cfg, resident_weight_transposes=False), 7)
+    proj = ("column_attn_weight", "linear_attn_weight", "column_mlp_weight", "linear_mlp_weight")
+    for k in proj:
+        v0 = w[k]._version
+        w[k].data.copy_(new[k])                                      # the optimizer's way: no version bump
+        assert w[k]._version == v0
+    runner.zero_grads()
+    outs, dxs = runner.run_double_strand(mbs)
+    ref = LayerRunner(dataclasses.replace(cfg, resident_weight_transposes=False), new)
+    outs_r, dxs_r = ref.run_double_strand([make_microbatch(cfg, i) for i in range(2)])
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(outs[i], outs_r[i]), f"out[{i}]"
+        assert torch.equal(dxs[i], dxs_r[i]), f"dx[{i}] was computed against a stale W^T"
+    for k in GRAD_KEYS:
+        assert torch.equal(w[k].main_grad, new[k].main_grad), k
+    # and a caller that opts out of the rebuild sees what the advice warns about: a stale W^T, silently
+    for k in proj:
+        w[k].data.copy_(make_weights(dataclasses.replace(cfg, resident_weight_transposes=False), 9)[k])
+    _, dxs_stale = runner.run_double_strand(mbs, refresh_transposes=False)
+    _, dxs_fresh = runner.run_double_strand(mbs)
+    torch.cuda.synchronize()
+    assert not torch.equal(dxs_stale[0], dxs_fresh[0])

@@ -24,7 +24,7 @@ def _sort(lib, idx, E, static):
     else:
         ws = torch.empty(lib.dh_moe_sort_workspace_bytes(n, E), dtype=torch.uint8, device=dev)
         _lib.check(lib.dh_moe_sort(idx.data_ptr(), tpe.data_ptr(), offs.data_ptr(), sidx.data_ptr(), dest.data_ptr(),
-                                   ws.data_ptr(), n, E, st))
+                                   ws.data_ptr(), ws.numel(), n, E, st))
     torch.cuda.synchronize()
     return [t.cpu().numpy() for t in (tpe, offs, sidx, dest)]
 

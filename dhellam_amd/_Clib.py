@@ -259,7 +259,13 @@ def wgrad_gemm(grad: torch.Tensor, data: torch.Tensor, out: torch.Tensor, accumu
 # version counter (any in-place torch op on the tensor itself) also triggers a rebuild at the next use.  A caller
 # that drives ``dgrad_gemm`` by hand and updates weights around the counter calls ``refresh_transposed`` itself;
 # weights that were never registered take the NN product as before.
-_kept_weights: "weakref.WeakSet" = weakref.WeakSet()
+_kept_weights: dict = {}        # id(weight) -> weak reference (tensors compare elementwise: no set of them)
+
+
+def _register_kept(weight: torch.Tensor) -> None:
+    key = id(weight)
+    if key not in _kept_weights:
+        _kept_weights[key] = weakref.ref(weight, lambda _r, key=key: _kept_weights.pop(key, None))
 
 
 class _Held:
@@ -300,7 +306,7 @@ def keep_transposed(weight: torch.Tensor, refresh: bool = False) -> Optional[tor
     ev = torch.cuda.Event()
     ev.record(stream)
     weight._dh_transposed = _Held(weight._version, wt, ev, stream.cuda_stream)
-    _kept_weights.add(weight)
+    _register_kept(weight)
     return wt
 
 
@@ -309,7 +315,7 @@ def refresh_transposed(weights=None) -> int:
     stream, whatever their version counters say: the call that follows an optimizer step.  Unregistered tensors in
     ``weights`` are skipped.  Returns how many copies were rebuilt."""
     n = 0
-    for w in (list(_kept_weights) if weights is None else weights):
+    for w in ([r() for r in list(_kept_weights.values())] if weights is None else weights):
         if isinstance(w, torch.Tensor) and getattr(w, "_dh_transposed", None) is not None:
             keep_transposed(w, refresh=True)
             n += 1

@@ -105,6 +105,6 @@ def pylayernorm_bwd(d_ln_out, inp, mu, rsigma, ln_weight, bwd_sm_margin, zero_ce
         add = add_to_dgrad.view((-1, in_features)) if add_to_dgrad is not None else None
         _lib.check(lib.dh_norm_bwd(d_ln_out.data_ptr(), inputmat.data_ptr(), _lib.ptr(mu), rsigma.data_ptr(),
                                    ln_weight.data_ptr(), _lib.ptr(add), dinp.data_ptr(), dgamma.data_ptr(),
-                                   _lib.ptr(dbeta), ws.data_ptr(), ws.numel(), rows, in_features,
+                                   _lib.ptr(dbeta), ws.data_ptr(), ws.numel() * ws.element_size(), rows, in_features,
                                    int(bool(zero_centered_gamma)), int(accumulate), _lib.dt(inp), st.cuda_stream))
     return dinp.view_as(inp), dgamma, dbeta, el[0]

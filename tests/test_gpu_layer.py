@@ -321,7 +321,8 @@ def test_weights_updated_around_the_version_counter_are_seen_by_the_next_step():
     """The projection weights are kept resident as W and W^T, and the data-gradient GEMMs read W^T.  An optimizer
     that writes through ``p.data`` (Megatron's do) does not move the tensor's version counter, so only an
     unconditional rebuild at the step boundary keeps W^T current: the step after such an update must give the
-    gradients of the NEW weights, bit for bit those of a layer that holds no resident transposes."""
+    gradients of the NEW weights: those of a layer that holds no resident transposes (the two take different GEMM
+    kernels for the data gradients, so they agree to rounding; against stale weights they would not agree at all)."""
     import dataclasses
     from dhellam_amd.core.dstb import LayerConfig
     from dhellam_amd.core.layer import LayerRunner, make_microbatch, make_weights
@@ -344,15 +345,16 @@ def test_weights_updated_around_the_version_counter_are_seen_by_the_next_step():
     ref = LayerRunner(dataclasses.replace(cfg, resident_weight_transposes=False), new)
     outs_r, dxs_r = ref.run_double_strand([make_microbatch(cfg, i) for i in range(2)])
     torch.cuda.synchronize()
+    from tests.util import rel_err
     for i in range(2):
         assert torch.equal(outs[i], outs_r[i]), f"out[{i}]"
-        assert torch.equal(dxs[i], dxs_r[i]), f"dx[{i}] was computed against a stale W^T"
+        assert_close(dxs[i], dxs_r[i].cpu(), cfg.params_dtype, f"dx[{i}] (a stale W^T would be off by ~1)")
     for k in GRAD_KEYS:
-        assert torch.equal(w[k].main_grad, new[k].main_grad), k
+        assert_close(w[k].main_grad, new[k].main_grad.cpu(), cfg.params_dtype, k)
     # and a caller that opts out of the rebuild sees what the advice warns about: a stale W^T, silently
     for k in proj:
         w[k].data.copy_(make_weights(dataclasses.replace(cfg, resident_weight_transposes=False), 9)[k])
     _, dxs_stale = runner.run_double_strand(mbs, refresh_transposes=False)
     _, dxs_fresh = runner.run_double_strand(mbs)
     torch.cuda.synchronize()
-    assert not torch.equal(dxs_stale[0], dxs_fresh[0])
+    assert rel_err(dxs_stale[0], dxs_fresh[0]) > 0.1

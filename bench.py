@@ -474,6 +474,27 @@ def _device_info():
     return info
 
 
+def _pick_plan(arg):
+    """(plan path or None, where it came from, whether the strands enter each block together): the plan that
+    ``python -m dhellam_amd.search.run`` emitted (its execute stage replays the DP's candidates and the built-in
+    plan and keeps the measured winner) unless ``--plan`` says otherwise."""
+    root = os.path.dirname(os.path.abspath(__file__))
+    emitted = os.path.join(root, "dhellam_amd", "search", "config", "best.json")
+    report = os.path.join(root, "dhellam_amd", "search", "config", "execute_report.json")
+    if arg == "builtin":
+        return None, "built-in plan (forced)", False
+    if arg:
+        return arg, f"--plan {arg}", False
+    if os.path.exists(emitted):
+        best = {}
+        if os.path.exists(report):
+            with open(report) as f:
+                best = json.load(f).get("best", {})
+        return emitted, (f"dhellam_amd/search/config/best.json (emitted by search + execute; winner "
+                         f"{best.get('name', '?')})"), bool(best.get("lockstep_blocks", False))
+    return None, "built-in plan (no emitted plan in the tree)", False
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -484,7 +505,10 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline section")
     ap.add_argument("--emulate-comm-us", type=float, default=55.0,
                     help="also time both schedules with each sequence-parallel stand-in taking this long (0: skip)")
-    ap.add_argument("--plan", default=None, help="plan JSON for the double-strand schedule (default: built-in)")
+    ap.add_argument("--plan", default=None,
+                    help="plan JSON for the double-strand schedule; default: the plan the search's execute stage "
+                         "emitted (dhellam_amd/search/config/best.json) when there is one, else the built-in plan; "
+                         "'builtin' forces the built-in plan")
     ap.add_argument("--profile-op", default=None,
                     help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, swiglu_t, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
     ap.add_argument("--analyze-trace", default=None,
@@ -511,7 +535,10 @@ def main():
     cfg = llama70b_tp8_shard()
     w = make_weights(cfg, 0, gen_device="cuda")
     mbs = [make_microbatch(cfg, i, gen_device="cuda") for i in range(args.micro_batches)]
-    plan = args.plan
+    plan, plan_source, plan_lockstep = _pick_plan(args.plan)
+    if plan_lockstep:
+        import dataclasses
+        cfg = dataclasses.replace(cfg, lockstep_blocks=True)
     runner = LayerRunner(cfg, w, plan=plan)
     tokens_per_step = cfg.tokens * len(mbs)
 
@@ -586,7 +613,13 @@ def main():
         "config": {"workload": "Llama-3.1-70B TP=8/SP rank share of one decoder layer fwd+bwd: hidden 8192, 8q+1kv "
                                "heads x128, SwiGLU shard 3584, seq 4096, SP rows 512, RoPE theta 5e5; "
                                f"{len(mbs)} micro-batches per step", "schedule": schedule,
-                   "tokens_per_step": tokens_per_step},
+                   "tokens_per_step": tokens_per_step, "plan_source": plan_source,
+                   # serial / double-strand / ceiling, and the same with stand-in collectives (also under
+                   # "schedules" and "schedules_with_emulated_collectives" below)
+                   "schedule_detail": {"serial_ms": round(ms_serial, 4), "double_strand_ms": round(ms_double, 4),
+                                       "double_strand_speedup": round(ms_serial / ms_double, 4),
+                                       "double_strand_ceiling": measured.get("double_strand_ceiling"),
+                                       "with_emulated_collectives": emulated}},
         "schedules": {"serial_ms": round(ms_serial, 4), "double_strand_ms": round(ms_double, 4),
                       "double_strand_speedup": round(ms_serial / ms_double, 4),
                       # what ANY co-schedule of these kernels could reach: idle compute-unit time of the serial trace

@@ -5,9 +5,14 @@ Counterpart of search/profiler.py:20-65,142-180.  The reference builds each op's
 from random tensors in per-op factories (search/op_table.py:127-361); here one real
 forward and backward of the layer is RECORDED (each op's input and the activation entries
 it consumes), and an op is re-issued from that record -- shapes, strides and dtypes are the
-ones the layer really uses.  Timing protocol as in the reference: one warm-up launch each
-for (s1,s2), (s1,s1), (s2,s2), then 5 serial and 5 two-stream repetitions of
-``benchmark_ms_ops``.
+ones the layer really uses.  Two timing protocols.  "reference": as in the reference, one warm-up launch
+each for (s1,s2), (s1,s1), (s2,s2), then 5 serial and 5 two-stream repetitions of ``benchmark_ms_ops`` (host
+clock, a device synchronisation around every repetition: right for a runtime that synchronises after every
+block, dhellam/core/dstb.py:1266).  "device" (the default here): the time the pair takes ON THE GPU when the
+launch queue is full, which is how this runtime executes a plan (nothing in ``exec`` waits for the device, so
+launch latency is hidden behind earlier work): the repetitions are queued behind a delay kernel that lets the
+host get ahead, separated by the same stream-to-stream event edges that ``lockstep_blocks`` puts between two
+blocks, and timed with events on the stream.
 """
 from __future__ import annotations
 
@@ -15,6 +20,7 @@ from typing import Dict, List, Optional
 
 import torch
 
+from .. import _lib
 from ..common.benchmark import benchmark_ms_ops
 from ..core import dstb
 from ..core.layer import LayerRunner, fresh_activation_dict
@@ -64,10 +70,54 @@ def op_factory(records, cfg, op_id: int):
     return factory
 
 
-def time_pair(records, cfg, fwd_ids: List[int], bwd_ids: List[int], s1, s2, repeat: int = 5):
-    """(speedup, seq_time, para_time) of one pair, protocol of search/profiler.py:46-56."""
+HOST_US_PER_OP = 150.0      # generous bound of what the host needs to queue one op (sizes the lead-in delay)
+
+
+def _device_ms(fn1, fn2, sa, sb, repeat: int) -> float:
+    """ms per repetition, on the device, of the ops of fn1 on ``sa`` and of fn2 on ``sb`` (``sa is sb``: one after
+    the other on one stream).  Every repetition starts with both streams joined, like a block of a lockstep plan."""
+    lib = _lib.load()
+    l1 = [op(sa) for op in fn1]
+    l2 = [op(sb) for op in fn2]
+    two = sb.cuda_stream != sa.cuda_stream
+
+    def join():
+        if two:
+            e1, e2 = torch.cuda.Event(), torch.cuda.Event()
+            e1.record(sa)
+            e2.record(sb)
+            sa.wait_event(e2)
+            sb.wait_event(e1)
+
+    join()
+    lead_ns = int((200.0 + HOST_US_PER_OP * repeat * (len(l1) + len(l2) + 2)) * 1e3)
+    _lib.check(lib.dh_delay(lead_ns, sa.cuda_stream))          # the host queues everything below meanwhile
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(sa)
+    for _ in range(repeat):
+        join()
+        for _, fn in l1:
+            fn()
+        for _, fn in l2:
+            fn()
+    join()
+    end.record(sa)
+    end.synchronize()
+    return start.elapsed_time(end) / repeat
+
+
+def time_pair(records, cfg, fwd_ids: List[int], bwd_ids: List[int], s1, s2, repeat: int = 5, mode: str = "device"):
+    """(speedup, seq_time, para_time) of one pair; ``mode`` "reference" is the protocol of
+    search/profiler.py:46-56, "device" times the pair on the GPU with the launch queue full (module docstring)."""
     fn1 = [op_factory(records, cfg, i) for i in fwd_ids]
     fn2 = [op_factory(records, cfg, i) for i in bwd_ids]
+    if mode == "device":
+        _device_ms(fn1, fn2, s1, s2, 1)                         # warm-up (first-use allocations, library plans)
+        seq = _device_ms(fn1, fn2, s1, s1, repeat)
+        par = _device_ms(fn1, fn2, s1, s2, repeat)
+        return (seq / par if par > 0 else 1.0), seq, par
+    if mode != "reference":
+        raise ValueError(f"unknown timing mode {mode!r}")
     benchmark_ms_ops(1, s1, s2, fn1, fn2, None)
     benchmark_ms_ops(1, s1, s1, fn1, fn2, None)
     benchmark_ms_ops(1, s2, s2, fn1, fn2, None)
@@ -76,7 +126,8 @@ def time_pair(records, cfg, fwd_ids: List[int], bwd_ids: List[int], s1, s2, repe
     return (seq / par if par > 0 else 1.0), seq, par
 
 
-def profile_pairs(runner: LayerRunner, mb: dict, out_path: Optional[str] = None, repeat: int = 5, progress=None):
+def profile_pairs(runner: LayerRunner, mb: dict, out_path: Optional[str] = None, repeat: int = 5, progress=None,
+                  mode: str = "device"):
     """Time every candidate pair; returns {(fwd ids, bwd ids): para_time ms} and, when
     ``out_path`` is given, appends the records to it in the op_profile_num.txt format."""
     records = record_layer(runner, mb)
@@ -89,7 +140,7 @@ def profile_pairs(runner: LayerRunner, mb: dict, out_path: Optional[str] = None,
             for b in bwd_c:
                 if not f and not b:
                     continue
-                sp, seq, par = time_pair(records, runner.cfg, f, b, s1, s2, repeat)
+                sp, seq, par = time_pair(records, runner.cfg, f, b, s1, s2, repeat, mode)
                 prof[(tuple(f), tuple(b))] = par
                 if fp:
                     fp.write(format_record(f, b, sp, seq, par))

@@ -55,54 +55,61 @@ def _starts(groups: List[List[int]]):
     return flat, start
 
 
-def search_plan(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_groups: List[List[int]],
-                illegal=None, alias=None) -> Tuple[float, List[Tuple[List[int], List[int]]]]:
-    """Best sequence of blocks [(fwd group, bwd group)], either possibly empty, that covers
-    both op lists in order and minimises the sum of the blocks' measured times.  ``illegal(f, b)``
-    forbids pairing two groups (the reference forbids pairs where both sides communicate,
-    search.py:13-21).  ``alias``: {op id: op id whose records time it} (a parked weight gradient
-    runs the kernel of the op it was parked from).  Raises KeyError if the profile lacks a needed record."""
+def search_plans(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_groups: List[List[int]],
+                 illegal=None, alias=None, k: int = 1) -> List[Tuple[float, List[Tuple[List[int], List[int]]]]]:
+    """The ``k`` cheapest sequences of blocks [(fwd group, bwd group)], either possibly empty, that cover both op
+    lists in order, by the sum of the blocks' measured times, cheapest first (the reference keeps every plan it
+    enumerates as a candidate file for its execute stage, search/execute.py:33-36; here the DP itself carries the k
+    best partial plans per cell).  ``illegal(f, b)`` forbids pairing two groups (the reference forbids pairs where
+    both sides communicate, search.py:13-21).  ``alias``: {op id: op id whose records time it} (a parked weight
+    gradient runs the kernel of the op it was parked from).  Raises KeyError if the profile lacks a needed
+    record."""
     F, fs = _starts(fwd_groups)
     B, bs = _starts(bwd_groups)
     nf, nb = len(F), len(B)
-    INF = float("inf")
-    cost = [[INF] * (nb + 1) for _ in range(nf + 1)]
-    back = [[None] * (nb + 1) for _ in range(nf + 1)]
-    cost[0][0] = 0.0
+    k = max(1, int(k))
+    # cell -> up to k entries (cost, (fg, bg), rank of the predecessor entry), cheapest first
+    cells = [[[] for _ in range(nb + 1)] for _ in range(nf + 1)]
+    cells[0][0] = [(0.0, None, -1)]
     al = alias or {}
     t = lambda f, b: profile[(tuple(al.get(x, x) for x in f), tuple(al.get(x, x) for x in b))]
     for i in range(nf + 1):
         for j in range(nb + 1):
             if i == 0 and j == 0:
                 continue
-            best, arg = INF, None
+            cand = []
             fgs = [F[a:i] for a in range(fs[i - 1], i)] if i > 0 else []
             bgs = [B[a:j] for a in range(bs[j - 1], j)] if j > 0 else []
-            for fg in fgs:
-                c = cost[i - len(fg)][j] + t(fg, [])
-                if c < best:
-                    best, arg = c, (fg, [])
-            for bg in bgs:
-                c = cost[i][j - len(bg)] + t([], bg)
-                if c < best:
-                    best, arg = c, ([], bg)
-            for fg in fgs:
-                for bg in bgs:
-                    if illegal is not None and illegal(fg, bg):
-                        continue
-                    c = cost[i - len(fg)][j - len(bg)] + t(fg, bg)
-                    if c < best:
-                        best, arg = c, (fg, bg)
-            cost[i][j], back[i][j] = best, arg
-    blocks = []
-    i, j = nf, nb
-    while i > 0 or j > 0:
-        fg, bg = back[i][j]
-        blocks.append((list(fg), list(bg)))
-        i -= len(fg)
-        j -= len(bg)
-    blocks.reverse()
-    return cost[nf][nb], blocks
+            moves = [(fg, []) for fg in fgs] + [([], bg) for bg in bgs]
+            moves += [(fg, bg) for fg in fgs for bg in bgs if illegal is None or not illegal(fg, bg)]
+            for fg, bg in moves:
+                prev = cells[i - len(fg)][j - len(bg)]
+                if not prev:
+                    continue
+                step = t(fg, bg)
+                cand.extend((c + step, (fg, bg), r) for r, (c, _, _) in enumerate(prev))
+            cand.sort(key=lambda e: e[0])
+            cells[i][j] = cand[:k]
+    out = []
+    for rank in range(len(cells[nf][nb])):
+        blocks, i, j, r = [], nf, nb, rank
+        total = cells[nf][nb][rank][0]
+        while i > 0 or j > 0:
+            _, (fg, bg), pr = cells[i][j][r]
+            blocks.append((list(fg), list(bg)))
+            i, j, r = i - len(fg), j - len(bg), pr
+        blocks.reverse()
+        out.append((total, blocks))
+    return out
+
+
+def search_plan(profile: Dict[Key, float], fwd_groups: List[List[int]], bwd_groups: List[List[int]],
+                illegal=None, alias=None) -> Tuple[float, List[Tuple[List[int], List[int]]]]:
+    """The cheapest plan of ``search_plans``: (cost, blocks)."""
+    found = search_plans(profile, fwd_groups, bwd_groups, illegal, alias, 1)
+    if not found:
+        raise KeyError("no plan covers the op lists")
+    return found[0]
 
 
 def park_choices(bwd_groups: List[List[int]], movable: Sequence[int]):
@@ -146,22 +153,29 @@ def park_choices(bwd_groups: List[List[int]], movable: Sequence[int]):
         yield groups, alias
 
 
-def search_plan_with_parking(profile: Dict[Key, float], fwd_groups, bwd_groups, movable=None, illegal=None):
-    """``search_plan`` over every choice of deferred weight gradients.  Returns (cost, blocks, alias): in the
-    blocks a deferred op appears as its placeholder id at the place where it runs; ``alias`` maps the
-    placeholders used to the ops they defer (``plan_to_json`` puts the op's own name back where it was parked)."""
+def search_candidates_with_parking(profile: Dict[Key, float], fwd_groups, bwd_groups, movable=None, illegal=None,
+                                   k: int = 1):
+    """``search_plans`` over every choice of deferred weight gradients: the ``k`` cheapest (cost, blocks, alias)
+    overall, cheapest first.  In the blocks a deferred op appears as its placeholder id at the place where it
+    runs; ``alias`` maps the placeholders used to the ops they defer (``plan_to_json`` puts the op's own name back
+    where it was parked)."""
     movable = list(PLACEHOLDER_OF) if movable is None else list(movable)
-    best = (float("inf"), None, None)
+    found = []
     for groups, alias in park_choices(bwd_groups, movable):
         try:
-            cost, blocks = search_plan(profile, fwd_groups, groups, illegal, alias)
+            for cost, blocks in search_plans(profile, fwd_groups, groups, illegal, alias, k):
+                found.append((cost, blocks, alias))
         except KeyError:
             continue                      # the profile has no record for a group this choice needs
-        if cost < best[0]:
-            best = (cost, blocks, alias)
-    if best[1] is None:
+    if not found:
         raise KeyError("the profile lacks the records of every candidate plan")
-    return best
+    found.sort(key=lambda e: e[0])
+    return found[:max(1, int(k))]
+
+
+def search_plan_with_parking(profile: Dict[Key, float], fwd_groups, bwd_groups, movable=None, illegal=None):
+    """The cheapest of ``search_candidates_with_parking``: (cost, blocks, alias)."""
+    return search_candidates_with_parking(profile, fwd_groups, bwd_groups, movable, illegal, 1)[0]
 
 
 def plan_to_json(blocks, with_comm_standins: bool = True, alias=None, bwd_order: Sequence[int] = ()) -> dict:
@@ -205,6 +219,12 @@ def plan_to_json(blocks, with_comm_standins: bool = True, alias=None, bwd_order:
     return {"DCBlocks": section(blocks),
             "fwd_only": section([(f, []) for f, _ in blocks if f]),
             "bwd_only": section([([], b) for _, b in blocks if b])}
+
+
+def unpaired_cost(profile: Dict[Key, float], fwd_groups, bwd_groups) -> Tuple[float, float]:
+    """(forward alone, backward alone): the boundary groups one after the other on their own, which is what the
+    ``fwd_only`` and ``bwd_only`` sections of a plan run for the first forward and the last backward."""
+    return (sum(profile[(tuple(g), ())] for g in fwd_groups), sum(profile[((), tuple(g))] for g in bwd_groups))
 
 
 def dump_plan(blocks, path: str, alias=None, bwd_order: Sequence[int] = ()) -> dict:

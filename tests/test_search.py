@@ -226,3 +226,79 @@ def test_context_parallel_groups_and_graph():
     blocks = [(fwd[i] if i < len(fwd) else [], bwd[i] if i < len(bwd) else []) for i in range(max(len(fwd), len(bwd)))]
     loaded = dstb.init_DCBlocks(search.plan_to_json(blocks), context_parallel_size=4)
     assert "cp_attn_block_bwd_5" in _ops_of(loaded.dcblocks, "stream2_op")
+
+
+def _all_plan_costs(profile, fwd_groups, bwd_groups):
+    """Cost of EVERY plan (every block sequence that covers both lists in order with groups inside the
+    boundaries), by plain recursion: the ground truth for the k-best DP."""
+    F, fs = search._starts(fwd_groups)
+    B, bs = search._starts(bwd_groups)
+    t = lambda f, b: profile[(tuple(f), tuple(b))]
+    out = []
+
+    def rec(i, j, acc):
+        if i == 0 and j == 0:
+            out.append(acc)
+            return
+        fgs = [F[a:i] for a in range(fs[i - 1], i)] if i > 0 else []
+        bgs = [B[a:j] for a in range(bs[j - 1], j)] if j > 0 else []
+        for fg in fgs:
+            rec(i - len(fg), j, acc + t(fg, []))
+        for bg in bgs:
+            rec(i, j - len(bg), acc + t([], bg))
+        for fg in fgs:
+            for bg in bgs:
+                rec(i - len(fg), j - len(bg), acc + t(fg, bg))
+
+    rec(len(F), len(B), 0.0)
+    return sorted(out)
+
+
+def test_k_best_plans_are_the_k_cheapest_of_all():
+    rng = random.Random(1)
+    fwd_groups, bwd_groups = [[1], [2, 3]], [[11, 12], [13]]
+    fc, bc = op_table.candidate_groups(fwd_groups), op_table.candidate_groups(bwd_groups)
+    prof = {(tuple(f), tuple(b)): rng.uniform(0.1, 1.0) for f in fc for b in bc if f or b}
+    truth = _all_plan_costs(prof, fwd_groups, bwd_groups)
+    for k in (1, 3, 7, len(truth) + 5):
+        found = search.search_plans(prof, fwd_groups, bwd_groups, k=k)
+        assert len(found) == min(k, len(truth))
+        assert all(abs(c - w) < 1e-12 for (c, _), w in zip(found, truth))
+        seen = set()
+        for cost, blocks in found:
+            assert [x for f, _ in blocks for x in f] == [1, 2, 3] and [x for _, b in blocks for x in b] == [11, 12, 13]
+            assert abs(sum(prof[(tuple(f), tuple(b))] for f, b in blocks) - cost) < 1e-12
+            seen.add(str(blocks))
+        assert len(seen) == len(found), "the k plans are k different plans"
+
+
+def test_execute_stage_keeps_the_measured_winner(tmp_path, monkeypatch):
+    """search/execute.py:54-116: every candidate is replayed, the fastest is copied to best.json; the built-in plan
+    is always among the candidates and wins ties, so the emitted plan is never slower than running without one."""
+    import json
+    from dhellam_amd.search import execute as ex
+    times = {"a": (10.0, 9.0), "b": (8.5, 9.5), ex.BUILTIN: (9.2, 9.3)}          # (free-running, lockstep)
+
+    def fake_replay(cfg, weights, mbs, plan, steps=20, warmup=3, lockstep=False):
+        name = ex.BUILTIN if plan is None else plan["name"]
+        return times[name][1 if lockstep else 0]
+
+    monkeypatch.setattr(ex, "replay", fake_replay)
+    monkeypatch.setattr(ex, "replay_serial", lambda *a, **k: 9.4)
+    cands = [{"name": n, "plan": {"name": n, "DCBlocks": []}, "paired_ms": 2.0} for n in ("a", "b")]
+    rep = ex.execute(None, None, [0, 1, 2, 3], cands, str(tmp_path), fwd_alone_ms=1.0, bwd_alone_ms=2.0, log=lambda m: None)
+    assert [r["name"] for r in rep["candidates"]] == ["a", "b", ex.BUILTIN]        # the built-in plan was added
+    assert rep["best"] == {"name": "b", "lockstep_blocks": False, "ms": 8.5}
+    assert rep["candidates"][0]["predicted_lockstep_ms"] == 1.0 + 3 * 2.0 + 2.0
+    assert json.load(open(tmp_path / "best.json"))["name"] == "b"
+    assert json.load(open(tmp_path / "execute_report.json"))["speedup_over_serial"] == round(9.4 / 8.5, 4)
+    # a candidate that only ties with the built-in plan does not displace it, and the built-in plan is written out
+    times["a"], times["b"] = (10.0, 9.6), (9.2, 9.5)
+    rep = ex.execute(None, None, [0, 1], cands, str(tmp_path), log=lambda m: None)
+    assert rep["best"]["name"] == ex.BUILTIN
+    written = json.load(open(tmp_path / "best.json"))
+    assert written == ex.builtin_plan() and dstb.init_DCBlocks(written).dcblocks
+    # lockstep wins where it is the faster mode
+    times["a"] = (10.0, 8.0)
+    rep = ex.execute(None, None, [0, 1], cands, None, log=lambda m: None)
+    assert rep["best"] == {"name": "a", "lockstep_blocks": True, "ms": 8.0}

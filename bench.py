@@ -267,30 +267,101 @@ def kernel_rooflines(cfg):
     return res
 
 
+def _median_s(fn, reps: int = 3, warmup: int = 1) -> float:
+    for _ in range(warmup):
+        fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2]
+
+
+def _oracle_cfg(cfg):
+    return dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
+                ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size,
+                tp=cfg.tensor_model_parallel_size, tp_rank=cfg.tp_rank, eps=cfg.layernorm_epsilon, theta=cfg.rope_theta)
+
+
 def cpu_baseline(cfg):
-    """The oracle's eager fp32 CPU layer (forward + backward by autograd) on this host's
-    cores, on a bounded sample: ONE micro-batch at the full 70B-shard shape."""
-    from dhellam_amd.core.layer import make_microbatch, make_weights
+    """The oracle's eager PyTorch path on this host's cores (the reference's own operators cannot run without a GPU:
+    every wrapper enters a CUDA stream), 1 warm-up + 3 timed repetitions, median, same seeded inputs as the GPU run.
+    The headline entry is ONE micro-batch of the 70B-shard layer at full shape (fp32, forward + backward by autograd);
+    ``others`` holds the fp32 parity layer at full shape, the MoE rank share's index / row-move operators at full
+    shape, and bounded, LABELLED samples of the two heavy ones (expert FFN: 512 of the ~4100 rows; ring attention:
+    one diagonal step of 4 of the 32 query heads), each with the figure scaled to the full size."""
+    import numpy as np
+    from dhellam_amd.core.layer import make_microbatch, make_weights, small_fp32_layer
+    from oracle import attention as OA
     from oracle import layer as OL
+    from oracle import moe as OM
     threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
     w = {k: v for k, v in make_weights(cfg, 0, device="cpu").items() if v.is_floating_point()}
     mb = make_microbatch(cfg, 0, device="cpu")
-    oc = dict(hidden=cfg.hidden_size, heads=cfg.heads_per_rank, groups=cfg.groups_per_rank, head_dim=cfg.head_dim,
-              ffn=cfg.ffn_per_rank, seq=cfg.seq_length, batch=cfg.micro_batch_size,
-              tp=cfg.tensor_model_parallel_size, tp_rank=cfg.tp_rank, eps=cfg.layernorm_epsilon, theta=cfg.rope_theta)
-    t0 = time.perf_counter()
-    OL.layer_fwd_bwd(oc, w, mb, dtype=torch.float32)
-    t1 = time.perf_counter() - t0
-    reps = 1 if t1 > 10 else 2
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        OL.layer_fwd_bwd(oc, w, mb, dtype=torch.float32)
-    t = (time.perf_counter() - t0) / reps
+    oc = _oracle_cfg(cfg)
+    t = _median_s(lambda: OL.layer_fwd_bwd(oc, w, mb, dtype=torch.float32))
+    others = []
+    # the fp32 parity layer (hidden 1024, 16 x 64 MHA, FFN 2816, batch 2 x seq 512), full shape
+    c0 = small_fp32_layer()
+    w0 = {k: v for k, v in make_weights(c0, 0, device="cpu").items() if v.is_floating_point()}
+    mb0 = make_microbatch(c0, 0, device="cpu")
+    t0 = _median_s(lambda: OL.layer_fwd_bwd(_oracle_cfg(c0), w0, mb0, dtype=torch.float32))
+    others.append({"what": "fp32 parity layer fwd+bwd (hidden 1024, 16x64 MHA, FFN 2816, 2x512 tokens), full shape",
+                   "ms": round(t0 * 1e3, 1), "tokens_per_s": round(c0.tokens / t0, 1), "scaled": False})
+    # MoE rank share: 8192 tokens, 8 experts, top-2, hidden 4096; route + sort, permute, unpermute at full shape
+    g = torch.Generator().manual_seed(0)
+    Tm, Hm, E, K, Fm = 8192, 4096, 8, 2, 14336
+    logits = torch.randn(Tm, E, generator=g).numpy()
+    xm = torch.randn(Tm, Hm, generator=g).to(torch.bfloat16)
+    idx, gates = OM.route_topk(logits, K)
+    tpe, offs, sidx, dest = OM.sort_assignments(idx, E)
+    t_route = _median_s(lambda: OM.sort_assignments(OM.route_topk(logits, K)[0], E))
+    t_perm = _median_s(lambda: OM.permute(xm, sidx, offs, 0, 2, K, dtype=torch.bfloat16))
+    xp = OM.permute(xm, sidx, offs, 0, 2, K, dtype=torch.bfloat16)
+    gt = torch.from_numpy(np.asarray(gates, dtype=np.float32))
+    t_unp = _median_s(lambda: OM.unpermute(xp, dest, offs, 0, 2, Tm, K, gates=gt, dtype=torch.float32))
+    R = int(offs[2] - offs[0])
+    others.append({"what": f"MoE route_topk + sort ({Tm} tokens x {E} experts, top-{K}), full shape",
+                   "ms": round(t_route * 1e3, 2), "scaled": False})
+    others.append({"what": f"MoE permute (R={R} rows x {Hm}, bf16), full shape", "ms": round(t_perm * 1e3, 2),
+                   "GB_per_s": round((2 * R * Hm * 2 + 8 * R) / t_perm / 1e9, 2), "scaled": False})
+    others.append({"what": f"MoE unpermute with gates (R={R} -> {Tm} tokens x {Hm}), full shape",
+                   "ms": round(t_unp * 1e3, 2), "GB_per_s": round((R * Hm * 2 + Tm * Hm * 2 + 8 * R) / t_unp / 1e9, 2),
+                   "scaled": False})
+    # expert FFN fwd+bwd on a sample of 512 rows (256 per expert), fp32, scaled by rows
+    rs = 512
+    w1 = torch.randn(2, 2 * Fm, Hm, generator=g) * 0.02
+    w2 = torch.randn(2, Hm, Fm, generator=g) * 0.02
+    xs = torch.randn(rs, Hm, generator=g, requires_grad=True)
+    so = np.array([0, rs // 2, rs])
+
+    def ffn():
+        y, _, _ = OM.grouped_ffn(xs, w1.requires_grad_(), w2.requires_grad_(), so, dtype=torch.float32)
+        y.sum().backward()
+    t_ffn = _median_s(ffn)
+    others.append({"what": f"MoE expert FFN fwd+bwd (2 experts, H {Hm}, F {Fm}): {rs} of {R} rows timed, SCALED to {R} rows",
+                   "ms": round(t_ffn * 1e3 * R / rs, 1), "sample_ms": round(t_ffn * 1e3, 1),
+                   "TFLOP_per_s": round(18.0 * rs * Hm * Fm / t_ffn / 1e12, 3), "scaled": True})
+    del w1, w2
+    # ring attention: one diagonal (causal 4096 x 4096) step, 4 of the 32 query heads on 1 of the 8 kv heads, fwd + bwd
+    S, hq, hk, d = 4096, 4, 1, 128
+    q, k, v, do = (torch.randn(S, h, d, generator=g) for h in (hq, hk, hk, hq))
+    cu = torch.tensor([0, S], dtype=torch.int32)
+
+    def ring_step():
+        o, l = OA.attn_fwd(q, k, v, cu, cu, d ** -0.5, True, torch.float32)
+        OA.attn_bwd(do, q, k, v, o, l, cu, cu, d ** -0.5, True, torch.float32)
+    t_ring = _median_s(ring_step, reps=3, warmup=1)
+    others.append({"what": "ring attention step fwd+bwd (diagonal, q 4096 x kv 4096, d 128): 4 of 32 query heads timed, "
+                           "SCALED to 32 heads x 4 steps",
+                   "ms": round(t_ring * 1e3 * 8 * 4, 1), "sample_ms": round(t_ring * 1e3, 1), "scaled": True})
     return {"value": round(cfg.tokens / t, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "ms_per_microbatch": round(t * 1e3, 1),
-            "sample": f"{reps} rep(s) of ONE micro-batch ({cfg.tokens} tokens) of the same layer, full shape, "
-                      f"fp32 eager PyTorch + autograd on the host (the oracle), after 1 warm-up"}
+            "sample": f"median of 3 reps after 1 warm-up of ONE micro-batch ({cfg.tokens} tokens) of the same layer, "
+                      f"full shape, fp32 eager PyTorch + autograd on the host (the oracle)",
+            "others": others}
 
 
 def profile_op(name: str, iters: int = 5):

@@ -5,7 +5,12 @@ import pytest
 import torch
 
 from oracle import layer as OL
-from tests.util import assert_close
+from tests.util import assert_close, rel_err
+
+# Bound on the distance between a 16-bit run of the whole layer and the oracle that keeps every intermediate exact
+# (fp64 / fp32): each of the ~12 tensors stored on the way carries a relative rounding error of up to 2^-9 (bf16),
+# and they add up roughly in quadrature through forward and backward.
+UNROUNDED_BOUND = {torch.bfloat16: 2.5e-2, torch.float16: 4e-3}
 
 pytestmark = pytest.mark.gpu
 
@@ -40,6 +45,16 @@ def _check_layer(cfg, oracle_dtype, round_to=None):
     for k in GRAD_KEYS:
         errs[k] = assert_close(w[k].main_grad, g_o[k], dt, f"d{k}")
     print("layer rel err:", {k: f"{v:.2e}" for k, v in errs.items()})
+    if round_to is not None:
+        # ... and against the oracle that rounds NOWHERE: the rounding oracle above places its rounding points where
+        # the pipeline stores 16-bit tensors, so a drift of the whole 16-bit pipeline would pass it.  The distance to
+        # the exact result is what a chain of a dozen 16-bit stores may cost, no more.
+        out_x, g_x = OL.layer_fwd_bwd(_oracle_cfg(cfg), w_cpu, mb_cpu, dtype=oracle_dtype, round_to=None)
+        far = {"out": rel_err(outs[0], out_x), "dx": rel_err(dxs[0], g_x["x"])}
+        far.update({k: rel_err(w[k].main_grad, g_x[k]) for k in GRAD_KEYS})
+        print("layer rel err vs the unrounded oracle:", {k: f"{v:.2e}" for k, v in far.items()})
+        for k, v in far.items():
+            assert v <= UNROUNDED_BOUND[dt], f"{k}: {v:.3e} from the unrounded oracle > {UNROUNDED_BOUND[dt]:.1e}"
 
 
 def test_layer_fp32_parity_config():
@@ -345,7 +360,6 @@ def test_weights_updated_around_the_version_counter_are_seen_by_the_next_step():
     ref = LayerRunner(dataclasses.replace(cfg, resident_weight_transposes=False), new)
     outs_r, dxs_r = ref.run_double_strand([make_microbatch(cfg, i) for i in range(2)])
     torch.cuda.synchronize()
-    from tests.util import rel_err
     for i in range(2):
         assert torch.equal(outs[i], outs_r[i]), f"out[{i}]"
         assert_close(dxs[i], dxs_r[i].cpu(), cfg.params_dtype, f"dx[{i}] (a stale W^T would be off by ~1)")

@@ -5,7 +5,11 @@ import pytest
 import torch
 
 from oracle import moe as OM
-from tests.util import assert_close, randn
+from tests.util import assert_close, randn, rel_err
+
+# Bound on the distance between the 16-bit expert FFN and the oracle that keeps h and a exact: two 16-bit stores
+# on the way forward and two gradients stored on the way back, each off by up to 2^-9 of itself.
+UNROUNDED_BOUND = 1.5e-2
 
 pytestmark = pytest.mark.gpu
 
@@ -167,6 +171,16 @@ def test_expert_ffn_fwd_bwd():
     assert_close(dxp, xr.grad, dtype, "dxp")
     assert_close(dw1, w1r.grad, dtype, "dw1")
     assert_close(dw2, w2r.grad, dtype, "dw2")
+    # ... and the distance to the oracle that rounds nowhere (fp64 throughout): what two 16-bit stores on the way
+    # forward and two on the way back may cost, so that a drift of the 16-bit pipeline cannot hide behind an oracle
+    # that rounds where the pipeline rounds
+    xe = xp.cpu().double().requires_grad_()
+    w1e, w2e = w1.double().requires_grad_(), w2.double().requires_grad_()
+    ye, _, _ = OM.grouped_ffn(xe, w1e, w2e, offs_cpu[e_lo:e_hi + 1], round_to=None)
+    (ye * dy.double()).sum().backward()
+    far = {"y": rel_err(y, ye), "dxp": rel_err(dxp, xe.grad), "dw1": rel_err(dw1, w1e.grad), "dw2": rel_err(dw2, w2e.grad)}
+    print("expert FFN rel err vs the unrounded oracle:", {k_: f"{v:.2e}" for k_, v in far.items()})
+    assert max(far.values()) <= UNROUNDED_BOUND, far
 
 
 def test_expert_ffn_full_size():
@@ -200,6 +214,15 @@ def test_expert_ffn_full_size():
     assert_close(dxp, xr.grad, dtype, "dxp")
     assert_close(dw1, w1r.grad, dtype, "dw1")
     assert_close(dw2, w2r.grad, dtype, "dw2")
+    # ... and the distance to the same oracle without any rounding of h and a (fp32 throughout)
+    del xr, w1r, w2r, yr
+    xe = xp.float().requires_grad_()
+    w1e, w2e = w1.float().requires_grad_(), w2.float().requires_grad_()
+    ye, _, _ = OM.grouped_ffn(xe, w1e, w2e, offs_cpu[0:3], dtype=torch.float32, round_to=None)
+    (ye * dy.float()).sum().backward()
+    far = {"y": rel_err(y, ye), "dxp": rel_err(dxp, xe.grad), "dw1": rel_err(dw1, w1e.grad), "dw2": rel_err(dw2, w2e.grad)}
+    print("expert FFN (full size) rel err vs the unrounded oracle:", {k_: f"{v:.2e}" for k_, v in far.items()})
+    assert max(far.values()) <= UNROUNDED_BOUND, far
 
 
 def test_expert_ffn_is_deterministic():

@@ -94,6 +94,7 @@ def kernel_rooflines(cfg):
     """Per-operator achieved rate against its roofline at the 70B-shard shapes (and the
     ring / MoE shapes).  Algorithmic work only: compulsory bytes, unmasked MACs."""
     from dhellam_amd import _Clib
+    from dhellam_amd import _lib as L_
     from dhellam_amd.operators import moe
     from dhellam_amd.operators.bda import bda_fwd
     from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
@@ -103,6 +104,20 @@ def kernel_rooflines(cfg):
     g = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(s, generator=g, device=dev, dtype=torch.float32).to(dt)
     res = []
+    lib = L_.load()
+    floors = {}
+
+    def copy_floor_ms(work_bytes):
+        """ms of the plain copy kernel (dh_copy_bytes) moving the same number of bytes (half read, half written),
+        timed the same way: what this machine gives a kernel of that size that does nothing but stream."""
+        n = int(work_bytes // 2) // 16 * 16
+        if n not in floors:
+            src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+            dst = torch.empty_like(src)
+            floors[n] = time_gpu_graph(lambda: L_.check(lib.dh_copy_bytes(src.data_ptr(), dst.data_ptr(), n,
+                                                                          torch.cuda.current_stream().cuda_stream)))
+            del src, dst
+        return floors[n]
 
     def add(name, bound, work, ms, unit_work):
         rate = work / (ms * 1e-3)
@@ -110,8 +125,15 @@ def kernel_rooflines(cfg):
             ach, peak, unit = rate / 1e9, HBM_PEAK_GBS, "GB/s"
         else:
             ach, peak, unit = rate / 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-        res.append({"kernel": name, "bound": bound, "ms": round(ms, 5), "achieved": round(ach, 2), "peak": peak,
-                    "unit": unit, "frac": round(ach / peak, 4), "work": unit_work})
+        row = {"kernel": name, "bound": bound, "ms": round(ms, 5), "achieved": round(ach, 2), "peak": peak,
+               "unit": unit, "frac": round(ach / peak, 4), "work": unit_work}
+        if bound == "hbm":
+            # the bar for a bandwidth kernel: 70 % of the HBM peak, or within 10 % of a plain copy of the same bytes
+            fl = copy_floor_ms(work)
+            row["copy_floor_ms"] = round(fl, 5)
+            row["vs_copy_floor"] = round(ms / fl, 3)
+            row["meets_bar"] = bool(ach / peak >= 0.70 or ms <= 1.10 * fl)
+        res.append(row)
 
     R, H, F, T = cfg.sp_rows, cfg.hidden_size, cfg.ffn_per_rank, cfg.tokens
     hq, hk, d = cfg.heads_per_rank, cfg.groups_per_rank, cfg.head_dim
@@ -432,6 +454,50 @@ def profile_op(name: str, iters: int = 5):
         else:
             src, dst = rn(4096, 8192), torch.empty(8192, 4096, device=dev, dtype=dt)
             fn = lambda: _Clib.transpose_2d(src, dst)
+    elif name in ("rope", "residual_add", "add_norm", "norm_shard", "merge", "permute", "unpermute", "copy_shard"):
+        # the bandwidth kernels at the configurations' own shapes (70B shard: 512 x 8192 norm rows, 4096 tokens of
+        # 8 q + 1 kv heads; ring: 4 steps of 4096 x 32 x 128; MoE: 8192 tokens, hidden 4096, this rank's 2 experts)
+        from dhellam_amd.operators import moe
+        from dhellam_amd.operators.bda import bda_fwd
+        from dhellam_amd.operators.layernorm import pylayernorm_bwd, pylayernorm_fwd
+        from dhellam_amd.operators.rope import rope_fwd
+        if name == "rope":
+            qkv = rn(4096, 1280)
+            q, k = qkv[:, :1024].view(4096, 8, 128), qkv[:, 1024:1152].view(4096, 1, 128)
+            fn = lambda: rope_fwd(q, k, None, 500000.0, 4096, None, False, inplace=True)
+        elif name == "residual_add":
+            a, b = rn(512, 8192), rn(512, 8192)
+            o = torch.empty_like(a)
+            fn = lambda: bda_fwd(a, b, out=o)
+        elif name == "add_norm":
+            a, b, gm = rn(512, 8192), rn(512, 8192), torch.ones(8192, device=dev, dtype=dt)
+            so = torch.empty_like(a)
+            fn = lambda: pylayernorm_fwd(a, gm, None, 1e-5, 0, False, None, residual=b, sum_out=so)
+        elif name == "norm_shard":
+            x, gm, dy = rn(512, 8192), torch.ones(8192, device=dev, dtype=dt), rn(512, 8192)
+            _, _, rs, _ = pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None)
+            fn = lambda: (pylayernorm_fwd(x, gm, None, 1e-5, 0, False, None), pylayernorm_bwd(dy, x, None, rs, gm, 0, False, None))
+        elif name == "copy_shard":      # the plain copy kernel on the norm's bytes: 8 MiB read, 8 MiB written
+            n = 512 * 8192 * 2
+            a = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+            b = torch.empty_like(a)
+            lib = _lib.load()
+            fn = lambda: _lib.check(lib.dh_copy_bytes(a.data_ptr(), b.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+        elif name == "merge":
+            outs = [rn(4096, 32, 128) for _ in range(4)]
+            lses = [torch.randn(1, 32, 4096, generator=g, device=dev) for _ in range(4)]
+            om, lm = torch.empty(4096, 32, 128, device=dev, dtype=dt), torch.empty(1, 32, 4096, device=dev)
+            fn = lambda: _Clib.pyattn_merge(outs, lses, [0] * 4, [4096] * 4, om, lm)
+        else:
+            Tm, Hm, E, K = 8192, 4096, 8, 2
+            logits = torch.randn(Tm, E, generator=g, device=dev)
+            xm = rn(Tm, Hm)
+            idx, gates, _ = moe.route_topk(logits, K)
+            plan, _ = moe.sort_assignments(idx, E)
+            Rm = int(plan.expert_offsets[2].item())
+            xp, _ = moe.permute_fwd(xm, plan, 0, 2, Rm)
+            print(f"moe rows of this rank: {Rm}", flush=True)
+            fn = (lambda: moe.permute_fwd(xm, plan, 0, 2, Rm)) if name == "permute" else (lambda: moe.unpermute_fwd(xp, plan, gates, 0, 2))
     elif name in ("gg_nt", "gemm_nt"):
         # one [4096, 8192] x [7168, 8192]^T product: the grouped GEMM kernel (two groups of 2048 rows, full tiles
         # only) and the library GEMM of the same shape, for side-by-side counter runs
@@ -581,7 +647,7 @@ def main():
                          "emitted (dhellam_amd/search/config/best.json) when there is one, else the built-in plan; "
                          "'builtin' forces the built-in plan")
     ap.add_argument("--profile-op", default=None,
-                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, swiglu_t, cross_entropy, transpose, gg_nt, gemm_nt, layer, copy) and exit")
+                    help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, swiglu_t, cross_entropy, transpose, rope, residual_add, add_norm, norm_shard, merge, permute, unpermute, copy_shard, gg_nt, gemm_nt, layer, copy) and exit")
     ap.add_argument("--analyze-trace", default=None,
                     help="kernel-trace CSV of `rocprofv3 --kernel-trace -- python bench.py --profile-op layer`: print the "
                          "overlap headroom of the serial schedule and exit (no GPU needed)")

@@ -364,6 +364,170 @@ norm_bwd_generic_wgrad_kernel(const T *__restrict__ dy, const T *__restrict__ x,
   }
 }
 
+// Backward in ONE launch for inputs that stay in the caches (a few hundred rows): no partial rows, no finalize.
+// dx needs a whole row (its two row sums), the weight gradients need a whole column:
+//     dgamma[c] = sum_r dy[r][c] * (x[r][c] - mu[r]) * rsigma[r],    dbeta[c] = sum_r dy[r][c],
+// and mu / rsigma are inputs (saved by the forward), so a column sum depends on no other workgroup.  Workgroup w
+// therefore does both: the rows w, w + G, ... for dx exactly as norm_bwd_kernel does (same arithmetic, same bits),
+// and the column slab [SW w, SW w + SW) over ALL rows for dgamma / dbeta, reading that slab a second time (from
+// L2 / the last-level cache: the operands were just streamed through it).  Row groups of the slab are added
+// through LDS in a fixed order.  1024 threads, one 16-byte vector of the row per thread (cols <= 1024 vectors).
+template <typename T, bool LN, bool ADD>
+__global__ void __launch_bounds__(1024)
+norm_bwd_onepass_kernel(const T *__restrict__ dy, const T *__restrict__ x, const float *__restrict__ mu,
+                        const float *__restrict__ rsigma, const T *__restrict__ gamma, const T *__restrict__ add_to_dx,
+                        T *__restrict__ dx, T *__restrict__ dgamma, T *__restrict__ dbeta, int64_t rows, int cols,
+                        float gamma_shift, int accumulate) {
+  constexpr int N = Vec<T>::N;
+  constexpr int BT = 1024;
+  constexpr int SW = 32;                 // columns of a slab
+  constexpr int L = SW / N;              // lanes across a slab row
+  constexpr int RG = BT / L;             // row groups of the column phase
+  constexpr int PRE = 2;                 // slab iterations requested before the row phase
+  __shared__ float red[BT / 64];
+  __shared__ float sg[RG][SW + 1];
+  __shared__ float sb[LN ? RG : 1][SW + 1];
+  const int nvec = cols / N;
+  const int tid = threadIdx.x;
+  const float inv_cols = 1.0f / (float)cols;
+
+  // ---- column phase, part 1: the first PRE row groups' loads go out now ----
+  const int cl = tid % L, rg = tid / L;
+  const int cv = (int)blockIdx.x * L + cl;             // vector index inside a row
+  const bool cvalid = cv < nvec;
+  Vec<T> sx[PRE], sd[PRE];
+  float srs[PRE], smu[PRE];
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) {
+    const int64_t r = rg + (int64_t)u * RG;
+    srs[u] = 0.f;
+    smu[u] = 0.f;
+    if (cvalid && r < rows) {
+      sx[u] = ldg(x + r * cols + (int64_t)cv * N);
+      sd[u] = ldg(dy + r * cols + (int64_t)cv * N);
+      srs[u] = rsigma[r];
+      if (LN) smu[u] = mu[r];
+    }
+  }
+
+  // ---- row phase: dx of rows blockIdx.x, blockIdx.x + gridDim.x, ... ----
+  {
+    const int v = tid;
+    const bool vvalid = v < nvec;
+    Vec<T> g;
+    if (vvalid) g = ldg(gamma + (int64_t)v * N);
+    Vec<T> xn, dn;
+    auto fetch = [&](int64_t row) {
+      if (row < rows && vvalid) {
+        xn = ldg(x + row * cols + (int64_t)v * N);
+        dn = ldg(dy + row * cols + (int64_t)v * N);
+      }
+    };
+    fetch(blockIdx.x);
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+      const Vec<T> xv = xn, dv = dn;
+      fetch(row + gridDim.x);
+      Vec<T> rv;
+      if (ADD && vvalid) rv = ldg(add_to_dx + row * cols + (int64_t)v * N);
+      const float rs = rsigma[row];
+      const float mean = LN ? mu[row] : 0.f;
+      float s1 = 0.f, s2 = 0.f;
+      if (vvalid) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float xh = (to_f(xv.v[j]) - mean) * rs;
+          const float gg = to_f(dv.v[j]) * (to_f(g.v[j]) + gamma_shift);
+          s1 += gg * xh;
+          if (LN) s2 += gg;
+        }
+      }
+      s1 = block_sum<BT>(s1, red);
+      if (LN) s2 = block_sum<BT>(s2, red);
+      const float c1 = s1 * inv_cols, c2 = s2 * inv_cols;
+      if (vvalid) {
+        Vec<T> o;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          const float xh = (to_f(xv.v[j]) - mean) * rs;
+          const float gg = to_f(dv.v[j]) * (to_f(g.v[j]) + gamma_shift);
+          float f = rs * (gg - xh * c1 - c2);
+          if (ADD) f += to_f(rv.v[j]);
+          o.v[j] = from_f<T>(f);
+        }
+        stg(dx + row * cols + (int64_t)v * N, o);
+      }
+    }
+  }
+
+  // ---- column phase, part 2: accumulate the slab over all rows, row groups in order ----
+  float dg[N], db[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    dg[j] = 0.f;
+    db[j] = 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) {
+    const int64_t r = rg + (int64_t)u * RG;
+    if (cvalid && r < rows) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const float d = to_f(sd[u].v[j]);
+        dg[j] += d * ((to_f(sx[u].v[j]) - smu[u]) * srs[u]);
+        if (LN) db[j] += d;
+      }
+    }
+  }
+  if (cvalid) {
+    for (int64_t r = rg + (int64_t)PRE * RG; r < rows; r += RG) {
+      const Vec<T> xv = ldg(x + r * cols + (int64_t)cv * N), dv = ldg(dy + r * cols + (int64_t)cv * N);
+      const float rs = rsigma[r];
+      const float mean = LN ? mu[r] : 0.f;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        const float d = to_f(dv.v[j]);
+        dg[j] += d * ((to_f(xv.v[j]) - mean) * rs);
+        if (LN) db[j] += d;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    sg[rg][cl * N + j] = dg[j];
+    if (LN) sb[rg][cl * N + j] = db[j];
+  }
+  __syncthreads();
+  // column c: 32 threads add RG / 32 row groups each (k, k + 32, ...), then thread k = 0 adds the 32 sums in order
+  {
+    const int c = tid / 32, k = tid % 32;
+    float ag = 0.f, ab = 0.f;
+#pragma unroll
+    for (int r = k; r < RG; r += 32) {
+      ag += sg[r][c];
+      if (LN) ab += sb[r][c];
+    }
+    __syncthreads();
+    sg[k][c] = ag;
+    if (LN) sb[k][c] = ab;
+    __syncthreads();
+    const int64_t col = (int64_t)blockIdx.x * SW + c;
+    if (k == 0 && col < cols) {
+      float tg = 0.f, tb = 0.f;
+#pragma unroll
+      for (int r = 0; r < 32; ++r) {
+        tg += sg[r][c];
+        if (LN) tb += sb[r][c];
+      }
+      if (accumulate) {
+        tg += to_f(dgamma[col]);
+        if (LN) tb += to_f(dbeta[col]);
+      }
+      dgamma[col] = from_f<T>(tg);
+      if (LN) dbeta[col] = from_f<T>(tb);
+    }
+  }
+}
+
 // Reduce partial rows: part [2][P][cols] -> dgamma (and dbeta) [cols].
 // Block = 16 float4 lanes (64 columns) x 16 row groups; each lane streams its rows with four
 // independent accumulators, the row groups are combined through LDS in a fixed order.
@@ -507,6 +671,13 @@ static int64_t bwd_blocks(int64_t rows, int64_t cols, int elt) {
   return nb;
 }
 
+// Whether the backward runs as one launch (norm_bwd_onepass_kernel): rows of 513 .. 1024 vectors (one vector per
+// thread of a 1024-thread workgroup) and operands small enough that the second, column-wise read of dy and x is
+// served by the caches (32 MiB of dy + x; the 512 x 8192 16-bit rows of a sequence-parallel shard are 16 MiB).
+static bool bwd_onepass(const NormPlan &p, int64_t rows, int64_t cols, int elt) {
+  return p.vec && p.tpr == 1024 && p.vpt == 1 && rows > 0 && 2 * rows * cols * elt <= (32ll << 20);
+}
+
 template <typename T, bool LN>
 static int launch_fwd(const NormPlan &p, const T *x, const T *residual, T *sum_out, const T *gamma, const T *beta, T *y,
                       float *mu, float *rs, int64_t rows, int64_t cols, float eps, float shift, hipStream_t st) {
@@ -559,6 +730,16 @@ static int launch_bwd(const NormPlan &p, const T *dy, const T *x, const float *m
                       const T *add, T *dx, T *dgamma, T *dbeta, float *part, int64_t rows, int64_t cols,
                       float shift, int accumulate, hipStream_t st) {
   const int64_t nb = bwd_blocks(rows, cols, sizeof(T));
+  if (bwd_onepass(p, rows, cols, sizeof(T))) {
+    const unsigned g = (unsigned)cdiv(cols, 32);
+    if (add)
+      hipLaunchKernelGGL((norm_bwd_onepass_kernel<T, LN, true>), dim3(g), dim3(1024), 0, st, dy, x, mu, rs, gamma, add,
+                         dx, dgamma, dbeta, rows, (int)cols, shift, accumulate);
+    else
+      hipLaunchKernelGGL((norm_bwd_onepass_kernel<T, LN, false>), dim3(g), dim3(1024), 0, st, dy, x, mu, rs, gamma, add,
+                         dx, dgamma, dbeta, rows, (int)cols, shift, accumulate);
+    return 0;
+  }
   if (!p.vec) {
     int64_t g = rows < 4096 ? rows : 4096;
     hipLaunchKernelGGL((norm_bwd_generic_kernel<T, LN>), dim3((unsigned)g), dim3(256), 0, st, dy, x, mu, rs, gamma,

@@ -10,7 +10,7 @@ from tests.util import assert_close, rel_err
 # Bound on the distance between a 16-bit run of the whole layer and the oracle that keeps every intermediate exact
 # (fp64 / fp32): each of the ~12 tensors stored on the way carries a relative rounding error of up to 2^-9 (bf16),
 # and they add up roughly in quadrature through forward and backward.
-UNROUNDED_BOUND = {torch.bfloat16: 2.5e-2, torch.float16: 4e-3}
+UNROUNDED_BOUND = {torch.bfloat16: 2e-2, torch.float16: 3e-3}    # measured: 2.5e-3 .. 1.3e-2 (bf16)
 
 pytestmark = pytest.mark.gpu
 

@@ -9,7 +9,7 @@ from tests.util import assert_close, randn, rel_err
 
 # Bound on the distance between the 16-bit expert FFN and the oracle that keeps h and a exact: two 16-bit stores
 # on the way forward and two gradients stored on the way back, each off by up to 2^-9 of itself.
-UNROUNDED_BOUND = 1.5e-2
+UNROUNDED_BOUND = 1e-2      # measured: 3.4e-3 .. 3.5e-3
 
 pytestmark = pytest.mark.gpu
 

@@ -724,6 +724,21 @@ def main():
             "double_strand_speedup": round(ser_h / dbl_h, 4),
             "serial_cost_us_per_standin": round((ser_h - ms_serial) * 1e3 / n_standins, 1),
             "double_strand_cost_us_per_standin": round((dbl_h - ms_double) * 1e3 / n_standins, 1)}
+        # ... and with the stand-ins carried out by the resident communication proxy: one kernel per step with a
+        # wavefront per strand, requests posted and waited for through the command processor (no kernel launch per
+        # collective, so a request does not queue behind the other strand's GEMM).  The proxy's own log gives how long
+        # each collective took on the device.
+        prox = dataclasses.replace(cfg, comm_standin_us=args.emulate_comm_us, comm_standin_engine="proxy")
+        runner_p = LayerRunner(prox, w, plan=plan)
+        ser_p, dbl_p = timed(runner_p.run_serial, runner_p), timed(runner_p.run_double_strand, runner_p)
+        durs = sorted(b - a for slot in (0, 1) for a, b in runner_p.proxy.log(slot))
+        emulated["resident_proxy_standins"] = {
+            "serial_ms": round(ser_p, 4), "double_strand_ms": round(dbl_p, 4),
+            "double_strand_speedup": round(ser_p / dbl_p, 4),
+            "serial_cost_us_per_standin": round((ser_p - ms_serial) * 1e3 / n_standins, 1),
+            "double_strand_cost_us_per_standin": round((dbl_p - ms_double) * 1e3 / n_standins, 1),
+            "standin_us_on_device": {"requested": args.emulate_comm_us, "median": round(durs[len(durs) // 2], 1),
+                                     "max": round(durs[-1], 1), "count_last_step": len(durs)} if durs else None}
     layer_flop = 2748.8e9 * len(mbs)   # GEMM 2628.5 + attention 120.3 GFLOP per 4096-token micro-batch
 
     measured = _measured()

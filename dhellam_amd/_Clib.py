@@ -403,6 +403,33 @@ def _attn_fwd_raw(q, k, v, out, lse, cu_q, cu_k, max_q, max_k, scale, causal, st
                                _tok_stride(out), float(scale), int(bool(causal)), _lib.dt(q), stream_ptr))
 
 
+HEAD_DIMS_16BIT = (64, 96, 128, 192, 256)      # head dims the 16-bit kernels are compiled for
+
+
+def _pad_head_dim(t: torch.Tensor, d_to: int) -> torch.Tensor:
+    """``t`` [tokens, heads, d] with zero columns appended up to ``d_to`` (the reference pads the head dim to a
+    multiple of 8 the same way, csrc/operators/flash_atten.cu:303-312: zero columns change neither the scores nor the
+    first d columns of the result)."""
+    d = t.shape[-1]
+    if d == d_to:
+        return t
+    out = t.new_zeros(t.shape[0], t.shape[1], d_to)
+    out[..., :d] = t
+    return out
+
+
+def _kernel_head_dim(t: torch.Tensor) -> int:
+    """The head dim the kernels run ``t`` at: its own for fp32 and for the compiled 16-bit sizes, else the next
+    compiled size (d <= 256 as in the reference, flash_atten.cu:284)."""
+    d = t.shape[-1]
+    if t.dtype == torch.float32 or d in HEAD_DIMS_16BIT:
+        return d
+    for s_ in HEAD_DIMS_16BIT:
+        if d < s_:
+            return s_
+    raise RuntimeError(f"attention supports head dims up to 256 (got {d})")
+
+
 _rng_zero: dict = {}
 
 
@@ -436,13 +463,17 @@ def pymha_varlen_fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
         raise RuntimeError("cu_seqlens must be int32")
     stream = torch.cuda.current_stream()
     b = cu_seqlens_q.numel() - 1
-    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    d, dk_ = q.shape[-1], _kernel_head_dim(q)
+    if dk_ != d:        # the padded tensors are what the "padded" slots of the return list hold (flash_atten.cu:429-433)
+        q, k, v = _pad_head_dim(q, dk_), _pad_head_dim(k, dk_), _pad_head_dim(v, dk_)
+    out_padded = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     lse = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
     ms = _timed(profiling, stream, lambda: _confined(stream, math_sm_count, lambda st: _attn_fwd_raw(
-        q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
+        q, k, v, out_padded, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, is_causal,
         st.cuda_stream)))
+    out = out_padded if dk_ == d else out_padded[..., :d]
     p = torch.empty(0, dtype=q.dtype, device=q.device)
-    res = [out, q, k, v, out, lse, p, _zero_rng_state(q.device)]
+    res = [out, q, k, v, out_padded, lse, p, _zero_rng_state(q.device)]
     if profiling:
         res.append(torch.tensor([ms], dtype=torch.float32))
     return res
@@ -500,13 +531,18 @@ def pymha_varlen_bwd(dout, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k
     b = cu_seqlens_q.numel() - 1
     ext = torch.cuda.ExternalStream(stream_ptr) if stream_ptr else torch.cuda.default_stream()
     with torch.cuda.stream(ext):
+        d, dk_ = q.shape[-1], _kernel_head_dim(q)
+        if dk_ != d:    # zero columns up to a compiled head dim, as flash_atten.cu:560-575 pads to a multiple of 8
+            dout, q, k, v, out = (_pad_head_dim(t, dk_) for t in (dout, q, k, v, out))
         dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
         dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-        softmax_d = torch.empty((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
+        softmax_d = torch.zeros((b, q.shape[1], int(max_seqlen_q)), dtype=torch.float32, device=q.device)
         ms = _timed(profiling, ext, lambda: _confined(ext, math_sm_count, lambda st: _attn_bwd_raw(
             dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
             max_seqlen_k, softmax_scale, is_causal, int(st.cuda_stream))))
+        if dk_ != d:
+            dq, dk, dv = dq[..., :d].contiguous(), dk[..., :d].contiguous(), dv[..., :d].contiguous()
     res = [dq, dk, dv, softmax_d]
     if profiling:
         res.append(torch.tensor([ms], dtype=torch.float32))

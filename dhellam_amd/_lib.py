@@ -25,6 +25,12 @@ SIGNATURES = {
     "dh_copy_bytes": (_i32, [_vp, _vp, _i64, _vp]),
     "dh_delay": (_i32, [_i64, _vp]),
     "dh_host_delay": (_i32, [_i64, _vp]),
+    "dh_comm_proxy_create": (_i32, [_i32, _vp]),
+    "dh_comm_proxy_launch": (_i32, [_vp, _i64, _i64, _vp]),
+    "dh_comm_proxy_post": (_i32, [_vp, _i32, _vp]),
+    "dh_comm_proxy_wait": (_i32, [_vp, _i32, _vp]),
+    "dh_comm_proxy_stop": (_i32, [_vp, _vp]),
+    "dh_comm_proxy_log": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp]),
     "dh_gemm": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _sz, _vp]),
     "dh_gemm_tt": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _sz, _vp]),
     "dh_stream_create_cu_mask": (_i32, [_vp, _i32, _vp]),

@@ -115,10 +115,14 @@ class LayerConfig:
     params_dtype: torch.dtype = torch.bfloat16
     layernorm_bias: bool = False      # False: RMSNorm (Llama); True: LayerNorm with bias (the reference's TE call)
     comm_standin_us: float = 0.0      # > 0: every sequence-parallel stand-in also occupies its stream this long
-    # what occupies the stream: "kernel" = a one-wavefront delay kernel (a collective made of kernels: it has to find
-    # a free wavefront slot next to whatever else runs), "host" = a host function of the stream (a transfer carried
-    # by a copy engine or a network adapter: needs no compute unit)
+    # what occupies the stream: "kernel" = a one-wavefront delay kernel launched per collective (it has to find a free
+    # wavefront slot next to whatever else runs, and a kernel launched beside a GEMM that owns every compute unit
+    # starts only when that GEMM has placed its last workgroup), "proxy" = a request to the resident communication
+    # proxy (one kernel per step with a wavefront per strand, reached through stream writes and stream waits:
+    # ``common/comm_proxy.py``; ``comm_proxy`` below must hold it -- ``LayerRunner`` sets it up), "host" = a host
+    # function of the stream (a transfer carried by a copy engine or a network adapter: needs no compute unit)
     comm_standin_engine: str = "kernel"
+    comm_proxy: Optional[object] = None
     lockstep_blocks: bool = False     # the two strands enter every plan block together (events between the streams)
     # (forward strand's, backward strand's) communication streams: the stand-ins' delays run there, with events
     # to and from the strand's own stream, instead of on the strand's stream itself
@@ -438,8 +442,14 @@ class DCFunc:
         if us > 0:
             st = stream if stream is not None else torch.cuda.current_stream()
             comm = getattr(config, "comm_streams", None)
-            delay = _lib.load().dh_host_delay if getattr(config, "comm_standin_engine", "kernel") == "host" \
-                else _lib.load().dh_delay
+            engine = getattr(config, "comm_standin_engine", "kernel")
+            if engine == "proxy":
+                proxy = getattr(config, "comm_proxy", None)
+                if proxy is None or not proxy.running:
+                    raise RuntimeError("comm_standin_engine='proxy' needs a launched CommProxy in config.comm_proxy")
+                proxy.collective(1 if bwd_strand else 0, st)
+                return
+            delay = _lib.load().dh_host_delay if engine == "host" else _lib.load().dh_delay
             if comm is None:
                 _lib.check(delay(int(us * 1000), st.cuda_stream))
                 return

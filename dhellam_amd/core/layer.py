@@ -99,11 +99,28 @@ def fresh_activation_dict(mb: Dict[str, torch.Tensor]) -> dict:
     return {k: v for k, v in mb.items() if k.startswith("sp_peer") or k == "cp_kv_chunks"}
 
 
+_PROXY = []
+
+
+def _shared_proxy():
+    if not _PROXY:
+        from ..common.comm_proxy import CommProxy
+        _PROXY.append(CommProxy(2))
+    return _PROXY[0]
+
+
 class LayerRunner:
     """Runs micro-batches through one layer, serially or double-stranded."""
 
     def __init__(self, cfg: LayerConfig, weights: Dict[str, torch.Tensor], plan=None,
                  stream1: Optional[torch.cuda.Stream] = None, stream2: Optional[torch.cuda.Stream] = None):
+        self.proxy = None
+        if cfg.comm_standin_engine == "proxy" and cfg.comm_standin_us > 0:
+            # the stand-in collectives go to the resident communication proxy (one per process: its flags are
+            # signal memory that stays allocated); slot 0 = forward strand, slot 1 = backward strand
+            import dataclasses
+            self.proxy = cfg.comm_proxy or _shared_proxy()
+            cfg = dataclasses.replace(cfg, comm_proxy=self.proxy)
         self.cfg = cfg
         self.weights = weights
         self.stream1 = stream1 or torch.cuda.Stream()
@@ -129,6 +146,7 @@ class LayerRunner:
             self.refresh_weight_transposes()
         s = self.stream1
         s.wait_stream(torch.cuda.current_stream())
+        self._proxy_begin()
         outs, dxs = [], []
         for mb in mbs:
             act = fresh_activation_dict(mb)
@@ -136,6 +154,7 @@ class LayerRunner:
             _, dx = self._exec(self.plan.bwd_only, None, mb["dy"], act, None, s, s)
             outs.append(out)
             dxs.append(dx)
+        self._proxy_end(s, s)
         torch.cuda.current_stream().wait_stream(s)
         return outs, dxs
 
@@ -148,6 +167,7 @@ class LayerRunner:
         cur = torch.cuda.current_stream()
         s1.wait_stream(cur)
         s2.wait_stream(cur)
+        self._proxy_begin()
         n = len(mbs)
         outs, dxs = [None] * n, [None] * n
         act = fresh_activation_dict(mbs[0])
@@ -157,9 +177,21 @@ class LayerRunner:
             outs[i], dxs[i - 1] = self._exec(self.plan.dcblocks, mbs[i]["x"], mbs[i - 1]["dy"], act, act_new, s1, s2)
             act = act_new
         _, dxs[n - 1] = self._exec(self.plan.bwd_only, None, mbs[n - 1]["dy"], act, None, s1, s2)
+        self._proxy_end(s1, s2)
         cur.wait_stream(s1)
         cur.wait_stream(s2)
         return outs, dxs
+
+    def _proxy_begin(self):
+        """Starts the step's communication proxy (stand-in collectives with ``comm_standin_engine='proxy'``)."""
+        if self.proxy is not None:
+            self.proxy.launch(self.cfg.comm_standin_us)
+
+    def _proxy_end(self, fwd_stream, bwd_stream):
+        """Ends it: no request follows what the two strands' streams hold now."""
+        if self.proxy is not None:
+            self.proxy.stop([fwd_stream, bwd_stream])
+            torch.cuda.current_stream().wait_stream(self.proxy.stream)
 
     def zero_grads(self):
         for t in self.weights.values():

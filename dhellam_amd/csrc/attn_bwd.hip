@@ -1454,6 +1454,8 @@ int attn_bwd_f32(const void *dout, const void *q, const void *k, const void *v, 
                  int dq_accumulate, hipStream_t st);
 
 constexpr int DKV_NW = 2;  // wavefronts per dK/dV workgroup (64 key rows)
+// the dQ kernel's 32-key tile must divide evenly over the workgroup's threads (head dim 96 does not over 256)
+constexpr bool dq_takes_4_waves(int d) { return (32 * (d / 8)) % 256 == 0; }
 
 // Keeping dS for the dQ product costs 2 bytes per (head, query, key) of workspace, written once and read once.
 // It pays where the recomputing dQ kernel runs its small-grid form (fewer than 256 workgroups of 128 query rows:
@@ -1572,7 +1574,8 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
                         max_seqlen_k, hq, hk, d, q_stride, k_stride, v_stride, do_stride, dq_stride, dk_stride,
                         dv_stride, softmax_scale, causal, dq_accumulate, st);
   }
-  DH_CHECK(d == 64 || d == 128, "bf16/fp16 attention supports head dim 64 or 128 (got %d)", d);
+  DH_CHECK(d == 64 || d == 96 || d == 128 || d == 192 || d == 256,
+           "bf16/fp16 attention supports head dims 64, 96, 128, 192 and 256 (got %d); pad other sizes with zero columns", d);
   DH_CHECK(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && dq_stride % 4 == 0 && dk_stride % 4 == 0 &&
                dv_stride % 4 == 0,
            "token strides must keep rows aligned");
@@ -1621,14 +1624,17 @@ static int attn_bwd_entry(const void *dout, const void *q, const void *k, const 
                          p.dv_part, (TT *)dk, (TT *)dv, total_k, hk, DD, p.hsplit, dk_stride, dv_stride);    \
     }                                                                                          \
     if (rc == DH_OK && max_seqlen_q > 0 && DD != 128)                                          \
-      rc = small_q ? launch_dq<TT, DD, 2>(p, batch, st) : launch_dq<TT, DD, 4>(p, batch, st);  \
+      rc = (small_q || !dq_takes_4_waves(DD)) ? launch_dq<TT, DD, 2>(p, batch, st)             \
+                                              : launch_dq<TT, DD, dq_takes_4_waves(DD) ? 4 : 2>(p, batch, st); \
     if (rc == DH_OK && max_seqlen_q > 0 && DD == 128 && keep_ds) rc = launch_dq2_d128<TT>(p, batch, st); \
   } while (0)
-  if (dtype == DH_BF16) {
-    if (d == 128) DH_BWD(bf16_t, 128); else DH_BWD(bf16_t, 64);
-  } else {
-    if (d == 128) DH_BWD(f16_t, 128); else DH_BWD(f16_t, 64);
-  }
+#define DH_BWD_D(TT)                                                                            \
+  do {                                                                                          \
+    if (d == 128) DH_BWD(TT, 128); else if (d == 64) DH_BWD(TT, 64); else if (d == 96) DH_BWD(TT, 96); \
+    else if (d == 192) DH_BWD(TT, 192); else DH_BWD(TT, 256);                                   \
+  } while (0)
+  if (dtype == DH_BF16) DH_BWD_D(bf16_t); else DH_BWD_D(f16_t);
+#undef DH_BWD_D
 #undef DH_BWD
   if (rc != DH_OK) return rc;
   DH_LAUNCH_CHECK();

@@ -627,7 +627,8 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
                         q_stride, k_stride, v_stride, o_stride, softmax_scale, causal, st);
   }
   DH_CHECK(dtype == DH_BF16 || dtype == DH_F16, "unknown dtype %d", dtype);
-  DH_CHECK(d == 64 || d == 128, "bf16/fp16 attention supports head dim 64 or 128 (got %d)", d);
+  DH_CHECK(d == 64 || d == 96 || d == 128 || d == 192 || d == 256,
+           "bf16/fp16 attention supports head dims 64, 96, 128, 192 and 256 (got %d); pad other sizes with zero columns", d);
   DH_CHECK(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && o_stride % 4 == 0,
            "token strides must keep rows 16-byte aligned");
   DH_CHECK(k_stride < (1ll << 31) && v_stride < (1ll << 31), "token stride too large");
@@ -651,8 +652,18 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
     // Few query tiles (small batch*heads) -> smaller workgroups so the grid still covers the chip.
     const int64_t blocks128 = cdiv(max_seqlen_q, 128) * hq * batch;
     const bool small = blocks128 < 2 * 256;
-    if (dtype == DH_BF16) rc = small ? launch_attn_fwd<bf16_t, 64, 2>(p, batch, st) : launch_attn_fwd<bf16_t, 64, 4>(p, batch, st);
-    else rc = small ? launch_attn_fwd<f16_t, 64, 2>(p, batch, st) : launch_attn_fwd<f16_t, 64, 4>(p, batch, st);
+#define DH_FWD_GENERIC(DD)                                                                                            \
+  do {                                                                                                                \
+    if (dtype == DH_BF16) rc = small ? launch_attn_fwd<bf16_t, DD, 2>(p, batch, st) : launch_attn_fwd<bf16_t, DD, 4>(p, batch, st); \
+    else rc = small ? launch_attn_fwd<f16_t, DD, 2>(p, batch, st) : launch_attn_fwd<f16_t, DD, 4>(p, batch, st);      \
+  } while (0)
+    // the register-staged kernel, compiled per head dim (the other head dims of the reference's d <= 256 reach
+    // these through zero padding in the binding, as flash_atten.cu:303-312 pads to a multiple of 8)
+    if (d == 64) DH_FWD_GENERIC(64);
+    else if (d == 96) DH_FWD_GENERIC(96);
+    else if (d == 192) DH_FWD_GENERIC(192);
+    else DH_FWD_GENERIC(256);
+#undef DH_FWD_GENERIC
   }
   if (rc != DH_OK) return rc;
   DH_LAUNCH_CHECK();

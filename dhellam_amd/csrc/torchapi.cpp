@@ -7,6 +7,7 @@
 // libdhellam_hip.so (dhellam_amd/build.py: build_torch_extension).
 #include <torch/extension.h>
 #include <c10/hip/HIPCachingAllocator.h>
+#include <c10/hip/HIPGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 
@@ -58,8 +59,8 @@ template <typename F> float timed(bool profiling, hipStream_t stream, F &&fn) {
   hip_check(hipEventSynchronize(b));
   float ms = 0.f;
   hip_check(hipEventElapsedTime(&ms, a, b));
-  hipEventDestroy(a);
-  hipEventDestroy(b);
+  (void)hipEventDestroy(a);
+  (void)hipEventDestroy(b);
   return ms;
 }
 
@@ -101,7 +102,7 @@ template <typename F> void confined(hipStream_t stream, int device, int math_sm_
   launch(m);
   hip_check(hipEventRecord(e, m));
   hip_check(hipStreamWaitEvent(stream, e, 0));
-  hipEventDestroy(e);     // the runtime keeps the event alive until the waits recorded on it are done
+  (void)hipEventDestroy(e);     // the runtime keeps the event alive until the waits recorded on it are done
 }
 
 // A tensor allocated on torch's current stream and used on another raw stream: tell the caching allocator.
@@ -109,6 +110,21 @@ void record_on(const at::Tensor &t, hipStream_t stream) {
   if (stream == c10::hip::getCurrentHIPStream().stream()) return;
   c10::hip::HIPCachingAllocator::recordStream(t.storage().data_ptr(),
                                               c10::hip::getStreamFromExternal(stream, t.device().index()));
+}
+
+// Head dims the 16-bit kernels are compiled for; other sizes up to 256 run zero-padded to the next one (the reference
+// pads to a multiple of 8 the same way, flash_atten.cu:303-312); fp32 takes any size as it is.
+int64_t kernel_head_dim(const at::Tensor &t) {
+  const int64_t d = t.size(-1);
+  if (t.scalar_type() == at::kFloat) return d;
+  for (int64_t s : {64, 96, 128, 192, 256})
+    if (d <= s) return s;
+  TORCH_CHECK(false, "attention supports head dims up to 256 (got ", d, ")");
+}
+
+at::Tensor pad_head_dim(const at::Tensor &t, int64_t d_to) {
+  if (t.size(-1) == d_to) return t;
+  return at::constant_pad_nd(t, {0, d_to - t.size(-1)}, 0);
 }
 
 at::Tensor ms_tensor(float ms) { return at::full({1}, ms, at::TensorOptions().dtype(at::kFloat)); }
@@ -119,27 +135,30 @@ at::Tensor ms_tensor(float ms) { return at::full({1}, ms, at::TensorOptions().dt
 // stream.  Returns [out, q, k, v, out, softmax_lse, p, rng_state] (+ a CPU fp32 [1] tensor of milliseconds when
 // profiling), the positions of flash_atten.cu:429-433; the supported head dims need no padding, so the "padded"
 // slots hold the inputs themselves; p is empty and rng_state zero (no dropout).
-std::vector<at::Tensor> pymha_varlen_fwd(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
+std::vector<at::Tensor> pymha_varlen_fwd(const at::Tensor &q_in, const at::Tensor &k_in, const at::Tensor &v_in,
                                          const at::Tensor &cu_seqlens_q, const at::Tensor &cu_seqlens_k,
                                          int max_seqlen_q, int max_seqlen_k, float p_dropout, float softmax_scale,
                                          bool is_causal, bool return_softmax, int math_sm_count, bool profiling) {
   TORCH_CHECK(p_dropout == 0.f, "pymha_varlen_fwd: dropout is not implemented (p_dropout must be 0)");
   TORCH_CHECK(!return_softmax, "pymha_varlen_fwd: return_softmax is only supported with dropout in the reference");
-  need_gpu({&q, &k, &v, &cu_seqlens_q, &cu_seqlens_k});
+  need_gpu({&q_in, &k_in, &v_in, &cu_seqlens_q, &cu_seqlens_k});
   TORCH_CHECK(cu_seqlens_q.scalar_type() == at::kInt && cu_seqlens_k.scalar_type() == at::kInt, "cu_seqlens must be int32");
   const int b = (int)cu_seqlens_q.numel() - 1;
-  auto out = at::empty(q.sizes(), q.options());
+  const int64_t d_og = q_in.size(-1), d_run = kernel_head_dim(q_in);
+  const at::Tensor q = pad_head_dim(q_in, d_run), k = pad_head_dim(k_in, d_run), v = pad_head_dim(v_in, d_run);
+  auto out_padded = at::empty(q.sizes(), q.options());
   auto lse = at::empty({b, q.size(1), max_seqlen_q}, q.options().dtype(at::kFloat));
   hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
   const float ms = timed(profiling, stream, [&] {
     confined(stream, q.device().index(), math_sm_count, [&](hipStream_t st) {
-      check(dh_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr<float>(),
+      check(dh_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_padded.data_ptr(), lse.data_ptr<float>(),
                         cu_seqlens_q.data_ptr<int>(), cu_seqlens_k.data_ptr<int>(), b, max_seqlen_q, max_seqlen_k,
                         (int)q.size(1), (int)k.size(1), (int)q.size(2), token_stride(q), token_stride(k),
-                        token_stride(v), token_stride(out), softmax_scale, is_causal ? 1 : 0, dt(q), st));
+                        token_stride(v), token_stride(out_padded), softmax_scale, is_causal ? 1 : 0, dt(q), st));
     });
   });
-  std::vector<at::Tensor> res = {out, q, k, v, out, lse, at::empty({0}, q.options()),
+  const at::Tensor out = d_run == d_og ? out_padded : out_padded.narrow(-1, 0, d_og);
+  std::vector<at::Tensor> res = {out, q, k, v, out_padded, lse, at::empty({0}, q.options()),
                                  at::zeros({2}, q.options().dtype(at::kLong))};
   if (profiling) res.push_back(ms_tensor(ms));
   return res;
@@ -149,8 +168,8 @@ std::vector<at::Tensor> pymha_varlen_fwd(const at::Tensor &q, const at::Tensor &
 // launches on the raw stream its caller hands over (flash_atten.cu:784; 0 = torch's current stream).  Returns
 // [dq, dk, dv, softmax_d] (+ the milliseconds tensor when profiling).  The result does not depend on
 // `deterministic`: no floating-point atomics are used either way.
-std::vector<at::Tensor> pymha_varlen_bwd(const at::Tensor &dout, const at::Tensor &q, const at::Tensor &k,
-                                         const at::Tensor &v, const at::Tensor &out, const at::Tensor &softmax_lse,
+std::vector<at::Tensor> pymha_varlen_bwd(const at::Tensor &dout_in, const at::Tensor &q_in, const at::Tensor &k_in,
+                                         const at::Tensor &v_in, const at::Tensor &out_in, const at::Tensor &softmax_lse,
                                          const at::Tensor &cu_seqlens_q, const at::Tensor &cu_seqlens_k,
                                          int max_seqlen_q, int max_seqlen_k, float p_dropout, float softmax_scale,
                                          bool is_causal, c10::optional<at::Tensor> rng_state, bool deterministic,
@@ -158,8 +177,11 @@ std::vector<at::Tensor> pymha_varlen_bwd(const at::Tensor &dout, const at::Tenso
   (void)rng_state;
   (void)deterministic;
   TORCH_CHECK(p_dropout == 0.f, "pymha_varlen_bwd: dropout is not implemented (p_dropout must be 0)");
-  need_gpu({&dout, &q, &k, &v, &out, &softmax_lse, &cu_seqlens_q, &cu_seqlens_k});
+  need_gpu({&dout_in, &q_in, &k_in, &v_in, &out_in, &softmax_lse, &cu_seqlens_q, &cu_seqlens_k});
   TORCH_CHECK(softmax_lse.scalar_type() == at::kFloat && softmax_lse.is_contiguous(), "softmax_lse must be contiguous fp32");
+  const int64_t d_og = q_in.size(-1), d_run = kernel_head_dim(q_in);
+  const at::Tensor dout = pad_head_dim(dout_in, d_run), q = pad_head_dim(q_in, d_run), k = pad_head_dim(k_in, d_run),
+                   v = pad_head_dim(v_in, d_run), out = pad_head_dim(out_in, d_run);
   const int b = (int)cu_seqlens_q.numel() - 1, hq = (int)q.size(1), hk = (int)k.size(1), d = (int)q.size(2);
   auto dq = at::empty(q.sizes(), q.options()), dk = at::empty(k.sizes(), k.options()), dv = at::empty(v.sizes(), v.options());
   auto softmax_d = at::zeros({b, hq, max_seqlen_q}, q.options().dtype(at::kFloat));
@@ -176,7 +198,7 @@ std::vector<at::Tensor> pymha_varlen_bwd(const at::Tensor &dout, const at::Tenso
       hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming));
       hip_check(hipEventRecord(e, cur));
       hip_check(hipStreamWaitEvent(stream, e, 0));
-      hipEventDestroy(e);
+      (void)hipEventDestroy(e);
     }
   }
   const float ms = timed(profiling, stream, [&] {
@@ -190,7 +212,14 @@ std::vector<at::Tensor> pymha_varlen_bwd(const at::Tensor &dout, const at::Tenso
                         dt(q), st));
     });
   });
-  for (const at::Tensor *t : {&ws, &dq, &dk, &dv, &softmax_d}) record_on(*t, stream);
+  for (const at::Tensor *t : std::initializer_list<const at::Tensor *>{&ws, &dq, &dk, &dv, &softmax_d, &dout, &q, &k, &v, &out})
+    record_on(*t, stream);
+  if (d_run != d_og) {       // the gradients of the columns that were given
+    c10::hip::HIPStreamGuard guard(c10::hip::getStreamFromExternal(stream, q.device().index()));
+    dq = dq.narrow(-1, 0, d_og).contiguous();
+    dk = dk.narrow(-1, 0, d_og).contiguous();
+    dv = dv.narrow(-1, 0, d_og).contiguous();
+  }
   std::vector<at::Tensor> res = {dq, dk, dv, softmax_d};
   if (profiling) res.push_back(ms_tensor(ms));
   return res;

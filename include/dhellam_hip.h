@@ -149,8 +149,11 @@ int dh_rope(const void *q, const void *k, void *q_out, void *k_out,
  * elements (head stride is d, last dim contiguous).  cu_seqlens_* int32 [b+1]
  * on device.  lse fp32 [b, hq, max_seqlen_q] = natural-log logsumexp of the
  * scaled scores (-inf rows never occur for causal sq == sk).  causal requires
- * per-sequence sq == sk.  hq % hk == 0 (GQA).  d in {64, 128} for bf16/fp16,
- * any d <= 256 with d % 4 == 0 for fp32.
+ * per-sequence sq == sk.  hq % hk == 0 (GQA).  d in {64, 96, 128, 192, 256}
+ * for bf16/fp16 (the reference takes any d <= 256 and pads it to a multiple
+ * of 8 above this boundary, flash_atten.cu:284,303-312: a binding pads other
+ * sizes with zero columns to the next of these, as dhellam._Clib does), any
+ * d <= 256 with d % 4 == 0 for fp32.
  * ---------------------------------------------------------------------- */
 int dh_attn_fwd(const void *q, const void *k, const void *v, void *out,
                 float *lse, const int32_t *cu_seqlens_q,
@@ -339,6 +342,43 @@ int dh_delay(int64_t nanoseconds, void *stream);
  * compute unit (copy engine, network adapter), so it starts while kernels of
  * another stream fill the device.  No counterpart in the reference. */
 int dh_host_delay(int64_t nanoseconds, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Resident communication proxy: collectives that a stream posts and waits for
+ * without a kernel launch per collective.  It stands where the reference has
+ * its third stream and communication handles (dhellam/core/dstb.py:1142-1188:
+ * the collective is posted on stream 3, the compute op waits for its handle);
+ * the reference's collectives themselves (dhellam/operators/comm.py) are NCCL
+ * kernels.  One kernel, launched at the start of a step, keeps one wavefront
+ * per slot (a slot = a strand's communication channel) resident; a request is
+ * posted with a stream write and waited for with a stream wait, both carried
+ * out by the command processor, so a request is seen within microseconds even
+ * while a kernel of another stream owns every compute unit (a collective
+ * launched as a kernel of its own then waits until that kernel has placed its
+ * last workgroup).  On one GPU a request is carried out by waiting
+ * `duration_ns`.  All waits of the kernel are bounded (see launch).
+ *
+ * create: allocates the proxy (host object + three 8-byte pieces of signal
+ *   memory per slot and a log, kept until the process ends); slots <= 8.
+ * launch: starts the kernel on `stream` (a stream of its own, not a strand's).
+ *   A slot that sees neither a request nor its stop for `limit_ns` gives up and
+ *   releases every stream wait behind it.  One launch at a time.
+ * post / wait: on the strand's stream; a wait refers to the slot's last post.
+ * stop: streams[slot] = the stream whose order ends the slot's requests of
+ *   this launch (the strand's stream); the kernel ends once every slot has
+ *   seen its stop with nothing pending.
+ * log: after the launch's streams have been synchronised, the (start, end)
+ *   times in ns (a 100 MHz device clock, arbitrary origin) of up to
+ *   max_entries collectives the slot carried out; clears the log.
+ * ---------------------------------------------------------------------- */
+int dh_comm_proxy_create(int slots, void **proxy_out);
+int dh_comm_proxy_launch(void *proxy, int64_t duration_ns, int64_t limit_ns,
+                         void *stream);
+int dh_comm_proxy_post(void *proxy, int slot, void *stream);
+int dh_comm_proxy_wait(void *proxy, int slot, void *stream);
+int dh_comm_proxy_stop(void *proxy, const void *const *streams);
+int dh_comm_proxy_log(void *proxy, int slot, int64_t max_entries,
+                      int64_t *start_ns, int64_t *end_ns, int64_t *n_out);
 
 /* Dense GEMM through hipBLASLt: cublas_gemm / pygemm, csrc/operators/gemm.cu:3-170 (csrc/operators/ops.h:54-65).
  * The reference's convention is kept: A [a_rows, a_cols], B [b_rows, b_cols] and D are contiguous row-major

@@ -187,9 +187,14 @@ def test_attention_profiling_and_errors():
     assert len(res) == 9 and res[8].device.type == "cpu" and res[8].item() > 0
     with pytest.raises(RuntimeError):
         _Clib.pymha_varlen_fwd(q, q, q, cu, cu, 256, 256, 0.1, 0.1, True, False, 0, False)   # dropout
-    q96 = randn((256, 4, 96), torch.bfloat16, 0).cuda()
-    with pytest.raises(RuntimeError, match="head dim"):
-        _Clib.pymha_varlen_fwd(q96, q96, q96, cu, cu, 256, 256, 0.0, 0.1, True, False, 0, False)
+    # the C ABI itself takes the compiled head dims only (the bindings pad other sizes before they call it)
+    from dhellam_amd import _lib
+    q72 = randn((256, 4, 72), torch.bfloat16, 0).cuda()
+    o72, l72 = torch.empty_like(q72), torch.empty(1, 4, 256, device="cuda")
+    rc = _lib.load().dh_attn_fwd(q72.data_ptr(), q72.data_ptr(), q72.data_ptr(), o72.data_ptr(), l72.data_ptr(),
+                                 cu.data_ptr(), cu.data_ptr(), 1, 256, 256, 4, 4, 72, 288, 288, 288, 288, 0.1, 1,
+                                 _lib.DH_BF16, torch.cuda.current_stream().cuda_stream)
+    assert rc == -1 and "head dim" in _lib.load().dh_last_error().decode()
     k3 = randn((256, 3, 128), torch.bfloat16, 0).cuda()
     with pytest.raises(RuntimeError, match="multiple"):
         _Clib.pymha_varlen_fwd(q, k3, k3, cu, cu, 256, 256, 0.0, 0.1, True, False, 0, False)
@@ -293,3 +298,61 @@ def test_ring_step_full_size(rank):
     for s in range(cp):
         assert_close(dkv[s][0], cr[s][0].grad, dtype, f"ring dk[{s}]")
         assert_close(dkv[s][1], cr[s][1].grad, dtype, f"ring dv[{s}]")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,lens,hq,hk,causal", [
+    (96, [160, 37], 4, 2, True),            # compiled head dims beside 64 / 128 ...
+    (192, [130, 64], 4, 1, True),
+    (256, [96, 71], 2, 2, True),
+    (256, [200], 4, 2, False),
+    (80, [150, 33], 4, 2, True),            # ... and sizes that run zero-padded to the next one (the reference takes
+    (40, [129], 2, 2, False),               # any d <= 256 and pads to a multiple of 8, flash_atten.cu:284,303-312)
+    (160, [100, 90], 2, 1, True),
+])
+def test_attention_other_head_dims(dtype, d, lens, hq, hk, causal):
+    """16-bit attention for head dims other than 64 / 128, forward and backward against the fp64 oracle, through
+    the Python mirror of the binding and through the compiled extension (same bits)."""
+    from dhellam_amd import _Clib
+    import dhellam._Clib as C
+    cu = _cu(lens)
+    t, m = int(cu[-1]), max(lens)
+    scale = 1.0 / math.sqrt(d)
+    q, k, v, do = (randn((t, h, d), dtype, s) for s, h in ((0, hq), (1, hk), (2, hk), (3, hq)))
+    qg, kg, vg, cug = q.cuda(), k.cuda(), v.cuda(), cu.cuda()
+    res = _Clib.pymha_varlen_fwd(qg, kg, vg, cug, cug, m, m, 0.0, scale, causal, False, 0, False)
+    out, lse = res[0], res[5]
+    assert out.shape == q.shape
+    d_run = res[4].shape[-1]
+    assert d_run in _Clib.HEAD_DIMS_16BIT and d_run >= d and res[1].shape[-1] == d_run      # the "padded" slots
+    oo, lo = OA.attn_fwd(q, k, v, cu, cu, scale, causal, torch.float64)
+    assert_close(out, oo, dtype, "out")
+    for i, n in enumerate(lens):
+        assert_close(lse[i, :, :n], lo[i, :, :n], torch.float32, f"lse[{i}]")
+    if d_run != d:
+        assert torch.count_nonzero(res[4][..., d:]) == 0                                    # padding columns stay zero
+    outc = out.contiguous()
+    sp = torch.cuda.current_stream().cuda_stream
+    dq, dk, dv, _ = _Clib.pymha_varlen_bwd(do.cuda(), qg, kg, vg, outc, lse, cug, cug, m, m, 0.0, scale, causal, None,
+                                           False, 0, False, sp)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    dqo, dko, dvo, _ = OA.attn_bwd(do, q, k, v, outc.cpu(), lse.cpu().double(), cu, cu, scale, causal, torch.float64)
+    assert_close(dq, dqo, dtype, "dq")
+    assert_close(dk, dko, dtype, "dk")
+    assert_close(dv, dvo, dtype, "dv")
+    # the compiled extension pads and runs the same kernels
+    rc = C.pymha_varlen_fwd(qg, kg, vg, cug, cug, m, m, 0.0, scale, causal, False, 0, False)
+    assert torch.equal(rc[0], out) and rc[4].shape[-1] == d_run
+    assert all(torch.equal(rc[5][i, :, :n], lse[i, :, :n]) for i, n in enumerate(lens))   # (entries past a sequence are not written)
+    gc = C.pymha_varlen_bwd(do.cuda(), qg, kg, vg, outc, lse, cug, cug, m, m, 0.0, scale, causal, None, False, 0, False, sp)
+    torch.cuda.synchronize()
+    for a, b_ in zip(gc[:3], (dq, dk, dv)):
+        assert torch.equal(a, b_)
+
+
+def test_attention_head_dim_above_256_is_refused():
+    from dhellam_amd import _Clib
+    q = torch.zeros(8, 1, 264, dtype=torch.bfloat16, device="cuda")
+    cu = _cu([8]).cuda()
+    with pytest.raises(RuntimeError, match="256"):
+        _Clib.pymha_varlen_fwd(q, q, q, cu, cu, 8, 8, 0.0, 1.0, True, False, 0, False)

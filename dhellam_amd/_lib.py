@@ -61,6 +61,7 @@ SIGNATURES = {
     "dh_attn_bwd_min_workspace_bytes": (_sz, [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]),
     "dh_attn_bwd": (_i32, [_vp] * 11 + [_sz] + [_vp] * 2 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _vp]),
     "dh_attn_bwd_set_ds_limit": (None, [_sz]),
+    "dh_attn_bwd_set_ds_when_full": (None, [_i32]),
     "dh_attn_bwd_acc": (_i32, [_vp] * 11 + [_sz] + [_vp] * 2 + [_i32] * 3 + [_i64] * 2 + [_i32] * 3 + [_i64] * 8 + [_f32, _i32, _i32, _i32, _vp]),
     "dh_attn_merge": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
     "dh_moe_route_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),

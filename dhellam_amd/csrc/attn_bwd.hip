@@ -1463,6 +1463,7 @@ constexpr bool dq_takes_4_waves(int d) { return (32 * (d / 8)) % 256 == 0; }
 // kernel is the faster one (32 heads x 4096: 610 against 669 us; 16 heads: 321 against 329), as the extra
 // memory traffic then costs more than the two products saved.  Above the byte limit dS is never kept.
 static std::atomic<size_t> g_ds_limit{(size_t)1280 << 20};
+static std::atomic<int> g_ds_when_full{0};   // 1: keep dS also where the recomputing dQ kernel would fill the chip
 
 // Whether the recomputing dQ kernel would fill the chip (its 128-row form).
 static bool dq_big_grid(int batch, int max_sq, int hq, int causal) {
@@ -1474,7 +1475,7 @@ static bool dq_big_grid(int batch, int max_sq, int hq, int causal) {
 // never keep dS, whatever space there is (other head dims, fp32, a chip-filling recomputing kernel).
 static size_t ds_bytes_wanted(int batch, int max_sq, int64_t max_sk, int hq, int d, int dtype, int causal) {
   if (dtype == DH_F32 || d != 128 || batch <= 0 || max_sq <= 0 || max_sk <= 0) return 0;
-  if (dq_big_grid(batch, max_sq, hq, causal)) return 0;
+  if (dq_big_grid(batch, max_sq, hq, causal) && !g_ds_when_full.load()) return 0;
   // one block more per row than needed: rows a power of two apart would meet on the same memory channels
   const size_t nqt = 2 * (size_t)cdiv(max_sq, 64), nkb = 2 * (size_t)cdiv(max_sk, 64) + 1;
   return (size_t)batch * hq * nqt * nkb * 2048;
@@ -1500,6 +1501,7 @@ static size_t bwd_base_bytes(int64_t total_k, int batch, int max_seqlen_q, int h
 }  // namespace dh
 
 extern "C" void dh_attn_bwd_set_ds_limit(size_t bytes) { dh::g_ds_limit.store(bytes); }
+extern "C" void dh_attn_bwd_set_ds_when_full(int on) { dh::g_ds_when_full.store(on ? 1 : 0); }
 
 extern "C" size_t dh_attn_bwd_min_workspace_bytes(int64_t total_q, int64_t total_k, int batch, int max_seqlen_q, int hq,
                                                   int hk, int d, int dtype) {

@@ -186,6 +186,9 @@ size_t dh_attn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int batch,
  * the workspace was sized.  No counterpart in the reference (flash-attention
  * always recomputes). */
 void dh_attn_bwd_set_ds_limit(size_t bytes);
+/* on != 0: calls large enough to fill the chip with the recomputing dQ kernel
+ * keep dS as well (same limit, same workspace check).  Process-wide. */
+void dh_attn_bwd_set_ds_when_full(int on);
 
 /* dq like q, dk/dv like k/v (GQA groups are reduced inside the kernel; the
  * reference sums an expanded buffer afterwards, flash_atten.cu:646-652).

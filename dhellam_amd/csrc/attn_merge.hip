@@ -28,18 +28,21 @@ struct MergeParams {
 __device__ __forceinline__ float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 __device__ __forceinline__ float log_pos(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
 
-template <typename T, int NS>
+// IDX: the type the item index is taken apart in (three divisions by run-time sizes stand in front of an item's
+// loads: 32-bit ones whenever the item count allows).
+template <typename T, int NS, typename IDX>
 __global__ void __launch_bounds__(256) attn_merge_kernel(const MergeParams p) {
   constexpr int N = Vec<T>::N;
-  const int cpr = p.d / N;  // chunks per (row, head)
-  const int64_t nitems = (int64_t)p.batch * p.sq * p.hq * cpr;
-  for (int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x; it < nitems; it += (int64_t)gridDim.x * 256) {
+  const IDX cpr = (IDX)(p.d / N);  // chunks per (row, head)
+  const IDX nitems = (IDX)p.batch * (IDX)p.sq * (IDX)p.hq * cpr;
+  const IDX hq_ = (IDX)p.hq, sq_ = (IDX)p.sq;
+  for (IDX it = (IDX)blockIdx.x * 256 + threadIdx.x; it < nitems; it += (IDX)gridDim.x * 256) {
     const int ch = (int)(it % cpr);
-    int64_t r = it / cpr;
-    const int h = (int)(r % p.hq);
-    r /= p.hq;
-    const int t = (int)(r % p.sq);
-    const int b = (int)(r / p.sq);
+    IDX r = it / cpr;
+    const int h = (int)(r % hq_);
+    r /= hq_;
+    const int t = (int)(r % sq_);
+    const int b = (int)(r / sq_);
     // every load of the item goes out before any arithmetic: the partial outputs do not depend on the weights
     float ls[NS];
     Vec<T> x[NS];
@@ -108,7 +111,12 @@ extern "C" int dh_attn_merge(const void *const *outs, const float *const *lses, 
   int64_t blocks = cdiv(nitems, 256);
   if (blocks > 256 * 32) blocks = 256 * 32;
   // steps beyond n_steps cover no rows (rows = 0), so a kernel compiled for more steps than given skips them
-#define DH_MERGE(NS) hipLaunchKernelGGL((attn_merge_kernel<T, NS>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p)
+  const bool small = nitems + blocks * 256 < (1ll << 32);
+#define DH_MERGE(NS)                                                                                                   \
+  do {                                                                                                                 \
+    if (small) hipLaunchKernelGGL((attn_merge_kernel<T, NS, uint32_t>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p); \
+    else hipLaunchKernelGGL((attn_merge_kernel<T, NS, int64_t>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, p);        \
+  } while (0)
   DH_DISPATCH_DTYPE(dtype, {
     if (n_steps <= 2) DH_MERGE(2); else if (n_steps <= 4) DH_MERGE(4); else DH_MERGE(8);
   });

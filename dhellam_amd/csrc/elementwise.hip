@@ -38,68 +38,77 @@ __device__ __forceinline__ void swiglu_grad(float y1, float y2, float gg, float 
 #define DH_EW_MAXGRID 65536
 #endif
 
-template <typename T, int UNROLL, bool NT>
+// IDX: the type the item index is computed in.  Splitting an item index into (row, column) is a division by the
+// run-time row length, and it stands in front of a workgroup's first load: in 64 bits it is some forty
+// instructions per vector, in 32 bits (whenever the item count allows) a handful.
+template <typename T, int UNROLL, bool NT, typename IDX>
 __global__ void __launch_bounds__(256)
-swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems, int fv) {
+swiglu_fwd_kernel(const T *__restrict__ y, T *__restrict__ out, int64_t nitems_, int fv_) {
   constexpr int N = Vec<T>::N;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  const int64_t ustride = DH_EW_BLOCKED ? 256 : stride;
-  int64_t it = (int64_t)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
+  const IDX nitems = (IDX)nitems_, fv = (IDX)fv_;
+  const IDX stride = (IDX)gridDim.x * 256;
+  const IDX ustride = DH_EW_BLOCKED ? 256 : stride;
+  IDX it = (IDX)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
   for (; it < nitems; it += stride * UNROLL) {
     Vec<T> a[UNROLL], b[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * ustride;
+      const IDX id = it + u * ustride;
       if (id < nitems) {
-        const int64_t r = id / fv;
+        const IDX r = id / fv;
         const int c = (int)(id - r * fv);
-        const T *row = y + r * (2 * (int64_t)fv * N);
+        const T *row = y + (int64_t)r * (2 * (int64_t)fv * N);
         a[u] = ldg_s<NT>(row + (int64_t)c * N);
         b[u] = ldg_s<NT>(row + ((int64_t)fv + c) * N);
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * ustride;
+      const IDX id = it + u * ustride;
       if (id < nitems) {
         Vec<T> o;
 #pragma unroll
         for (int j = 0; j < N; ++j) {
           o.v[j] = from_f<T>(swiglu_value(to_f(a[u].v[j]), to_f(b[u].v[j])));
         }
-        stg_s<NT>(out + id * N, o);
+        stg_s<NT>(out + (int64_t)id * N, o);
       }
     }
   }
 }
 
-template <typename T, int UNROLL, bool NT>
+template <typename T, int UNROLL, bool NT, typename IDX>
 __global__ void __launch_bounds__(256)
-swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, int64_t nitems, int fv) {
+swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restrict__ dy, int64_t nitems_, int fv_) {
   constexpr int N = Vec<T>::N;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  const int64_t ustride = DH_EW_BLOCKED ? 256 : stride;
-  int64_t it = (int64_t)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
+  const IDX nitems = (IDX)nitems_, fv = (IDX)fv_;
+  const IDX stride = (IDX)gridDim.x * 256;
+  const IDX ustride = DH_EW_BLOCKED ? 256 : stride;
+  IDX it = (IDX)blockIdx.x * (DH_EW_BLOCKED ? 256 * UNROLL : 256) + threadIdx.x;
   for (; it < nitems; it += stride * UNROLL) {
     Vec<T> a[UNROLL], b[UNROLL], gv[UNROLL];
+    IDX rr[UNROLL];
+    int cc[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * ustride;
+      const IDX id = it + u * ustride;
       if (id < nitems) {
-        const int64_t r = id / fv;
+        const IDX r = id / fv;
         const int c = (int)(id - r * fv);
-        const T *row = y + r * (2 * (int64_t)fv * N);
+        rr[u] = r;
+        cc[u] = c;
+        const T *row = y + (int64_t)r * (2 * (int64_t)fv * N);
         a[u] = ldg_s<NT>(row + (int64_t)c * N);
         b[u] = ldg_s<NT>(row + ((int64_t)fv + c) * N);
-        gv[u] = ldg_s<NT>(g + id * N);
+        gv[u] = ldg_s<NT>(g + (int64_t)id * N);
       }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int64_t id = it + u * ustride;
+      const IDX id = it + u * ustride;
       if (id < nitems) {
-        const int64_t r = id / fv;
-        const int c = (int)(id - r * fv);
+        const IDX r = rr[u];
+        const int c = cc[u];
         Vec<T> d1, d2;
 #pragma unroll
         for (int j = 0; j < N; ++j) {
@@ -108,7 +117,7 @@ swiglu_bwd_kernel(const T *__restrict__ g, const T *__restrict__ y, T *__restric
           d1.v[j] = from_f<T>(v1);
           d2.v[j] = from_f<T>(v2);
         }
-        T *row = dy + r * (2 * (int64_t)fv * N);
+        T *row = dy + (int64_t)r * (2 * (int64_t)fv * N);
         stg_s<NT>(row + (int64_t)c * N, d1);
         stg_s<NT>(row + ((int64_t)fv + c) * N, d2);
       }
@@ -350,21 +359,39 @@ static int launch_ew(const void *x, const void *bias, const void *res, const voi
 }
 
 // nitems 16-byte output vectors; the forward touches 3 of them per item, the backward 5.
-template <typename T>
-static void launch_swiglu_fwd(const T *y, T *out, int64_t nitems, int fv, hipStream_t st) {
-  const dim3 grid(stream_grid(nitems, 4));
-  if (stream_hint(3 * 16 * nitems))
-    hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4, true>), grid, dim3(256), 0, st, y, out, nitems, fv);
-  else
-    hipLaunchKernelGGL((swiglu_fwd_kernel<T, 4, false>), grid, dim3(256), 0, st, y, out, nitems, fv);
+// Vectors in flight per lane: measured on [rows, 2 x 3584] bf16 (forward, us at 512 / 4096 / 16384 / 65536 rows):
+// one 3.6 / 15.5 / 54.8 / 231, two 3.7 / 16.4 / 56.3 / 222, four 4.2 / 18.5 / 61.4 / 234.  Below a few hundred MB
+// more, smaller workgroups win (the whole tensor is in flight at once and what counts is how soon the first loads
+// go out); beyond that two vectors per lane do.
+template <typename T, int U>
+static void launch_swiglu_fwd_u(const T *y, T *out, int64_t nitems, int fv, hipStream_t st) {
+  const dim3 grid(stream_grid(nitems, U));
+  // 32-bit item arithmetic while an index one trip past the end still fits
+  const bool small = nitems + (int64_t)grid.x * 256 * U < (1ll << 32);
+#define L(NT, IDX) hipLaunchKernelGGL((swiglu_fwd_kernel<T, U, NT, IDX>), grid, dim3(256), 0, st, y, out, nitems, fv)
+  if (stream_hint(3 * 16 * nitems)) { if (small) L(true, uint32_t); else L(true, int64_t); }
+  else { if (small) L(false, uint32_t); else L(false, int64_t); }
+#undef L
 }
 template <typename T>
+static void launch_swiglu_fwd(const T *y, T *out, int64_t nitems, int fv, hipStream_t st) {
+  if (3 * 16 * nitems <= (512ll << 20)) launch_swiglu_fwd_u<T, 1>(y, out, nitems, fv, st);
+  else launch_swiglu_fwd_u<T, 2>(y, out, nitems, fv, st);
+}
+template <typename T, int U>
+static void launch_swiglu_bwd_u(const T *g, const T *y, T *dy, int64_t nitems, int fv, hipStream_t st) {
+  const dim3 grid(stream_grid(nitems, U));
+  const bool small = nitems + (int64_t)grid.x * 256 * U < (1ll << 32);
+#define L(NT, IDX) hipLaunchKernelGGL((swiglu_bwd_kernel<T, U, NT, IDX>), grid, dim3(256), 0, st, g, y, dy, nitems, fv)
+  if (stream_hint(5 * 16 * nitems)) { if (small) L(true, uint32_t); else L(true, int64_t); }
+  else { if (small) L(false, uint32_t); else L(false, int64_t); }
+#undef L
+}
+// (backward, same shapes: one vector per lane 4.4 / 22.8 / 91.3 / 390 us, two 4.9 / 23.5 / 92.8 / 381)
+template <typename T>
 static void launch_swiglu_bwd(const T *g, const T *y, T *dy, int64_t nitems, int fv, hipStream_t st) {
-  const dim3 grid(stream_grid(nitems, 2));
-  if (stream_hint(5 * 16 * nitems))
-    hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2, true>), grid, dim3(256), 0, st, g, y, dy, nitems, fv);
-  else
-    hipLaunchKernelGGL((swiglu_bwd_kernel<T, 2, false>), grid, dim3(256), 0, st, g, y, dy, nitems, fv);
+  if (5 * 16 * nitems <= (768ll << 20)) launch_swiglu_bwd_u<T, 1>(g, y, dy, nitems, fv, st);
+  else launch_swiglu_bwd_u<T, 2>(g, y, dy, nitems, fv, st);
 }
 
 }  // namespace dh

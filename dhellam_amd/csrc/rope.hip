@@ -116,6 +116,8 @@ extern "C" int dh_rope(const void *q, const void *k, void *q_out, void *k_out, c
   const int heads = hq + hk;
   // Split the heads over several lanes while the grid is too small to fill the chip.
   int hsplit = 1;
+  // (splitting further costs more than it gives: every lane of a split evaluates the chunk's cos / sin again;
+  // 4096 tokens x 9 heads: 5.8 us with this bound, 6.9 / 7.6 us with twice / four times as many lanes)
   while (hsplit < heads && tokens * chunks * hsplit < 256ll * 256 * 2) ++hsplit;
   const int64_t nitems = tokens * hsplit * chunks;
   int64_t blocks = cdiv(nitems, 256);

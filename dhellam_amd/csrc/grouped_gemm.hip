@@ -567,6 +567,272 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGPar
   }
 }
 
+// ---- 256x256 tiles with ONE wavefront per SIMD: four wavefronts of 128x128 outputs ------------------------------
+// The 256 accumulator registers of a wavefront live in AGPRs, and the loop is written slot by slot: after every
+// MFMA exactly one LDS or memory instruction (fragment read, staging-register write to LDS, buffer load), so that
+// the matrix pipe never waits for a burst of them and the LDS queue never fills.  A 64-deep k slice is loaded
+// into registers THREE slices ahead (two staging sets of 16 x 16 bytes per lane), written to the LDS stage that
+// is not being read during the first half of a slice, published by the slice's one barrier and read as fragments
+// one k step (16) ahead of the MFMAs that use them.  Against the eight-wavefront kernel above: a third fewer
+// fragment reads per MFMA, MFMAs of one wavefront back to back instead of two wavefronts alternating on the pipe.
+//
+// The loads are buffer loads issued from assembly: the compiler does not count them, every use of a staging
+// register is ordered by a hand-written s_waitcnt vmcnt (loads return in order), and between its load and its
+// LDS write a staging register is touched by nothing else.  The buffer descriptors do the edge handling: one per
+// 32-row block of a tile, its length cut at the group's (or n's) last row, so that rows past the end read as
+// zero and no access leaves the operands, whatever the offsets table says.
+typedef int gg_i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ gg_i32x4 gg_rsrc(const void *ptr, int64_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)ptr;
+  const uint32_t nb = bytes <= 0 ? 0u : (bytes > 0x7fffffffll ? 0x7fffffffu : (uint32_t)bytes);
+  gg_i32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu));   // stride 0: raw buffer
+  r[2] = __builtin_amdgcn_readfirstlane((int)nb);
+  r[3] = 0x00020000;
+  return r;
+}
+
+template <typename T, bool BKS>
+__global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) {
+  using M = Mma<T>;
+  using Frag = typename M::Frag;
+  constexpr int BM = 256, ROWB = 128, BROWB = 512, TILEB = 256 * ROWB, STAGEB = 2 * TILEB;
+  constexpr int NRD = BKS ? 12 : 8;                     // LDS read instructions per k step
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
+
+  const int ntiles = p.tiles_m * p.tiles_n;
+  int pid = blockIdx.x;
+  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  int tm = pid % p.tiles_m;
+  const int tn = pid / p.tiles_m;
+  const int base = p.offs[0];
+  int g = 0, row_begin = 0, row_end = 0;
+  {
+    bool found = false;
+    for (int gi = 0; gi < p.groups; ++gi) {
+      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
+      const int t = (re - rb + BM - 1) / BM;
+      if (!found && tm < t) {
+        g = gi; row_begin = rb; row_end = re; found = true;
+      } else if (!found) {
+        tm -= t;
+      }
+    }
+    if (!found) return;
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, hh = lane >> 5;
+  const int wm = w >> 1, wn = w & 1;
+  const int n0 = tn * 256, m0 = row_begin + tm * BM;
+  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
+  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
+  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+  const int nsl = (int)(p.k_dim / 64);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const uint32_t lda_b = (uint32_t)p.lda * (uint32_t)sizeof(T), ldb_b = (uint32_t)p.ldb * (uint32_t)sizeof(T);
+
+  // ---- copies ----------------------------------------------------------------------------------------------
+  // k-contiguous tile [256 rows][64 k]: a lane copies chunk lc of rows lr + 32 i; descriptor i starts at row 32 i.
+  // k-strided tile [64 k][256 n]: a lane copies chunk cx of k rows kr + 8 i; descriptor i starts at k row 8 i.
+  const int lc = tid & 7, lr = tid >> 3, cx = tid & 31, kr = tid >> 5;
+  gg_i32x4 rsa[8], rsb[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    rsa[i] = gg_rsrc(ag + (int64_t)(32 * i) * p.lda, (int64_t)(a_rext - 32 * i) * lda_b);
+    if (BKS) rsb[i] = gg_rsrc(bg + (int64_t)(8 * i) * p.ldb, 0x7fffffffll);
+    else rsb[i] = gg_rsrc(bg + (int64_t)(32 * i) * p.ldb, (int64_t)(b_rext - 32 * i) * ldb_b);
+  }
+  const uint32_t goff_a = (uint32_t)lr * lda_b + (uint32_t)(lc * 16);
+  const uint32_t goff_b = BKS ? (uint32_t)kr * ldb_b + (uint32_t)(cx * 16) : (uint32_t)lr * ldb_b + (uint32_t)(lc * 16);
+  const uint32_t kstep_a = 64 * (uint32_t)sizeof(T);                          // bytes from one k slice to the next
+  const uint32_t kstep_b = BKS ? 64 * ldb_b : 64 * (uint32_t)sizeof(T);
+  const uint32_t wr_a = (uint32_t)(lr * ROWB + ((lc ^ ((lr >> 1) & 7)) << 4));                      // + i * 4096
+  // k-strided tile: chunk XOR 4 (k % 4) + (k / 4) % 4 with k = kr + 8 i: the i part is bit 1 of the chunk for odd i
+  const uint32_t wr_b = BKS ? (uint32_t)(TILEB + kr * BROWB + (cx >> 4) * 256 + (((cx & 15) ^ (4 * (kr & 3) + (kr >> 2))) << 4))
+                            : (uint32_t)TILEB + wr_a;
+
+  // ---- fragment reads --------------------------------------------------------------------------------------
+  const uint32_t sw = (uint32_t)((hh ^ ((c >> 1) & 7)) << 4);
+  const uint32_t fa_lane = (uint32_t)((wm * 128 + c) * ROWB) + sw;                  // k step: XOR 32 ks; block i: + 4096 i
+  const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 128 + c) * ROWB) + sw;
+  const int r16 = lane & 15;
+  const int t_lc = 2 * ((lane >> 4) & 1) + ((r16 & 3) >> 1);
+  const int tx = 4 * (r16 >> 2) + 2 * hh;
+  const uint32_t t_row = (uint32_t)(TILEB + wn * 256 + (8 * hh + (r16 >> 2)) * BROWB + ((r16 & 3) & 1) * 8);
+  const uint32_t tb_a = t_row + (uint32_t)((t_lc ^ tx) << 4);                       // k rows 8 hh + 0..3 of a step
+  const uint32_t tb_b = t_row + 4 * BROWB + (uint32_t)((t_lc ^ (tx + 1)) << 4);     // k rows 8 hh + 4..7
+  typedef __attribute__((address_space(3))) const Frag *lds_frag;
+  typedef short4v __attribute__((address_space(3))) *lds_tr;
+  typedef __attribute__((address_space(3))) gg_i32x4 *lds_w;
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  gg_i32x4 stg[2][16];
+  Frag fa[2][4];
+  Frag fbr[2][4];                                       // B fragments, k-contiguous form
+  short4v fbt[2][4][2];                                 // k-strided form: the two transpose reads of a fragment
+
+  auto gload = [&](int set, int idx, uint32_t ka, uint32_t kb) {   // idx 0..7: A, 8..15: B; ka, kb: byte offsets of the slice
+    if (idx < 8) asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_a), "s"(rsa[idx]), "s"(ka) : "memory");
+    else asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_b), "s"(rsb[idx - 8]), "s"(kb) : "memory");
+  };
+  auto swrite = [&](int set, int idx, uint32_t stage) {  // stage: LDS byte address of the stage
+    if (idx < 8) *(lds_w)(stage + wr_a + idx * 4096) = stg[set][idx];
+    else if (!BKS) *(lds_w)(stage + wr_b + (idx - 8) * 4096) = stg[set][idx];
+    else *(lds_w)(((stage + wr_b) ^ (uint32_t)(((idx - 8) & 1) << 5)) + (idx - 8) * 4096) = stg[set][idx];
+  };
+  // read r of a k step, in the order in which the MFMAs first need the data: B0 A0 B1 B2 B3 A1 A2 A3 (a k-strided
+  // B fragment is two transpose reads).  abase/bbase: lane addresses of the stage with the k step applied.
+  auto fread = [&](int set, int r, uint32_t stage, int ks) {
+    if constexpr (!BKS) {
+      constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
+      if (!isb[r]) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      else fbr[set][blk[r]] = *(lds_frag)(((stage + fb_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+    } else {
+      constexpr int kind[12] = {1, 2, 0, 1, 2, 1, 2, 1, 2, 0, 0, 0}, blk[12] = {0, 0, 0, 1, 1, 2, 2, 3, 3, 1, 2, 3};
+      if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      else if (kind[r] == 1)
+        fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + tb_a) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+      else
+        fbt[set][blk[r]][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + tb_b) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+    }
+  };
+
+  // prologue: slice 0 into stage 0 (through set 0), slice 1 into set 1, slice 2 into set 0.  Loads of slices that
+  // do not exist repeat the last slice (their data is written to a stage nobody reads).
+  const int last = nsl > 0 ? nsl - 1 : 0;
+  auto kof = [&](int s) { return (uint32_t)(s < last ? s : last); };
+#pragma unroll
+  for (int x = 0; x < 16; ++x) gload(0, x, 0, 0);
+#pragma unroll
+  for (int x = 0; x < 16; ++x) gload(1, x, kof(1) * kstep_a, kof(1) * kstep_b);
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+#pragma unroll
+  for (int x = 0; x < 16; ++x) swrite(0, x, lds0);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // issue order of a staging set inside the loop: 0..7, 15, 8..14
+#pragma unroll
+  for (int x = 0; x < 8; ++x) gload(0, x, kof(2) * kstep_a, kof(2) * kstep_b);
+  gload(0, 15, kof(2) * kstep_a, kof(2) * kstep_b);
+#pragma unroll
+  for (int x = 8; x < 15; ++x) gload(0, x, kof(2) * kstep_a, kof(2) * kstep_b);
+  asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+  for (int x = 0; x < NRD; ++x) fread(0, x, lds0, 0);
+
+  // Slice s reads stage s % 2, writes slice s + 1 (staging set (s + 1) % 2, loaded two slices ago) into the other
+  // stage during its first half and then loads slice s + 3 into the same set.
+  int st = 0;
+  auto slice = [&](auto xc, auto lastc, int s) {
+    constexpr int X = decltype(xc)::value;              // s % 2
+    constexpr bool LAST = decltype(lastc)::value;       // the last slice of an odd count: nothing to prepare
+    uint32_t cur = lds0 + (uint32_t)(st * STAGEB), nxt = lds0 + (uint32_t)((st ^ 1) * STAGEB);
+    const uint32_t ka = kof(s + 3) * kstep_a, kb = kof(s + 3) * kstep_b;
+    asm volatile("" : "+s"(cur), "+s"(nxt));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mi = 0; mi < 64; ++mi) {
+      const int ks = mi >> 4, i = (mi >> 2) & 3, j = mi & 3, q = mi & 15;
+      if constexpr (BKS) acc[i][j] = M::mma(frag_join<T>(fbt[ks & 1][j][0], fbt[ks & 1][j][1]), fa[ks & 1][i], acc[i][j]);
+      else acc[i][j] = M::mma(fbr[ks & 1][j], fa[ks & 1][i], acc[i][j]);
+      // fragment reads of the next k step, spread over the quarter (the last quarter: behind the barrier, from the next stage)
+      if (ks < 3) {
+        if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, cur, ks + 1); }
+        else { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1); }
+      } else if (!LAST) {
+        if (mi == 50) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (NRD == 8) {
+          if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, nxt, 0);
+          if (mi == 63) fread(0, 7, nxt, 0);
+        } else {
+          if (mi >= 50 && mi < 62) fread(0, mi - 50, nxt, 0);
+        }
+      }
+      if (!LAST && mi < 32 && mi % 2 == 1) {            // LDS writes of slice s + 1: the older of the two sets in flight
+        const int k = mi / 2;
+        if (k == 0) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+        if (k == 8) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        swrite(X ^ 1, k, nxt);
+      }
+      if (!LAST && mi >= 33 && mi <= 61 && mi % 2 == 1) gload(X ^ 1, (mi - 33) / 2, ka, kb);
+      if (!LAST && mi == 48) gload(X ^ 1, 15, ka, kb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    st ^= 1;
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  int s = 0;
+#pragma unroll 1
+  for (; s + 1 < nsl; s += 2) {
+    slice(I0{}, std::false_type{}, s);
+    slice(I1{}, std::false_type{}, s + 1);
+  }
+  // The loads of the last slices (unused data) still target the staging registers: wait for them, and keep the
+  // registers reserved until then (for the compiler a load whose result nobody reads frees its register at once).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int x = 0; x < 16; ++x) asm volatile("" ::"v"(stg[0][x]), "v"(stg[1][x]));
+  if (s < nsl) slice(I0{}, std::true_type{}, s);
+  __syncthreads();                                      // everyone is done with the stages: they stage the output below
+
+  // Epilogue: each wavefront passes its 128x128 block through a private LDS region, 64 rows at a time, and stores
+  // whole 256-byte row segments (16 lanes a row, 4 rows per instruction).  Rows of 264 bytes: the 8-byte writes of
+  // 32 lanes (32 rows, one column) fall on different banks.
+  constexpr int EP = 264;
+  static_assert(4 * 64 * EP <= 2 * STAGEB, "epilogue staging fits in the stage buffers");
+  unsigned char *ep = smem + w * (64 * EP);
+  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 128;
+  struct alignas(8) Q4 { T v[4]; };
+  const int er = lane >> 4, ec = lane & 15;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int i2 = 0; i2 < 2; ++i2)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const floatx16 av = acc[2 * h + i2][j];
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          Q4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
+          *reinterpret_cast<Q4 *>(ep + (32 * i2 + c) * EP + (32 * j + 8 * vb + 4 * hh) * (int)sizeof(T)) = o;
+        }
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const int mh = wm * 128 + 64 * h;                   // first row of this half in the tile
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int r = 4 * it + er;
+      const dh_u32x4 o = *reinterpret_cast<const dh_u32x4 *>(ep + r * EP + ec * 16);
+      if (mh + r < a_rext && wn * 128 + 8 * ec < b_rext)
+        *reinterpret_cast<dh_u32x4 *>(cg + (int64_t)(mh + r) * p.ldc + 8 * ec) = o;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <typename T, bool BKS>
+static int launch_gg_w4(GGParams p, int64_t m_extent, hipStream_t st) {
+  p.tiles_n = (int)cdiv(p.n_dim, 256);
+  p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
+  if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
+  hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
+  return DH_OK;
+}
+
 template <typename T, int WVN, int BKT, int NST, bool BKS>
 static int launch_gg_dma(GGParams p, int64_t m_extent, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
@@ -649,7 +915,10 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
-  if (big && k % 64 == 0 && k < (1ll << 30))
+  if (big && k % 64 == 0 && k <= (1ll << 21))
+    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, false>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_w4<f16_t, false>(p, max_rows, (hipStream_t)stream);
+  else if (big && k % 64 == 0 && k < (1ll << 30))
     rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream)
                           : launch_gg_dma<f16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream);
   else
@@ -673,7 +942,10 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
-  if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
+  if (big && k % 64 == 0 && n % 256 == 0 && k <= (1ll << 21) && k * n * (int64_t)dtype_size(dtype) < (1ll << 31))
+    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, true>(p, max_rows, (hipStream_t)stream)
+                          : launch_gg_w4<f16_t, true>(p, max_rows, (hipStream_t)stream);
+  else if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
     rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream)
                           : launch_gg_dma<f16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream);
   else

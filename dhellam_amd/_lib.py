@@ -72,8 +72,9 @@ SIGNATURES = {
     "dh_moe_gather_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
     "dh_moe_scatter_rows": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
     "dh_moe_gate_grad": (_i32, [_vp] * 5 + [_i32, _i32, _i64, _i32, _i64, _i32, _vp]),
-    "dh_grouped_gemm_nt": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp]),
-    "dh_grouped_gemm_nn": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp]),
+    "dh_grouped_gemm_workspace_bytes": (_sz, []),
+    "dh_grouped_gemm_nt": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp, _sz, _vp]),
+    "dh_grouped_gemm_nn": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _vp, _sz, _vp]),
     "dh_grouped_gemm_tn": (_i32, [_vp] * 4 + [_i32, _i64, _i64, _i64, _i32, _i32, _vp]),
 }
 

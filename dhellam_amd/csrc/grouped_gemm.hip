@@ -6,12 +6,11 @@
 //   NT  c[r, n]  = sum_k a[r, k] * w[g][n, k]      forward  (both k-contiguous)
 //   NN  c[r, n]  = sum_k a[r, k] * w[g][k, n]      dgrad    (w strided in k)
 //   TN  c[g][m,n] = sum_r a[r, m] * b[r, n]        wgrad    (both strided in k = r)
-// A workgroup is 2 x WVN wavefronts, each owning a (32*WM) x (32*WN) output block
-// kept in accumulators (256x256 tiles: 2x4 wavefronts of 128x64, two wavefronts per
-// SIMD, so that one wavefront's loads, LDS stores and barrier waits overlap the other's
-// MFMAs; with one wavefront per SIMD those phases simply added up); 64-deep k slices of
-// both operands are staged in LDS
-// (two stages, one barrier per slice).  k-contiguous operands are read from LDS
+// Two kernels.  grouped_gemm_w4_kernel (NT and NN at sizes that fill the chip): 256x256 tiles, four
+// wavefronts of 128x128 with hand-placed copies, optionally one workgroup per compute unit that takes
+// whole tiles in rounds and a k piece of a tile of the last round.  grouped_gemm_kernel (everything else, and TN): a workgroup is 2 x WVN wavefronts, each
+// owning a (32*WM) x (32*WN) output block kept in accumulators; 64-deep k slices of both operands are
+// staged in LDS through registers (two stages, one barrier per slice).  k-contiguous operands are read from LDS
 // as 16-byte row fragments; k-strided operands stay row-major in LDS and are
 // read with transpose loads, so no operand is ever transposed in memory.
 // The product is formed as C^T (weights in the MFMA A slot) so that each lane
@@ -19,18 +18,6 @@
 // Group row ranges are read on the device from the offsets table.
 #include "mma.h"
 #include <atomic>
-#ifndef DH_GG_WVN
-#define DH_GG_WVN 4
-#endif
-#ifndef DH_GG_CPI
-#define DH_GG_CPI 2
-#endif
-#ifndef DH_GG_BKT
-#define DH_GG_BKT 64
-#endif
-#ifndef DH_GG_NST
-#define DH_GG_NST 2
-#endif
 
 namespace dh {
 
@@ -50,6 +37,7 @@ struct GGParams {
   int tiles_m, tiles_n;  // grid extents (tiles_m is an upper bound for NT/NN)
   int accumulate;
   int max_rows;          // rows the stacked operands hold: group ranges read from offs are cut off there
+  float *ws;             // split last round: fp32 partial tiles, one per workgroup
 };
 
 // A group's row range as the kernels use it: relative to the first group and never past the rows the caller's
@@ -274,313 +262,25 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
   }
 }
 
-// ---- NT with direct global->LDS copies --------------------------------------------------------------
-// The forward product at 256x256 tiles when K is a multiple of 64.  The register-staged kernel above
-// runs its phases one after the other (wait for the global loads, store them to LDS, barrier, MFMAs):
-// switching off one phase at a time showed their times simply add up.  Here the next k slice goes
-// global -> LDS by assembly copies issued between the MFMAs of the current slice (no staging registers,
-// no LDS stores, the wavefront never waits for its own loads before the end of the slice).
-// Tiles are [256 rows][64 k] with unpadded 128-byte rows; the 16-byte chunk index is XORed with
-// (row / 2) % 8, applied on the global side of the copy, which makes the 16-byte row-fragment reads
-// conflict-free.  8 wavefronts = 2 (m) x 4 (n), 128x64 outputs each; wavefronts 0-3 copy the A tile
-// (64 rows each), wavefronts 4-7 the B tile.
-// WVN = 4: 8 wavefronts of 128x64 (two per SIMD, accumulators in VGPRs).
-// BKT: k depth of a slice (64 or 32); NST: LDS stages.  The copies of slice s + NST - 1 are issued during
-// slice s, so with NST > 2 a copy has more than a whole slice to land before anyone waits for it (with two
-// stages the copies issued late in a slice are waited for almost at once: their latency is exposed).
-// BKS: the B operand is k-strided ([k][n] row-major, the NN product).  Its tile is then [64 k][256 n] with
-// 512-byte rows, copied two k rows per block with the transpose-read swizzle (chunk ^= 4 * (k % 4) +
-// (k / 4) % 4 inside each 256-byte half row), and its fragments come from LDS transpose reads.
-template <bool B> struct BoolC { static constexpr bool value = B; };
-
-template <typename T, int WVN, int BKT, int NST, bool BKS>
-__global__ void __launch_bounds__(128 * WVN) grouped_gemm_dma_kernel(const GGParams p) {
-  using M = Mma<T>;
-  using Frag = typename M::Frag;
-  constexpr int BM = 256, BN = 256, WM = 4, WN = 8 / WVN, NW = 2 * WVN;
-  static_assert(WVN == 4, "eight wavefronts of 128x64");
-  static_assert(!BKS || BKT == 64, "the k-strided B tile is 64 k rows of 512 bytes");
-  constexpr int BROWB = 256 * (int)sizeof(T);           // bytes of a row of the k-strided B tile
-  constexpr int ROWB = BKT * (int)sizeof(T);            // bytes of a tile row (128 or 64)
-  constexpr int CHUNKS = ROWB / 16;                     // 16-byte chunks per row
-  constexpr int RP = 256 / ROWB;                        // rows per 256 bytes: the swizzle is (row / RP) % CHUNKS
-  constexpr int RPB = 1024 / ROWB;                      // rows per 1 KB copy block
-  constexpr int CPB = 2 * 256 / RPB / NW;               // copy blocks per wavefront and slice
-  constexpr int KS = BKT / 16;                          // MFMA k steps per slice
-  constexpr int DIST = NST - 1;                         // copies run this many slices ahead
-  // With four stages a slice is published one slice BEFORE it is used, so its first fragments are
-  // requested before the barrier that ends the previous slice (no LDS latency at the start of a slice).
-  constexpr bool CROSS = NST >= 4;
-  constexpr int WAITD = CROSS ? 2 : 1;                  // the barrier at the end of slice s publishes slice s + WAITD
-  static_assert(!CROSS || KS % 2 == 0, "fragment sets alternate across slices");
-  constexpr int TILEB = 256 * ROWB;                     // one operand tile
-  constexpr int STAGEB = 2 * TILEB;                     // A tile, then B tile
-  static_assert(NST * STAGEB <= 160 * 1024 && (DIST - 1) * CPB < 64, "LDS budget / wait counter range");
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[NST * STAGEB];
-
-  // A contiguous run of tiles per XCD, m fastest (tiles that share a weight panel run together).
-  // Cutting the grid into 4 x 8 super-tiles per XCD instead lowers the L2 miss traffic by a third
-  // (measured) but is slower: the bound is not the fabric.  Running every full tile first and the groups'
-  // cheap last tiles afterwards (long jobs first) is slower too, by 10 %: a last tile then re-reads from HBM
-  // the weight panel that its group's full tiles shared through L2 long before.
-  const int ntiles = p.tiles_m * p.tiles_n;
-  int pid = blockIdx.x;
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-  int tm = pid % p.tiles_m;
-  const int tn = pid / p.tiles_m;
-  const int base = p.offs[0];
-  int g = 0, row_begin = 0, row_end = 0;
-  {
-    bool found = false;
-    for (int gi = 0; gi < p.groups; ++gi) {
-      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
-      const int t = (re - rb + BM - 1) / BM;
-      if (!found && tm < t) {
-        g = gi; row_begin = rb; row_end = re; found = true;
-      } else if (!found) {
-        tm -= t;
-      }
-    }
-    if (!found) return;
-  }
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int c = lane & 31, hh = lane >> 5;
-  const int wm = w / WVN, wn = w % WVN;   // 2 x WVN wavefronts
-  const int n0 = tn * BN, m0 = row_begin + tm * BM;
-  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
-  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
-  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
-  const int nslices = (int)(p.k_dim / BKT);
-  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-
-  // ---- copies ------------------------------------------------------------------------------------
-  const int cp_b = w / (NW / 2);                        // 0: A tile, 1: B tile
-  const bool cp_ks = BKS && cp_b;                       // this wavefront copies rows of the k-strided tile
-  const int cp_row0 = cp_ks ? (64 / (NW / 2)) * (w % (NW / 2)) : RPB * CPB * (w % (NW / 2));
-  const int cp_ld = (int)(cp_b ? p.ldb : p.lda);
-  const int cp_ext = cp_ks ? 64 : (cp_b ? b_rext : a_rext);   // valid rows of the tile
-  const T *cp_t = cp_b ? bg : ag;
-  const char *cp_g = reinterpret_cast<const char *>(cp_t + (int64_t)cp_row0 * cp_ld);
-  const uint32_t cp_dst0 = (uint32_t)(cp_b * TILEB + cp_row0 * (cp_ks ? BROWB : ROWB));
-  const uint32_t cp_step = (uint32_t)((cp_ks ? 2 : RPB) * cp_ld) * (uint32_t)sizeof(T);
-  const int64_t cp_slice = cp_ks ? (int64_t)64 * cp_ld * (int)sizeof(T) : (int64_t)ROWB;   // bytes from one k slice to the next
-  const bool cp_fast = cp_ks || cp_row0 + RPB * CPB <= cp_ext;   // every row this wavefront copies exists
-  const int lr = cp_ks ? lane >> 5 : lane / CHUNKS, lc = cp_ks ? lane & 15 : lane % CHUNKS;
-  // row-fragment tiles: block i has swizzle (row / RP) % CHUNKS = (RPB / RP * (i % 2) + lr / RP) % CHUNKS (two values).
-  // k-strided tile: block i holds k rows 2 i + lr, swizzle 4 * ((2 i + lr) % 4) + (i / 2) % 4, i.e. the lane part
-  // lc ^ (4 lr) XOR the block constant ((i & 1) << 3) | ((i >> 1) & 3).
-  uint32_t cp_off[2];
-#pragma unroll
-  for (int x = 0; x < 2; ++x)
-    cp_off[x] = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)((lc ^ ((RPB / RP * x + lr / RP) % CHUNKS)) << 4);
-  const uint32_t ks_base = (uint32_t)(lr * cp_ld) * (uint32_t)sizeof(T) + (uint32_t)(((lane >> 4) & 1) * 256);
-  const uint32_t ks_chunk = (uint32_t)(lc ^ (4 * lr));
-  auto block_off = [&](int i) -> uint32_t {
-    if (cp_ks) return ks_base + ((ks_chunk ^ (uint32_t)(((i & 1) << 3) | ((i >> 1) & 3))) << 4);
-    return cp_off[i & 1];
-  };
-  // general form (tiles at the edge of a group or of n): rows past the end re-read the last valid row
-  auto copy_general = [&](uint32_t stage, int slice) {
-#pragma unroll 1
-    for (int i = 0; i < CPB; ++i) {
-      const T *src;
-      if (cp_ks) {
-        const int row = cp_row0 + 2 * i + lr;
-        const int f = 4 * (row & 3) + ((row >> 2) & 3);
-        src = cp_t + ((int64_t)slice * 64 + row) * cp_ld + ((lane >> 4) & 1) * 128 + ((lc ^ f) * 8);
-      } else {
-        int row = cp_row0 + RPB * i + lr;
-        const int f = (row / RP) % CHUNKS;
-        row = row < cp_ext ? row : cp_ext - 1;
-        src = cp_t + (int64_t)row * cp_ld + (int64_t)slice * BKT + ((lc ^ f) * 8);
-      }
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                       (__attribute__((address_space(3))) void *)(smem + stage + cp_dst0 + i * 1024), 16, 0, 0);
-    }
-  };
-  // ---- fragment reads: byte offsets inside a stage; other k steps by XOR, other 32-row blocks by + 32 rows ----
-  const uint32_t sw = (uint32_t)((hh ^ ((c / RP) % CHUNKS)) << 4);
-  const uint32_t fa_lane = (uint32_t)((wm * 32 * WM + c) * ROWB) + sw;            // A tile rows (m)
-  const uint32_t fb_lane = (uint32_t)(TILEB + (wn * 32 * WN + c) * ROWB) + sw;    // B tile rows (n)
-  // k-strided B tile: transpose reads.  A read with the lane address &tile[k0 + r / 4][n0 + 4 * (r % 4)]
-  // (r = lane % 16) returns tile[k0 + 0..3][n0 + r] to the lane, so the fragment's k values 8 hh + 0..3 come
-  // from a read at k0 = 8 hh and 8 hh + 4..7 from one at k0 = 8 hh + 4: the natural k order, matching the
-  // row fragments of A.  t_lc: 16-byte chunk inside the 64-byte run of the 32-column block.
-  const int r16 = lane & 15;
-  const int t_lc = 2 * ((lane >> 4) & 1) + ((r16 & 3) >> 1);
-  const int tx = 4 * (r16 >> 2) + 2 * hh;              // swizzle of k row 8 hh + r / 4; the row 4 further down has tx + 1
-  const uint32_t t_row = (uint32_t)(TILEB + (8 * hh + (r16 >> 2)) * BROWB + ((r16 & 3) & 1) * 8);
-  const uint32_t tb_a = t_row + (uint32_t)((t_lc ^ tx) << 4);
-  const uint32_t tb_b = t_row + 4 * BROWB + (uint32_t)((t_lc ^ (tx + 1)) << 4);
-  typedef __attribute__((address_space(3))) const Frag *lds_frag;
-  typedef short4v __attribute__((address_space(3))) *lds_tr;
-  // B fragment j of k step ks in the stage at byte offset `stage` (BKS form): the k step is an immediate offset
-  auto ld_b_tr = [&](uint32_t stage, int ks, int j) -> Frag {
-    const int nb = wn * WN + j;                         // 32-column block of the tile
-    const uint32_t o = stage + (uint32_t)((nb >> 2) * 256);
-    const uint32_t a0 = (tb_a ^ (uint32_t)((nb & 3) << 6)) + o, a1 = (tb_b ^ (uint32_t)((nb & 3) << 6)) + o;
-    const short4v x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a0 + (uint32_t)(ks * 16 * BROWB)));
-    const short4v x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(a1 + (uint32_t)(ks * 16 * BROWB)));
-    return frag_join<T>(x0, x1);
-  };
-
-  floatx16 acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  for (int s = 0; s < DIST; ++s)
-    if (s < nslices && cp_ext > 0) copy_general((uint32_t)(s * STAGEB), s);
-  dma_wait_all();
-  __syncthreads();
-
-  Frag fa[2][WM], fb[2][WN];
-  // fragments of k step ks of the stage whose row-fragment bases are fa_/fb_ (byte offset stage_ for the BKS form)
-  // nvi: how many of this wavefront's WM 32-row blocks hold rows of the group (WM except in a group's last tile)
-  auto load_frags = [&](int buf, uint32_t fa_, uint32_t fb_, uint32_t stage_, int ks, int nvi) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-      if (i < nvi) fa[buf][i] = *(lds_frag)((fa_ ^ (uint32_t)(ks << 5)) + i * 32 * ROWB);
-    if (nvi > 0) {
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        if constexpr (BKS) fb[buf][j] = ld_b_tr(stage_, ks, j);
-        else fb[buf][j] = *(lds_frag)((fb_ ^ (uint32_t)(ks << 5)) + j * 32 * ROWB);
-      }
-    }
-  };
-  // A group's last tile usually holds fewer than 256 rows.  Its wavefronts skip the 32-row blocks past the end
-  // (fragment reads and MFMAs; the copies and barriers stay), so such a tile costs what its copies cost,
-  // about a quarter of a full one, instead of a full tile's time.  The full tile keeps a branch-free loop.
-  auto slices = [&](auto partial) {
-  constexpr bool PARTIAL = decltype(partial)::value;
-  const int nvi = PARTIAL ? min(WM, max(0, (a_rext - wm * 32 * WM + 31) >> 5)) : WM;
-  if constexpr (CROSS) {
-    if (nslices > 0) load_frags(0, lds0 + fa_lane, lds0 + fb_lane, lds0, 0, nvi);
-  }
-  int st_cur = 0, st_nxt = DIST % NST;                  // stage of slice s, stage of slice s + DIST
-#pragma unroll 1
-  for (int s = 0; s < nslices; ++s) {
-    const uint32_t cur = (uint32_t)(st_cur * STAGEB), nxt = (uint32_t)(st_nxt * STAGEB);
-    const bool copy = s + DIST < nslices && cp_ext > 0;
-    const bool fcopy = copy && cp_fast;
-    const char *cp_src = cp_g + (int64_t)(s + DIST) * cp_slice;
-    uint32_t cp_dst = lds0 + nxt + cp_dst0;
-    if (copy && !fcopy) copy_general(nxt, s + DIST);
-    uint32_t fa0 = lds0 + cur + fa_lane, fb0 = lds0 + cur + fb_lane;
-    const uint32_t nst1 = (uint32_t)((st_cur + 1 == NST ? 0 : st_cur + 1) * STAGEB);   // stage of slice s + 1
-    uint32_t fa1 = lds0 + nst1 + fa_lane, fb1 = lds0 + nst1 + fb_lane;
-    uint32_t sg0 = lds0 + cur, sg1 = lds0 + nst1;
-    asm volatile("" : "+v"(fa0), "+v"(fb0), "+v"(fa1), "+v"(fb1), "+v"(sg0), "+v"(sg1));   // derive the other addresses here, not ahead of the loop
-    if constexpr (!CROSS) load_frags(0, fa0, fb0, sg0, 0, nvi);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int cu = ks & 1, nx = cu ^ 1;
-      if (ks + 1 < KS) load_frags(nx, fa0, fb0, sg0, ks + 1, nvi);
-      else if (CROSS && s + 1 < nslices) load_frags(nx, fa1, fb1, sg1, 0, nvi);   // first fragments of the next slice (already published)
-#pragma unroll
-      for (int i = 0; i < WM; ++i) {
-#pragma unroll
-        for (int j = 0; j < WN; ++j) {  // C^T block: rows n, cols m
-          if (!PARTIAL || i < nvi) acc[i][j] = M::mma(fb[cu][j], fa[cu][i], acc[i][j]);
-          // one 1 KB copy block after every DH_GG_CPI MFMAs until the slice's CPB blocks are out
-          const int mi = (ks * WM + i) * WN + j;
-          if (mi % DH_GG_CPI == DH_GG_CPI - 1 && mi / DH_GG_CPI < CPB && fcopy) {
-            __builtin_amdgcn_sched_barrier(0);
-            dma_block_fast(cp_src, block_off(mi / DH_GG_CPI), cp_dst);
-            cp_src += cp_step;
-            cp_dst += 1024;
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-      }
-    }
-    // slice s + WAITD must have landed; the copies of the DIST - WAITD slices after it may still be in
-    // flight (copies complete in order), unless fewer were issued (tail of k) or this wavefront uses
-    // the general copies
-    if (DIST > WAITD && fcopy) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DIST - WAITD) * CPB) : "memory");
-    else dma_wait_all();
-    st_cur = st_cur + 1 == NST ? 0 : st_cur + 1;
-    st_nxt = st_nxt + 1 == NST ? 0 : st_nxt + 1;
-    // A bare barrier: __syncthreads() would also wait for EVERY outstanding memory operation, i.e. drain
-    // the copies that are meant to stay in flight across it.  What the barrier has to order is covered by
-    // the waits above (this wavefront's copies of the slice being published) and by the fact that a
-    // wavefront's fragment reads of slice s have returned before its last MFMAs of slice s were issued.
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  }
-  };
-  if (a_rext >= BM) slices(BoolC<false>{});
-  else slices(BoolC<true>{});
-
-  // Epilogue.  A lane owns output row (m) c of each 32x32 block and 4 consecutive columns per register quad;
-  // stored straight from there, an instruction would touch 32 rows with two 8-byte pieces each, and such
-  // scattered partial-line stores run at a fraction of the memory system's rate (the stores were 5 % of the
-  // kernel).  Each wavefront instead passes its 128x64 block through a private LDS region, 64 rows at a time,
-  // and stores whole 128-byte lines: 8 adjacent lanes cover one row, 8 rows per instruction.  The stage
-  // buffers are free: the barrier that ended the last slice came after every wavefront's last fragment read.
-  // Rows of 136 bytes: the 8-byte writes of 32 lanes (32 rows, one column) fall on 64 different banks.
-  constexpr int EP = 136;
-  static_assert(NW * 64 * EP <= NST * STAGEB, "epilogue staging fits in the stage buffers");
-  unsigned char *ep = smem + w * (64 * EP);
-  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 32 * WN;
-  struct alignas(8) Q4 { T v[4]; };
-  struct alignas(8) Q8 { Q4 lo, hi; };
-  const int er = lane >> 3, ec = lane & 7;              // row inside a step of 8 rows, 16-byte chunk of the row
-#pragma unroll
-  for (int h = 0; h < WM / 2; ++h) {
-#pragma unroll
-    for (int i2 = 0; i2 < 2; ++i2) {
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        const floatx16 av = acc[2 * h + i2][j];
-#pragma unroll
-        for (int vb = 0; vb < 4; ++vb) {
-          Q4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
-          *reinterpret_cast<Q4 *>(ep + (32 * i2 + c) * EP + (32 * j + 8 * vb + 4 * hh) * (int)sizeof(T)) = o;
-        }
-      }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
-    const int mh = wm * 32 * WM + 64 * h;               // first row of this half in the tile
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int r = 8 * it + er;
-      const unsigned char *src = ep + r * EP + ec * 16;
-      Q8 o;
-      o.lo = *reinterpret_cast<const Q4 *>(src);
-      o.hi = *reinterpret_cast<const Q4 *>(src + 8);
-      const int n = wn * 32 * WN + 8 * ec;
-      if (mh + r < a_rext && n < b_rext) {
-        T *dst = cg + (int64_t)(mh + r) * p.ldc + 8 * ec;
-        *reinterpret_cast<dh_u32x4 *>(dst) = __builtin_bit_cast(dh_u32x4, o);
-      }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
-  }
-}
-
 // ---- 256x256 tiles with ONE wavefront per SIMD: four wavefronts of 128x128 outputs ------------------------------
 // The 256 accumulator registers of a wavefront live in AGPRs, and the loop is written slot by slot: after every
 // MFMA exactly one LDS or memory instruction (fragment read, staging-register write to LDS, buffer load), so that
 // the matrix pipe never waits for a burst of them and the LDS queue never fills.  A 64-deep k slice is loaded
 // into registers THREE slices ahead (two staging sets of 16 x 16 bytes per lane), written to the LDS stage that
 // is not being read during the first half of a slice, published by the slice's one barrier and read as fragments
-// one k step (16) ahead of the MFMAs that use them.  Against the eight-wavefront kernel above: a third fewer
-// fragment reads per MFMA, MFMAs of one wavefront back to back instead of two wavefronts alternating on the pipe.
+// one k step (16) ahead of the MFMAs that use them.  Against eight wavefronts of 128x64 (two per SIMD): a third
+// fewer fragment reads per MFMA, and the MFMAs of one wavefront run back to back instead of two wavefronts
+// alternating on the pipe.
+// Tiles in LDS: k-contiguous operands as [256 rows][64 k] with unpadded 128-byte rows, the 16-byte chunk index
+// XORed with (row / 2) % 8 (conflict-free 16-byte row-fragment reads); a k-strided operand (B of the NN product,
+// [k][n] row-major) as [64 k][256 n] with 512-byte rows, chunk ^= 4 (k % 4) + (k / 4) % 4 inside each 256-byte
+// half row, read as fragments by LDS transpose reads.
 //
 // The loads are buffer loads issued from assembly: the compiler does not count them, every use of a staging
 // register is ordered by a hand-written s_waitcnt vmcnt (loads return in order), and between its load and its
-// LDS write a staging register is touched by nothing else.  The buffer descriptors do the edge handling: one per
-// 32-row block of a tile, its length cut at the group's (or n's) last row, so that rows past the end read as
-// zero and no access leaves the operands, whatever the offsets table says.
+// LDS write a staging register is touched by nothing else.  The buffer descriptors do the edge handling: their
+// length is cut at the group's (or n's) last row, so that rows past the end read as zero and no access leaves
+// the operands, whatever the offsets table says.
 typedef int gg_i32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ gg_i32x4 gg_rsrc(const void *ptr, int64_t bytes) {
@@ -594,7 +294,62 @@ __device__ __forceinline__ gg_i32x4 gg_rsrc(const void *ptr, int64_t bytes) {
   return r;
 }
 
-template <typename T, bool BKS>
+// Stores a 256x256 tile held in the accumulator layout of grouped_gemm_w4_kernel (wavefront w = 2 wm + wn owns the
+// 128x128 block (wm, wn); acc[i][j] is its 32x32 block (i, j), transposed: lane column c is output row c).
+template <typename T>
+__device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigned char *smem, const GGParams &p, int m0, int n0,
+                                            int a_rext, int b_rext) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 31, hh = lane >> 5;
+  const int wm = w >> 1, wn = w & 1;
+  // Epilogue: each wavefront passes its 128x128 block through a private LDS region, 64 rows at a time, and stores
+  // whole 256-byte row segments (16 lanes a row, 4 rows per instruction).  Rows of 264 bytes: the 8-byte writes of
+  // 32 lanes (32 rows, one column) fall on different banks.
+  constexpr int EP = 264;
+  static_assert(4 * 64 * EP <= 128 * 1024, "epilogue staging fits in the stage buffers");
+  unsigned char *ep = smem + w * (64 * EP);
+  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 128;
+  struct alignas(8) Q4 { T v[4]; };
+  const int er = lane >> 4, ec = lane & 15;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int i2 = 0; i2 < 2; ++i2)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const floatx16 av = acc[2 * h + i2][j];
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          Q4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
+          *reinterpret_cast<Q4 *>(ep + (32 * i2 + c) * EP + (32 * j + 8 * vb + 4 * hh) * (int)sizeof(T)) = o;
+        }
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const int mh = wm * 128 + 64 * h;                   // first row of this half in the tile
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int r = 4 * it + er;
+      const dh_u32x4 o = *reinterpret_cast<const dh_u32x4 *>(ep + r * EP + ec * 16);
+      if (mh + r < a_rext && wn * 128 + 8 * ec < b_rext)
+        *reinterpret_cast<dh_u32x4 *>(cg + (int64_t)(mh + r) * p.ldc + 8 * ec) = o;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// k pieces per tile of the last round: as many as there are workgroups per tile, each at least one slice.
+__device__ __forceinline__ int gg_sk_pieces(int grid, int rem, int nsl) {
+  if (rem <= 0) return 1;
+  const int pc = grid / rem;
+  return pc < 1 ? 1 : (pc > nsl ? (nsl > 0 ? nsl : 1) : pc);
+}
+
+template <typename T, bool BKS, bool SK>
 __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) {
   using M = Mma<T>;
   using Frag = typename M::Frag;
@@ -602,53 +357,24 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   constexpr int NRD = BKS ? 12 : 8;                     // LDS read instructions per k step
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
 
-  const int ntiles = p.tiles_m * p.tiles_n;
-  int pid = blockIdx.x;
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-  int tm = pid % p.tiles_m;
-  const int tn = pid / p.tiles_m;
-  const int base = p.offs[0];
-  int g = 0, row_begin = 0, row_end = 0;
-  {
-    bool found = false;
-    for (int gi = 0; gi < p.groups; ++gi) {
-      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
-      const int t = (re - rb + BM - 1) / BM;
-      if (!found && tm < t) {
-        g = gi; row_begin = rb; row_end = re; found = true;
-      } else if (!found) {
-        tm -= t;
-      }
-    }
-    if (!found) return;
-  }
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hh = lane >> 5;
   const int wm = w >> 1, wn = w & 1;
-  const int n0 = tn * 256, m0 = row_begin + tm * BM;
-  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
-  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
-  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
   const int nsl = (int)(p.k_dim / 64);
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const uint32_t lda_b = (uint32_t)p.lda * (uint32_t)sizeof(T), ldb_b = (uint32_t)p.ldb * (uint32_t)sizeof(T);
+  const int base = p.offs[0];
 
   // ---- copies ----------------------------------------------------------------------------------------------
-  // k-contiguous tile [256 rows][64 k]: a lane copies chunk lc of rows lr + 32 i; descriptor i starts at row 32 i.
-  // k-strided tile [64 k][256 n]: a lane copies chunk cx of k rows kr + 8 i; descriptor i starts at k row 8 i.
+  // k-contiguous tile [256 rows][64 k]: a lane copies chunk lc of rows lr + 32 i.
+  // k-strided tile [64 k][256 n]: a lane copies chunk cx of k rows kr + 8 i.
   const int lc = tid & 7, lr = tid >> 3, cx = tid & 31, kr = tid >> 5;
-  gg_i32x4 rsa[8], rsb[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    rsa[i] = gg_rsrc(ag + (int64_t)(32 * i) * p.lda, (int64_t)(a_rext - 32 * i) * lda_b);
-    if (BKS) rsb[i] = gg_rsrc(bg + (int64_t)(8 * i) * p.ldb, 0x7fffffffll);
-    else rsb[i] = gg_rsrc(bg + (int64_t)(32 * i) * p.ldb, (int64_t)(b_rext - 32 * i) * ldb_b);
-  }
   const uint32_t goff_a = (uint32_t)lr * lda_b + (uint32_t)(lc * 16);
   const uint32_t goff_b = BKS ? (uint32_t)kr * ldb_b + (uint32_t)(cx * 16) : (uint32_t)lr * ldb_b + (uint32_t)(lc * 16);
   const uint32_t kstep_a = 64 * (uint32_t)sizeof(T);                          // bytes from one k slice to the next
   const uint32_t kstep_b = BKS ? 64 * ldb_b : 64 * (uint32_t)sizeof(T);
+  const uint32_t rstep_a = 32 * lda_b, rstep_b = BKS ? 8 * ldb_b : 32 * ldb_b;     // bytes from one copy of a lane to its next
   const uint32_t wr_a = (uint32_t)(lr * ROWB + ((lc ^ ((lr >> 1) & 7)) << 4));                      // + i * 4096
   // k-strided tile: chunk XOR 4 (k % 4) + (k / 4) % 4 with k = kr + 8 i: the i part is bit 1 of the chunk for odd i
   const uint32_t wr_b = BKS ? (uint32_t)(TILEB + kr * BROWB + (cx >> 4) * 256 + (((cx & 15) ^ (4 * (kr & 3) + (kr >> 2))) << 4))
@@ -668,6 +394,20 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   typedef short4v __attribute__((address_space(3))) *lds_tr;
   typedef __attribute__((address_space(3))) gg_i32x4 *lds_w;
 
+  // One segment: slices [s0, s1) of the tile (g, tm, tn).  part == nullptr: the segment is the whole k range and the
+  // result goes to c; else the fp32 partial sums go to part (accumulator layout: 1 KB per wavefront instruction;
+  // gg_split_reduce_kernel sums the pieces of a tile in k order).
+  auto segment = [&](int g, int row_begin, int row_end, int tm, int tn, int s0, int s1, float *part) {
+  const int n0 = tn * 256, m0 = row_begin + tm * BM;
+  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
+  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
+  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+  // One descriptor per operand, cut at the last row of the group (of n): the hardware compares the lane offset plus
+  // the scalar offset with the length, so a row past the end reads as zero whichever 32-row block it is in.
+  const gg_i32x4 rsa = gg_rsrc(ag, (int64_t)(a_rext < 256 ? a_rext : 256) * lda_b);
+  const gg_i32x4 rsb = BKS ? gg_rsrc(bg, (int64_t)p.k_dim * ldb_b - (int64_t)n0 * (int)sizeof(T))
+                           : gg_rsrc(bg, (int64_t)(b_rext < 256 ? b_rext : 256) * ldb_b);
+  const int cnt = s1 - s0;                              // slices of this segment
   floatx16 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -682,8 +422,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   short4v fbt[2][4][2];                                 // k-strided form: the two transpose reads of a fragment
 
   auto gload = [&](int set, int idx, uint32_t ka, uint32_t kb) {   // idx 0..7: A, 8..15: B; ka, kb: byte offsets of the slice
-    if (idx < 8) asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_a), "s"(rsa[idx]), "s"(ka) : "memory");
-    else asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_b), "s"(rsb[idx - 8]), "s"(kb) : "memory");
+    if (idx < 8) asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_a), "s"(rsa), "s"(ka + idx * rstep_a) : "memory");
+    else asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_b), "s"(rsb), "s"(kb + (idx - 8) * rstep_b) : "memory");
   };
   auto swrite = [&](int set, int idx, uint32_t stage) {  // stage: LDS byte address of the stage
     if (idx < 8) *(lds_w)(stage + wr_a + idx * 4096) = stg[set][idx];
@@ -709,10 +449,10 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
 
   // prologue: slice 0 into stage 0 (through set 0), slice 1 into set 1, slice 2 into set 0.  Loads of slices that
   // do not exist repeat the last slice (their data is written to a stage nobody reads).
-  const int last = nsl > 0 ? nsl - 1 : 0;
-  auto kof = [&](int s) { return (uint32_t)(s < last ? s : last); };
+  const int last = cnt > 0 ? cnt - 1 : 0;
+  auto kof = [&](int s) { return (uint32_t)(s0 + (s < last ? s : last)); };
 #pragma unroll
-  for (int x = 0; x < 16; ++x) gload(0, x, 0, 0);
+  for (int x = 0; x < 16; ++x) gload(0, x, kof(0) * kstep_a, kof(0) * kstep_b);
 #pragma unroll
   for (int x = 0; x < 16; ++x) gload(1, x, kof(1) * kstep_a, kof(1) * kstep_b);
   asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
@@ -773,7 +513,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   using I1 = std::integral_constant<int, 1>;
   int s = 0;
 #pragma unroll 1
-  for (; s + 1 < nsl; s += 2) {
+  for (; s + 1 < cnt; s += 2) {
     slice(I0{}, std::false_type{}, s);
     slice(I1{}, std::false_type{}, s + 1);
   }
@@ -782,63 +522,167 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int x = 0; x < 16; ++x) asm volatile("" ::"v"(stg[0][x]), "v"(stg[1][x]));
-  if (s < nsl) slice(I0{}, std::true_type{}, s);
+  if (s < cnt) slice(I0{}, std::true_type{}, s);
   __syncthreads();                                      // everyone is done with the stages: they stage the output below
 
-  // Epilogue: each wavefront passes its 128x128 block through a private LDS region, 64 rows at a time, and stores
-  // whole 256-byte row segments (16 lanes a row, 4 rows per instruction).  Rows of 264 bytes: the 8-byte writes of
-  // 32 lanes (32 rows, one column) fall on different banks.
-  constexpr int EP = 264;
-  static_assert(4 * 64 * EP <= 2 * STAGEB, "epilogue staging fits in the stage buffers");
-  unsigned char *ep = smem + w * (64 * EP);
-  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 128;
-  struct alignas(8) Q4 { T v[4]; };
-  const int er = lane >> 4, ec = lane & 15;
+  if (SK && part != nullptr) {
+    // 16 bytes per lane and instruction: piece ((w * 16 + i * 4 + j) * 4 + vb) of the tile, 1 KB each
+    float *dst = part + ((size_t)w * 64 * 4 + 0) * 64 + (size_t)lane * 4;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int i2 = 0; i2 < 2; ++i2)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const floatx16 av = acc[2 * h + i2][j];
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int vb = 0; vb < 4; ++vb) {
-          Q4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(av[4 * vb + e]);
-          *reinterpret_cast<Q4 *>(ep + (32 * i2 + c) * EP + (32 * j + 8 * vb + 4 * hh) * (int)sizeof(T)) = o;
+          const floatx16 av = acc[i][j];
+          const floatx4 o = {av[4 * vb], av[4 * vb + 1], av[4 * vb + 2], av[4 * vb + 3]};
+          *reinterpret_cast<floatx4 *>(dst + (size_t)(((i * 4 + j) * 4 + vb) * 256)) = o;
         }
+    __syncthreads();                                    // the next segment's copies reuse the stages
+    return;
+  }
+  gg_w4_store<T>(acc, smem, p, m0, n0, a_rext, b_rext);
+    __syncthreads();                                    // the next segment's copies reuse the staging area
+  };
+
+  if constexpr (!SK) {
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int pid = blockIdx.x;
+    if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+    int tm = pid % p.tiles_m;
+    const int tn = pid / p.tiles_m;
+    for (int gi = 0; gi < p.groups; ++gi) {
+      const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
+      const int t = (re - rb + BM - 1) / BM;
+      if (tm < t) {
+        segment(gi, rb, re, tm, tn, 0, nsl, nullptr);
+        return;
       }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
-    const int mh = wm * 128 + 64 * h;                   // first row of this half in the tile
-#pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int r = 4 * it + er;
-      const dh_u32x4 o = *reinterpret_cast<const dh_u32x4 *>(ep + r * EP + ec * 16);
-      if (mh + r < a_rext && wn * 128 + 8 * ec < b_rext)
-        *reinterpret_cast<dh_u32x4 *>(cg + (int64_t)(mh + r) * p.ldc + 8 * ec) = o;
+      tm -= t;
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_wave_barrier();
+  } else {
+    // One workgroup per compute unit.  The tiles (m fastest) are dealt out in rounds of gridDim.x: round j gives
+    // workgroup w the tile j * gridDim.x + w, so that the tiles in flight are neighbours and share their operand
+    // panels through L2.  When the last round holds at most half as many tiles as there are workgroups, its tiles
+    // are split along k into as many pieces as fit (workgroup w: tile w % rem, piece w / rem, so that neighbours
+    // still work on neighbouring tiles); the pieces are summed afterwards, in k order.  288 tiles on 256 compute
+    // units then take 1 1/8 tile times instead of 2.
+    int tiles_m = 0;
+    for (int gi = 0; gi < p.groups; ++gi)
+      tiles_m += (gg_clamp_row(p.offs[gi + 1] - base, p.max_rows) - gg_clamp_row(p.offs[gi] - base, p.max_rows) + BM - 1) / BM;
+    const int tiles = tiles_m * p.tiles_n;
+    const int grid = (int)gridDim.x, full = tiles / grid, rem = tiles - full * grid;
+    const int pieces = gg_sk_pieces(grid, rem, nsl);
+    int wg = blockIdx.x;
+    if (grid % 8 == 0) wg = (wg % 8) * (grid / 8) + wg / 8;            // neighbouring tiles on one XCD
+    const int rounds = full + (wg < rem * pieces ? 1 : 0);
+#pragma unroll 1
+    for (int it = 0; it < rounds; ++it) {
+      int t = it * grid + wg, s0 = 0, s1 = nsl;
+      float *part = nullptr;
+      if (it == full) {                                                 // the last round
+        const int ts = wg % rem, pc = wg / rem;
+        t = full * grid + ts;
+        s0 = pc * nsl / pieces;
+        s1 = (pc + 1) * nsl / pieces;
+        if (pieces > 1) part = p.ws + (size_t)wg * (256 * 256);
+      }
+      int tm = t % tiles_m;
+      const int tn = t / tiles_m;
+      int g = 0, rb = 0, re = 0;
+      for (int gi = 0; gi < p.groups; ++gi) {
+        rb = gg_clamp_row(p.offs[gi] - base, p.max_rows); re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
+        const int nt = (re - rb + BM - 1) / BM;
+        if (tm < nt) { g = gi; break; }
+        tm -= nt;
+      }
+      segment(g, rb, re, tm, tn, s0, s1, part);
+    }
   }
 }
 
-template <typename T, bool BKS>
-static int launch_gg_w4(GGParams p, int64_t m_extent, hipStream_t st) {
-  p.tiles_n = (int)cdiv(p.n_dim, 256);
-  p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
-  if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
-  hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
-  return DH_OK;
+// Sums the k pieces of the tiles of a split last round, in k order (deterministic), and stores the tiles.
+// 16 workgroups per tile of that round: a wavefront takes one 32x32 block (w, i, j) of the accumulator layout,
+// reads its 4 KB of every piece (1 KB per instruction) and writes 4 columns per lane and register quad.
+template <typename T>
+__global__ void __launch_bounds__(256) gg_split_reduce_kernel(const GGParams p, int sk_grid) {
+  constexpr int BM = 256;
+  const int nsl = (int)(p.k_dim / 64);
+  const int base = p.offs[0];
+  int tiles_m = 0;
+  for (int gi = 0; gi < p.groups; ++gi)
+    tiles_m += (gg_clamp_row(p.offs[gi + 1] - base, p.max_rows) - gg_clamp_row(p.offs[gi] - base, p.max_rows) + BM - 1) / BM;
+  const int tiles = tiles_m * p.tiles_n, full = tiles / sk_grid, rem = tiles - full * sk_grid;
+  const int ts = blockIdx.x / 16;                       // tile of the last round
+  if (ts >= rem || nsl == 0) return;
+  const int pieces = gg_sk_pieces(sk_grid, rem, nsl);
+  if (pieces == 1) return;
+  const int t = full * sk_grid + ts;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int blk = (blockIdx.x % 16) * 4 + (tid >> 6);   // (w * 4 + i) * 4 + j
+  const int w = blk >> 4, i = (blk >> 2) & 3, j = blk & 3;
+  floatx4 acc[4];
+#pragma unroll
+  for (int vb = 0; vb < 4; ++vb) acc[vb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int pc = 0; pc < pieces; ++pc) {
+    const float *src = p.ws + (size_t)(pc * rem + ts) * (256 * 256) + (size_t)blk * (4 * 256) + (size_t)lane * 4;
+#pragma unroll
+    for (int vb = 0; vb < 4; ++vb) acc[vb] += *reinterpret_cast<const floatx4 *>(src + vb * 256);
+  }
+  int tm = t % tiles_m;
+  const int tn = t / tiles_m;
+  int rb = 0, re = 0;
+  for (int gi = 0; gi < p.groups; ++gi) {
+    rb = gg_clamp_row(p.offs[gi] - base, p.max_rows); re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
+    const int nt = (re - rb + BM - 1) / BM;
+    if (tm < nt) break;
+    tm -= nt;
+  }
+  const int c = lane & 31, hh = lane >> 5;
+  const int m = (w >> 1) * 128 + 32 * i + c, n = (w & 1) * 128 + 32 * j + 4 * hh;    // + 8 vb
+  const int m0 = rb + tm * BM, n0 = tn * 256;
+  if (m0 + m >= re) return;
+  T *dst = reinterpret_cast<T *>(p.c) + (int64_t)(m0 + m) * p.ldc + n0 + n;
+  struct alignas(8) Q4 { T v[4]; };
+#pragma unroll
+  for (int vb = 0; vb < 4; ++vb)
+    if (n0 + n + 8 * vb < p.n_dim) {
+      Q4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[vb][e]);
+      *reinterpret_cast<Q4 *>(dst + 8 * vb) = o;
+    }
 }
 
-template <typename T, int WVN, int BKT, int NST, bool BKS>
-static int launch_gg_dma(GGParams p, int64_t m_extent, hipStream_t st) {
+// Workspace of the split last round: one fp32 tile per workgroup of the grid.
+constexpr int GG_SK_MAX_GRID = 256;
+constexpr size_t GG_SK_WS_BYTES = (size_t)GG_SK_MAX_GRID * 256 * 256 * sizeof(float);
+
+template <typename T, bool BKS>
+static int launch_gg_w4(GGParams p, int64_t m_extent, void *workspace, size_t workspace_bytes, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
   p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
-  hipLaunchKernelGGL((grouped_gemm_dma_kernel<T, WVN, BKT, NST, BKS>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(128 * WVN), 0, st, p);
+  int grid = 0;
+  if (workspace != nullptr && p.k_dim >= 64) {
+    int dev = 0, cus = 0;
+    DH_HIP(hipGetDevice(&dev));
+    DH_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    grid = cus < GG_SK_MAX_GRID ? cus : GG_SK_MAX_GRID;
+    if (workspace_bytes < (size_t)grid * 256 * 256 * sizeof(float)) grid = 0;
+  }
+  // One workgroup per compute unit costs a few percent against one workgroup per tile (its tile loop is not
+  // overlapped with anything); it pays where the split of the last round can save half a tile time or more of a
+  // short job: at most one and a half rounds of tiles (the host knows the tile count only up to the groups'
+  // partial tiles, so it cannot tell how full the last round of a longer job is).
+  if (grid > 0 && 2 * (int64_t)p.tiles_m * p.tiles_n > 3 * (int64_t)grid) grid = 0;
+  if (grid > 0) {
+    p.ws = reinterpret_cast<float *>(workspace);
+    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS, true>), dim3((unsigned)grid), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((gg_split_reduce_kernel<T>), dim3((unsigned)(16 * grid / 2)), dim3(256), 0, st, p, grid);   // at most grid / 2 tiles are split
+  } else {
+    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS, false>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
+  }
   return DH_OK;
 }
 
@@ -901,8 +745,11 @@ static int gg_common_checks(const void *a, const void *b, void *c, const int32_t
 
 }  // namespace dh
 
+extern "C" size_t dh_grouped_gemm_workspace_bytes(void) { return dh::GG_SK_WS_BYTES; }
+
 extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const int32_t *offs, int groups,
-                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
+                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *workspace,
+                                  size_t workspace_bytes, void *stream) {
   using namespace dh;
   DH_CHECK(max_rows >= 0 && max_rows < (1ll << 31) && n >= 0 && k >= 0, "size out of range");
   if (max_rows == 0 || n == 0) return DH_OK;
@@ -916,11 +763,8 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && k <= (1ll << 21))
-    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, false>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_w4<f16_t, false>(p, max_rows, (hipStream_t)stream);
-  else if (big && k % 64 == 0 && k < (1ll << 30))
-    rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_dma<f16_t, DH_GG_WVN, DH_GG_BKT, DH_GG_NST, false>(p, max_rows, (hipStream_t)stream);
+    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, false>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream)
+                          : launch_gg_w4<f16_t, false>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream);
   else
     rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;
@@ -929,7 +773,8 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
 }
 
 extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const int32_t *offs, int groups,
-                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *stream) {
+                                  int64_t max_rows, int64_t n, int64_t k, int dtype, void *workspace,
+                                  size_t workspace_bytes, void *stream) {
   using namespace dh;
   DH_CHECK(max_rows >= 0 && max_rows < (1ll << 31) && n >= 0 && k >= 0, "size out of range");
   if (max_rows == 0 || n == 0) return DH_OK;
@@ -943,11 +788,8 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
   if (big && k % 64 == 0 && n % 256 == 0 && k <= (1ll << 21) && k * n * (int64_t)dtype_size(dtype) < (1ll << 31))
-    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, true>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_w4<f16_t, true>(p, max_rows, (hipStream_t)stream);
-  else if (big && k % 64 == 0 && n % 256 == 0 && DH_GG_BKT == 64 && n * (int64_t)dtype_size(dtype) < (1ll << 30))
-    rc = dtype == DH_BF16 ? launch_gg_dma<bf16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream)
-                          : launch_gg_dma<f16_t, DH_GG_WVN, 64, DH_GG_NST, true>(p, max_rows, (hipStream_t)stream);
+    rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, true>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream)
+                          : launch_gg_w4<f16_t, true>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream);
   else
     rc = dispatch_gg<false, true, false>(p, max_rows, dtype, (hipStream_t)stream);
   if (rc) return rc;

@@ -123,6 +123,23 @@ def unpermute_bwd(dout, y, plan, gates, e_lo, e_hi, max_rows, stream=None, profi
 # ---------------------------------------------------------------------------------------
 # grouped GEMM and the expert FFN built from it
 # ---------------------------------------------------------------------------------------
+_gg_workspaces: dict = {}
+
+
+def _gg_workspace(rows, n, device, stream):
+    """(pointer, bytes) of the split-k workspace for a product of this size on this stream: one buffer per
+    (device, stream), since calls on different streams may overlap.  Small products (fewer 256x256 tiles than
+    compute units) do not use one."""
+    if -(-rows // 256) * -(-n // 256) < 256:
+        return None, 0
+    key = (device, stream.cuda_stream)
+    ws = _gg_workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(_lib.load().dh_grouped_gemm_workspace_bytes(), dtype=torch.uint8, device=device)
+        _gg_workspaces[key] = ws
+    return ws.data_ptr(), ws.numel()
+
+
 def grouped_gemm_nt(a, b, offs, max_rows=None, out=None, stream=None):
     """c[rows_g] = a[rows_g] @ b[g].T ; a [R, K], b [G, N, K] -> c [R, N]."""
     lib = _lib.load()
@@ -134,9 +151,10 @@ def grouped_gemm_nt(a, b, offs, max_rows=None, out=None, stream=None):
         c = out if out is not None else torch.empty((a.shape[0], n), dtype=a.dtype, device=a.device)
         if out is None and max_rows is not None and max_rows < a.shape[0]:
             c[max_rows:].zero_()
-        _lib.check(lib.dh_grouped_gemm_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g,
-                                          a.shape[0] if max_rows is None else max_rows, n, k, _lib.dt(a),
-                                          st.cuda_stream))
+        rows = a.shape[0] if max_rows is None else max_rows
+        ws, ws_bytes = _gg_workspace(rows, n, a.device, st)
+        _lib.check(lib.dh_grouped_gemm_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g, rows, n, k,
+                                          _lib.dt(a), ws, ws_bytes, st.cuda_stream))
     return c
 
 
@@ -151,9 +169,10 @@ def grouped_gemm_nn(a, b, offs, max_rows=None, out=None, stream=None):
         c = out if out is not None else torch.empty((a.shape[0], n), dtype=a.dtype, device=a.device)
         if out is None and max_rows is not None and max_rows < a.shape[0]:
             c[max_rows:].zero_()
-        _lib.check(lib.dh_grouped_gemm_nn(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g,
-                                          a.shape[0] if max_rows is None else max_rows, n, k, _lib.dt(a),
-                                          st.cuda_stream))
+        rows = a.shape[0] if max_rows is None else max_rows
+        ws, ws_bytes = _gg_workspace(rows, n, a.device, st)
+        _lib.check(lib.dh_grouped_gemm_nn(a.data_ptr(), b.data_ptr(), c.data_ptr(), offs.data_ptr(), g, rows, n, k,
+                                          _lib.dt(a), ws, ws_bytes, st.cuda_stream))
     return c
 
 

@@ -276,7 +276,7 @@ def test_offsets_past_the_callers_bound_touch_nothing_beyond_it():
     for name, fn, bb in (("nt", lib.dh_grouped_gemm_nt, b), ("nn", lib.dh_grouped_gemm_nn, b.transpose(1, 2).contiguous())):
         c = torch.full((max_rows + guard, N), 3.0, dtype=dt, device="cuda")
         _lib.check(fn(a.data_ptr(), bb.data_ptr(), c.data_ptr(), plan.expert_offsets.data_ptr(), E, max_rows, N, H,
-                      _lib.dt(a), st))
+                      _lib.dt(a), None, 0, st))
         torch.cuda.synchronize()
         assert (c[max_rows:] == 3.0).all(), f"grouped GEMM {name} wrote past max_rows"
         ref = torch.zeros((max_rows, N), dtype=torch.float64)
@@ -338,3 +338,46 @@ def test_expert_ffn_bwd_with_resident_weight_transposes():
         assert torch.equal(a, b)
     w2.mul_(0.5)
     assert torch.equal(_Clib.transposed_of(w2), w2.transpose(1, 2).contiguous())
+
+
+@pytest.mark.parametrize("K", [192, 1024])
+@pytest.mark.parametrize("form", ["nt", "nn"])
+def test_grouped_gemm_split_last_round(form, K):
+    """The chip-filling kernels through the C ABI, with and without a workspace (last round split along k / one workgroup per tile):
+    both within the bound of the fp64 product, the split result the same on every run, rows cut off at max_rows
+    (the offsets describe more rows than the operands hold), nothing written past them."""
+    from dhellam_amd import _lib
+    lib = _lib.load()
+    dt = torch.bfloat16
+    rows, N = [2100, 0, 1990, 37, 500], 4096
+    G, R = len(rows), sum(rows)
+    max_rows, guard = 4200, 64                      # the last group is cut off: 73 of its 500 rows exist
+    offs_np = np.concatenate(([5], 5 + np.cumsum(rows))).astype(np.int32)
+    offs = torch.from_numpy(offs_np).cuda()
+    a = randn((max_rows, K), dt, 11, std=0.5).cuda()
+    b = randn((G, N, K), dt, 12, std=0.5).cuda()
+    bb = b if form == "nt" else b.transpose(1, 2).contiguous()
+    fn = lib.dh_grouped_gemm_nt if form == "nt" else lib.dh_grouped_gemm_nn
+    st = torch.cuda.current_stream().cuda_stream
+    ws = torch.empty(lib.dh_grouped_gemm_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    ref = torch.zeros((max_rows, N), dtype=torch.float64)
+    for g in range(G):
+        lo, hi = min(int(offs_np[g]) - 5, max_rows), min(int(offs_np[g + 1]) - 5, max_rows)
+        ref[lo:hi] = a[lo:hi].cpu().double() @ b[g].cpu().double().T
+    outs = []
+    for wsp, nbytes in ((None, 0), (ws.data_ptr(), ws.numel()), (ws.data_ptr(), ws.numel())):
+        ws.fill_(0x7f)                              # the workspace's contents on entry do not matter
+        c = torch.full((max_rows + guard, N), 3.0, dtype=dt, device="cuda")
+        _lib.check(fn(a.data_ptr(), bb.data_ptr(), c.data_ptr(), offs.data_ptr(), G, max_rows, N, K, _lib.dt(a),
+                      wsp, nbytes, st))
+        torch.cuda.synchronize()
+        assert (c[max_rows:] == 3.0).all(), "wrote past max_rows"
+        assert_close(c[:max_rows], ref, dt, f"grouped GEMM {form}, workspace {nbytes}")
+        outs.append(c)
+    assert torch.equal(outs[1], outs[2]), "split result differs between runs"
+    # a workspace that is too small is not used (the product falls back to one workgroup per tile)
+    c = torch.full((max_rows + guard, N), 3.0, dtype=dt, device="cuda")
+    _lib.check(fn(a.data_ptr(), bb.data_ptr(), c.data_ptr(), offs.data_ptr(), G, max_rows, N, K, _lib.dt(a),
+                  ws.data_ptr(), 1 << 20, st))
+    torch.cuda.synchronize()
+    assert torch.equal(c, outs[0])

@@ -296,9 +296,9 @@ __device__ __forceinline__ gg_i32x4 gg_rsrc(const void *ptr, int64_t bytes) {
 
 // Stores a 256x256 tile held in the accumulator layout of grouped_gemm_w4_kernel (wavefront w = 2 wm + wn owns the
 // 128x128 block (wm, wn); acc[i][j] is its 32x32 block (i, j), transposed: lane column c is output row c).
-template <typename T>
-__device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigned char *smem, const GGParams &p, int m0, int n0,
-                                            int a_rext, int b_rext) {
+template <typename T, bool MAY_ACCUMULATE>
+__device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigned char *smem, const GGParams &p, T *cbase, int m0,
+                                            int n0, int a_rext, int b_rext) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hh = lane >> 5;
@@ -309,8 +309,31 @@ __device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigne
   constexpr int EP = 264;
   static_assert(4 * 64 * EP <= 128 * 1024, "epilogue staging fits in the stage buffers");
   unsigned char *ep = smem + w * (64 * EP);
-  T *cg = reinterpret_cast<T *>(p.c) + (int64_t)m0 * p.ldc + n0 + wn * 128;
+  T *cg = cbase + (int64_t)m0 * p.ldc + n0 + wn * 128;
   struct alignas(8) Q4 { T v[4]; };
+  if (MAY_ACCUMULATE && p.accumulate) {
+    // c += product with one rounding: straight from the accumulators (a lane owns output row c of each 32x32 block
+    // and 4 consecutive columns per register quad)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = wm * 128 + 32 * i + c;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int vb = 0; vb < 4; ++vb) {
+          const int n = 32 * j + 8 * vb + 4 * hh;
+          if (m < a_rext && wn * 128 + n < b_rext) {
+            Q4 *dst = reinterpret_cast<Q4 *>(cg + (int64_t)m * p.ldc + n);
+            const Q4 old = *dst;
+            Q4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o.v[e] = static_cast<T>(acc[i][j][4 * vb + e] + static_cast<float>(old.v[e]));
+            *dst = o;
+          }
+        }
+    }
+    return;
+  }
   const int er = lane >> 4, ec = lane & 15;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -349,12 +372,16 @@ __device__ __forceinline__ int gg_sk_pieces(int grid, int rem, int nsl) {
   return pc < 1 ? 1 : (pc > nsl ? (nsl > 0 ? nsl : 1) : pc);
 }
 
-template <typename T, bool BKS, bool SK>
+// FORM 0: NT (both operands k-contiguous); 1: NN (b k-strided); 2: TN (both k-strided, k = the group's rows, one output
+// per group).
+template <typename T, int FORM, bool SK>
 __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) {
+  constexpr bool BKS = FORM >= 1, AKS = FORM == 2;
+  static_assert(!(AKS && SK), "the wgrad form has many tiles and a short k: it is never split");
   using M = Mma<T>;
   using Frag = typename M::Frag;
   constexpr int BM = 256, ROWB = 128, BROWB = 512, TILEB = 256 * ROWB, STAGEB = 2 * TILEB;
-  constexpr int NRD = BKS ? 12 : 8;                     // LDS read instructions per k step
+  constexpr int NRD = AKS ? 16 : (BKS ? 12 : 8);        // LDS read instructions per k step
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGEB];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -370,15 +397,15 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   // k-contiguous tile [256 rows][64 k]: a lane copies chunk lc of rows lr + 32 i.
   // k-strided tile [64 k][256 n]: a lane copies chunk cx of k rows kr + 8 i.
   const int lc = tid & 7, lr = tid >> 3, cx = tid & 31, kr = tid >> 5;
-  const uint32_t goff_a = (uint32_t)lr * lda_b + (uint32_t)(lc * 16);
+  const uint32_t goff_a = AKS ? (uint32_t)kr * lda_b + (uint32_t)(cx * 16) : (uint32_t)lr * lda_b + (uint32_t)(lc * 16);
   const uint32_t goff_b = BKS ? (uint32_t)kr * ldb_b + (uint32_t)(cx * 16) : (uint32_t)lr * ldb_b + (uint32_t)(lc * 16);
-  const uint32_t kstep_a = 64 * (uint32_t)sizeof(T);                          // bytes from one k slice to the next
+  const uint32_t kstep_a = AKS ? 64 * lda_b : 64 * (uint32_t)sizeof(T);       // bytes from one k slice to the next
   const uint32_t kstep_b = BKS ? 64 * ldb_b : 64 * (uint32_t)sizeof(T);
-  const uint32_t rstep_a = 32 * lda_b, rstep_b = BKS ? 8 * ldb_b : 32 * ldb_b;     // bytes from one copy of a lane to its next
-  const uint32_t wr_a = (uint32_t)(lr * ROWB + ((lc ^ ((lr >> 1) & 7)) << 4));                      // + i * 4096
+  const uint32_t rstep_a = AKS ? 8 * lda_b : 32 * lda_b, rstep_b = BKS ? 8 * ldb_b : 32 * ldb_b;   // bytes from one copy of a lane to its next
+  const uint32_t wr_kc = (uint32_t)(lr * ROWB + ((lc ^ ((lr >> 1) & 7)) << 4));                     // + i * 4096
   // k-strided tile: chunk XOR 4 (k % 4) + (k / 4) % 4 with k = kr + 8 i: the i part is bit 1 of the chunk for odd i
-  const uint32_t wr_b = BKS ? (uint32_t)(TILEB + kr * BROWB + (cx >> 4) * 256 + (((cx & 15) ^ (4 * (kr & 3) + (kr >> 2))) << 4))
-                            : (uint32_t)TILEB + wr_a;
+  const uint32_t wr_ks = (uint32_t)(kr * BROWB + (cx >> 4) * 256 + (((cx & 15) ^ (4 * (kr & 3) + (kr >> 2))) << 4));
+  const uint32_t wr_a = AKS ? wr_ks : wr_kc, wr_b = (uint32_t)TILEB + (BKS ? wr_ks : wr_kc);
 
   // ---- fragment reads --------------------------------------------------------------------------------------
   const uint32_t sw = (uint32_t)((hh ^ ((c >> 1) & 7)) << 4);
@@ -387,9 +414,11 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   const int r16 = lane & 15;
   const int t_lc = 2 * ((lane >> 4) & 1) + ((r16 & 3) >> 1);
   const int tx = 4 * (r16 >> 2) + 2 * hh;
-  const uint32_t t_row = (uint32_t)(TILEB + wn * 256 + (8 * hh + (r16 >> 2)) * BROWB + ((r16 & 3) & 1) * 8);
-  const uint32_t tb_a = t_row + (uint32_t)((t_lc ^ tx) << 4);                       // k rows 8 hh + 0..3 of a step
-  const uint32_t tb_b = t_row + 4 * BROWB + (uint32_t)((t_lc ^ (tx + 1)) << 4);     // k rows 8 hh + 4..7
+  const uint32_t t_row = (uint32_t)((8 * hh + (r16 >> 2)) * BROWB + ((r16 & 3) & 1) * 8);
+  const uint32_t t_lo = t_row + (uint32_t)((t_lc ^ tx) << 4);                       // k rows 8 hh + 0..3 of a step
+  const uint32_t t_hi = t_row + 4 * BROWB + (uint32_t)((t_lc ^ (tx + 1)) << 4);     // k rows 8 hh + 4..7
+  const uint32_t tb_a = (uint32_t)(TILEB + wn * 256) + t_lo, tb_b = (uint32_t)(TILEB + wn * 256) + t_hi;   // B tile, this wavefront's 128 columns
+  const uint32_t ta_a = (uint32_t)(wm * 256) + t_lo, ta_b = (uint32_t)(wm * 256) + t_hi;                   // A tile (TN)
   typedef __attribute__((address_space(3))) const Frag *lds_frag;
   typedef short4v __attribute__((address_space(3))) *lds_tr;
   typedef __attribute__((address_space(3))) gg_i32x4 *lds_w;
@@ -398,14 +427,20 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   // result goes to c; else the fp32 partial sums go to part (accumulator layout: 1 KB per wavefront instruction;
   // gg_split_reduce_kernel sums the pieces of a tile in k order).
   auto segment = [&](int g, int row_begin, int row_end, int tm, int tn, int s0, int s1, float *part) {
-  const int n0 = tn * 256, m0 = row_begin + tm * BM;
-  const int a_rext = row_end - m0, b_rext = (int)(p.n_dim - n0);
-  const T *ag = reinterpret_cast<const T *>(p.a) + (int64_t)m0 * p.lda;
-  const T *bg = reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
+  // NT / NN: output rows m0.. of the stacked rows; TN: output rows m0.. of group g's own [m_dim, n_dim] result
+  const int n0 = tn * 256, m0 = AKS ? tm * BM : row_begin + tm * BM;
+  const int a_rext = AKS ? (int)(p.m_dim - m0) : row_end - m0, b_rext = (int)(p.n_dim - n0);
+  const T *ag = reinterpret_cast<const T *>(p.a) + (AKS ? (int64_t)row_begin * p.lda + m0 : (int64_t)m0 * p.lda);
+  const T *bg = AKS ? reinterpret_cast<const T *>(p.b) + (int64_t)row_begin * p.ldb + n0
+                    : reinterpret_cast<const T *>(p.b) + (int64_t)g * p.b_group_stride + (BKS ? (int64_t)n0 : (int64_t)n0 * p.ldb);
   // One descriptor per operand, cut at the last row of the group (of n): the hardware compares the lane offset plus
   // the scalar offset with the length, so a row past the end reads as zero whichever 32-row block it is in.
-  const gg_i32x4 rsa = gg_rsrc(ag, (int64_t)(a_rext < 256 ? a_rext : 256) * lda_b);
-  const gg_i32x4 rsb = BKS ? gg_rsrc(bg, (int64_t)p.k_dim * ldb_b - (int64_t)n0 * (int)sizeof(T))
+  // (k-strided operands: cut at the last k row, i.e. the group's last row for TN; their tiles are whole in the
+  // other direction, which the host checks)
+  const gg_i32x4 rsa = AKS ? gg_rsrc(ag, (int64_t)(row_end - row_begin) * lda_b - (int64_t)m0 * (int)sizeof(T))
+                           : gg_rsrc(ag, (int64_t)(a_rext < 256 ? a_rext : 256) * lda_b);
+  const gg_i32x4 rsb = AKS ? gg_rsrc(bg, (int64_t)(row_end - row_begin) * ldb_b - (int64_t)n0 * (int)sizeof(T))
+                     : BKS ? gg_rsrc(bg, (int64_t)p.k_dim * ldb_b - (int64_t)n0 * (int)sizeof(T))
                            : gg_rsrc(bg, (int64_t)(b_rext < 256 ? b_rext : 256) * ldb_b);
   const int cnt = s1 - s0;                              // slices of this segment
   floatx16 acc[4][4];
@@ -417,7 +452,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   gg_i32x4 stg[2][16];
-  Frag fa[2][4];
+  Frag fa[2][4];                                        // A fragments, k-contiguous form
+  short4v fat[2][4][2];                                 // k-strided form
   Frag fbr[2][4];                                       // B fragments, k-contiguous form
   short4v fbt[2][4][2];                                 // k-strided form: the two transpose reads of a fragment
 
@@ -426,7 +462,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     else asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_b), "s"(rsb), "s"(kb + (idx - 8) * rstep_b) : "memory");
   };
   auto swrite = [&](int set, int idx, uint32_t stage) {  // stage: LDS byte address of the stage
-    if (idx < 8) *(lds_w)(stage + wr_a + idx * 4096) = stg[set][idx];
+    if (idx < 8 && !AKS) *(lds_w)(stage + wr_a + idx * 4096) = stg[set][idx];
+    else if (idx < 8) *(lds_w)(((stage + wr_a) ^ (uint32_t)((idx & 1) << 5)) + idx * 4096) = stg[set][idx];
     else if (!BKS) *(lds_w)(stage + wr_b + (idx - 8) * 4096) = stg[set][idx];
     else *(lds_w)(((stage + wr_b) ^ (uint32_t)(((idx - 8) & 1) << 5)) + (idx - 8) * 4096) = stg[set][idx];
   };
@@ -437,6 +474,14 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
       if (!isb[r]) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
       else fbr[set][blk[r]] = *(lds_frag)(((stage + fb_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+    } else if constexpr (AKS) {
+      // B0 A0 B1 B2 B3 A1 A2 A3, two transpose reads each
+      constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
+      const int f = r >> 1, half = r & 1;
+      const uint32_t lane_addr = isb[f] ? (half ? tb_b : tb_a) : (half ? ta_b : ta_a);
+      const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + lane_addr) ^ (uint32_t)(blk[f] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+      if (isb[f]) fbt[set][blk[f]][half] = x;
+      else fat[set][blk[f]][half] = x;
     } else {
       constexpr int kind[12] = {1, 2, 0, 1, 2, 1, 2, 1, 2, 0, 0, 0}, blk[12] = {0, 0, 0, 1, 1, 2, 2, 3, 3, 1, 2, 3};
       if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
@@ -482,19 +527,25 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
 #pragma unroll
     for (int mi = 0; mi < 64; ++mi) {
       const int ks = mi >> 4, i = (mi >> 2) & 3, j = mi & 3, q = mi & 15;
-      if constexpr (BKS) acc[i][j] = M::mma(frag_join<T>(fbt[ks & 1][j][0], fbt[ks & 1][j][1]), fa[ks & 1][i], acc[i][j]);
+      if constexpr (AKS) acc[i][j] = M::mma(frag_join<T>(fbt[ks & 1][j][0], fbt[ks & 1][j][1]), frag_join<T>(fat[ks & 1][i][0], fat[ks & 1][i][1]), acc[i][j]);
+      else if constexpr (BKS) acc[i][j] = M::mma(frag_join<T>(fbt[ks & 1][j][0], fbt[ks & 1][j][1]), fa[ks & 1][i], acc[i][j]);
       else acc[i][j] = M::mma(fbr[ks & 1][j], fa[ks & 1][i], acc[i][j]);
       // fragment reads of the next k step, spread over the quarter (the last quarter: behind the barrier, from the next stage)
       if (ks < 3) {
         if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, cur, ks + 1); }
-        else { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1); }
+        else if (NRD == 12) { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1); }
+        else fread((ks + 1) & 1, q, cur, ks + 1);
       } else if (!LAST) {
         if (mi == 50) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         if (NRD == 8) {
           if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, nxt, 0);
           if (mi == 63) fread(0, 7, nxt, 0);
-        } else {
+        } else if (NRD == 12) {
           if (mi >= 50 && mi < 62) fread(0, mi - 50, nxt, 0);
+        } else {
+          if (mi >= 50) fread(0, mi - 50, nxt, 0);
+          if (mi == 50) fread(0, 14, nxt, 0);
+          if (mi == 51) fread(0, 15, nxt, 0);
         }
       }
       if (!LAST && mi < 32 && mi % 2 == 1) {            // LDS writes of slice s + 1: the older of the two sets in flight
@@ -541,11 +592,19 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     __syncthreads();                                    // the next segment's copies reuse the stages
     return;
   }
-  gg_w4_store<T>(acc, smem, p, m0, n0, a_rext, b_rext);
+  gg_w4_store<T, AKS>(acc, smem, p, AKS ? reinterpret_cast<T *>(p.c) + (int64_t)g * p.c_group_stride : reinterpret_cast<T *>(p.c), m0, n0, a_rext, b_rext);
     __syncthreads();                                    // the next segment's copies reuse the staging area
   };
 
-  if constexpr (!SK) {
+  if constexpr (AKS) {
+    // one output of tiles_m x tiles_n tiles per group (blockIdx.y); k = the group's rows, the last slice cut there
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int pid = blockIdx.x;
+    if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+    const int g = blockIdx.y;
+    const int rb = gg_clamp_row(p.offs[g] - base, p.max_rows), re = gg_clamp_row(p.offs[g + 1] - base, p.max_rows);
+    segment(g, rb, re, pid % p.tiles_m, pid / p.tiles_m, 0, (re - rb + 63) / 64, nullptr);
+  } else if constexpr (!SK) {
     const int ntiles = p.tiles_m * p.tiles_n;
     int pid = blockIdx.x;
     if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
@@ -658,6 +717,14 @@ __global__ void __launch_bounds__(256) gg_split_reduce_kernel(const GGParams p, 
 constexpr int GG_SK_MAX_GRID = 256;
 constexpr size_t GG_SK_WS_BYTES = (size_t)GG_SK_MAX_GRID * 256 * 256 * sizeof(float);
 
+template <typename T>
+static int launch_gg_w4_tn(GGParams p, hipStream_t st) {
+  p.tiles_m = (int)(p.m_dim / 256);
+  p.tiles_n = (int)(p.n_dim / 256);
+  hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, 2, false>), dim3((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.groups), dim3(256), 0, st, p);
+  return DH_OK;
+}
+
 template <typename T, bool BKS>
 static int launch_gg_w4(GGParams p, int64_t m_extent, void *workspace, size_t workspace_bytes, hipStream_t st) {
   p.tiles_n = (int)cdiv(p.n_dim, 256);
@@ -678,10 +745,10 @@ static int launch_gg_w4(GGParams p, int64_t m_extent, void *workspace, size_t wo
   if (grid > 0 && 2 * (int64_t)p.tiles_m * p.tiles_n > 3 * (int64_t)grid) grid = 0;
   if (grid > 0) {
     p.ws = reinterpret_cast<float *>(workspace);
-    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS, true>), dim3((unsigned)grid), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS ? 1 : 0, true>), dim3((unsigned)grid), dim3(256), 0, st, p);
     hipLaunchKernelGGL((gg_split_reduce_kernel<T>), dim3((unsigned)(16 * grid / 2)), dim3(256), 0, st, p, grid);   // at most grid / 2 tiles are split
   } else {
-    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS, false>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
+    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS ? 1 : 0, false>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
   }
   return DH_OK;
 }
@@ -809,7 +876,11 @@ extern "C" int dh_grouped_gemm_tn(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.m_dim = m; p.n_dim = n; p.lda = m; p.ldb = n; p.ldc = n;
   p.c_group_stride = m * n; p.accumulate = accumulate; p.max_rows = (int)max_rows;
-  rc = dispatch_gg<true, true, true>(p, m, dtype, (hipStream_t)stream);
+  // whole 256x256 tiles, enough of them to fill the chip, and offsets that fit the 32-bit buffer addressing
+  if (m % 256 == 0 && n % 256 == 0 && (m / 256) * (n / 256) * groups >= 256 && max_rows * (m > n ? m : n) * (int64_t)dtype_size(dtype) < (1ll << 31))
+    rc = dtype == DH_BF16 ? launch_gg_w4_tn<bf16_t>(p, (hipStream_t)stream) : launch_gg_w4_tn<f16_t>(p, (hipStream_t)stream);
+  else
+    rc = dispatch_gg<true, true, true>(p, m, dtype, (hipStream_t)stream);
   if (rc) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;

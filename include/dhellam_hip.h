@@ -37,7 +37,8 @@ typedef enum {
 
 /* Library version (major*100 + minor).  2.0: dh_attn_bwd, dh_attn_bwd_acc,
  * dh_norm_bwd and dh_moe_sort take the size of the caller's workspace and
- * check it (1.x trusted the caller). */
+ * check it (1.x trusted the caller); dh_grouped_gemm_nt / _nn take an optional
+ * workspace. */
 int dh_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *dh_last_error(void);

@@ -340,16 +340,16 @@ def test_expert_ffn_bwd_with_resident_weight_transposes():
     assert torch.equal(_Clib.transposed_of(w2), w2.transpose(1, 2).contiguous())
 
 
-@pytest.mark.parametrize("K", [192, 1024])
-@pytest.mark.parametrize("form", ["nt", "nn"])
-def test_grouped_gemm_split_last_round(form, K):
+@pytest.mark.parametrize("form,K,N", [("nt", 192, 4096), ("nt", 1024, 4096), ("nn", 192, 4096), ("nn", 1024, 4096),
+                                      ("nt", 320, 4232)])     # n ends inside a tile: 4232 = 16 * 256 + 136
+def test_grouped_gemm_split_last_round(form, K, N):
     """The chip-filling kernels through the C ABI, with and without a workspace (last round split along k / one workgroup per tile):
     both within the bound of the fp64 product, the split result the same on every run, rows cut off at max_rows
     (the offsets describe more rows than the operands hold), nothing written past them."""
     from dhellam_amd import _lib
     lib = _lib.load()
     dt = torch.bfloat16
-    rows, N = [2100, 0, 1990, 37, 500], 4096
+    rows = [2100, 0, 1990, 37, 500]
     G, R = len(rows), sum(rows)
     max_rows, guard = 4200, 64                      # the last group is cut off: 73 of its 500 rows exist
     offs_np = np.concatenate(([5], 5 + np.cumsum(rows))).astype(np.int32)

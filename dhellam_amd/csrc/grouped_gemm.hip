@@ -608,8 +608,12 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     const int ntiles = p.tiles_m * p.tiles_n;
     int pid = blockIdx.x;
     if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-    int tm = pid % p.tiles_m;
-    const int tn = pid / p.tiles_m;
+    // Inside an XCD's run of tiles: bands of 8 m tiles, n fastest inside a band, so that the 32 tiles an XCD has
+    // in flight are 8 x 4 and share 12 operand panels through its L2 instead of 18 + 2 (1-2 % on the FFN products).
+    constexpr int GM = 8;
+    const int band = pid / (GM * p.tiles_n), first = band * GM, gm = min(GM, p.tiles_m - first);
+    int tm = first + (pid - band * GM * p.tiles_n) % gm;
+    const int tn = (pid - band * GM * p.tiles_n) / gm;
     for (int gi = 0; gi < p.groups; ++gi) {
       const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
       const int t = (re - rb + BM - 1) / BM;

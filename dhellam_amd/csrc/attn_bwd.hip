@@ -844,7 +844,13 @@ __global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdPar
 #pragma unroll
     for (int x = 0; x < 4; ++x) cp_off[x] = rowb + (chunk ^ (uint32_t)(x << 4));
   }
-  const uint32_t ds_lane = (uint32_t)lane * 16u;
+  // The dK/dV kernel wrote a dS block as two fragments of 64 lanes x 16 bytes (piece 64 s + L is lane L of fragment
+  // s).  The transpose reads below fetch, per instruction, the pieces L = 32 b + 8 t + 4 hh + j of both fragments
+  // (t fixed; j = 0..3, b = 0..1): copied as they lie, the four 64-byte runs (s, b) of a half wavefront fall on the
+  // same 16 banks.  So the copy permutes: LDS position 64 hh + 16 t + 8 s + 4 b + j holds that piece (lane l of the
+  // copy for half hh fetches the piece with j = l % 4, b = l / 4 % 2, s = l / 8 % 2, t = l / 16), and the 16 pieces of
+  // a half wavefront's read are 256 consecutive bytes.
+  const uint32_t ds_lane = 16u * (uint32_t)(64 * ((lane >> 3) & 1) + 32 * ((lane >> 2) & 1) + 8 * ((lane >> 4) & 3) + (lane & 3));
   const int64_t ds_head = ((int64_t)b * p.hq + h) * p.ds_nqt;
   const char *ds_b = reinterpret_cast<const char *>(p.ds);
 
@@ -856,8 +862,8 @@ __global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdPar
   const uint32_t ta_lane = t_row + (uint32_t)((t_lc ^ ta_x) << 4);
   const uint32_t tb_lane = t_row + 8 * 256 + (uint32_t)((t_lc ^ (ta_x + 2)) << 4);
   // dS block: piece (s = 16-lane group, hh_p = r % 2) of key 4 hh + r / 4, half u = (r % 4) / 2 of the piece
-  const uint32_t db_lane = (uint32_t)(sp * DSB + rg * 2048 + ((((lane >> 4) & 1) * 64 + (r & 1) * 32 + 4 * hh + (r >> 2)) * 16) +
-                                      ((r & 3) >> 1) * 8);
+  const uint32_t db_lane = (uint32_t)(sp * DSB + rg * 2048 + ((64 * hh + 8 * ((lane >> 4) & 1) + 4 * (r & 1) + (r >> 2)) * 16) +
+                                      ((r & 3) >> 1) * 8);        // + 256 t
 
   for (int qi = 0; qi < nq; ++qi) {
     const int m0 = qt[qi] * BM;
@@ -897,7 +903,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdPar
       const char *dsrc = ds_b + (ds_row + tile) * 2048;
       const uint32_t ddst = ldsD + stD + (uint32_t)(csp * DSB + half * 2048);
       dma_block_fast(dsrc, ds_lane, ddst);
-      dma_block_fast(dsrc + 1024, ds_lane, ddst + 1024);
+      dma_block_fast(dsrc + 64, ds_lane, ddst + 1024);
     };
 
     // Steps 0 and 1 go out now; in the loop, step it + 2 goes out at the top of step it and the wait at the bottom
@@ -930,7 +936,7 @@ __global__ void __launch_bounds__(512) attn_bwd_dq2_d128_kernel(const AttnBwdPar
           ad[2 * t + 1] = tb ^ (uint32_t)(t << 6);
         }
         short4v bq[4], f0[8], f1[8];
-        lds_read_tr4<128>(bq, db);
+        lds_read_tr4<256>(bq, db);
         lds_read_tr8<0>(f0, ad);
         lds_wait<4>(bq[0], bq[1], bq[2], bq[3]);
         lds_wait<4>(f0[0], f0[1], f0[2], f0[3]);

@@ -82,6 +82,91 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     return LIB_PATH
 
 
+def check_grouped_gemm_loops(verbose: bool = False) -> int:
+    """The chip-filling grouped GEMM kernel (``grouped_gemm_w4_kernel``) issues its loads from assembly, so the compiler
+    does not know that their results arrive later: the kernel is only correct if, between a load and the LDS write
+    that consumes it, NO instruction names the loaded registers (a register copy or a spill there would move data
+    that has not arrived).  The source arranges that; this check holds the generated code to it.  It compiles
+    ``grouped_gemm.hip`` to device assembly and, in the main loop of every instantiation of the kernel (the innermost
+    loop with 32 loads), follows each ``buffer_load_dwordx4`` destination to its ``ds_write_b128`` across the loop's
+    back edge; it also refuses scratch accesses and register copies inside that loop.  Returns the number of loops
+    checked; raises on a violation."""
+    import re
+    import tempfile
+    with tempfile.TemporaryDirectory() as td:
+        out = Path(td) / "gg.s"
+        cmd = [HIPCC, *[f for f in CXXFLAGS if f != "-fPIC"], "--cuda-device-only", "-S", str(CSRC / "grouped_gemm.hip"), "-o", str(out)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc -S failed for grouped_gemm.hip:\n" + res.stderr)
+        lines = out.read_text().split("\n")
+
+    def regs(tok: str) -> set:
+        m = re.match(r"v\[(\d+):(\d+)\]$", tok)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.match(r"v(\d+)$", tok)
+        return {int(m.group(1))} if m else set()
+
+    checked = 0
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_ZN2dh22grouped_gemm_w4_kernel\w+:", l)]
+    for a in starts:
+        b = next(i for i in range(a, len(lines)) if "s_endpgm" in lines[i])
+        fn = lines[a:b]
+        labels = {m.group(1): i for i, l in enumerate(fn) if (m := re.match(r"^(\.LBB\d+_\d+):", l))}
+        loops = []
+        for i, l in enumerate(fn):
+            m = re.match(r"\s+s_cbranch_\w+ (\.LBB\d+_\d+)", l)
+            if m and m.group(1) in labels and labels[m.group(1)] < i:
+                body = fn[labels[m.group(1)]:i]
+                if sum("buffer_load_dwordx4" in x for x in body) == 32:
+                    loops.append(body)
+        if not loops:
+            raise RuntimeError(f"{fn[0].split(':')[0]}: no main loop with 32 loads found (the kernel's structure changed: "
+                               "update check_grouped_gemm_loops)")
+        body = min(loops, key=len)
+        name = fn[0].split(":")[0]
+        for l in body:
+            if "scratch_" in l or re.match(r"\s+v_mov_b\d+", l) or "v_accvgpr" in l:
+                raise RuntimeError(f"{name}: '{l.strip()}' inside the main loop")
+        if sum("v_mfma" in x for x in body) != 128:
+            raise RuntimeError(f"{name}: {sum('v_mfma' in x for x in body)} MFMAs in the main loop, expected 128")
+        # the same rule from the first load of the function up to the loop (the prologue's loads, whose results the
+        # loop's first slices write to LDS) and from the loop's end to the wait for every load that follows it
+        lo = next(i for i, l in enumerate(fn) if l is body[0])
+        first = next(i for i, l in enumerate(fn) if "buffer_load_dwordx4" in l)
+        hi = lo + len(body)
+        end = next((i for i in range(hi, len(fn)) if "s_waitcnt vmcnt(0)" in fn[i]), None)
+        if first >= lo or end is None:
+            raise RuntimeError(f"{name}: prologue loads or the wait behind the loop not found")
+        pending: dict = {}
+        for n, l in enumerate(fn[first:lo] + body + body + fn[hi:end]):   # the loop twice: values live across the back edge
+            t = l.replace(",", " ").split()
+            if not t or t[0].startswith((";", ".")):
+                continue
+            if t[0] == "buffer_load_dwordx4":
+                for r in regs(t[1]):
+                    if r in pending:
+                        raise RuntimeError(f"{name}: v{r} is loaded again before the LDS write of its previous load")
+                    pending[r] = n
+                continue
+            if t[0] == "s_waitcnt" and "vmcnt(0)" in l:     # everything has arrived
+                pending.clear()
+                continue
+            touched = set().union(*[regs(x) for x in t[1:]]) & set(pending)
+            if touched:
+                if t[0] != "ds_write_b128":
+                    raise RuntimeError(f"{name}: '{l.strip()}' names a register whose load may still be in flight")
+                for r in touched:
+                    pending.pop(r)
+        checked += 1
+        if verbose:
+            print(f"checked {name}: {len(body)} lines", flush=True)
+    if checked == 0:
+        raise RuntimeError("no grouped_gemm_w4_kernel instantiation found in the assembly")
+    return checked
+
+
 EXT_SRC = CSRC / "torchapi.cpp"
 EXT_PKG = ROOT / "dhellam"
 
@@ -126,5 +211,6 @@ def build_torch_extension(verbose: bool = False) -> Path:
 if __name__ == "__main__":
     path = build(verbose="-v" in sys.argv)
     print(path)
+    print(f"grouped GEMM main loops checked: {check_grouped_gemm_loops(verbose='-v' in sys.argv)}")
     if "--no-ext" not in sys.argv:
         print(build_torch_extension(verbose="-v" in sys.argv))

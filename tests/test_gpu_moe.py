@@ -381,3 +381,27 @@ def test_grouped_gemm_split_last_round(form, K, N):
                   ws.data_ptr(), 1 << 20, st))
     torch.cuda.synchronize()
     assert torch.equal(c, outs[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_grouped_gemm_tn_chip_filling(dtype):
+    """Weight-gradient products large enough for the 256x256-tile kernel (m, n multiples of 256, >= 256 tiles): an
+    empty group (its output must be zeros), groups of 1, 65 and 300 rows (k not a multiple of the 64-deep slice),
+    rows of the operands past the last group (not read), accumulation into an existing output, same result twice."""
+    from dhellam_amd.operators import moe
+    rows, M, N = [300, 0, 65, 1], 4096, 2048
+    G, R = len(rows), sum(rows)
+    offs = torch.tensor(np.concatenate(([3], 3 + np.cumsum(rows))), dtype=torch.int32).cuda()
+    a = randn((R + 7, M), dtype, 21, std=0.5).cuda()
+    b = randn((R + 7, N), dtype, 22, std=0.5).cuda()
+    st = np.concatenate(([0], np.cumsum(rows)))
+    ref = torch.stack([a[st[g]:st[g + 1]].cpu().double().T @ b[st[g]:st[g + 1]].cpu().double() for g in range(G)])
+    w = moe.grouped_gemm_tn(a, b, offs)
+    assert_close(w, ref, dtype, "TN")
+    assert bool((w[1] == 0).all()), "empty group"
+    assert torch.equal(w, moe.grouped_gemm_tn(a, b, offs))
+    acc0 = randn((G, M, N), dtype, 23)
+    acc = acc0.clone().cuda()
+    moe.grouped_gemm_tn(a, b, offs, out=acc, accumulate=True)
+    assert_close(acc, ref + acc0.double(), dtype, "TN accumulate")
+    assert torch.equal(acc[1].cpu(), acc0[1]), "accumulating an empty group must leave the output as it was"

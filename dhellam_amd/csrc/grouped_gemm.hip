@@ -278,7 +278,8 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
 //
 // The loads are buffer loads issued from assembly: the compiler does not count them, every use of a staging
 // register is ordered by a hand-written s_waitcnt vmcnt (loads return in order), and between its load and its
-// LDS write a staging register is touched by nothing else.  The buffer descriptors do the edge handling: their
+// LDS write a staging register is touched by nothing else (every build checks the generated assembly for this:
+// check_grouped_gemm_loops in dhellam_amd/build.py).  The buffer descriptors do the edge handling: their
 // length is cut at the group's (or n's) last row, so that rows past the end read as zero and no access leaves
 // the operands, whatever the offsets table says.
 typedef int gg_i32x4 __attribute__((ext_vector_type(4)));

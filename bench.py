@@ -48,26 +48,36 @@ def _ensure_built():
         build()
 
 
-def time_gpu(fn, iters=20, warmup=3, stream=None):
-    """Median-free mean ms per call of fn() measured with HIP events recorded on the stream
-    the kernels are launched on."""
+def time_gpu(fn, iters=20, warmup=3, stream=None, min_ms=50.0):
+    """Mean ms per call of fn() measured with HIP events recorded on the stream the kernels are
+    launched on.  The chip's clock follows the load of the last tens of milliseconds (a kernel timed
+    right after idle or after light kernels runs 10-20 % slower than in a loop that has been going
+    for a while), so a timing that covers less than ``min_ms`` counts as warm-up and is repeated with
+    as many calls as fill that time."""
     stream = stream or torch.cuda.current_stream()
     for _ in range(warmup):
         fn()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
-    start.record(stream)
-    for _ in range(iters):
-        fn()
-    end.record(stream)
-    end.synchronize()
-    return start.elapsed_time(end) / iters
+    for attempt in range(4):                              # the first pass is warm-up whatever it covers
+        start.record(stream)
+        for _ in range(iters):
+            fn()
+        end.record(stream)
+        end.synchronize()
+        total = start.elapsed_time(end)
+        if total >= min_ms and attempt > 0:
+            break
+        if total < min_ms:
+            iters = min(20000, int(iters * min_ms / max(total, 1e-3) * 1.2) + 1)
+    return total / iters
 
 
-def time_gpu_graph(fn, iters=20):
-    """Mean ms per call with ``iters`` calls captured in one HIP graph and the replay bracketed by
+def time_gpu_graph(fn, iters=50, min_ms=20.0):
+    """Mean ms per call with ``iters`` calls captured in one HIP graph and the replays bracketed by
     HIP events on the replay stream: for kernels of a few microseconds this measures the kernels,
-    not the Python launch path."""
+    not the Python launch path.  The graph is replayed for ``min_ms`` untimed (clock settled, as in
+    time_gpu) and then for ``min_ms`` timed."""
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(s):
@@ -78,16 +88,22 @@ def time_gpu_graph(fn, iters=20):
         with torch.cuda.graph(g, stream=s):
             for _ in range(iters):
                 fn()
-        g.replay()
-        torch.cuda.synchronize()
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
         start.record(s)
         g.replay()
         end.record(s)
         end.synchronize()
+        reps = max(1, min(2000, int(min_ms / max(start.elapsed_time(end), 1e-3)) + 1))
+        for _ in range(reps):
+            g.replay()
+        start.record(s)
+        for _ in range(reps):
+            g.replay()
+        end.record(s)
+        end.synchronize()
     torch.cuda.current_stream().wait_stream(s)
-    return start.elapsed_time(end) / iters
+    return start.elapsed_time(end) / (iters * reps)
 
 
 def kernel_rooflines(cfg):
@@ -646,6 +662,8 @@ def main():
                     help="plan JSON for the double-strand schedule; default: the plan the search's execute stage "
                          "emitted (dhellam_amd/search/config/best.json) when there is one, else the built-in plan; "
                          "'builtin' forces the built-in plan")
+    ap.add_argument("--profile-iters", type=int, default=5,
+                    help="launches of --profile-op (a few hundred put a kernel trace's average at the settled clock)")
     ap.add_argument("--profile-op", default=None,
                     help="run only this operator a few times (attn_fwd, attn_bwd, ring_fwd, ring_bwd, moe_ffn_fwd, moe_ffn_bwd, norm, swiglu, swiglu_t, cross_entropy, transpose, rope, residual_add, add_norm, norm_shard, merge, permute, unpermute, copy_shard, gg_nt, gemm_nt, layer, copy) and exit")
     ap.add_argument("--analyze-trace", default=None,
@@ -665,7 +683,7 @@ def main():
     _ensure_built()
     if args.profile_op:
         torch.cuda.set_device(0)
-        profile_op(args.profile_op)
+        profile_op(args.profile_op, args.profile_iters)
         return
     from dhellam_amd.core.layer import LayerRunner, llama70b_tp8_shard, make_microbatch, make_weights
     torch.cuda.set_device(0)

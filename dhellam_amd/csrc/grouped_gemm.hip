@@ -38,6 +38,7 @@ struct GGParams {
   int accumulate;
   int max_rows;          // rows the stacked operands hold: group ranges read from offs are cut off there
   float *ws;             // split last round: fp32 partial tiles, one per workgroup
+  int zero_tail;         // NT/NN on grouped_gemm_w4_kernel: the kernel itself zeroes the rows of c past the last group
 };
 
 // A group's row range as the kernels use it: relative to the first group and never past the rows the caller's
@@ -366,6 +367,13 @@ __device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigne
   }
 }
 
+// Workgroup ids go round the 8 XCDs; this gives XCD x (the ids x, x + 8, ...) the x-th of 8 contiguous chunks of
+// 0..n-1, so that neighbouring tiles share an L2 (a bijection for any n: the first n % 8 chunks are one longer).
+__device__ __forceinline__ int gg_xcd_chunk(int id, int n) {
+  const int q8 = n / 8, r8 = n % 8, x = id % 8;
+  return x * q8 + (x < r8 ? x : r8) + id / 8;
+}
+
 // k pieces per tile of the last round: as many as there are workgroups per tile, each at least one slice.
 __device__ __forceinline__ int gg_sk_pieces(int grid, int rem, int nsl) {
   if (rem <= 0) return 1;
@@ -393,6 +401,19 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const uint32_t lda_b = (uint32_t)p.lda * (uint32_t)sizeof(T), ldb_b = (uint32_t)p.ldb * (uint32_t)sizeof(T);
   const int base = p.offs[0];
+
+  // Rows of c past the last group, up to max_rows (usually none): zeroed here, a row per workgroup at a time, instead
+  // of by a kernel of its own in front of this one (5 us per product).
+  if constexpr (!AKS) {
+    if (p.zero_tail) {
+      const int first = gg_clamp_row(p.offs[p.groups] - base, p.max_rows);
+      const int nv = (int)(p.n_dim / 8);
+      for (int r = first + (int)blockIdx.x; r < p.max_rows; r += (int)gridDim.x) {
+        T *row = reinterpret_cast<T *>(p.c) + (int64_t)r * p.ldc;
+        for (int v = tid; v < nv; v += 256) *reinterpret_cast<dh_u32x4 *>(row + 8 * v) = dh_u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  }
 
   // ---- copies ----------------------------------------------------------------------------------------------
   // k-contiguous tile [256 rows][64 k]: a lane copies chunk lc of rows lr + 32 i.
@@ -462,19 +483,21 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     if (idx < 8) asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_a), "s"(rsa), "s"(ka + idx * rstep_a) : "memory");
     else asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(stg[set][idx]) : "v"(goff_b), "s"(rsb), "s"(kb + (idx - 8) * rstep_b) : "memory");
   };
-  auto swrite = [&](int set, int idx, uint32_t stage) {  // stage: LDS byte address of the stage
-    if (idx < 8 && !AKS) *(lds_w)(stage + wr_a + idx * 4096) = stg[set][idx];
+  // kc_w / kc_a / kc_b: the stage's lane addresses for the k-contiguous operands' writes and fragment reads, formed once
+  // per slice and kept in registers (left to the compiler they are re-added in front of every LDS instruction)
+  auto swrite = [&](int set, int idx, uint32_t stage, uint32_t kc_w) {  // stage: LDS byte address of the stage
+    if (idx < 8 && !AKS) *(lds_w)(kc_w + idx * 4096) = stg[set][idx];
     else if (idx < 8) *(lds_w)(((stage + wr_a) ^ (uint32_t)((idx & 1) << 5)) + idx * 4096) = stg[set][idx];
-    else if (!BKS) *(lds_w)(stage + wr_b + (idx - 8) * 4096) = stg[set][idx];
+    else if (!BKS) *(lds_w)(kc_w + TILEB + (idx - 8) * 4096) = stg[set][idx];
     else *(lds_w)(((stage + wr_b) ^ (uint32_t)(((idx - 8) & 1) << 5)) + (idx - 8) * 4096) = stg[set][idx];
   };
   // read r of a k step, in the order in which the MFMAs first need the data: B0 A0 B1 B2 B3 A1 A2 A3 (a k-strided
   // B fragment is two transpose reads).  abase/bbase: lane addresses of the stage with the k step applied.
-  auto fread = [&](int set, int r, uint32_t stage, int ks) {
+  auto fread = [&](int set, int r, uint32_t stage, int ks, uint32_t kc_a, uint32_t kc_b) {
     if constexpr (!BKS) {
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
-      if (!isb[r]) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
-      else fbr[set][blk[r]] = *(lds_frag)(((stage + fb_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      if (!isb[r]) fa[set][blk[r]] = *(lds_frag)((kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      else fbr[set][blk[r]] = *(lds_frag)((kc_b ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
     } else if constexpr (AKS) {
       // B0 A0 B1 B2 B3 A1 A2 A3, two transpose reads each
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
@@ -485,7 +508,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       else fat[set][blk[f]][half] = x;
     } else {
       constexpr int kind[12] = {1, 2, 0, 1, 2, 1, 2, 1, 2, 0, 0, 0}, blk[12] = {0, 0, 0, 1, 1, 2, 2, 3, 3, 1, 2, 3};
-      if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)(((stage + fa_lane) ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)((kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
       else if (kind[r] == 1)
         fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + tb_a) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
       else
@@ -503,7 +526,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   for (int x = 0; x < 16; ++x) gload(1, x, kof(1) * kstep_a, kof(1) * kstep_b);
   asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
 #pragma unroll
-  for (int x = 0; x < 16; ++x) swrite(0, x, lds0);
+  for (int x = 0; x < 16; ++x) swrite(0, x, lds0, lds0 + wr_kc);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   // issue order of a staging set inside the loop: 0..7, 15, 8..14
 #pragma unroll
@@ -513,7 +536,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   for (int x = 8; x < 15; ++x) gload(0, x, kof(2) * kstep_a, kof(2) * kstep_b);
   asm volatile("s_barrier" ::: "memory");
 #pragma unroll
-  for (int x = 0; x < NRD; ++x) fread(0, x, lds0, 0);
+  for (int x = 0; x < NRD; ++x) fread(0, x, lds0, 0, lds0 + fa_lane, lds0 + fb_lane);
 
   // Slice s reads stage s % 2, writes slice s + 1 (staging set (s + 1) % 2, loaded two slices ago) into the other
   // stage during its first half and then loads slice s + 3 into the same set.
@@ -524,6 +547,9 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     uint32_t cur = lds0 + (uint32_t)(st * STAGEB), nxt = lds0 + (uint32_t)((st ^ 1) * STAGEB);
     const uint32_t ka = kof(s + 3) * kstep_a, kb = kof(s + 3) * kstep_b;
     asm volatile("" : "+s"(cur), "+s"(nxt));
+    uint32_t ac = cur + fa_lane, bc = cur + fb_lane, an = nxt + fa_lane, bn = nxt + fb_lane, wn_ = nxt + wr_kc;
+    if constexpr (!AKS) asm volatile("" : "+v"(ac), "+v"(an), "+v"(wn_));
+    if constexpr (!BKS) asm volatile("" : "+v"(bc), "+v"(bn));
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mi = 0; mi < 64; ++mi) {
@@ -533,27 +559,27 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       else acc[i][j] = M::mma(fbr[ks & 1][j], fa[ks & 1][i], acc[i][j]);
       // fragment reads of the next k step, spread over the quarter (the last quarter: behind the barrier, from the next stage)
       if (ks < 3) {
-        if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, cur, ks + 1); }
-        else if (NRD == 12) { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1); }
-        else fread((ks + 1) & 1, q, cur, ks + 1);
+        if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, cur, ks + 1, ac, bc); }
+        else if (NRD == 12) { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1, ac, bc); }
+        else fread((ks + 1) & 1, q, cur, ks + 1, ac, bc);
       } else if (!LAST) {
         if (mi == 50) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         if (NRD == 8) {
-          if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, nxt, 0);
-          if (mi == 63) fread(0, 7, nxt, 0);
+          if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, nxt, 0, an, bn);
+          if (mi == 63) fread(0, 7, nxt, 0, an, bn);
         } else if (NRD == 12) {
-          if (mi >= 50 && mi < 62) fread(0, mi - 50, nxt, 0);
+          if (mi >= 50 && mi < 62) fread(0, mi - 50, nxt, 0, an, bn);
         } else {
-          if (mi >= 50) fread(0, mi - 50, nxt, 0);
-          if (mi == 50) fread(0, 14, nxt, 0);
-          if (mi == 51) fread(0, 15, nxt, 0);
+          if (mi >= 50) fread(0, mi - 50, nxt, 0, an, bn);
+          if (mi == 50) fread(0, 14, nxt, 0, an, bn);
+          if (mi == 51) fread(0, 15, nxt, 0, an, bn);
         }
       }
       if (!LAST && mi < 32 && mi % 2 == 1) {            // LDS writes of slice s + 1: the older of the two sets in flight
         const int k = mi / 2;
         if (k == 0) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
         if (k == 8) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        swrite(X ^ 1, k, nxt);
+        swrite(X ^ 1, k, nxt, wn_);
       }
       if (!LAST && mi >= 33 && mi <= 61 && mi % 2 == 1) gload(X ^ 1, (mi - 33) / 2, ka, kb);
       if (!LAST && mi == 48) gload(X ^ 1, 15, ka, kb);
@@ -601,18 +627,23 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     // one output of tiles_m x tiles_n tiles per group (blockIdx.y); k = the group's rows, the last slice cut there
     const int ntiles = p.tiles_m * p.tiles_n;
     int pid = blockIdx.x;
-    if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+    pid = gg_xcd_chunk(pid, ntiles);
     const int g = blockIdx.y;
     const int rb = gg_clamp_row(p.offs[g] - base, p.max_rows), re = gg_clamp_row(p.offs[g + 1] - base, p.max_rows);
     segment(g, rb, re, pid % p.tiles_m, pid / p.tiles_m, 0, (re - rb + 63) / 64, nullptr);
   } else if constexpr (!SK) {
-    const int ntiles = p.tiles_m * p.tiles_n;
-    int pid = blockIdx.x;
-    if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-    // Inside an XCD's run of tiles: bands of 8 m tiles, n fastest inside a band, so that the 32 tiles an XCD has
+    // The grid is sized for the host's upper bound of the tile count (it does not know how the rows split into
+    // groups); the chunks of the XCDs are cut from the real count, so that every XCD gets its share of real tiles.
+    int tiles_m = 0;
+    for (int gi = 0; gi < p.groups; ++gi)
+      tiles_m += (gg_clamp_row(p.offs[gi + 1] - base, p.max_rows) - gg_clamp_row(p.offs[gi] - base, p.max_rows) + BM - 1) / BM;
+    const int ntiles = tiles_m * p.tiles_n;
+    if ((int)blockIdx.x >= ntiles) return;
+    const int pid = gg_xcd_chunk((int)blockIdx.x, ntiles);
+    // Inside an XCD's run of tiles: bands of 8 m tiles, m fastest inside a band, so that the 32 tiles an XCD has
     // in flight are 8 x 4 and share 12 operand panels through its L2 instead of 18 + 2 (1-2 % on the FFN products).
     constexpr int GM = 8;
-    const int band = pid / (GM * p.tiles_n), first = band * GM, gm = min(GM, p.tiles_m - first);
+    const int band = pid / (GM * p.tiles_n), first = band * GM, gm = min(GM, tiles_m - first);
     int tm = first + (pid - band * GM * p.tiles_n) % gm;
     const int tn = (pid - band * GM * p.tiles_n) / gm;
     for (int gi = 0; gi < p.groups; ++gi) {
@@ -638,7 +669,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     const int grid = (int)gridDim.x, full = tiles / grid, rem = tiles - full * grid;
     const int pieces = gg_sk_pieces(grid, rem, nsl);
     int wg = blockIdx.x;
-    if (grid % 8 == 0) wg = (wg % 8) * (grid / 8) + wg / 8;            // neighbouring tiles on one XCD
+    wg = gg_xcd_chunk(wg, grid);                                       // neighbouring tiles on one XCD
     const int rounds = full + (wg < rem * pieces ? 1 : 0);
 #pragma unroll 1
     for (int it = 0; it < rounds; ++it) {
@@ -735,6 +766,7 @@ static int launch_gg_w4(GGParams p, int64_t m_extent, void *workspace, size_t wo
   p.tiles_n = (int)cdiv(p.n_dim, 256);
   p.tiles_m = (int)(cdiv(m_extent, 256) + p.groups);
   if (p.tiles_m <= 0 || p.tiles_n <= 0) return DH_OK;
+  p.zero_tail = 1;
   int grid = 0;
   if (workspace != nullptr && p.k_dim >= 64) {
     int dev = 0, cus = 0;
@@ -832,13 +864,14 @@ extern "C" int dh_grouped_gemm_nt(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = k; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
-  gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
-  if (big && k % 64 == 0 && k <= (1ll << 21))
+  if (big && k % 64 == 0 && k <= (1ll << 21)) {
     rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, false>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream)
                           : launch_gg_w4<f16_t, false>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream);
-  else
+  } else {
+    gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
     rc = dispatch_gg<false, false, false>(p, max_rows, dtype, (hipStream_t)stream);
+  }
   if (rc) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;
@@ -857,13 +890,14 @@ extern "C" int dh_grouped_gemm_nn(const void *a, const void *b, void *c, const i
   p.a = a; p.b = b; p.c = c; p.offs = offs; p.groups = groups;
   p.n_dim = n; p.k_dim = k; p.lda = k; p.ldb = n; p.ldc = n;
   p.b_group_stride = n * k; p.accumulate = 0; p.max_rows = (int)max_rows;
-  gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
   const bool big = cdiv(max_rows, 256) * cdiv(n, 256) >= 256;
-  if (big && k % 64 == 0 && n % 256 == 0 && k <= (1ll << 21) && k * n * (int64_t)dtype_size(dtype) < (1ll << 31))
+  if (big && k % 64 == 0 && n % 256 == 0 && k <= (1ll << 21) && k * n * (int64_t)dtype_size(dtype) < (1ll << 31)) {
     rc = dtype == DH_BF16 ? launch_gg_w4<bf16_t, true>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream)
                           : launch_gg_w4<f16_t, true>(p, max_rows, workspace, workspace_bytes, (hipStream_t)stream);
-  else
+  } else {
+    gg_zero_tail(c, offs, groups, max_rows, n, (hipStream_t)stream);
     rc = dispatch_gg<false, true, false>(p, max_rows, dtype, (hipStream_t)stream);
+  }
   if (rc) return rc;
   DH_LAUNCH_CHECK();
   return DH_OK;

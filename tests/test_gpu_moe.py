@@ -340,18 +340,21 @@ def test_expert_ffn_bwd_with_resident_weight_transposes():
     assert torch.equal(_Clib.transposed_of(w2), w2.transpose(1, 2).contiguous())
 
 
-@pytest.mark.parametrize("form,K,N", [("nt", 192, 4096), ("nt", 1024, 4096), ("nn", 192, 4096), ("nn", 1024, 4096),
-                                      ("nt", 320, 4232)])     # n ends inside a tile: 4232 = 16 * 256 + 136
-def test_grouped_gemm_split_last_round(form, K, N):
+@pytest.mark.parametrize("form,K,N,last", [("nt", 192, 4096, 500), ("nt", 1024, 4096, 500), ("nn", 192, 4096, 500),
+                                           ("nn", 1024, 4096, 500),
+                                           ("nt", 320, 4232, 500),    # n ends inside a tile: 4232 = 16 * 256 + 136
+                                           ("nt", 256, 4096, 10), ("nn", 256, 4096, 10)])   # groups end before max_rows
+def test_grouped_gemm_split_last_round(form, K, N, last):
     """The chip-filling kernels through the C ABI, with and without a workspace (last round split along k / one workgroup per tile):
     both within the bound of the fp64 product, the split result the same on every run, rows cut off at max_rows
-    (the offsets describe more rows than the operands hold), nothing written past them."""
+    (the offsets describe more rows than the operands hold), nothing written past them; rows between the last
+    group's end and max_rows come back as zeros (the output starts out as 3.0 everywhere)."""
     from dhellam_amd import _lib
     lib = _lib.load()
     dt = torch.bfloat16
-    rows = [2100, 0, 1990, 37, 500]
+    rows = [2100, 0, 1990, 37, last]
     G, R = len(rows), sum(rows)
-    max_rows, guard = 4200, 64                      # the last group is cut off: 73 of its 500 rows exist
+    max_rows, guard = 4200, 64                      # last = 500: the last group is cut off, 73 of its rows exist
     offs_np = np.concatenate(([5], 5 + np.cumsum(rows))).astype(np.int32)
     offs = torch.from_numpy(offs_np).cuda()
     a = randn((max_rows, K), dt, 11, std=0.5).cuda()

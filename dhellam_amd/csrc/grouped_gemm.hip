@@ -493,26 +493,28 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   };
   // read r of a k step, in the order in which the MFMAs first need the data: B0 A0 B1 B2 B3 A1 A2 A3 (a k-strided
   // B fragment is two transpose reads).  abase/bbase: lane addresses of the stage with the k step applied.
-  auto fread = [&](int set, int r, uint32_t stage, int ks, uint32_t kc_a, uint32_t kc_b) {
+  struct Bases { uint32_t kc_a, kc_b, ta_a, ta_b, tb_a, tb_b; };   // a stage's lane addresses, k-contiguous / k-strided reads
+  auto bases_of = [&](uint32_t stage) { return Bases{stage + fa_lane, stage + fb_lane, stage + ta_a, stage + ta_b, stage + tb_a, stage + tb_b}; };
+  auto fread = [&](int set, int r, int ks, const Bases &ba) {
     if constexpr (!BKS) {
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
-      if (!isb[r]) fa[set][blk[r]] = *(lds_frag)((kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
-      else fbr[set][blk[r]] = *(lds_frag)((kc_b ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      if (!isb[r]) fa[set][blk[r]] = *(lds_frag)((ba.kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      else fbr[set][blk[r]] = *(lds_frag)((ba.kc_b ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
     } else if constexpr (AKS) {
       // B0 A0 B1 B2 B3 A1 A2 A3, two transpose reads each
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
       const int f = r >> 1, half = r & 1;
-      const uint32_t lane_addr = isb[f] ? (half ? tb_b : tb_a) : (half ? ta_b : ta_a);
-      const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + lane_addr) ^ (uint32_t)(blk[f] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+      const uint32_t lane_addr = isb[f] ? (half ? ba.tb_b : ba.tb_a) : (half ? ba.ta_b : ba.ta_a);
+      const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((lane_addr ^ (uint32_t)(blk[f] << 6)) + (uint32_t)(ks * 16 * BROWB)));
       if (isb[f]) fbt[set][blk[f]][half] = x;
       else fat[set][blk[f]][half] = x;
     } else {
       constexpr int kind[12] = {1, 2, 0, 1, 2, 1, 2, 1, 2, 0, 0, 0}, blk[12] = {0, 0, 0, 1, 1, 2, 2, 3, 3, 1, 2, 3};
-      if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)((kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
+      if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)((ba.kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
       else if (kind[r] == 1)
-        fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + tb_a) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+        fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((ba.tb_a ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
       else
-        fbt[set][blk[r]][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((stage + tb_b) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+        fbt[set][blk[r]][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((ba.tb_b ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
     }
   };
 
@@ -535,8 +537,11 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
 #pragma unroll
   for (int x = 8; x < 15; ++x) gload(0, x, kof(2) * kstep_a, kof(2) * kstep_b);
   asm volatile("s_barrier" ::: "memory");
+  {
+    const Bases b0 = bases_of(lds0);
 #pragma unroll
-  for (int x = 0; x < NRD; ++x) fread(0, x, lds0, 0, lds0 + fa_lane, lds0 + fb_lane);
+    for (int x = 0; x < NRD; ++x) fread(0, x, 0, b0);
+  }
 
   // Slice s reads stage s % 2, writes slice s + 1 (staging set (s + 1) % 2, loaded two slices ago) into the other
   // stage during its first half and then loads slice s + 3 into the same set.
@@ -547,9 +552,11 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     uint32_t cur = lds0 + (uint32_t)(st * STAGEB), nxt = lds0 + (uint32_t)((st ^ 1) * STAGEB);
     const uint32_t ka = kof(s + 3) * kstep_a, kb = kof(s + 3) * kstep_b;
     asm volatile("" : "+s"(cur), "+s"(nxt));
-    uint32_t ac = cur + fa_lane, bc = cur + fb_lane, an = nxt + fa_lane, bn = nxt + fb_lane, wn_ = nxt + wr_kc;
-    if constexpr (!AKS) asm volatile("" : "+v"(ac), "+v"(an), "+v"(wn_));
-    if constexpr (!BKS) asm volatile("" : "+v"(bc), "+v"(bn));
+    Bases bc = bases_of(cur), bn = bases_of(nxt);
+    uint32_t wn_ = nxt + wr_kc;
+    if constexpr (!AKS) asm volatile("" : "+v"(bc.kc_a), "+v"(bn.kc_a), "+v"(wn_));
+    if constexpr (!BKS) asm volatile("" : "+v"(bc.kc_b), "+v"(bn.kc_b));
+    // (the k-strided operands' addresses are left to the compiler: pinned, they cost more additions than they save)
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mi = 0; mi < 64; ++mi) {
@@ -559,20 +566,20 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       else acc[i][j] = M::mma(fbr[ks & 1][j], fa[ks & 1][i], acc[i][j]);
       // fragment reads of the next k step, spread over the quarter (the last quarter: behind the barrier, from the next stage)
       if (ks < 3) {
-        if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, cur, ks + 1, ac, bc); }
-        else if (NRD == 12) { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, cur, ks + 1, ac, bc); }
-        else fread((ks + 1) & 1, q, cur, ks + 1, ac, bc);
+        if (NRD == 8) { if (q % 2 == 0) fread((ks + 1) & 1, q / 2, ks + 1, bc); }
+        else if (NRD == 12) { if (q % 4 != 3) fread((ks + 1) & 1, q - q / 4, ks + 1, bc); }
+        else fread((ks + 1) & 1, q, ks + 1, bc);
       } else if (!LAST) {
         if (mi == 50) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         if (NRD == 8) {
-          if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, nxt, 0, an, bn);
-          if (mi == 63) fread(0, 7, nxt, 0, an, bn);
+          if (mi >= 50 && mi % 2 == 0) fread(0, (mi - 50) / 2, 0, bn);
+          if (mi == 63) fread(0, 7, 0, bn);
         } else if (NRD == 12) {
-          if (mi >= 50 && mi < 62) fread(0, mi - 50, nxt, 0, an, bn);
+          if (mi >= 50 && mi < 62) fread(0, mi - 50, 0, bn);
         } else {
-          if (mi >= 50) fread(0, mi - 50, nxt, 0, an, bn);
-          if (mi == 50) fread(0, 14, nxt, 0, an, bn);
-          if (mi == 51) fread(0, 15, nxt, 0, an, bn);
+          if (mi >= 50) fread(0, mi - 50, 0, bn);
+          if (mi == 50) fread(0, 14, 0, bn);
+          if (mi == 51) fread(0, 15, 0, bn);
         }
       }
       if (!LAST && mi < 32 && mi % 2 == 1) {            // LDS writes of slice s + 1: the older of the two sets in flight

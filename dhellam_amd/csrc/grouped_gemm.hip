@@ -41,6 +41,13 @@ struct GGParams {
   int zero_tail;         // NT/NN on grouped_gemm_w4_kernel: the kernel itself zeroes the rows of c past the last group
 };
 
+// Workgroup ids go round the 8 XCDs; this gives XCD x (the ids x, x + 8, ...) the x-th of 8 contiguous chunks of
+// 0..n-1, so that neighbouring tiles share an L2 (a bijection for any n: the first n % 8 chunks are one longer).
+__device__ __forceinline__ int gg_xcd_chunk(int id, int n) {
+  const int q8 = n / 8, r8 = n % 8, x = id % 8;
+  return x * q8 + (x < r8 ? x : r8) + id / 8;
+}
+
 // A group's row range as the kernels use it: relative to the first group and never past the rows the caller's
 // buffers hold, whatever the offsets say (they live on the device, so the host cannot check them).
 __device__ __forceinline__ int gg_clamp_row(int r, int max_rows) { return r < 0 ? 0 : (r > max_rows ? max_rows : r); }
@@ -112,7 +119,7 @@ __global__ void __launch_bounds__(128 * WVN) grouped_gemm_kernel(const GGParams 
   // that share a weight panel are neighbours in one L2).
   const int ntiles = p.tiles_m * p.tiles_n;
   int pid = blockIdx.x;
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  pid = gg_xcd_chunk(pid, ntiles);
   int tm = pid % p.tiles_m;
   const int tn = pid / p.tiles_m;
 
@@ -365,13 +372,6 @@ __device__ __forceinline__ void gg_w4_store(const floatx16 (&acc)[4][4], unsigne
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
   }
-}
-
-// Workgroup ids go round the 8 XCDs; this gives XCD x (the ids x, x + 8, ...) the x-th of 8 contiguous chunks of
-// 0..n-1, so that neighbouring tiles share an L2 (a bijection for any n: the first n % 8 chunks are one longer).
-__device__ __forceinline__ int gg_xcd_chunk(int id, int n) {
-  const int q8 = n / 8, r8 = n % 8, x = id % 8;
-  return x * q8 + (x < r8 ? x : r8) + id / 8;
 }
 
 // k pieces per tile of the last round: as many as there are workgroups per tile, each at least one slice.

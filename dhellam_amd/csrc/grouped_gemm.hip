@@ -493,8 +493,9 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   };
   // read r of a k step, in the order in which the MFMAs first need the data: B0 A0 B1 B2 B3 A1 A2 A3 (a k-strided
   // B fragment is two transpose reads).  abase/bbase: lane addresses of the stage with the k step applied.
-  struct Bases { uint32_t kc_a, kc_b, ta_a, ta_b, tb_a, tb_b; };   // a stage's lane addresses, k-contiguous / k-strided reads
-  auto bases_of = [&](uint32_t stage) { return Bases{stage + fa_lane, stage + fb_lane, stage + ta_a, stage + ta_b, stage + tb_a, stage + tb_b}; };
+  // a stage's lane addresses for k-contiguous fragment reads, and its base for the k-strided ones
+  struct Bases { uint32_t kc_a, kc_b, stage; };
+  auto bases_of = [&](uint32_t stage) { return Bases{stage + fa_lane, stage + fb_lane, stage}; };
   auto fread = [&](int set, int r, int ks, const Bases &ba) {
     if constexpr (!BKS) {
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
@@ -504,17 +505,17 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       // B0 A0 B1 B2 B3 A1 A2 A3, two transpose reads each
       constexpr int isb[8] = {1, 0, 1, 1, 1, 0, 0, 0}, blk[8] = {0, 0, 1, 2, 3, 1, 2, 3};
       const int f = r >> 1, half = r & 1;
-      const uint32_t lane_addr = isb[f] ? (half ? ba.tb_b : ba.tb_a) : (half ? ba.ta_b : ba.ta_a);
-      const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((lane_addr ^ (uint32_t)(blk[f] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+      const uint32_t lane_addr = isb[f] ? (half ? tb_b : tb_a) : (half ? ta_b : ta_a);
+      const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((ba.stage + lane_addr) ^ (uint32_t)(blk[f] << 6)) + (uint32_t)(ks * 16 * BROWB)));
       if (isb[f]) fbt[set][blk[f]][half] = x;
       else fat[set][blk[f]][half] = x;
     } else {
       constexpr int kind[12] = {1, 2, 0, 1, 2, 1, 2, 1, 2, 0, 0, 0}, blk[12] = {0, 0, 0, 1, 1, 2, 2, 3, 3, 1, 2, 3};
       if (kind[r] == 0) fa[set][blk[r]] = *(lds_frag)((ba.kc_a ^ (uint32_t)(ks << 5)) + blk[r] * 4096);
       else if (kind[r] == 1)
-        fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((ba.tb_a ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+        fbt[set][blk[r]][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((ba.stage + tb_a) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
       else
-        fbt[set][blk[r]][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)((ba.tb_b ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
+        fbt[set][blk[r]][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr)(((ba.stage + tb_b) ^ (uint32_t)(blk[r] << 6)) + (uint32_t)(ks * 16 * BROWB)));
     }
   };
 

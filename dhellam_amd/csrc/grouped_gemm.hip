@@ -48,6 +48,15 @@ __device__ __forceinline__ int gg_xcd_chunk(int id, int n) {
   return x * q8 + (x < r8 ? x : r8) + id / 8;
 }
 
+// Tile t of the list -> (m tile, n tile): bands of 8 m tiles, m fastest inside a band, so that the 32 tiles an XCD has in
+// flight are 8 x 4 and share 12 operand panels through its L2 instead of 18 + 2 (1-2 % on the FFN products).
+__device__ __forceinline__ void gg_tile_of(int t, int tiles_m, int tiles_n, int &tm, int &tn) {
+  constexpr int GM = 8;
+  const int band = t / (GM * tiles_n), first = band * GM, gm = min(GM, tiles_m - first), in_band = t - band * GM * tiles_n;
+  tm = first + in_band % gm;
+  tn = in_band / gm;
+}
+
 // A group's row range as the kernels use it: relative to the first group and never past the rows the caller's
 // buffers hold, whatever the offsets say (they live on the device, so the host cannot check them).
 __device__ __forceinline__ int gg_clamp_row(int r, int max_rows) { return r < 0 ? 0 : (r > max_rows ? max_rows : r); }
@@ -648,12 +657,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     const int ntiles = tiles_m * p.tiles_n;
     if ((int)blockIdx.x >= ntiles) return;
     const int pid = gg_xcd_chunk((int)blockIdx.x, ntiles);
-    // Inside an XCD's run of tiles: bands of 8 m tiles, m fastest inside a band, so that the 32 tiles an XCD has
-    // in flight are 8 x 4 and share 12 operand panels through its L2 instead of 18 + 2 (1-2 % on the FFN products).
-    constexpr int GM = 8;
-    const int band = pid / (GM * p.tiles_n), first = band * GM, gm = min(GM, tiles_m - first);
-    int tm = first + (pid - band * GM * p.tiles_n) % gm;
-    const int tn = (pid - band * GM * p.tiles_n) / gm;
+    int tm, tn;
+    gg_tile_of(pid, tiles_m, p.tiles_n, tm, tn);
     for (int gi = 0; gi < p.groups; ++gi) {
       const int rb = gg_clamp_row(p.offs[gi] - base, p.max_rows), re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
       const int t = (re - rb + BM - 1) / BM;
@@ -664,7 +669,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
       tm -= t;
     }
   } else {
-    // One workgroup per compute unit.  The tiles (m fastest) are dealt out in rounds of gridDim.x: round j gives
+    // One workgroup per compute unit.  The tiles (in the order of gg_tile_of) are dealt out in rounds of gridDim.x: round j gives
     // workgroup w the tile j * gridDim.x + w, so that the tiles in flight are neighbours and share their operand
     // panels through L2.  When the last round holds at most half as many tiles as there are workgroups, its tiles
     // are split along k into as many pieces as fit (workgroup w: tile w % rem, piece w / rem, so that neighbours
@@ -690,8 +695,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
         s1 = (pc + 1) * nsl / pieces;
         if (pieces > 1) part = p.ws + (size_t)wg * (256 * 256);
       }
-      int tm = t % tiles_m;
-      const int tn = t / tiles_m;
+      int tm, tn;
+      gg_tile_of(t, tiles_m, p.tiles_n, tm, tn);
       int g = 0, rb = 0, re = 0;
       for (int gi = 0; gi < p.groups; ++gi) {
         rb = gg_clamp_row(p.offs[gi] - base, p.max_rows); re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);
@@ -732,8 +737,8 @@ __global__ void __launch_bounds__(256) gg_split_reduce_kernel(const GGParams p, 
 #pragma unroll
     for (int vb = 0; vb < 4; ++vb) acc[vb] += *reinterpret_cast<const floatx4 *>(src + vb * 256);
   }
-  int tm = t % tiles_m;
-  const int tn = t / tiles_m;
+  int tm, tn;
+  gg_tile_of(t, tiles_m, p.tiles_n, tm, tn);
   int rb = 0, re = 0;
   for (int gi = 0; gi < p.groups; ++gi) {
     rb = gg_clamp_row(p.offs[gi] - base, p.max_rows); re = gg_clamp_row(p.offs[gi + 1] - base, p.max_rows);

@@ -647,7 +647,9 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     pid = gg_xcd_chunk(pid, ntiles);
     const int g = blockIdx.y;
     const int rb = gg_clamp_row(p.offs[g] - base, p.max_rows), re = gg_clamp_row(p.offs[g + 1] - base, p.max_rows);
-    segment(g, rb, re, pid % p.tiles_m, pid / p.tiles_m, 0, (re - rb + 63) / 64, nullptr);
+    int tm, tn;
+    gg_tile_of(pid, p.tiles_m, p.tiles_n, tm, tn);
+    segment(g, rb, re, tm, tn, 0, (re - rb + 63) / 64, nullptr);
   } else if constexpr (!SK) {
     // The grid is sized for the host's upper bound of the tile count (it does not know how the rows split into
     // groups); the chunks of the XCDs are cut from the real count, so that every XCD gets its share of real tiles.

@@ -386,6 +386,32 @@ def test_grouped_gemm_split_last_round(form, K, N, last):
     assert torch.equal(c, outs[0])
 
 
+@pytest.mark.parametrize("form", ["nt", "nn"])
+def test_grouped_gemm_sixty_four_groups(form):
+    """The largest group count the kernels take (one group per lane of the workgroup's group table), on the
+    chip-filling kernels: groups of 0 to 130 rows, most of them one partial tile, a first offset that is not 0."""
+    from dhellam_amd.operators import moe
+    dt = torch.bfloat16
+    rng = np.random.default_rng(5)
+    rows = rng.integers(0, 131, size=64)
+    rows[7] = 0
+    rows[63] = 130
+    R, K, N = int(rows.sum()), 192, 4096
+    offs_np = np.concatenate(([11], 11 + np.cumsum(rows))).astype(np.int32)
+    offs = torch.from_numpy(offs_np).cuda()
+    a = randn((R, K), dt, 31, std=0.5).cuda()
+    b = randn((64, N, K), dt, 32, std=0.5).cuda()
+    ref = torch.zeros((R, N), dtype=torch.float64)
+    st = np.concatenate(([0], np.cumsum(rows)))
+    for g in range(64):
+        ref[st[g]:st[g + 1]] = a[st[g]:st[g + 1]].cpu().double() @ b[g].cpu().double().T
+    if form == "nt":
+        c = moe.grouped_gemm_nt(a, b, offs)
+    else:
+        c = moe.grouped_gemm_nn(a, b.transpose(1, 2).contiguous(), offs)
+    assert_close(c, ref, dt, f"64 groups, {form}")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_grouped_gemm_tn_chip_filling(dtype):
     """Weight-gradient products large enough for the 256x256-tile kernel (m, n multiples of 256, >= 256 tiles): an

@@ -591,6 +591,11 @@ static int launch_attn_fwd_d128(const AttnFwdParams &p, int batch, hipStream_t s
   return DH_OK;
 }
 
+// fewest workgroups of 128 query rows for which the 128-row kernel is taken
+#ifndef DH_FWD_128ROW_MIN_WG
+#define DH_FWD_128ROW_MIN_WG 256
+#endif
+
 template <typename T, int D, int NW>
 static int launch_attn_fwd(const AttnFwdParams &p, int batch, hipStream_t st) {
   constexpr int BM = 32 * NW, BN = 64;
@@ -645,7 +650,7 @@ extern "C" int dh_attn_fwd(const void *q, const void *k, const void *v, void *ou
   if (d == 128) {
     // 128-row query tiles when that still gives every CU a workgroup, else 64-row tiles.
     const int64_t wg128 = (causal ? (cdiv(max_seqlen_q, 128) + 1) / 2 : cdiv(max_seqlen_q, 128)) * hq * batch;
-    const bool big = wg128 >= 256;
+    const bool big = wg128 >= DH_FWD_128ROW_MIN_WG;
     if (dtype == DH_BF16) rc = big ? launch_attn_fwd_d128<bf16_t, 4, 2, 64, DH_FWD_LAG>(p, batch, st) : launch_attn_fwd_d128<bf16_t, 2, 4, 32, DH_FWD_LAG>(p, batch, st);
     else rc = big ? launch_attn_fwd_d128<f16_t, 4, 2, 64, DH_FWD_LAG>(p, batch, st) : launch_attn_fwd_d128<f16_t, 2, 4, 32, DH_FWD_LAG>(p, batch, st);
   } else {

@@ -111,7 +111,7 @@ def check_grouped_gemm_loops(verbose: bool = False) -> int:
     checked = 0
     starts = [i for i, l in enumerate(lines) if re.match(r"^_ZN2dh22grouped_gemm_w4_kernel\w+:", l)]
     for a in starts:
-        b = next(i for i in range(a, len(lines)) if "s_endpgm" in lines[i])
+        b = next(i for i in range(a, len(lines)) if lines[i].startswith(".Lfunc_end"))   # (a kernel may hold several s_endpgm)
         fn = lines[a:b]
         labels = {m.group(1): i for i, l in enumerate(fn) if (m := re.match(r"^(\.LBB\d+_\d+):", l))}
         loops = []

@@ -39,6 +39,7 @@ struct GGParams {
   int max_rows;          // rows the stacked operands hold: group ranges read from offs are cut off there
   float *ws;             // split last round: fp32 partial tiles, one per workgroup
   int zero_tail;         // NT/NN on grouped_gemm_w4_kernel: the kernel itself zeroes the rows of c past the last group
+  int sk_grid;           // > 0: a split kernel of that many workgroups follows and takes the last round of tiles if it splits it
 };
 
 // Workgroup ids go round the 8 XCDs; this gives XCD x (the ids x, x + 8, ...) the x-th of 8 contiguous chunks of
@@ -648,7 +649,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
   if (s < cnt) slice(I0{}, std::true_type{}, s);
   __syncthreads();                                      // everyone is done with the stages: they stage the output below
 
-  if (SK && part != nullptr) {
+  if constexpr (SK) {
     // 16 bytes per lane and instruction: piece ((w * 16 + i * 4 + j) * 4 + vb) of the tile, 1 KB each
     float *dst = part + ((size_t)w * 64 * 4 + 0) * 64 + (size_t)lane * 4;
 #pragma unroll
@@ -684,43 +685,38 @@ __global__ void __launch_bounds__(256) grouped_gemm_w4_kernel(const GGParams p) 
     int tiles_m;
     const GGGroupTable gt = gg_group_table(p, base, tiles_m);
     const int ntiles = tiles_m * p.tiles_n;
-    if ((int)blockIdx.x >= ntiles) return;
-    const int pid = gg_xcd_chunk((int)blockIdx.x, ntiles);
+    int kept = ntiles;
+    if (p.sk_grid > 0) {
+      // the tiles past the last full round of sk_grid tiles belong to the split kernel, if it splits them
+      const int full = ntiles / p.sk_grid, rem = ntiles - full * p.sk_grid;
+      if (gg_sk_pieces(p.sk_grid, rem, nsl) > 1) kept = full * p.sk_grid;
+    }
+    if ((int)blockIdx.x >= kept) return;
+    const int pid = gg_xcd_chunk((int)blockIdx.x, kept);              // (the XCDs share the tiles that are computed here)
     int tm_all, tn, g, rb, re, tm;
     gg_tile_of(pid, tiles_m, p.tiles_n, tm_all, tn);
     gg_locate(gt, tm_all, g, rb, re, tm);
     segment(g, rb, re, tm, tn, 0, nsl, nullptr);
   } else {
-    // One workgroup per compute unit.  The tiles (in the order of gg_tile_of) are dealt out in rounds of gridDim.x: round j gives
-    // workgroup w the tile j * gridDim.x + w, so that the tiles in flight are neighbours and share their operand
-    // panels through L2.  When the last round holds at most half as many tiles as there are workgroups, its tiles
-    // are split along k into as many pieces as fit (workgroup w: tile w % rem, piece w / rem, so that neighbours
-    // still work on neighbouring tiles); the pieces are summed afterwards, in k order.  288 tiles on 256 compute
-    // units then take 1 1/8 tile times instead of 2.
+    // The last round of tiles, split along k.  The tiles (in the order of gg_tile_of) run in rounds of gridDim.x = the
+    // number of compute units; grouped_gemm_w4_kernel<.., false> in front of this kernel takes the full rounds, one
+    // workgroup per tile.  When the last round holds at most half as many tiles as there are workgroups, it is left to
+    // this kernel: as many k pieces per tile as fit (workgroup w: tile w % rem, piece w / rem, so that neighbours work
+    // on neighbouring tiles), summed afterwards in k order.  288 tiles on 256 compute units then take 1 1/8 tile
+    // times instead of 2.  (A resident workgroup that also looped over the full rounds was 3-6 % slower on them than
+    // one workgroup per tile.)
     int tiles_m;
     const GGGroupTable gt = gg_group_table(p, base, tiles_m);
     const int tiles = tiles_m * p.tiles_n;
     const int grid = (int)gridDim.x, full = tiles / grid, rem = tiles - full * grid;
     const int pieces = gg_sk_pieces(grid, rem, nsl);
-    int wg = blockIdx.x;
-    wg = gg_xcd_chunk(wg, grid);                                       // neighbouring tiles on one XCD
-    const int rounds = full + (wg < rem * pieces ? 1 : 0);
-#pragma unroll 1
-    for (int it = 0; it < rounds; ++it) {
-      int t = it * grid + wg, s0 = 0, s1 = nsl;
-      float *part = nullptr;
-      if (it == full) {                                                 // the last round
-        const int ts = wg % rem, pc = wg / rem;
-        t = full * grid + ts;
-        s0 = pc * nsl / pieces;
-        s1 = (pc + 1) * nsl / pieces;
-        if (pieces > 1) part = p.ws + (size_t)wg * (256 * 256);
-      }
-      int tm_all, tn, g, rb, re, tm;
-      gg_tile_of(t, tiles_m, p.tiles_n, tm_all, tn);
-      gg_locate(gt, tm_all, g, rb, re, tm);
-      segment(g, rb, re, tm, tn, s0, s1, part);
-    }
+    const int wg = gg_xcd_chunk((int)blockIdx.x, grid);                // neighbouring tiles on one XCD
+    if (pieces == 1 || wg >= rem * pieces) return;
+    const int ts = wg % rem, pc = wg / rem;
+    int tm_all, tn, g, rb, re, tm;
+    gg_tile_of(full * grid + ts, tiles_m, p.tiles_n, tm_all, tn);
+    gg_locate(gt, tm_all, g, rb, re, tm);
+    segment(g, rb, re, tm, tn, pc * nsl / pieces, (pc + 1) * nsl / pieces, p.ws + (size_t)wg * (256 * 256));
   }
 }
 
@@ -803,17 +799,16 @@ static int launch_gg_w4(GGParams p, int64_t m_extent, void *workspace, size_t wo
     grid = cus < GG_SK_MAX_GRID ? cus : GG_SK_MAX_GRID;
     if (workspace_bytes < (size_t)grid * 256 * 256 * sizeof(float)) grid = 0;
   }
-  // One workgroup per compute unit costs a few percent against one workgroup per tile (its tile loop is not
-  // overlapped with anything); it pays where the split of the last round can save half a tile time or more of a
-  // short job: at most one and a half rounds of tiles (the host knows the tile count only up to the groups'
-  // partial tiles, so it cannot tell how full the last round of a longer job is).
-  if (grid > 0 && 2 * (int64_t)p.tiles_m * p.tiles_n > 3 * (int64_t)grid) grid = 0;
+  // With a workspace the last round of tiles may be split along k (decided on the device, where the tile count is
+  // known): the first kernel then leaves that round to the split kernel.  When nothing is split the two extra
+  // launches cost a few microseconds; a split saves up to half a tile time (45 us and more).
+  p.sk_grid = grid;
+  hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS ? 1 : 0, false>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
   if (grid > 0) {
     p.ws = reinterpret_cast<float *>(workspace);
+    p.zero_tail = 0;                                    // done by the kernel above
     hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS ? 1 : 0, true>), dim3((unsigned)grid), dim3(256), 0, st, p);
     hipLaunchKernelGGL((gg_split_reduce_kernel<T>), dim3((unsigned)(16 * grid / 2)), dim3(256), 0, st, p, grid);   // at most grid / 2 tiles are split
-  } else {
-    hipLaunchKernelGGL((grouped_gemm_w4_kernel<T, BKS ? 1 : 0, false>), dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(256), 0, st, p);
   }
   return DH_OK;
 }

@@ -318,10 +318,11 @@ int dh_moe_gate_grad(const void *dout, const void *y, const int32_t *dest_row,
  * from offs are cut off there (no row past it is read or written), and NT / NN zero the rows of c from the
  * last group's end up to max_rows, so c may be uninitialised on entry.
  * workspace (NT, NN; may be NULL): device memory of at least dh_grouped_gemm_workspace_bytes() bytes.  With it,
- * products that fill the chip run one workgroup per compute unit: whole tiles are dealt out in rounds, and when the
- * last round holds at most half as many tiles as there are compute units its tiles are split along k into as many
- * pieces as fit, whose fp32 sums go through the workspace and are added in k order by a second kernel
- * (deterministic).  288 tiles on 256 compute units then cost 1 1/8 tile times instead of 2.  Without a workspace a
+ * a product that fills the chip may have its last round of tiles split along k: the tiles run in rounds of one
+ * per compute unit, and when the last round holds at most half as many tiles as there are compute units a second
+ * kernel computes them in as many k pieces as fit, whose fp32 sums go through the workspace and are added in k order
+ * by a third kernel (deterministic).  288 tiles on 256 compute units then cost 1 1/8 tile times instead of 2; when
+ * nothing is split the two extra launches find nothing to do.  Without a workspace a
  * tile is one workgroup and the last round is as full as it happens to be.  The contents of the workspace do not
  * matter on entry; calls that overlap on one device need workspaces of their own.
  * ---------------------------------------------------------------------- */

@@ -343,7 +343,8 @@ def test_expert_ffn_bwd_with_resident_weight_transposes():
 @pytest.mark.parametrize("form,K,N,last", [("nt", 192, 4096, 500), ("nt", 1024, 4096, 500), ("nn", 192, 4096, 500),
                                            ("nn", 1024, 4096, 500),
                                            ("nt", 320, 4232, 500),    # n ends inside a tile: 4232 = 16 * 256 + 136
-                                           ("nt", 256, 4096, 10), ("nn", 256, 4096, 10)])   # groups end before max_rows
+                                           ("nt", 256, 4096, 10), ("nn", 256, 4096, 10),    # groups end before max_rows
+                                           ("nt", 192, 8192, 500), ("nn", 320, 8192, 500)]) # two full rounds, then a split one
 def test_grouped_gemm_split_last_round(form, K, N, last):
     """The chip-filling kernels through the C ABI, with and without a workspace (last round split along k / one workgroup per tile):
     both within the bound of the fp64 product, the split result the same on every run, rows cut off at max_rows

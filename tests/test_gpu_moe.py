@@ -413,13 +413,14 @@ def test_grouped_gemm_sixty_four_groups(form):
     assert_close(c, ref, dt, f"64 groups, {form}")
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_grouped_gemm_tn_chip_filling(dtype):
+@pytest.mark.parametrize("dtype,M,N", [(torch.bfloat16, 4096, 2048), (torch.float16, 4096, 2048),
+                                       (torch.bfloat16, 2304, 7424)])    # 9 x 29 tiles: a last band of one m tile, odd counts
+def test_grouped_gemm_tn_chip_filling(dtype, M, N):
     """Weight-gradient products large enough for the 256x256-tile kernel (m, n multiples of 256, >= 256 tiles): an
     empty group (its output must be zeros), groups of 1, 65 and 300 rows (k not a multiple of the 64-deep slice),
     rows of the operands past the last group (not read), accumulation into an existing output, same result twice."""
     from dhellam_amd.operators import moe
-    rows, M, N = [300, 0, 65, 1], 4096, 2048
+    rows = [300, 0, 65, 1]
     G, R = len(rows), sum(rows)
     offs = torch.tensor(np.concatenate(([3], 3 + np.cumsum(rows))), dtype=torch.int32).cuda()
     a = randn((R + 7, M), dtype, 21, std=0.5).cuda()
